@@ -1,0 +1,320 @@
+"""Pins the CPU oracle: reference golden vectors, known-answer cases, and what the
+mathematics fixes (brute force, numpy int64 products, float64 closed forms)."""
+import numpy as np
+import pytest
+
+import oracle as O
+
+
+# ----------------------------------------------------------------- quantize
+def test_quantize_fold_golden_vectors(golden):
+    """disc-fold-quantize.mlir: the folder's double arithmetic, every dtype."""
+    for case in golden["quantize_fold"]:
+        x = np.array(case["x"], np.float32)
+        got = O.quantize(x, case["scale"], case["zp"], axis=case["axis"],
+                         qmin=case["qmin"], qmax=case["qmax"],
+                         round_mode=case["round_mode"],
+                         dtype=np.dtype(case["dtype"]), fold=True)
+        np.testing.assert_array_equal(got, np.array(case["expect"], case["dtype"]),
+                                      err_msg=case["src"])
+
+
+def test_quantize_runtime_f32_matches_golden_for_8_and_16_bit(golden):
+    """The runtime decomposition (f32 divide/add/round/clamp) must give the same
+    vectors wherever qmin/qmax are exactly representable in f32."""
+    for case in golden["quantize_fold"]:
+        if case["dtype"] in ("int32", "uint32"):
+            continue
+        x = np.array(case["x"], np.float32)
+        got = O.quantize(x, case["scale"], case["zp"], axis=case["axis"],
+                         qmin=case["qmin"], qmax=case["qmax"],
+                         round_mode=case["round_mode"],
+                         dtype=np.dtype(case["dtype"]), fold=False)
+        np.testing.assert_array_equal(got, np.array(case["expect"], case["dtype"]),
+                                      err_msg=case["src"])
+
+
+def test_quantize_edge_values(golden):
+    """quantize_v2.cc edge vector: 1.25/1.75 exercise rounding, -255/500 saturation."""
+    x = np.array(golden["quantize_v2_edge_values"]["x"], np.float32)
+    got = O.quantize(x, 1.0, 0)
+    np.testing.assert_array_equal(got, [-128, 0, 1, 1, 2, 64, 127, 127])
+    got = O.quantize(x, 0.5, 0, round_mode=O.ROUND_HALF_AWAY_FROM_ZERO)
+    # x/0.5 = -510, 0, 2, 2.5, 3.5, 128, 254, 1000 -> away-from-zero: 3, 4
+    np.testing.assert_array_equal(got, [-128, 0, 2, 3, 4, 127, 127, 127])
+    got = O.quantize(x, 0.5, 0, round_mode=O.ROUND_HALF_TO_EVEN)
+    np.testing.assert_array_equal(got, [-128, 0, 2, 2, 4, 127, 127, 127])
+
+
+def test_quantize_is_true_division_not_reciprocal():
+    """x/scale and x*(1/scale) differ at ties; the reference divides."""
+    rng = np.random.default_rng(0)
+    scale = np.float32(0.0473)
+    # construct x = (k+0.5)*scale rounded to f32: a near-tie for every k
+    k = np.arange(-120, 120, dtype=np.float32)
+    x = ((k + np.float32(0.5)) * scale).astype(np.float32)
+    got = O.quantize(x, scale, 0)
+    want = np.clip(np.rint((x / scale).astype(np.float32)), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(got, want)
+    recip = np.clip(np.rint(x * (np.float32(1) / scale)), -128, 127).astype(np.int8)
+    assert (recip != want).any(), "probe vector no longer separates the two"
+    del rng
+
+
+@pytest.mark.parametrize("axis", [None, 0, 1, 2])
+def test_quantize_per_channel_vs_numpy(axis):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((5, 7, 6)).astype(np.float32) * 3
+    n = 1 if axis is None else x.shape[axis]
+    scale = rng.uniform(0.01, 0.1, n).astype(np.float32)
+    zp = rng.integers(-5, 5, n).astype(np.int32)
+    shape = [1, 1, 1]
+    if axis is not None:
+        shape[axis] = n
+    s = scale.reshape(shape)
+    z = zp.reshape(shape).astype(np.float32)
+    want = np.clip(np.rint((x / s).astype(np.float32) + z), -128, 127).astype(np.int8)
+    got = O.quantize(x, scale, zp, axis=axis)
+    np.testing.assert_array_equal(got, want)
+    # dequantize: (q - zp) * scale with an integer subtract
+    dq = O.dequantize(got, scale, zp, axis=axis)
+    want_dq = ((got.astype(np.int32) - zp.reshape(shape)).astype(np.float32) * s)
+    np.testing.assert_array_equal(dq, want_dq.astype(np.float32))
+
+
+def test_dequantize_uint8():
+    q = np.array([[0, 10, 255]], np.uint8)
+    got = O.dequantize(q, 0.5, 10)
+    np.testing.assert_array_equal(got, [[-5.0, 0.0, 122.5]])
+
+
+# -------------------------------------------------------------------- qgemm
+@pytest.mark.parametrize("tp_a,tp_b", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_s32_vs_int64(tp_a, tp_b):
+    rng = np.random.default_rng(7)
+    m, k, n = 9, 37, 11
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    zx, zw = 3, -2
+    want = (a.astype(np.int64) - zx) @ (w.astype(np.int64) - zw)
+    got = O.gemm_s32(a.T.copy() if tp_a else a, w.T.copy() if tp_b else w,
+                     tp_a=tp_a, tp_b=tp_b, zx=zx, zw=zw)
+    np.testing.assert_array_equal(got, want.astype(np.int32))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (4, 4, 64), (5, 7, 63), (13, 9, 200),
+                                   (8, 12, 768), (3, 5, 65)])
+def test_gemm_fast_equals_plain(m, n, k):
+    rng = np.random.default_rng(m * 1000 + n * 10 + k)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    want = a.astype(np.int64) @ w.astype(np.int64).T
+    got, threads = O.gemm_s32_fast(a, w)
+    assert threads >= 1
+    np.testing.assert_array_equal(got, want.astype(np.int32))
+
+
+def test_gemm_fast_extreme_values():
+    """-128 * -128 * K must not overflow the a+128 trick."""
+    k = 4096
+    a = np.full((4, k), -128, np.int8)
+    w = np.full((4, k), -128, np.int8)
+    got, _ = O.gemm_s32_fast(a, w)
+    assert (got == 128 * 128 * k).all()
+    a[:] = 127
+    got, _ = O.gemm_s32_fast(a, w)
+    assert (got == -127 * 128 * k).all()
+
+
+def test_gemm_mismatched_contraction_dim():
+    with pytest.raises(ValueError):
+        O.gemm_s32(np.zeros((2, 3), np.int8), np.zeros((4, 5), np.int8))
+
+
+def test_qgemm_known_answers(golden):
+    """quantized_matmul.cc: 4x25x71 -> 12.0; GPU per-tensor 32x64x128 -> 128.0."""
+    for case in golden["qgemm"]:
+        m, k, n = case["m"], case["k"], case["n"]
+        x = np.full((m, k), case["x"], np.float32)
+        w = np.full((k, n), case["w"], np.float32)
+        sw = np.full(n if case["per_channel"] else 1, case["sw"], np.float32)
+        qx = O.quantize(x, case["sx"], 0)
+        qw = O.quantize(w, sw, np.zeros_like(sw, np.int32),
+                        axis=1 if case["per_channel"] else None)
+        assert (qx == case["qx"]).all() and (qw == case["qw"]).all()
+        acc = O.gemm_s32(qx, qw)
+        assert (acc == case["acc"]).all()
+        for out in (O.requant_cpu(acc, case["sx"], sw, case["so"]),
+                    O.requant_gpu(acc, case["sx"], sw[:1], case["so"])):
+            assert (out == case["q_out"]).all()
+            f = O.dequantize(out, case["so"], 0)
+            assert (f == case["expect_f32"]).all(), case["src"]
+
+
+def test_requant_cpu_closed_form_and_order():
+    """E1 = (acc + b32) * os: distinguishes the order from acc*os + b32*os and from
+    acc*os + b32 on constructed values; checked against exact rational arithmetic."""
+    from fractions import Fraction
+    rng = np.random.default_rng(11)
+    m, n = 64, 48
+    acc = rng.integers(-300000, 300000, (m, n)).astype(np.int32)
+    b32 = rng.integers(-50000, 50000, n).astype(np.int32)
+    sx = np.float32(0.021)
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    so = np.float32(0.37)
+    got = O.requant_cpu(acc, sx, sw, so, b32=b32)
+    os_ = ((sx * sw).astype(np.float32) / so).astype(np.float32)
+    # the sum acc+b32 is exact in f32 only below 2^24: emulate f32 rounding
+    s = (acc.astype(np.float32) + b32.astype(np.float32)).astype(np.float32)
+    d = (s * os_[None, :]).astype(np.float32)
+    want = np.clip(np.rint(d), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(got, want)
+    # and the f32 pipeline stays within half an LSB + 2^-10 of the exact value
+    for i in range(0, m, 9):
+        for j in range(0, n, 7):
+            exact = (Fraction(int(acc[i, j])) + int(b32[j])) * Fraction(float(os_[j]))
+            if -128 < exact < 127:
+                assert abs(Fraction(int(got[i, j])) - exact) <= Fraction(1, 2) + Fraction(1, 1024)
+
+
+def test_requant_cpu_output_zero_point_and_saturation():
+    acc = np.array([[0, 1000, -1000, 10**9, -10**9]], np.int32)
+    out = O.requant_cpu(acc, 1.0, np.float32(0.1), 1.0, zo=5)
+    np.testing.assert_array_equal(out, [[5, 105, -95, 127, -128]])
+
+
+def test_requant_ties_round_half_to_even():
+    # os = 0.5 exactly: acc odd -> x.5 ties
+    acc = np.array([[1, 3, 5, -1, -3, -5, 7]], np.int32)
+    out = O.requant_cpu(acc, 1.0, np.float32(0.5), 1.0)
+    np.testing.assert_array_equal(out, [[0, 2, 2, 0, -2, -2, 4]])
+    out = O.requant_gpu(acc, 1.0, np.float32(0.5), 1.0)
+    np.testing.assert_array_equal(out, [[0, 2, 2, 0, -2, -2, 4]])
+
+
+def test_bias_f32_to_s32():
+    sx = np.float32(0.02)
+    sw = np.array([0.01, 0.05, 0.001], np.float32)
+    bias = np.array([0.5, -0.25, 1e9], np.float32)
+    got = O.bias_f32_to_s32(bias, sx, sw)
+    bs = np.float32(1.0) / (sx * sw).astype(np.float32)
+    want = np.rint((bias * bs).astype(np.float32).astype(np.float64))
+    want = np.clip(want, -2**31, 2147483520).astype(np.int64)
+    np.testing.assert_array_equal(got.astype(np.int64), want)
+    assert got[2] == 2147483520  # saturates at the largest float below 2^31
+
+
+def test_requant_gpu_per_channel_and_bias():
+    rng = np.random.default_rng(5)
+    m, n = 17, 23
+    acc = rng.integers(-200000, 200000, (m, n)).astype(np.int32)
+    sx = rng.uniform(0.01, 0.03, n).astype(np.float32)
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    so = rng.uniform(0.2, 0.5, n).astype(np.float32)
+    bi8 = rng.integers(-128, 128, n).astype(np.int8)
+    alpha = ((sx * sw).astype(np.float32) / so).astype(np.float32)
+    d = (alpha[None, :] * acc.astype(np.float32)).astype(np.float32)
+    d = (d + bi8.astype(np.float32)[None, :]).astype(np.float32)
+    want = np.clip(np.rint(d), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(O.requant_gpu(acc, sx, sw, so, bias_i8=bi8), want)
+    bf = rng.standard_normal(n).astype(np.float32) * 10
+    d = (alpha[None, :] * acc.astype(np.float32)).astype(np.float32)
+    d = (d + bf[None, :]).astype(np.float32)
+    want = np.clip(np.rint(d), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(O.requant_gpu(acc, sx, sw, so, bias_f32=bf), want)
+
+
+def test_dequant_acc_within_1e5_of_float64():
+    rng = np.random.default_rng(9)
+    acc = rng.integers(-10**6, 10**6, (8, 16)).astype(np.int32)
+    sw = rng.uniform(0.001, 0.05, 16).astype(np.float32)
+    bias = rng.standard_normal(16).astype(np.float32)
+    got = O.dequant_acc(acc, 0.02, sw, bias)
+    want = acc.astype(np.float64) * (np.float64(np.float32(0.02)) * sw.astype(np.float64)) + bias
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+
+
+# --------------------------------------------------------------------- conv
+def _hwio_to_ohwi(w):
+    return np.ascontiguousarray(np.transpose(w, (3, 0, 1, 2)))
+
+
+def test_conv_known_answers(golden):
+    for case in golden["qconv"]:
+        fmt = case["data_format"]
+        x = np.full(case["in_shape"], case["x"], np.float32)
+        w = np.full(case["w_hwio"], case["w"], np.float32)
+        co = w.shape[3]
+        sw = np.full(co, case["sw"], np.float32)
+        qx = O.quantize(x, case["sx"], 0)
+        qw = _hwio_to_ohwi(O.quantize(w, sw, np.zeros(co, np.int32), axis=3))
+        pad, md, out_shape = O.conv_attrs(qx.shape, qw.shape, fmt, case["strides"],
+                                          case["dilations"], case["padding"])
+        assert out_shape == case["out_shape"], case["src"]
+        acc = O.conv_s32(qx, qw, pad, md, out_shape)
+        ch_axis = fmt.index("C")
+        acc2 = np.moveaxis(acc, ch_axis, -1).reshape(-1, co)
+        q = O.requant_cpu(acc2, case["sx"], sw, case["so"])
+        f = O.dequantize(q, case["so"], 0)
+        if case["padding"] == "VALID" or case["w_hwio"][0] == 1 or case["x"] == 0.0:
+            assert (f == case["expect_f32"]).all(), case["src"]
+
+
+def test_conv_layout_probe(golden):
+    c = golden["qconv_layout_probe"]
+    x = np.array(c["x"], np.float32).reshape(c["in_shape"])
+    w = np.array(c["w_hwio"], np.float32).reshape(c["w_hwio_shape"])
+    qx = O.quantize(x, c["sx"], 0)
+    qw = _hwio_to_ohwi(O.quantize(w, [c["sw"]], [0], axis=3))
+    pad, md, out_shape = O.conv_attrs(qx.shape, qw.shape, "NHWC", c["strides"],
+                                      c["dilations"], c["padding"])
+    assert out_shape == c["out_shape"]
+    acc = O.conv_s32(qx, qw, pad, md, out_shape)
+    assert (acc == 0).all()
+
+
+def test_conv_metadata_matches_lowering_test():
+    """disc-lower-to-library-call.mlir:472-475 expects, for NHWC x OHWI,
+    {0,3,1,2, 3,0,1,2, 0,3,1,2, strides, dilations, const}."""
+    pad, md, out = O.conv_attrs([2, 8, 8, 16], [4, 3, 3, 16], "NHWC", [1, 2, 2, 1],
+                                [1, 1, 1, 1], "SAME", weight_is_const=True)
+    assert md == [0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2, 2, 2, 1, 1, 1]
+    assert pad == [0, 1, 0, 1] and out == [2, 4, 4, 4]
+    pad, md, out = O.conv_attrs([2, 16, 8, 8], [4, 3, 3, 16], "NCHW", [1], [1],
+                                "EXPLICIT", explicit_paddings=[1, 1, 2, 2])
+    assert md[:4] == [0, 1, 2, 3] and pad == [1, 1, 2, 2] and out == [2, 4, 8, 10]
+
+
+@pytest.mark.parametrize("stride,dil,pad", [(1, 1, 1), (2, 1, 0), (1, 2, 2), (2, 2, 1)])
+def test_conv_equals_im2col_gemm(stride, dil, pad):
+    """Textbook identity: conv = im2col + matmul (independent numpy im2col)."""
+    rng = np.random.default_rng(stride * 100 + dil * 10 + pad)
+    nb, h, w_, ci, co, kh, kw = 2, 9, 7, 5, 6, 3, 3
+    x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+    wt = rng.integers(-128, 128, (co, kh, kw, ci), dtype=np.int8)
+    ho = (h + 2 * pad - dil * (kh - 1) - 1) // stride + 1
+    wo = (w_ + 2 * pad - dil * (kw - 1) - 1) // stride + 1
+    md = list(O.NHWC_OHWI_METADATA) + [stride, stride, dil, dil, 1]
+    got = O.conv_s32(x, wt, [pad, pad, pad, pad], md, [nb, ho, wo, co])
+    xp = np.zeros((nb, h + 2 * pad, w_ + 2 * pad, ci), np.int64)
+    xp[:, pad:pad + h, pad:pad + w_, :] = x
+    cols = np.zeros((nb, ho, wo, kh, kw, ci), np.int64)
+    for r in range(kh):
+        for q in range(kw):
+            cols[:, :, :, r, q, :] = xp[:, r * dil:r * dil + stride * ho:stride,
+                                        q * dil:q * dil + stride * wo:stride, :]
+    want = cols.reshape(-1, kh * kw * ci) @ wt.reshape(co, -1).astype(np.int64).T
+    np.testing.assert_array_equal(got.reshape(-1, co), want.astype(np.int32))
+
+
+def test_conv_nchw_oihw_layout_via_metadata():
+    rng = np.random.default_rng(21)
+    x = rng.integers(-128, 128, (2, 6, 6, 4), dtype=np.int8)        # NHWC
+    wt = rng.integers(-128, 128, (3, 3, 3, 4), dtype=np.int8)       # OHWI
+    md_nhwc = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    ref = O.conv_s32(x, wt, [1, 1, 1, 1], md_nhwc, [2, 6, 6, 3])
+    x2 = np.ascontiguousarray(x.transpose(0, 3, 1, 2))              # NCHW
+    w2 = np.ascontiguousarray(wt.transpose(0, 3, 1, 2))             # OIHW
+    md = [0, 1, 2, 3, 1, 0, 2, 3, 0, 1, 2, 3, 1, 1, 1, 1, 1]
+    got = O.conv_s32(x2, w2, [1, 1, 1, 1], md, [2, 3, 6, 6])
+    np.testing.assert_array_equal(got.transpose(0, 2, 3, 1), ref)
