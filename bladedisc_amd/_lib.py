@@ -1,0 +1,61 @@
+"""Loads libdisc_q8_ral.so (the HIP kernels + RAL runtime) through ctypes.
+
+There is no fallback: if the library has not been built, loading raises.
+"""
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libdisc_q8_ral.so")
+
+_lib = None
+
+_I64, _I32, _INT, _VP, _SZ = C.c_int64, C.c_int32, C.c_int, C.c_void_p, C.c_size_t
+
+# name -> (restype, argtypes); mirrors include/disc_q8.h
+_PROTOS = {
+    "dq8_last_error": (C.c_char_p, []),
+    "dq8_version": (_INT, []),
+    "dq8_device_info": (_INT, [C.POINTER(_INT)] * 3),
+    "dq8_quantize": (_INT, [_VP, _VP, _INT, _I64, _I64, _I64, _VP, _VP, _I64, _I32,
+                            _I32, _INT, _VP]),
+    "dq8_dequantize": (_INT, [_VP, _INT, _VP, _I64, _I64, _I64, _VP, _VP, _I64, _VP]),
+    "dq8_qgemm_workspace_bytes": (_SZ, [_I64, _I64, _I64, _INT, _INT]),
+    "dq8_qgemm": (_INT, [_VP, _I64, _VP, _I64, _VP, _I64, _I64, _I64, _I64, _INT, _INT,
+                         _INT, _VP, _INT, _VP, _I64, _VP, _I64, _VP, _I64, _I32, _I32,
+                         _I32, _VP, _SZ, _VP]),
+    "dq8_qgemm_variant": (_INT, [_INT, _VP, _I64, _VP, _I64, _VP, _I64, _I64, _I64, _I64,
+                                 _INT, _INT, _INT, _VP, _INT, _VP, _I64, _VP, _I64, _VP,
+                                 _I64, _I32, _I32, _I32, _VP, _SZ, _VP]),
+    "dq8_qgemm_num_variants": (_INT, []),
+    "dq8_qgemm_variant_name": (C.c_char_p, [_INT]),
+    "dq8_qconv2d": (_INT, [_VP, C.POINTER(_I64), _VP, C.POINTER(_I64), C.POINTER(_I32),
+                           C.POINTER(_I32), _VP, C.POINTER(_I64), _INT, _VP, _INT, _VP,
+                           _VP, _I64, _VP, _I32, _VP]),
+    "dq8_qconv2d_variant": (_INT, [_INT, _VP, C.POINTER(_I64), _VP, C.POINTER(_I64),
+                                   C.POINTER(_I32), C.POINTER(_I32), _VP,
+                                   C.POINTER(_I64), _INT, _VP, _INT, _VP, _VP, _I64,
+                                   _VP, _I32, _VP]),
+    "dq8_mfma_probe": (_INT, [_VP] * 7),
+}
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -m bladedisc_amd.build` "
+                "(there is no CPU fallback)" % LIB_PATH)
+        _lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+        for name, (res, args) in _PROTOS.items():
+            fn = getattr(_lib, name)
+            fn.restype = res
+            fn.argtypes = args
+    return _lib
+
+
+def check(status, what):
+    if status != 0:
+        msg = lib().dq8_last_error().decode()
+        raise RuntimeError("%s failed: %s" % (what, msg))

@@ -1,0 +1,88 @@
+"""Builds libdisc_q8_ral.so: the gfx950 kernels, their C ABI and the RAL runtime.
+
+Everything is compiled in-tree with hipcc for gfx950 only (hipcc cross-compiles
+without a GPU).  Usage: ``python -m bladedisc_amd.build [--force]``.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+OBJ = os.path.join(PKG, "build")
+LIB = os.path.join(PKG, "libdisc_q8_ral.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -ffp-contract=off: the requantisation epilogue and quantize are defined as
+#   separately rounded binary32 operations.
+# packed-fp32-ops disabled: never let the compiler form v_pk_*_f32.
+COMMON = [
+    "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
+    "-Wall", "-Wno-unused-function",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+    "-I" + os.path.join(CSRC, "kernels"),
+]
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+          "-packed-fp32-ops"]
+
+
+def sources():
+    out = []
+    for d, _, files in os.walk(CSRC):
+        for f in sorted(files):
+            if f.endswith((".hip", ".cc")):
+                out.append(os.path.join(d, f))
+    return sorted(out)
+
+
+def _headers_mtime():
+    m = 0.0
+    for base in (CSRC, os.path.join(ROOT, "include")):
+        for d, _, files in os.walk(base):
+            for f in files:
+                if f.endswith(".h"):
+                    m = max(m, os.path.getmtime(os.path.join(d, f)))
+    return m
+
+
+def _compile(src, force, hdr_m):
+    rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
+    obj = os.path.join(OBJ, rel + ".o")
+    if (not force and os.path.exists(obj)
+            and os.path.getmtime(obj) > max(os.path.getmtime(src), hdr_m)):
+        return obj, ""
+    cmd = [HIPCC] + COMMON + DEVICE + ["-x", "hip", "-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    log = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
+                    if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    return obj, log
+
+
+def build(force=False, verbose=False, jobs=8):
+    os.makedirs(OBJ, exist_ok=True)
+    srcs = sources()
+    hdr_m = _headers_mtime()
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(lambda s: _compile(s, force, hdr_m), srcs))
+    objs = [o for o, _ in results]
+    if verbose:
+        for _, log in results:
+            if log.strip():
+                print(log)
+    newest = max(os.path.getmtime(o) for o in objs)
+    if force or not os.path.exists(LIB) or os.path.getmtime(LIB) < newest:
+        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    path = build(force="--force" in sys.argv, verbose=True)
+    print("built", path)

@@ -1,0 +1,553 @@
+// Host launchers of the int8 GEMM / convolution kernels for gfx950, the generic
+// (any layout, any alignment, zero points) scalar kernels, and the MFMA layout
+// probe.  The tile shape is chosen at run time from the dynamic M.
+#include <algorithm>
+#include <mutex>
+
+#include "dq8_common.h"
+#include "disc_q8.h"
+#include "qgemm_device.h"
+
+#pragma clang fp contract(off)
+
+namespace dq8 {
+namespace {
+
+// ------------------------------------------------------------ generic kernels
+struct GenericParams {
+  const int8_t* A;
+  const int8_t* W;
+  int64_t a_sm, a_sk;  // element strides of A along m and k
+  int64_t w_sn, w_sk;  // element strides of W along n and k
+  int K;
+  int zx, zw;
+  EpiParams epi;
+};
+
+template <int EPI>
+__device__ __forceinline__ void store_one(const EpiParams& e, int m, int n, int acc) {
+  const ColParams c = col_params<EPI>(e, n);
+  const int64_t off = (int64_t)m * e.ldo + n;
+  if (EPI == DQ8_EPI_ACC_S32)
+    ((int32_t*)e.out)[off] = acc;
+  else if (EPI == DQ8_EPI_DEQUANT_F32)
+    ((float*)e.out)[off] = dequant_one(e, c, acc);
+  else
+    ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, acc);
+}
+
+template <int EPI>
+__global__ void __launch_bounds__(256) qgemm_generic_kernel(const GenericParams p) {
+  const int64_t total = (int64_t)p.epi.M * p.epi.N;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * 256) {
+    const int m = (int)(idx / p.epi.N), n = (int)(idx % p.epi.N);
+    const int8_t* a = p.A + (int64_t)m * p.a_sm;
+    const int8_t* w = p.W + (int64_t)n * p.w_sn;
+    int acc = 0;
+    for (int k = 0; k < p.K; ++k)
+      acc += ((int)a[(int64_t)k * p.a_sk] - p.zx) * ((int)w[(int64_t)k * p.w_sk] - p.zw);
+    store_one<EPI>(p.epi, m, n, acc);
+  }
+}
+
+struct GenericConvParams {
+  const int8_t* in;
+  const int8_t* w;
+  int64_t i_sb, i_sc, i_sh, i_sw;  // input element strides: batch, channel, h, w
+  int64_t w_si, w_so, w_sh, w_sw;  // kernel strides: in ch, out ch, h, w
+  int64_t o_sb, o_sc, o_sh, o_sw;  // output strides
+  int NB, H, Wd, Ci, Co, Kh, Kw, Ho, Wo;
+  int pad_t, pad_l, sh, sw_, dh, dw;
+  EpiParams epi;  // M = NB*Ho*Wo, N = Co; ldo unused
+};
+
+template <int EPI>
+__global__ void __launch_bounds__(256) qconv_generic_kernel(const GenericConvParams p) {
+  const int64_t total = (int64_t)p.NB * p.Ho * p.Wo * p.Co;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * 256) {
+    const int co = (int)(idx % p.Co);
+    int64_t r = idx / p.Co;
+    const int x = (int)(r % p.Wo);
+    r /= p.Wo;
+    const int y = (int)(r % p.Ho);
+    const int b = (int)(r / p.Ho);
+    int acc = 0;
+    for (int kh = 0; kh < p.Kh; ++kh) {
+      const int yy = y * p.sh - p.pad_t + kh * p.dh;
+      if (yy < 0 || yy >= p.H) continue;
+      for (int kw = 0; kw < p.Kw; ++kw) {
+        const int xx = x * p.sw_ - p.pad_l + kw * p.dw;
+        if (xx < 0 || xx >= p.Wd) continue;
+        const int8_t* pi = p.in + b * p.i_sb + yy * p.i_sh + xx * p.i_sw;
+        const int8_t* pw = p.w + co * p.w_so + kh * p.w_sh + kw * p.w_sw;
+        for (int ci = 0; ci < p.Ci; ++ci)
+          acc += (int)pi[ci * p.i_sc] * (int)pw[ci * p.w_si];
+      }
+    }
+    const ColParams c = col_params<EPI>(p.epi, co);
+    const int64_t off = b * p.o_sb + co * p.o_sc + y * p.o_sh + x * p.o_sw;
+    if (EPI == DQ8_EPI_ACC_S32)
+      ((int32_t*)p.epi.out)[off] = acc;
+    else if (EPI == DQ8_EPI_DEQUANT_F32)
+      ((float*)p.epi.out)[off] = dequant_one(p.epi, c, acc);
+    else
+      ((int8_t*)p.epi.out)[off] = (int8_t)requant_one<EPI>(p.epi, c, acc);
+  }
+}
+
+// int8 [R, C] (row stride ld) -> [C, R] contiguous, 64x64 tiles through LDS
+__global__ void __launch_bounds__(256)
+transpose_s8_kernel(const int8_t* __restrict__ src, int64_t ld, int8_t* __restrict__ dst,
+                    int R, int C) {
+  __shared__ int8_t tile[64][65];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    tile[i][tx] = (r < R && c < C) ? src[(int64_t)r * ld + c] : (int8_t)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, r = r0 + tx;
+    if (c < C && r < R) dst[(int64_t)c * R + r] = tile[tx][i];
+  }
+}
+
+// one MFMA of each shape, operands straight from global memory
+__global__ void __launch_bounds__(64)
+mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* a16,
+                  const int8_t* b16, int32_t* d16) {
+  const int lane = threadIdx.x;
+  {
+    // 32x32x32: lane holds 16 consecutive k of row/column lane%32, k group lane/32
+    v4i fa = *(const v4i*)(a + (lane & 31) * 32 + (lane >> 5) * 16);
+    v4i fb = *(const v4i*)(b + (lane & 31) * 32 + (lane >> 5) * 16);
+    v16i c;
+    for (int v = 0; v < 16; ++v) c[v] = 0;
+    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, c, 0, 0, 0);
+    for (int v = 0; v < 16; ++v) {
+      const int i = 8 * (v / 4) + 4 * (lane >> 5) + (v % 4), j = lane & 31;
+      d32[i * 32 + j] = c[v];
+    }
+  }
+  {
+    // 16x16x64: lane holds 16 consecutive k of row/column lane%16, k group lane/16
+    v4i fa = *(const v4i*)(a16 + (lane & 15) * 64 + (lane >> 4) * 16);
+    v4i fb = *(const v4i*)(b16 + (lane & 15) * 64 + (lane >> 4) * 16);
+    v4i c = {0, 0, 0, 0};
+    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fb, c, 0, 0, 0);
+    for (int v = 0; v < 4; ++v) {
+      const int i = 4 * (lane >> 4) + v, j = lane & 15;
+      d16[i * 16 + j] = c[v];
+    }
+  }
+}
+
+// ------------------------------------------------------------- tile variants
+struct Variant {
+  const char* name;
+  int bm, bn, bk, threads;
+};
+// index 0 is the generic scalar kernel
+const Variant kVariants[] = {
+    {"generic", 1, 1, 1, 256},
+    {"mfma_256x256x64_w2x2", 256, 256, 64, 256},
+    {"mfma_128x128x64_w2x2", 128, 128, 64, 256},
+    {"mfma_64x64x64_w2x2", 64, 64, 64, 256},
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
+int launch_mfma(const MainParams& p, hipStream_t st) {
+  constexpr int lds = 2 * (BM + BN) * (BK + 16);
+  auto kern = qgemm_mfma_kernel<BM, BN, BK, WM, WN, CONV, EPI>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  });
+  DQ8_HIP(attr_err);
+  const int grid = p.tiles_m * p.tiles_n;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, st, p);
+  return check_hip(hipGetLastError(), "qgemm_mfma launch");
+}
+
+template <bool CONV, int EPI>
+int launch_variant(int variant, MainParams& p, hipStream_t st) {
+  const Variant& v = kVariants[variant];
+  p.tiles_m = (int)ceil_div(p.M, v.bm);
+  p.tiles_n = (int)ceil_div(p.N, v.bn);
+  switch (variant) {
+    case 1: return launch_mfma<256, 256, 64, 2, 2, CONV, EPI>(p, st);
+    case 2: return launch_mfma<128, 128, 64, 2, 2, CONV, EPI>(p, st);
+    case 3: return launch_mfma<64, 64, 64, 2, 2, CONV, EPI>(p, st);
+  }
+  return fail("unknown qgemm variant");
+}
+
+template <bool CONV>
+int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
+  switch (epilogue) {
+    case DQ8_EPI_ACC_S32: return launch_variant<CONV, DQ8_EPI_ACC_S32>(variant, p, st);
+    case DQ8_EPI_REQUANT_CPU: return launch_variant<CONV, DQ8_EPI_REQUANT_CPU>(variant, p, st);
+    case DQ8_EPI_REQUANT_GPU: return launch_variant<CONV, DQ8_EPI_REQUANT_GPU>(variant, p, st);
+    case DQ8_EPI_DEQUANT_F32: return launch_variant<CONV, DQ8_EPI_DEQUANT_F32>(variant, p, st);
+  }
+  return fail("unknown epilogue");
+}
+
+// Picks the MFMA tile from the dynamic problem size: the largest tile that still
+// yields at least about one workgroup per compute unit; small problems take the
+// smallest tile to spread the weight stream over as many CUs as possible.
+int pick_variant(int64_t M, int64_t N) {
+  constexpr int64_t kCus = 256;
+  for (int v = 1; v < kNumVariants; ++v) {
+    const int64_t tiles = ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn);
+    if (tiles >= kCus - kCus / 8) return v;
+  }
+  return kNumVariants - 1;
+}
+
+int elem_size(int epilogue) {
+  return (epilogue == DQ8_EPI_ACC_S32 || epilogue == DQ8_EPI_DEQUANT_F32) ? 4 : 1;
+}
+
+int check_epilogue(const char* who, int epilogue, const void* bias, int bias_kind,
+                   const float* sx, const float* sw, const float* so, int64_t n_sx,
+                   int64_t n_sw, int64_t n_so, int64_t N) {
+  const std::string w(who);
+  DQ8_REQUIRE(epilogue >= DQ8_EPI_ACC_S32 && epilogue <= DQ8_EPI_DEQUANT_F32,
+              w + ": unknown epilogue");
+  DQ8_REQUIRE(bias_kind >= DQ8_BIAS_NONE && bias_kind <= DQ8_BIAS_S8,
+              w + ": unknown bias kind");
+  DQ8_REQUIRE((bias_kind == DQ8_BIAS_NONE) == (bias == nullptr) ||
+                  (bias_kind == DQ8_BIAS_NONE),
+              w + ": bias pointer missing");
+  if (epilogue == DQ8_EPI_ACC_S32) {
+    DQ8_REQUIRE(bias_kind == DQ8_BIAS_NONE, w + ": ACC_S32 takes no bias");
+    return 0;
+  }
+  DQ8_REQUIRE(sx && sw, w + ": scale pointer missing");
+  DQ8_REQUIRE((n_sx == 1 || n_sx == N) && (n_sw == 1 || n_sw == N),
+              w + ": scale vectors must have 1 or N entries");
+  if (epilogue == DQ8_EPI_DEQUANT_F32) {
+    DQ8_REQUIRE(bias_kind == DQ8_BIAS_NONE || bias_kind == DQ8_BIAS_F32,
+                w + ": DEQUANT_F32 takes an f32 bias or none");
+    return 0;
+  }
+  DQ8_REQUIRE(so && (n_so == 1 || n_so == N), w + ": output scale missing or mis-sized");
+  if (epilogue == DQ8_EPI_REQUANT_CPU)
+    DQ8_REQUIRE(bias_kind != DQ8_BIAS_S8, w + ": REQUANT_CPU takes s32/f32 bias or none");
+  if (epilogue == DQ8_EPI_REQUANT_GPU)
+    DQ8_REQUIRE(bias_kind != DQ8_BIAS_S32, w + ": REQUANT_GPU takes f32/s8 bias or none");
+  return 0;
+}
+
+template <typename P>
+int launch_generic_epi(void (*k0)(const P), void (*k1)(const P), void (*k2)(const P),
+                       void (*k3)(const P), int epilogue, const P& p, int64_t total,
+                       hipStream_t st) {
+  int64_t blocks = std::min<int64_t>(ceil_div(total, 256), 256 * 32);
+  void (*k)(const P) = epilogue == DQ8_EPI_ACC_S32       ? k0
+                       : epilogue == DQ8_EPI_REQUANT_CPU ? k1
+                       : epilogue == DQ8_EPI_REQUANT_GPU ? k2
+                                                         : k3;
+  hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), 0, st, p);
+  return check_hip(hipGetLastError(), "generic kernel launch");
+}
+
+}  // namespace
+}  // namespace dq8
+
+using namespace dq8;
+
+extern "C" int dq8_qgemm_num_variants(void) { return kNumVariants; }
+
+extern "C" const char* dq8_qgemm_variant_name(int variant) {
+  if (variant < 0 || variant >= kNumVariants) return "";
+  return kVariants[variant].name;
+}
+
+extern "C" size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
+                                            int tp_b) {
+  size_t bytes = 0;
+  auto pad = [](int64_t v) { return (size_t)((v + 255) / 256 * 256); };
+  if (tp_a) bytes += pad(M * K);
+  if (!tp_b) bytes += pad(N * K);
+  return bytes;
+}
+
+extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
+                                 const int8_t* W, int64_t ldw, void* out, int64_t ldo,
+                                 int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
+                                 int epilogue, const void* bias, int bias_kind,
+                                 const float* sx, int64_t n_sx, const float* sw,
+                                 int64_t n_sw, const float* so, int64_t n_so,
+                                 int32_t zx, int32_t zw, int32_t zo, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(M >= 0 && N >= 0 && K >= 0, "dq8_qgemm: negative size");
+  DQ8_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
+              "dq8_qgemm: dimension exceeds 2^31-1");
+  DQ8_REQUIRE(variant >= -1 && variant < kNumVariants, "dq8_qgemm: unknown variant");
+  if (int s = check_epilogue("dq8_qgemm", epilogue, bias, bias_kind, sx, sw, so, n_sx,
+                             n_sw, n_so, N))
+    return s;
+  if (M == 0 || N == 0) return 0;
+  DQ8_REQUIRE(out != nullptr, "dq8_qgemm: null output");
+  DQ8_REQUIRE(K == 0 || (A && W), "dq8_qgemm: null operand");
+  DQ8_REQUIRE(lda >= (tp_a ? M : K) && ldw >= (tp_b ? K : N) && ldo >= N,
+              "dq8_qgemm: leading dimension smaller than the row length");
+  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
+              "dq8_qgemm: an output zero point needs the REQUANT_CPU epilogue");
+  hipStream_t st = (hipStream_t)stream;
+
+  EpiParams e;
+  e.out = out;
+  e.ldo = ldo;
+  e.M = (int)M;
+  e.N = (int)N;
+  e.bias = bias;
+  e.bias_kind = bias_kind;
+  e.sx = sx;
+  e.sw = sw;
+  e.so = so;
+  e.sx_stride = n_sx > 1;
+  e.sw_stride = n_sw > 1;
+  e.so_stride = n_so > 1;
+  e.zo = zo;
+  const int es = elem_size(epilogue);
+  e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
+
+  const bool need_generic = zx != 0 || zw != 0;
+  if (variant == -1) variant = need_generic ? 0 : pick_variant(M, N);
+  if (variant == 0) {
+    GenericParams g;
+    g.A = A;
+    g.W = W;
+    g.a_sm = tp_a ? 1 : lda;
+    g.a_sk = tp_a ? lda : 1;
+    g.w_sn = tp_b ? ldw : 1;
+    g.w_sk = tp_b ? 1 : ldw;
+    g.K = (int)K;
+    g.zx = zx;
+    g.zw = zw;
+    g.epi = e;
+    return launch_generic_epi<GenericParams>(
+        qgemm_generic_kernel<DQ8_EPI_ACC_S32>, qgemm_generic_kernel<DQ8_EPI_REQUANT_CPU>,
+        qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
+        epilogue, g, M * N, st);
+  }
+  DQ8_REQUIRE(!need_generic,
+              "dq8_qgemm: input/weight zero points are only supported by the generic variant");
+
+  // MFMA path wants A [M,K] and W [N,K], both k-contiguous: transpose the others
+  // into the workspace.
+  const int8_t* a_use = A;
+  const int8_t* w_use = W;
+  int64_t lda_use = lda, ldw_use = ldw;
+  size_t ws_off = 0;
+  auto pad = [](int64_t v) { return (size_t)((v + 255) / 256 * 256); };
+  if (K > 0 && (tp_a || !tp_b)) {
+    DQ8_REQUIRE(workspace != nullptr &&
+                    workspace_bytes >= dq8_qgemm_workspace_bytes(M, N, K, tp_a, tp_b),
+                "dq8_qgemm: workspace too small for the requested transposes");
+    if (tp_a) {  // A is [K, M] -> [M, K]
+      int8_t* dst = (int8_t*)workspace + ws_off;
+      hipLaunchKernelGGL(transpose_s8_kernel, dim3((unsigned)ceil_div(M, 64), (unsigned)ceil_div(K, 64)),
+                         dim3(256), 0, st, A, lda, dst, (int)K, (int)M);
+      a_use = dst;
+      lda_use = K;
+      ws_off += pad(M * K);
+    }
+    if (!tp_b) {  // W is [K, N] -> [N, K]
+      int8_t* dst = (int8_t*)workspace + ws_off;
+      hipLaunchKernelGGL(transpose_s8_kernel, dim3((unsigned)ceil_div(N, 64), (unsigned)ceil_div(K, 64)),
+                         dim3(256), 0, st, W, ldw, dst, (int)K, (int)N);
+      w_use = dst;
+      ldw_use = K;
+    }
+    DQ8_HIP(hipGetLastError());
+  }
+  // 16-byte loads: rows must start 16-byte aligned and K must be a multiple of 16
+  const bool fast_ok = K % 16 == 0 && (K == 0 || (aligned(a_use, 16) && aligned(w_use, 16) &&
+                                                  lda_use % 16 == 0 && ldw_use % 16 == 0));
+  if (!fast_ok) {
+    GenericParams g;
+    g.A = a_use;
+    g.W = w_use;
+    g.a_sm = lda_use;
+    g.a_sk = 1;
+    g.w_sn = ldw_use;
+    g.w_sk = 1;
+    g.K = (int)K;
+    g.zx = 0;
+    g.zw = 0;
+    g.epi = e;
+    return launch_generic_epi<GenericParams>(
+        qgemm_generic_kernel<DQ8_EPI_ACC_S32>, qgemm_generic_kernel<DQ8_EPI_REQUANT_CPU>,
+        qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
+        epilogue, g, M * N, st);
+  }
+
+  MainParams p = {};
+  p.A = a_use;
+  p.W = w_use;
+  p.lda = lda_use;
+  p.ldw = ldw_use;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.epi = e;
+  return launch_epi<false>(variant, p, epilogue, st);
+}
+
+extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
+                         void* out, int64_t ldo, int64_t M, int64_t N, int64_t K,
+                         int tp_a, int tp_b, int epilogue, const void* bias,
+                         int bias_kind, const float* sx, int64_t n_sx, const float* sw,
+                         int64_t n_sw, const float* so, int64_t n_so, int32_t zx,
+                         int32_t zw, int32_t zo, void* workspace, size_t workspace_bytes,
+                         void* stream) {
+  return dq8_qgemm_variant(-1, A, lda, W, ldw, out, ldo, M, N, K, tp_a, tp_b, epilogue,
+                           bias, bias_kind, sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo,
+                           workspace, workspace_bytes, stream);
+}
+
+extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t in_sizes[4],
+                                   const int8_t* w, const int64_t w_sizes[4],
+                                   const int32_t padding[4], const int32_t md[17],
+                                   void* out, const int64_t out_sizes[4], int epilogue,
+                                   const void* bias, int bias_kind, const float* sx,
+                                   const float* sw, int64_t n_sw, const float* so,
+                                   int32_t zo, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(in_sizes && w_sizes && padding && md && out_sizes, "dq8_qconv2d: null descriptor");
+  DQ8_REQUIRE(variant >= -1 && variant < kNumVariants, "dq8_qconv2d: unknown variant");
+  for (int i = 0; i < 12; ++i)
+    DQ8_REQUIRE(md[i] >= 0 && md[i] < 4, "dq8_qconv2d: metadata dimension index out of range");
+  for (int g = 0; g < 3; ++g) {
+    int seen = 0;
+    for (int i = 0; i < 4; ++i) seen |= 1 << md[4 * g + i];
+    DQ8_REQUIRE(seen == 15, "dq8_qconv2d: metadata layout is not a permutation");
+  }
+  const int ib = md[0], ic = md[1], ih = md[2], iw = md[3];
+  const int ki = md[4], ko = md[5], kh = md[6], kw = md[7];
+  const int ob = md[8], oc = md[9], oh = md[10], ow = md[11];
+  const int64_t NB = in_sizes[ib], Ci = in_sizes[ic], H = in_sizes[ih], Wd = in_sizes[iw];
+  const int64_t Co = w_sizes[ko], Kh = w_sizes[kh], Kw = w_sizes[kw];
+  const int64_t Ho = out_sizes[oh], Wo = out_sizes[ow];
+  DQ8_REQUIRE(w_sizes[ki] == Ci, "dq8_qconv2d: kernel input features differ from the input's");
+  DQ8_REQUIRE(out_sizes[ob] == NB && out_sizes[oc] == Co,
+              "dq8_qconv2d: output batch/channel mismatch");
+  const int sh = md[12], sw_ = md[13], dh = md[14], dw = md[15];
+  DQ8_REQUIRE(sh > 0 && sw_ > 0 && dh > 0 && dw > 0, "dq8_qconv2d: strides/dilations must be > 0");
+  DQ8_REQUIRE(padding[0] >= 0 && padding[1] >= 0 && padding[2] >= 0 && padding[3] >= 0,
+              "dq8_qconv2d: negative padding");
+  // the output extent must be what the geometry produces
+  auto out_len = [](int64_t i, int64_t p0, int64_t p1, int64_t k, int64_t d, int64_t s) {
+    return (i + p0 + p1 - k * d + d + s - 1) / s;
+  };
+  DQ8_REQUIRE(Ho == out_len(H, padding[0], padding[1], Kh, dh, sh) &&
+                  Wo == out_len(Wd, padding[2], padding[3], Kw, dw, sw_),
+              "dq8_qconv2d: output spatial size inconsistent with padding/stride/dilation");
+  if (int s = check_epilogue("dq8_qconv2d", epilogue, bias, bias_kind, sx, sw, so, 1, n_sw, 1, Co))
+    return s;
+  const int64_t Mg = NB * Ho * Wo, Kg = Kh * Kw * Ci;
+  DQ8_REQUIRE(Mg < (1LL << 31) && Kg < (1LL << 31) && Co < (1LL << 31) &&
+                  NB * H * Wd * Ci < (1LL << 40),
+              "dq8_qconv2d: problem too large");
+  if (Mg == 0 || Co == 0) return 0;
+  DQ8_REQUIRE(in && w && out, "dq8_qconv2d: null tensor");
+  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
+              "dq8_qconv2d: an output zero point needs the REQUANT_CPU epilogue");
+  hipStream_t st = (hipStream_t)stream;
+
+  EpiParams e;
+  e.out = out;
+  e.ldo = Co;
+  e.M = (int)Mg;
+  e.N = (int)Co;
+  e.bias = bias;
+  e.bias_kind = bias_kind;
+  e.sx = sx;
+  e.sw = sw;
+  e.so = so;
+  e.sx_stride = 0;
+  e.sw_stride = n_sw > 1;
+  e.so_stride = 0;
+  e.zo = zo;
+  const int es = elem_size(epilogue);
+  e.vec_store = aligned(out, 4 * es) && (Co % 4 == 0);
+
+  const bool nhwc_ohwi = ib == 0 && ic == 3 && ih == 1 && iw == 2 && ki == 3 && ko == 0 &&
+                         kh == 1 && kw == 2 && ob == 0 && oc == 3 && oh == 1 && ow == 2;
+  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16);
+  if (variant == -1) variant = fast_ok ? pick_variant(Mg, Co) : 0;
+  if (variant != 0)
+    DQ8_REQUIRE(fast_ok, "dq8_qconv2d: the MFMA variants need NHWC x OHWI, Ci % 16 == 0 and "
+                         "16-byte aligned tensors");
+  if (variant == 0) {
+    auto strides = [](const int64_t s[4], int64_t st4[4]) {
+      st4[3] = 1;
+      for (int i = 3; i > 0; --i) st4[i - 1] = st4[i] * s[i];
+    };
+    int64_t is[4], ws[4], os[4];
+    strides(in_sizes, is);
+    strides(w_sizes, ws);
+    strides(out_sizes, os);
+    GenericConvParams g;
+    g.in = in;
+    g.w = w;
+    g.i_sb = is[ib]; g.i_sc = is[ic]; g.i_sh = is[ih]; g.i_sw = is[iw];
+    g.w_si = ws[ki]; g.w_so = ws[ko]; g.w_sh = ws[kh]; g.w_sw = ws[kw];
+    g.o_sb = os[ob]; g.o_sc = os[oc]; g.o_sh = os[oh]; g.o_sw = os[ow];
+    g.NB = (int)NB; g.H = (int)H; g.Wd = (int)Wd; g.Ci = (int)Ci; g.Co = (int)Co;
+    g.Kh = (int)Kh; g.Kw = (int)Kw; g.Ho = (int)Ho; g.Wo = (int)Wo;
+    g.pad_t = padding[0]; g.pad_l = padding[2];
+    g.sh = sh; g.sw_ = sw_; g.dh = dh; g.dw = dw;
+    g.epi = e;
+    return launch_generic_epi<GenericConvParams>(
+        qconv_generic_kernel<DQ8_EPI_ACC_S32>, qconv_generic_kernel<DQ8_EPI_REQUANT_CPU>,
+        qconv_generic_kernel<DQ8_EPI_REQUANT_GPU>, qconv_generic_kernel<DQ8_EPI_DEQUANT_F32>,
+        epilogue, g, Mg * Co, st);
+  }
+
+  MainParams p = {};
+  p.A = in;
+  p.W = w;
+  p.lda = 0;
+  p.ldw = Kg;
+  p.M = (int)Mg;
+  p.N = (int)Co;
+  p.K = (int)Kg;
+  p.H = (int)H; p.Wd = (int)Wd; p.Ci = (int)Ci; p.Ho = (int)Ho; p.Wo = (int)Wo;
+  p.Kh = (int)Kh; p.Kw = (int)Kw;
+  p.pad_t = padding[0]; p.pad_l = padding[2];
+  p.sh = sh; p.sw_ = sw_; p.dh = dh; p.dw = dw;
+  p.epi = e;
+  return launch_epi<true>(variant, p, epilogue, st);
+}
+
+extern "C" int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                           const int64_t w_sizes[4], const int32_t padding[4],
+                           const int32_t metadata[17], void* out, const int64_t out_sizes[4],
+                           int epilogue, const void* bias, int bias_kind, const float* sx,
+                           const float* sw, int64_t n_sw, const float* so, int32_t zo,
+                           void* stream) {
+  return dq8_qconv2d_variant(-1, in, in_sizes, w, w_sizes, padding, metadata, out, out_sizes,
+                             epilogue, bias, bias_kind, sx, sw, n_sw, so, zo, stream);
+}
+
+extern "C" int dq8_mfma_probe(const int8_t* a, const int8_t* b, int32_t* d32,
+                              const int8_t* a16, const int8_t* b16, int32_t* d16,
+                              void* stream) {
+  clear_error();
+  DQ8_REQUIRE(a && b && d32 && a16 && b16 && d16, "dq8_mfma_probe: null pointer");
+  hipLaunchKernelGGL(mfma_probe_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, a, b, d32,
+                     a16, b16, d16);
+  return check_hip(hipGetLastError(), "dq8_mfma_probe launch");
+}

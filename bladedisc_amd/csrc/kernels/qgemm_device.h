@@ -1,0 +1,370 @@
+// Device-side building blocks shared by the int8 GEMM and the implicit-GEMM
+// convolution for gfx950: parameter blocks, the fused requantisation epilogue and
+// the LDS-tiled MFMA main loop.
+//
+// Arithmetic contract of the epilogue (binary32, no contraction, IEEE division):
+//   REQUANT_CPU  os = (sx*sw[n]) / (1*so);  d = (f32(acc) + b[n]) * os + zo
+//                b[n] = f32(bias_s32[n])  or  f32(sat32(rne(bias_f32[n] * (1/(sx*sw[n])))))
+//                (reference: ral/context/mkldnn/ideep/ideep/operators/matmul.hpp:532-535)
+//   REQUANT_GPU  os = (sx[n]*sw[n]) / so[n];  d = os * f32(acc) + bias[n]
+//                (reference: ral/context/quantized_gpu_kernel_impl.cc:262-265,385,416-420)
+//   DEQUANT_F32  d = f32(acc) * (sx*sw[n]) + bias[n]
+// followed, for the two requant modes, by saturation to [-128,127] and
+// round-half-to-even.
+#ifndef DQ8_QGEMM_DEVICE_H_
+#define DQ8_QGEMM_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "disc_q8.h"
+
+#pragma clang fp contract(off)
+
+namespace dq8 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct EpiParams {
+  void* out;
+  int64_t ldo;  // elements
+  int M, N;
+  const void* bias;
+  int bias_kind;
+  const float* sx;
+  const float* sw;
+  const float* so;
+  int sx_stride, sw_stride, so_stride;  // 0 (rank-0 scale) or 1 (per channel)
+  int zo;
+  int vec_store;  // 1: a group of 4 consecutive n may be stored as one 4/16-byte word
+};
+
+// Operand description.  GEMM: A [M,K] (row stride lda), W [N,K] (row stride ldw).
+// Convolution (NHWC x OHWI): GEMM row m = (batch, ho, wo), k = (kh, kw, ci).
+struct MainParams {
+  const int8_t* A;
+  const int8_t* W;
+  int64_t lda, ldw;
+  int M, N, K;
+  // convolution geometry (unused by the plain GEMM)
+  int H, Wd, Ci, Ho, Wo, Kh, Kw;
+  int pad_t, pad_l, sh, sw_, dh, dw;
+  int tiles_m, tiles_n;
+  EpiParams epi;
+};
+
+// ------------------------------------------------------------------ epilogue
+struct ColParams {  // per output channel
+  float os;   // output scale (requant) or dequant scale
+  float b;    // additive term, already in the units the mode needs
+};
+
+__device__ __forceinline__ float sat_rne_s32_as_float(float v) {
+  // saturate to int32 in float (the largest float below 2^31 is 2147483520), then
+  // round to nearest even; the result is integral, so the later int->float
+  // conversion of the stored s32 bias is the identity on it.
+  v = fminf(fmaxf(v, -2147483648.0f), 2147483520.0f);
+  return (float)(int)rintf(v);
+}
+
+template <int EPI>
+__device__ __forceinline__ ColParams col_params(const EpiParams& p, int n) {
+  ColParams c;
+  c.os = 1.0f;
+  c.b = 0.0f;
+  if (EPI == DQ8_EPI_ACC_S32) return c;
+  const float sx = p.sx[(int64_t)n * p.sx_stride];
+  const float sw = p.sw[(int64_t)n * p.sw_stride];
+  const float prod = sx * sw;
+  if (EPI == DQ8_EPI_DEQUANT_F32) {
+    c.os = prod;
+    if (p.bias_kind == DQ8_BIAS_F32) c.b = ((const float*)p.bias)[n];
+    return c;
+  }
+  const float so = p.so[(int64_t)n * p.so_stride];
+  if (EPI == DQ8_EPI_REQUANT_CPU) {
+    c.os = prod / (1.0f * so);
+    if (p.bias_kind == DQ8_BIAS_S32) {
+      c.b = (float)((const int32_t*)p.bias)[n];
+    } else if (p.bias_kind == DQ8_BIAS_F32) {
+      const float bs = (1.0f * 1.0f) / prod;
+      c.b = sat_rne_s32_as_float(((const float*)p.bias)[n] * bs);
+    }
+  } else {  // REQUANT_GPU
+    c.os = prod / so;
+    if (p.bias_kind == DQ8_BIAS_F32)
+      c.b = ((const float*)p.bias)[n];
+    else if (p.bias_kind == DQ8_BIAS_S8)
+      c.b = (float)((const int8_t*)p.bias)[n];
+  }
+  return c;
+}
+
+__device__ __forceinline__ int sat_rne_s8(float d) {
+  d = fminf(fmaxf(d, -128.0f), 127.0f);  // NaN -> -128, like the CPU path
+  return (int)rintf(d);
+}
+
+// int8 result of one accumulator for the two requant modes
+template <int EPI>
+__device__ __forceinline__ int requant_one(const EpiParams& p, const ColParams& c,
+                                           int acc) {
+  float d = (float)acc;
+  if (EPI == DQ8_EPI_REQUANT_CPU) {
+    if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
+    d = d * c.os;
+    if (p.zo != 0) d = d + (float)p.zo;
+  } else {
+    d = c.os * d;
+    if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
+  }
+  return sat_rne_s8(d);
+}
+
+__device__ __forceinline__ float dequant_one(const EpiParams& p, const ColParams& c,
+                                             int acc) {
+  float d = (float)acc * c.os;
+  if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
+  return d;
+}
+
+// Stores the results for row m, columns n .. n+3 (n % 4 == 0).
+template <int EPI>
+__device__ __forceinline__ void store_group4(const EpiParams& p, int m, int n,
+                                             const ColParams (&c)[4], int a0, int a1,
+                                             int a2, int a3) {
+  const int acc[4] = {a0, a1, a2, a3};
+  const int64_t off = (int64_t)m * p.ldo + n;
+  const bool full = n + 3 < p.N;
+  if (EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU) {
+    int8_t* out = (int8_t*)p.out;
+    int q[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q[e] = requant_one<EPI>(p, c[e], acc[e]);
+    if (full && p.vec_store) {
+      uint32_t w = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) |
+                   ((uint32_t)(q[2] & 0xff) << 16) | ((uint32_t)(q[3] & 0xff) << 24);
+      *(uint32_t*)(out + off) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < p.N) out[off + e] = (int8_t)q[e];
+    }
+  } else if (EPI == DQ8_EPI_ACC_S32) {
+    int32_t* out = (int32_t*)p.out;
+    if (full && p.vec_store) {
+      v4i w = {a0, a1, a2, a3};
+      *(v4i*)(out + off) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < p.N) out[off + e] = acc[e];
+    }
+  } else {
+    float* out = (float*)p.out;
+    float f[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = dequant_one(p, c[e], acc[e]);
+    if (full && p.vec_store) {
+      v4f w = {f[0], f[1], f[2], f[3]};
+      *(v4f*)(out + off) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < p.N) out[off + e] = f[e];
+    }
+  }
+}
+
+// ----------------------------------------------------------------- main loop
+// Workgroups are handed to the 8 XCDs round-robin; consecutive logical tiles
+// share operand rows, so give each XCD a contiguous range of logical tiles to
+// keep that reuse inside one L2.
+__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
+  constexpr int kXcd = 8;
+  if (nblocks % kXcd != 0) return bid;
+  return (bid % kXcd) * (nblocks / kXcd) + bid / kXcd;
+}
+
+// LDS-tiled int8 GEMM on v_mfma_i32_32x32x32_i8.
+//   block tile BM x BN x BK, WM x WN waves, each wave a (BM/WM) x (BN/WN) tile
+//   built from 32x32 MFMA fragments; two LDS stages, global loads for stage
+//   t+1 are in flight while stage t is multiplied.
+// The weight rows are fed as the MFMA's row operand and the activation rows as
+// its column operand, so each lane ends up with 4 consecutive output channels
+// of one output row per accumulator quad: an aligned 4-byte (int8) or 16-byte
+// (int32 / f32) store.
+template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
+__global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParams p) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM, TN = BN / WN;
+  constexpr int FM = TM / 32, FN = TN / 32;
+  constexpr int KC = BK / 16;        // 16-byte chunks per tile row
+  constexpr int ROW = BK + 16;       // padded LDS row: conflict-free b128 reads
+  constexpr int RPP = NT / KC;       // tile rows covered by one pass of the block
+  constexpr int A_LD = BM / RPP, B_LD = BN / RPP;
+  constexpr int STAGE = (BM + BN) * ROW;
+  static_assert(BM % RPP == 0 && BN % RPP == 0, "tile/thread mismatch");
+  static_assert(TM % 32 == 0 && TN % 32 == 0 && BK % 32 == 0, "fragment mismatch");
+
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int kc = tid % KC;
+  const int lrow = tid / KC;
+
+  // ---- per-thread global row descriptors (fixed for the whole K loop)
+  const int8_t* a_ptr[A_LD];
+  bool a_ok[A_LD];
+  int a_hi0[A_LD], a_wi0[A_LD];  // conv only
+#pragma unroll
+  for (int i = 0; i < A_LD; ++i) {
+    const int m = m0 + lrow + i * RPP;
+    a_ok[i] = m < p.M;
+    const int mm = a_ok[i] ? m : 0;
+    if (CONV) {
+      const int hw = p.Ho * p.Wo;
+      const int b = mm / hw;
+      const int r = mm - b * hw;
+      const int ho = r / p.Wo, wo = r - ho * p.Wo;
+      a_hi0[i] = ho * p.sh - p.pad_t;
+      a_wi0[i] = wo * p.sw_ - p.pad_l;
+      a_ptr[i] = p.A + (int64_t)b * p.H * p.Wd * p.Ci;
+    } else {
+      a_hi0[i] = a_wi0[i] = 0;
+      a_ptr[i] = p.A + (int64_t)mm * p.lda + kc * 16;
+    }
+  }
+  const int8_t* b_ptr[B_LD];
+  bool b_ok[B_LD];
+#pragma unroll
+  for (int i = 0; i < B_LD; ++i) {
+    const int n = n0 + lrow + i * RPP;
+    b_ok[i] = n < p.N;
+    b_ptr[i] = p.W + (int64_t)(b_ok[i] ? n : 0) * p.ldw + kc * 16;
+  }
+  // conv: position of this thread's chunk inside the (kh, kw, ci) index space
+  int c_ci = kc * 16, c_kw = 0, c_kh = 0;
+  if (CONV) {
+    while (c_ci >= p.Ci) {
+      c_ci -= p.Ci;
+      if (++c_kw == p.Kw) { c_kw = 0; ++c_kh; }
+    }
+  }
+
+  v4i ra[A_LD], rb[B_LD];
+  const v4i zero4 = {0, 0, 0, 0};
+
+  auto gload = [&](int kt) {
+    const bool k_ok = kt * BK + kc * 16 < p.K;
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i) {
+      if (CONV) {
+        const int hi = a_hi0[i] + c_kh * p.dh, wi = a_wi0[i] + c_kw * p.dw;
+        const bool ok = a_ok[i] && k_ok && hi >= 0 && hi < p.H && wi >= 0 && wi < p.Wd;
+        const int8_t* src = a_ptr[i] + ((int64_t)(ok ? hi : 0) * p.Wd + (ok ? wi : 0)) * p.Ci + c_ci;
+        ra[i] = ok ? *(const v4i*)src : zero4;
+      } else {
+        ra[i] = (a_ok[i] && k_ok) ? *(const v4i*)(a_ptr[i] + (int64_t)kt * BK) : zero4;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i)
+      rb[i] = (b_ok[i] && k_ok) ? *(const v4i*)(b_ptr[i] + (int64_t)kt * BK) : zero4;
+    if (CONV) {  // advance this thread's chunk by BK along k
+      c_ci += BK;
+      while (c_ci >= p.Ci) {
+        c_ci -= p.Ci;
+        if (++c_kw == p.Kw) { c_kw = 0; ++c_kh; }
+      }
+    }
+  };
+  auto lstore = [&](int buf) {
+    int8_t* As = smem + buf * STAGE;
+    int8_t* Bs = As + BM * ROW;
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i)
+      *(v4i*)(As + (lrow + i * RPP) * ROW + kc * 16) = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i)
+      *(v4i*)(Bs + (lrow + i * RPP) * ROW + kc * 16) = rb[i];
+  };
+
+  v16i acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  const int KT = (p.K + BK - 1) / BK;
+  const int frag_off = (lane & 31) * ROW + (lane >> 5) * 16;
+
+  if (KT > 0) {
+    gload(0);
+    lstore(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) gload(kt + 1);
+    const int8_t* As = smem + buf * STAGE + (wm * TM) * ROW + frag_off;
+    const int8_t* Bs = smem + buf * STAGE + BM * ROW + (wn * TN) * ROW + frag_off;
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      v4i fa[FM], fb[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) fa[i] = *(const v4i*)(As + i * 32 * ROW + ks * 32);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) fb[j] = *(const v4i*)(Bs + j * 32 * ROW + ks * 32);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) lstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: accumulator v of fragment (i,j) is output row
+  // m = m0 + wm*TM + i*32 + lane%32, channel n = n0 + wn*TN + j*32 + 8*(v/4) +
+  // 4*(lane/32) + v%4.
+  const EpiParams& e = p.epi;
+  const int m_base = m0 + wm * TM + (lane & 31);
+  const int n_base = n0 + wn * TN + 4 * (lane >> 5);
+#pragma unroll
+  for (int j = 0; j < FN; ++j) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int n = n_base + j * 32 + 8 * g;
+      if (n >= e.N) continue;
+      ColParams c[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) c[q] = col_params<EPI>(e, n + q < e.N ? n + q : n);
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        const int m = m_base + i * 32;
+        if (m < e.M)
+          store_group4<EPI>(e, m, n, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
+                            acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+      }
+    }
+  }
+}
+
+}  // namespace dq8
+
+#endif  // DQ8_QGEMM_DEVICE_H_

@@ -1,0 +1,392 @@
+// quantize / dequantize for gfx950: bandwidth-bound, 5 bytes of HBM traffic per
+// element.  Semantics follow the reference's runtime decomposition of
+// mhlo_disc.quantize / mhlo_disc.dequantize
+// (tao_compiler/mlir/disc/transforms/disc_lower_quantize_and_dequantize.cc:77-94,
+// 131-136): every step is a separately rounded binary32 operation and the
+// division is a true IEEE division, so this file is compiled with
+// -ffp-contract=off.
+//
+// Three access patterns, all without per-element integer division:
+//   per tensor            1-D grid-stride over float4 / packed-4 elements
+//   per channel, inner==1 (channel is the last axis) 2-D tiles [rows, 4*threads];
+//                         each thread keeps its four scales / zero points in
+//                         registers while it walks down the rows
+//   per channel, inner%4==0 one (outer, channel) row per blockIdx.y
+// Anything else (odd sizes, unaligned pointers) takes the scalar kernel.
+#include <algorithm>
+
+#include "dq8_common.h"
+#include "disc_q8.h"
+
+#pragma clang fp contract(off)
+
+namespace {
+
+constexpr int kThreads = 256;
+
+template <int ROUND>
+__device__ __forceinline__ int quant_one(float x, float s, float z, float lo,
+                                         float hi) {
+  float t0 = x / s;
+  float t1 = t0 + z;
+  float t2 = ROUND == DQ8_ROUND_HALF_TO_EVEN ? rintf(t1) : roundf(t1);
+  float t3 = fminf(fmaxf(t2, lo), hi);  // clamp; NaN -> lo like the CPU loop
+  return (int)t3;
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+  return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) |
+         ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+
+// ---------------------------------------------------------------- per tensor
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+quantize_tensor_v4(const float4* __restrict__ x, uint32_t* __restrict__ out,
+                   int64_t n4, const float* __restrict__ scale,
+                   const int32_t* __restrict__ zp, float lo, float hi) {
+  const float s = scale[0];
+  const float z = (float)zp[0];
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  // four independent 16-byte loads in flight per thread
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    float4 v0 = x[i], v1 = x[i + stride], v2 = x[i + 2 * stride],
+           v3 = x[i + 3 * stride];
+    out[i] = pack4(quant_one<ROUND>(v0.x, s, z, lo, hi), quant_one<ROUND>(v0.y, s, z, lo, hi),
+                   quant_one<ROUND>(v0.z, s, z, lo, hi), quant_one<ROUND>(v0.w, s, z, lo, hi));
+    out[i + stride] = pack4(quant_one<ROUND>(v1.x, s, z, lo, hi), quant_one<ROUND>(v1.y, s, z, lo, hi),
+                            quant_one<ROUND>(v1.z, s, z, lo, hi), quant_one<ROUND>(v1.w, s, z, lo, hi));
+    out[i + 2 * stride] = pack4(quant_one<ROUND>(v2.x, s, z, lo, hi), quant_one<ROUND>(v2.y, s, z, lo, hi),
+                                quant_one<ROUND>(v2.z, s, z, lo, hi), quant_one<ROUND>(v2.w, s, z, lo, hi));
+    out[i + 3 * stride] = pack4(quant_one<ROUND>(v3.x, s, z, lo, hi), quant_one<ROUND>(v3.y, s, z, lo, hi),
+                                quant_one<ROUND>(v3.z, s, z, lo, hi), quant_one<ROUND>(v3.w, s, z, lo, hi));
+  }
+  for (; i < n4; i += stride) {
+    float4 v = x[i];
+    out[i] = pack4(quant_one<ROUND>(v.x, s, z, lo, hi), quant_one<ROUND>(v.y, s, z, lo, hi),
+                   quant_one<ROUND>(v.z, s, z, lo, hi), quant_one<ROUND>(v.w, s, z, lo, hi));
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+dequantize_tensor_v4(const uint32_t* __restrict__ q, float4* __restrict__ out,
+                     int64_t n4, const float* __restrict__ scale,
+                     const int32_t* __restrict__ zp, int is_signed) {
+  const float s = scale[0];
+  const int z = zp[0];
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  auto one = [&](uint32_t w) {
+    int b0, b1, b2, b3;
+    if (is_signed) {
+      b0 = (int8_t)(w & 0xff); b1 = (int8_t)((w >> 8) & 0xff);
+      b2 = (int8_t)((w >> 16) & 0xff); b3 = (int8_t)(w >> 24);
+    } else {
+      b0 = w & 0xff; b1 = (w >> 8) & 0xff; b2 = (w >> 16) & 0xff; b3 = w >> 24;
+    }
+    return make_float4((float)(b0 - z) * s, (float)(b1 - z) * s,
+                       (float)(b2 - z) * s, (float)(b3 - z) * s);
+  };
+  int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  for (; i + 3 * stride < n4; i += 4 * stride) {
+    uint32_t w0 = q[i], w1 = q[i + stride], w2 = q[i + 2 * stride],
+             w3 = q[i + 3 * stride];
+    out[i] = one(w0);
+    out[i + stride] = one(w1);
+    out[i + 2 * stride] = one(w2);
+    out[i + 3 * stride] = one(w3);
+  }
+  for (; i < n4; i += stride) out[i] = one(q[i]);
+}
+
+// ------------------------------------------- per channel, channel = last axis
+// x: [rows, nch], nch % 4 == 0.  blockIdx.x tiles channels (4 per thread),
+// blockIdx.y tiles rows; each block walks rows_per_block rows.
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+quantize_lastaxis_v4(const float4* __restrict__ x, uint32_t* __restrict__ out,
+                     int64_t rows, int nch4, int rows_per_block,
+                     const float4* __restrict__ scale,
+                     const int4* __restrict__ zp, float lo, float hi) {
+  const int c4 = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c4 >= nch4) return;
+  const float4 s = scale[c4];
+  const int4 zi = zp[c4];
+  const float4 z = make_float4((float)zi.x, (float)zi.y, (float)zi.z, (float)zi.w);
+  int64_t r = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end = r + rows_per_block < rows ? r + rows_per_block : rows;
+  const float4* px = x + r * nch4 + c4;
+  uint32_t* po = out + r * nch4 + c4;
+  for (; r + 3 < r_end; r += 4, px += 4 * (int64_t)nch4, po += 4 * (int64_t)nch4) {
+    float4 v0 = px[0], v1 = px[nch4], v2 = px[2 * (int64_t)nch4],
+           v3 = px[3 * (int64_t)nch4];
+    po[0] = pack4(quant_one<ROUND>(v0.x, s.x, z.x, lo, hi), quant_one<ROUND>(v0.y, s.y, z.y, lo, hi),
+                  quant_one<ROUND>(v0.z, s.z, z.z, lo, hi), quant_one<ROUND>(v0.w, s.w, z.w, lo, hi));
+    po[nch4] = pack4(quant_one<ROUND>(v1.x, s.x, z.x, lo, hi), quant_one<ROUND>(v1.y, s.y, z.y, lo, hi),
+                     quant_one<ROUND>(v1.z, s.z, z.z, lo, hi), quant_one<ROUND>(v1.w, s.w, z.w, lo, hi));
+    po[2 * (int64_t)nch4] = pack4(quant_one<ROUND>(v2.x, s.x, z.x, lo, hi), quant_one<ROUND>(v2.y, s.y, z.y, lo, hi),
+                                  quant_one<ROUND>(v2.z, s.z, z.z, lo, hi), quant_one<ROUND>(v2.w, s.w, z.w, lo, hi));
+    po[3 * (int64_t)nch4] = pack4(quant_one<ROUND>(v3.x, s.x, z.x, lo, hi), quant_one<ROUND>(v3.y, s.y, z.y, lo, hi),
+                                  quant_one<ROUND>(v3.z, s.z, z.z, lo, hi), quant_one<ROUND>(v3.w, s.w, z.w, lo, hi));
+  }
+  for (; r < r_end; ++r, px += nch4, po += nch4) {
+    float4 v = px[0];
+    po[0] = pack4(quant_one<ROUND>(v.x, s.x, z.x, lo, hi), quant_one<ROUND>(v.y, s.y, z.y, lo, hi),
+                  quant_one<ROUND>(v.z, s.z, z.z, lo, hi), quant_one<ROUND>(v.w, s.w, z.w, lo, hi));
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+dequantize_lastaxis_v4(const uint32_t* __restrict__ q, float4* __restrict__ out,
+                       int64_t rows, int nch4, int rows_per_block,
+                       const float4* __restrict__ scale,
+                       const int4* __restrict__ zp, int is_signed) {
+  const int c4 = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c4 >= nch4) return;
+  const float4 s = scale[c4];
+  const int4 z = zp[c4];
+  int64_t r = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end = r + rows_per_block < rows ? r + rows_per_block : rows;
+  auto one = [&](uint32_t w) {
+    int b0, b1, b2, b3;
+    if (is_signed) {
+      b0 = (int8_t)(w & 0xff); b1 = (int8_t)((w >> 8) & 0xff);
+      b2 = (int8_t)((w >> 16) & 0xff); b3 = (int8_t)(w >> 24);
+    } else {
+      b0 = w & 0xff; b1 = (w >> 8) & 0xff; b2 = (w >> 16) & 0xff; b3 = w >> 24;
+    }
+    return make_float4((float)(b0 - z.x) * s.x, (float)(b1 - z.y) * s.y,
+                       (float)(b2 - z.z) * s.z, (float)(b3 - z.w) * s.w);
+  };
+  const uint32_t* pq = q + r * nch4 + c4;
+  float4* po = out + r * nch4 + c4;
+  for (; r + 3 < r_end; r += 4, pq += 4 * (int64_t)nch4, po += 4 * (int64_t)nch4) {
+    uint32_t w0 = pq[0], w1 = pq[nch4], w2 = pq[2 * (int64_t)nch4],
+             w3 = pq[3 * (int64_t)nch4];
+    po[0] = one(w0);
+    po[nch4] = one(w1);
+    po[2 * (int64_t)nch4] = one(w2);
+    po[3 * (int64_t)nch4] = one(w3);
+  }
+  for (; r < r_end; ++r, pq += nch4, po += nch4) po[0] = one(pq[0]);
+}
+
+// ------------------------------------- per channel, inner % 4 == 0 (any axis)
+// One (outer, channel) row of `inner` contiguous elements per blockIdx.y.
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+quantize_rows_v4(const float4* __restrict__ x, uint32_t* __restrict__ out,
+                 int64_t rows, int64_t inner4, int nch,
+                 const float* __restrict__ scale,
+                 const int32_t* __restrict__ zp, float lo, float hi) {
+  const int64_t row = (int64_t)blockIdx.y + (int64_t)blockIdx.z * gridDim.y;
+  if (row >= rows) return;
+  const int c = (int)(row % nch);
+  const float s = scale[c];
+  const float z = (float)zp[c];
+  const float4* px = x + row * inner4;
+  uint32_t* po = out + row * inner4;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < inner4;
+       i += (int64_t)gridDim.x * kThreads) {
+    float4 v = px[i];
+    po[i] = pack4(quant_one<ROUND>(v.x, s, z, lo, hi), quant_one<ROUND>(v.y, s, z, lo, hi),
+                  quant_one<ROUND>(v.z, s, z, lo, hi), quant_one<ROUND>(v.w, s, z, lo, hi));
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+dequantize_rows_v4(const uint32_t* __restrict__ q, float4* __restrict__ out,
+                   int64_t rows, int64_t inner4, int nch,
+                   const float* __restrict__ scale,
+                   const int32_t* __restrict__ zp, int is_signed) {
+  const int64_t row = (int64_t)blockIdx.y + (int64_t)blockIdx.z * gridDim.y;
+  if (row >= rows) return;
+  const int c = (int)(row % nch);
+  const float s = scale[c];
+  const int z = zp[c];
+  const uint32_t* pq = q + row * inner4;
+  float4* po = out + row * inner4;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < inner4;
+       i += (int64_t)gridDim.x * kThreads) {
+    uint32_t w = pq[i];
+    int b0, b1, b2, b3;
+    if (is_signed) {
+      b0 = (int8_t)(w & 0xff); b1 = (int8_t)((w >> 8) & 0xff);
+      b2 = (int8_t)((w >> 16) & 0xff); b3 = (int8_t)(w >> 24);
+    } else {
+      b0 = w & 0xff; b1 = (w >> 8) & 0xff; b2 = (w >> 16) & 0xff; b3 = w >> 24;
+    }
+    po[i] = make_float4((float)(b0 - z) * s, (float)(b1 - z) * s,
+                        (float)(b2 - z) * s, (float)(b3 - z) * s);
+  }
+}
+
+// ------------------------------------------------------------ scalar fallback
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+quantize_scalar(const float* __restrict__ x, uint8_t* __restrict__ out,
+                int64_t begin, int64_t n, int64_t nch, int64_t inner,
+                int per_channel, const float* __restrict__ scale,
+                const int32_t* __restrict__ zp, float lo, float hi) {
+  for (int64_t i = begin + (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kThreads) {
+    int64_t c = per_channel ? (i / inner) % nch : 0;
+    out[i] = (uint8_t)(quant_one<ROUND>(x[i], scale[c], (float)zp[c], lo, hi) & 0xff);
+  }
+}
+
+__global__ void __launch_bounds__(kThreads)
+dequantize_scalar(const uint8_t* __restrict__ q, float* __restrict__ out,
+                  int64_t begin, int64_t n, int64_t nch, int64_t inner,
+                  int per_channel, const float* __restrict__ scale,
+                  const int32_t* __restrict__ zp, int is_signed) {
+  for (int64_t i = begin + (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kThreads) {
+    int64_t c = per_channel ? (i / inner) % nch : 0;
+    int v = is_signed ? (int)(int8_t)q[i] : (int)q[i];
+    out[i] = (float)(v - zp[c]) * scale[c];
+  }
+}
+
+int grid_for(int64_t work_items, int per_thread) {
+  // enough blocks to cover the work with `per_thread` items per thread, capped at
+  // 16 blocks per CU (256 CUs) so the grid-stride loops keep loads in flight
+  int64_t blocks = dq8::ceil_div(work_items, (int64_t)kThreads * per_thread);
+  if (blocks < 1) blocks = 1;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  return (int)blocks;
+}
+
+}  // namespace
+
+extern "C" int dq8_quantize(const float* x, void* out, int out_kind,
+                            int64_t outer, int64_t nch, int64_t inner,
+                            const float* scale, const int32_t* zp, int64_t n_q,
+                            int32_t qmin, int32_t qmax, int round_mode,
+                            void* stream) {
+  dq8::clear_error();
+  DQ8_REQUIRE(outer >= 0 && nch >= 0 && inner >= 0, "dq8_quantize: negative size");
+  DQ8_REQUIRE(out_kind == DQ8_I8 || out_kind == DQ8_U8,
+              "dq8_quantize: out_kind must be DQ8_I8 or DQ8_U8");
+  DQ8_REQUIRE(round_mode == DQ8_ROUND_HALF_TO_EVEN ||
+                  round_mode == DQ8_ROUND_HALF_AWAY_FROM_ZERO,
+              "dq8_quantize: unknown round_mode");
+  DQ8_REQUIRE(n_q == 1 || n_q == nch, "dq8_quantize: n_q must be 1 or nch");
+  const int lim_lo = out_kind == DQ8_I8 ? -128 : 0;
+  const int lim_hi = out_kind == DQ8_I8 ? 127 : 255;
+  DQ8_REQUIRE(qmin <= qmax && qmin >= lim_lo && qmax <= lim_hi,
+              "dq8_quantize: quant_min/quant_max outside the output type");
+  const int64_t n = outer * nch * inner;
+  if (n == 0) return 0;
+  DQ8_REQUIRE(x && out && scale && zp, "dq8_quantize: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const float lo = (float)qmin, hi = (float)qmax;
+  const bool per_channel = n_q > 1;
+  const bool vec_ok = dq8::aligned(x, 16) && dq8::aligned(out, 4);
+  const bool rne = round_mode == DQ8_ROUND_HALF_TO_EVEN;
+
+#define LAUNCH_RND(kernel, grid, block, ...)                                        \
+  do {                                                                              \
+    if (rne)                                                                        \
+      hipLaunchKernelGGL((kernel<DQ8_ROUND_HALF_TO_EVEN>), grid, block, 0, st,      \
+                         __VA_ARGS__);                                              \
+    else                                                                            \
+      hipLaunchKernelGGL((kernel<DQ8_ROUND_HALF_AWAY_FROM_ZERO>), grid, block, 0,   \
+                         st, __VA_ARGS__);                                          \
+  } while (0)
+
+  if (!per_channel) {
+    const int64_t n4 = vec_ok ? n / 4 : 0;
+    if (n4 > 0)
+      LAUNCH_RND(quantize_tensor_v4, dim3(grid_for(n4, 4)), dim3(kThreads),
+                 (const float4*)x, (uint32_t*)out, n4, scale, zp, lo, hi);
+    if (n4 * 4 < n)
+      LAUNCH_RND(quantize_scalar, dim3(grid_for(n - n4 * 4, 1)), dim3(kThreads), x,
+                 (uint8_t*)out, n4 * 4, n, (int64_t)1, (int64_t)1, 0, scale, zp, lo, hi);
+  } else if (vec_ok && inner == 1 && nch % 4 == 0 && nch / 4 < (1 << 30) &&
+             dq8::aligned(scale, 16) && dq8::aligned(zp, 16)) {
+    const int nch4 = (int)(nch / 4);
+    int bx = nch4 >= kThreads ? kThreads : (int)(dq8::ceil_div(nch4, 64) * 64);
+    int gx = (int)dq8::ceil_div(nch4, bx);
+    // about 4096 blocks in flight, at least 8 rows each, grid.y <= 65535
+    int64_t rpb = dq8::ceil_div(outer * gx, 4096);
+    if (rpb < 8) rpb = 8;
+    if (dq8::ceil_div(outer, rpb) > 65535) rpb = dq8::ceil_div(outer, 65535);
+    int gy = (int)dq8::ceil_div(outer, rpb);
+    LAUNCH_RND(quantize_lastaxis_v4, dim3(gx, gy), dim3(bx), (const float4*)x,
+               (uint32_t*)out, outer, nch4, (int)rpb, (const float4*)scale,
+               (const int4*)zp, lo, hi);
+  } else if (vec_ok && inner % 4 == 0 && nch < (1LL << 31)) {
+    const int64_t rows = outer * nch;
+    const int64_t inner4 = inner / 4;
+    int gx = (int)std::min<int64_t>(dq8::ceil_div(inner4, kThreads), 1024);
+    int gy = (int)std::min<int64_t>(rows, 32768);
+    int64_t gz = dq8::ceil_div(rows, gy);
+    DQ8_REQUIRE(gz <= 65535, "dq8_quantize: too many rows for one launch");
+    LAUNCH_RND(quantize_rows_v4, dim3(gx, gy, (unsigned)gz), dim3(kThreads),
+               (const float4*)x, (uint32_t*)out, rows, inner4, (int)nch, scale, zp,
+               lo, hi);
+  } else {
+    LAUNCH_RND(quantize_scalar, dim3(grid_for(n, 1)), dim3(kThreads), x,
+               (uint8_t*)out, (int64_t)0, n, nch, inner, 1, scale, zp, lo, hi);
+  }
+#undef LAUNCH_RND
+  return dq8::check_hip(hipGetLastError(), "dq8_quantize launch");
+}
+
+extern "C" int dq8_dequantize(const void* q, int in_kind, float* out,
+                              int64_t outer, int64_t nch, int64_t inner,
+                              const float* scale, const int32_t* zp,
+                              int64_t n_q, void* stream) {
+  dq8::clear_error();
+  DQ8_REQUIRE(outer >= 0 && nch >= 0 && inner >= 0, "dq8_dequantize: negative size");
+  DQ8_REQUIRE(in_kind == DQ8_I8 || in_kind == DQ8_U8,
+              "dq8_dequantize: in_kind must be DQ8_I8 or DQ8_U8");
+  DQ8_REQUIRE(n_q == 1 || n_q == nch, "dq8_dequantize: n_q must be 1 or nch");
+  const int64_t n = outer * nch * inner;
+  if (n == 0) return 0;
+  DQ8_REQUIRE(q && out && scale && zp, "dq8_dequantize: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int is_signed = in_kind == DQ8_I8;
+  const bool per_channel = n_q > 1;
+  const bool vec_ok = dq8::aligned(q, 4) && dq8::aligned(out, 16);
+
+  if (!per_channel) {
+    const int64_t n4 = vec_ok ? n / 4 : 0;
+    if (n4 > 0)
+      hipLaunchKernelGGL(dequantize_tensor_v4, dim3(grid_for(n4, 4)), dim3(kThreads),
+                         0, st, (const uint32_t*)q, (float4*)out, n4, scale, zp,
+                         is_signed);
+    if (n4 * 4 < n)
+      hipLaunchKernelGGL(dequantize_scalar, dim3(grid_for(n - n4 * 4, 1)),
+                         dim3(kThreads), 0, st, (const uint8_t*)q, out, n4 * 4, n,
+                         (int64_t)1, (int64_t)1, 0, scale, zp, is_signed);
+  } else if (vec_ok && inner == 1 && nch % 4 == 0 && nch / 4 < (1 << 30) &&
+             dq8::aligned(scale, 16) && dq8::aligned(zp, 16)) {
+    const int nch4 = (int)(nch / 4);
+    int bx = nch4 >= kThreads ? kThreads : (int)(dq8::ceil_div(nch4, 64) * 64);
+    int gx = (int)dq8::ceil_div(nch4, bx);
+    int64_t rpb = dq8::ceil_div(outer * gx, 4096);
+    if (rpb < 8) rpb = 8;
+    if (dq8::ceil_div(outer, rpb) > 65535) rpb = dq8::ceil_div(outer, 65535);
+    int gy = (int)dq8::ceil_div(outer, rpb);
+    hipLaunchKernelGGL(dequantize_lastaxis_v4, dim3(gx, gy), dim3(bx), 0, st,
+                       (const uint32_t*)q, (float4*)out, outer, nch4, (int)rpb,
+                       (const float4*)scale, (const int4*)zp, is_signed);
+  } else if (vec_ok && inner % 4 == 0 && nch < (1LL << 31)) {
+    const int64_t rows = outer * nch;
+    const int64_t inner4 = inner / 4;
+    int gx = (int)std::min<int64_t>(dq8::ceil_div(inner4, kThreads), 1024);
+    int gy = (int)std::min<int64_t>(rows, 32768);
+    int64_t gz = dq8::ceil_div(rows, gy);
+    DQ8_REQUIRE(gz <= 65535, "dq8_dequantize: too many rows for one launch");
+    hipLaunchKernelGGL(dequantize_rows_v4, dim3(gx, gy, (unsigned)gz), dim3(kThreads),
+                       0, st, (const uint32_t*)q, (float4*)out, rows, inner4,
+                       (int)nch, scale, zp, is_signed);
+  } else {
+    hipLaunchKernelGGL(dequantize_scalar, dim3(grid_for(n, 1)), dim3(kThreads), 0,
+                       st, (const uint8_t*)q, out, (int64_t)0, n, nch, inner, 1,
+                       scale, zp, is_signed);
+  }
+  return dq8::check_hip(hipGetLastError(), "dq8_dequantize launch");
+}

@@ -1,0 +1,158 @@
+"""torch-tensor front-end of the raw kernel C ABI (include/disc_q8.h).
+
+PyTorch only supplies device memory and the current stream here; every function
+launches the hand-written HIP kernels in libdisc_q8_ral.so.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+EPI_ACC_S32, EPI_REQUANT_CPU, EPI_REQUANT_GPU, EPI_DEQUANT_F32 = 0, 1, 2, 3
+BIAS_NONE, BIAS_S32, BIAS_F32, BIAS_S8 = 0, 1, 2, 3
+ROUND_HALF_AWAY_FROM_ZERO, ROUND_HALF_TO_EVEN = 0, 1
+
+_BIAS_KIND = {torch.int32: BIAS_S32, torch.float32: BIAS_F32, torch.int8: BIAS_S8}
+_OUT_DTYPE = {EPI_ACC_S32: torch.int32, EPI_REQUANT_CPU: torch.int8,
+              EPI_REQUANT_GPU: torch.int8, EPI_DEQUANT_F32: torch.float32}
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("expected device tensors")
+
+
+def _scale(t, device):
+    if not torch.is_tensor(t):
+        t = torch.tensor(t, dtype=torch.float32, device=device)
+    return t.reshape(-1).contiguous().float()
+
+
+def variant_names():
+    L = _lib.lib()
+    return [L.dq8_qgemm_variant_name(i).decode() for i in range(L.dq8_qgemm_num_variants())]
+
+
+def _view3(shape, axis):
+    n = 1
+    for s in shape:
+        n *= s
+    if axis is None:
+        return 1, 1, n
+    outer = 1
+    for s in shape[:axis]:
+        outer *= s
+    inner = 1
+    for s in shape[axis + 1:]:
+        inner *= s
+    return outer, shape[axis], inner
+
+
+def quantize(x, scale, zero_point, axis=None, qmin=-128, qmax=127,
+             round_mode=ROUND_HALF_TO_EVEN, dtype=torch.int8, out=None):
+    """mhlo_disc.quantize on the GPU.  scale/zero_point: device tensors (f32 / i32)."""
+    _need_cuda(x, scale, zero_point)
+    x = x.contiguous()
+    outer, nch, inner = _view3(tuple(x.shape), axis)
+    if out is None:
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    kind = 0 if out.dtype == torch.int8 else 1
+    n_q = scale.numel() if axis is not None else 1
+    st = _lib.lib().dq8_quantize(_ptr(x), _ptr(out), kind, outer, nch, inner, _ptr(scale),
+                                 _ptr(zero_point), n_q, qmin, qmax, round_mode, _stream())
+    _lib.check(st, "dq8_quantize")
+    return out
+
+
+def dequantize(q, scale, zero_point, axis=None, out=None):
+    _need_cuda(q, scale, zero_point)
+    q = q.contiguous()
+    outer, nch, inner = _view3(tuple(q.shape), axis)
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    kind = 0 if q.dtype == torch.int8 else 1
+    n_q = scale.numel() if axis is not None else 1
+    st = _lib.lib().dq8_dequantize(_ptr(q), kind, _ptr(out), outer, nch, inner, _ptr(scale),
+                                   _ptr(zero_point), n_q, _stream())
+    _lib.check(st, "dq8_dequantize")
+    return out
+
+
+def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b=True,
+          zx=0, zw=0, zo=0, variant=-1, out=None):
+    """int8 GEMM with a fused epilogue.  a: [M,K] ([K,M] if tp_a); w: [N,K] if tp_b
+    else [K,N]; scales are device f32 tensors with 1 or N entries."""
+    _need_cuda(a, w, bias)
+    L = _lib.lib()
+    a = a.contiguous()
+    w = w.contiguous()
+    m, k = (a.shape[1], a.shape[0]) if tp_a else a.shape
+    n = w.shape[0] if tp_b else w.shape[1]
+    kw = w.shape[1] if tp_b else w.shape[0]
+    if k != kw:
+        raise ValueError("mismatch contraction dim")
+    dev = a.device
+    if out is None:
+        out = torch.empty((m, n), dtype=_OUT_DTYPE[epilogue], device=dev)
+    sx = _scale(sx, dev) if sx is not None else None
+    sw = _scale(sw, dev) if sw is not None else None
+    so = _scale(so, dev) if so is not None else None
+    bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
+    ws_bytes = L.dq8_qgemm_workspace_bytes(m, n, k, int(tp_a), int(tp_b))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    st = L.dq8_qgemm_variant(
+        variant, _ptr(a), a.shape[1], _ptr(w), w.shape[1], _ptr(out), out.stride(0) if m else n,
+        m, n, k, int(tp_a), int(tp_b), epilogue, _ptr(bias), bias_kind,
+        _ptr(sx), sx.numel() if sx is not None else 0,
+        _ptr(sw), sw.numel() if sw is not None else 0,
+        _ptr(so), so.numel() if so is not None else 0,
+        zx, zw, zo, _ptr(ws), ws_bytes, _stream())
+    _lib.check(st, "dq8_qgemm")
+    return out
+
+
+NHWC_OHWI = (0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2)
+
+
+def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=None,
+            bias=None, zo=0, variant=-1, out=None):
+    """int8 convolution; layouts/strides/dilations from the 17-entry ral_qconv
+    metadata, padding = (top, bottom, left, right)."""
+    _need_cuda(x, w, bias)
+    L = _lib.lib()
+    x = x.contiguous()
+    w = w.contiguous()
+    dev = x.device
+    if out is None:
+        out = torch.empty(tuple(out_shape), dtype=_OUT_DTYPE[epilogue], device=dev)
+    sx = _scale(sx, dev) if sx is not None else None
+    sw = _scale(sw, dev) if sw is not None else None
+    so = _scale(so, dev) if so is not None else None
+    bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
+    i64x4 = C.c_int64 * 4
+    st = L.dq8_qconv2d_variant(
+        variant, _ptr(x), i64x4(*x.shape), _ptr(w), i64x4(*w.shape),
+        (C.c_int32 * 4)(*padding), (C.c_int32 * 17)(*metadata), _ptr(out),
+        i64x4(*out_shape), epilogue, _ptr(bias), bias_kind, _ptr(sx), _ptr(sw),
+        sw.numel() if sw is not None else 0, _ptr(so), zo, _stream())
+    _lib.check(st, "dq8_qconv2d")
+    return out
+
+
+def mfma_probe(a32, b32, a16, b16):
+    d32 = torch.empty((32, 32), dtype=torch.int32, device=a32.device)
+    d16 = torch.empty((16, 16), dtype=torch.int32, device=a32.device)
+    st = _lib.lib().dq8_mfma_probe(_ptr(a32), _ptr(b32), _ptr(d32), _ptr(a16), _ptr(b16),
+                                   _ptr(d16), _stream())
+    _lib.check(st, "dq8_mfma_probe")
+    return d32, d16

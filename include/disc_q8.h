@@ -1,0 +1,159 @@
+/*
+ * disc_q8.h -- C ABI of the MI355X (gfx950) quantized-inference kernels.
+ *
+ * These are the launchers the RAL entries in include/tao_ral_api.h are built on.
+ * Every pointer marked "device" is HBM-resident; nothing here dereferences a
+ * device pointer on the host, synchronises a stream, or allocates memory.
+ * All launches go to `stream` (a hipStream_t passed as void*; NULL = the null
+ * stream).  Return value: 0 on success, non-zero on error with the message
+ * available from dq8_last_error() (thread-local).
+ *
+ * Reference interfaces replaced (R = alibaba/BladeDISC, tao_compiler/mlir/):
+ *   dq8_qgemm      -> the vendor GEMM behind ral_qgemm
+ *                     (R ral/context/stream_executor_based_impl.cc:427-483, bladnn::gemm)
+ *                     and behind ral_pdll_qgemm[_per_channel]
+ *                     (R ral/context/quantized_gpu_kernel_impl.cc:129-158 cublasLtMatmul,
+ *                     :197-321, :329-422), plus the CPU-signature variants
+ *                     (R ral/context/common_context_impl_quantization.cc:1196-1672).
+ *   dq8_qconv2d    -> the fused int8 convolution behind ral_qconv
+ *                     (R ral/context/stream_executor_based_impl.cc:1506-1588, 1831-1948).
+ *   dq8_quantize / dq8_dequantize
+ *                  -> the loops the compiler generates from mhlo_disc.quantize /
+ *                     mhlo_disc.dequantize
+ *                     (R disc/transforms/disc_lower_quantize_and_dequantize.cc:36-139, 141-215).
+ */
+#ifndef DISC_Q8_H_
+#define DISC_Q8_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- enums (plain ints in the ABI) ------------------------------------ */
+
+/* epilogue applied to the int32 accumulators */
+#define DQ8_EPI_ACC_S32 0     /* out: int32  acc                                          */
+#define DQ8_EPI_REQUANT_CPU 1 /* out: int8   sat(rne((f32(acc)+b32[n])*os[n] + zo))        */
+#define DQ8_EPI_REQUANT_GPU 2 /* out: int8   sat(rne(os[n]*f32(acc) + bias[n]))            */
+#define DQ8_EPI_DEQUANT_F32 3 /* out: float  f32(acc)*(sx*sw[n]) + bias[n]                 */
+/* os[n] = (sx*sw[n])/so evaluated in binary32, left to right.                            */
+
+/* bias operand kinds */
+#define DQ8_BIAS_NONE 0
+#define DQ8_BIAS_S32 1 /* REQUANT_CPU: used as is                                          */
+#define DQ8_BIAS_F32 2 /* REQUANT_CPU: b32 = sat32(rne(bias/(sx*sw[n]))) first;
+                          REQUANT_GPU / DEQUANT_F32: added as is                           */
+#define DQ8_BIAS_S8 3  /* REQUANT_GPU: (float)bias                                          */
+
+/* element kinds of quantized tensors */
+#define DQ8_I8 0
+#define DQ8_U8 1
+
+/* mhlo_disc round_mode (R disc/IR/hlo_disc_enums.td) */
+#define DQ8_ROUND_HALF_AWAY_FROM_ZERO 0
+#define DQ8_ROUND_HALF_TO_EVEN 1
+
+/* ---- library ---------------------------------------------------------- */
+
+const char* dq8_last_error(void);
+/* packed version: major*10000 + minor*100 + patch */
+int dq8_version(void);
+/* Number of compute units / LDS bytes / clock the library sees on the current
+ * device; fills what it can, returns 0 on success. */
+int dq8_device_info(int* compute_units, int* lds_bytes_per_cu, int* clock_khz);
+
+/* ---- quantize / dequantize -------------------------------------------- */
+
+/* x (device, f32) is viewed as [outer, nch, inner]; scale (device f32) and zp
+ * (device i32) hold n_q = 1 (per tensor) or nch (per channel along the middle
+ * axis) entries.  out[i] = convert(clamp(round(x[i]/scale + (f32)zp), qmin, qmax)). */
+int dq8_quantize(const float* x, void* out, int out_kind, int64_t outer,
+                 int64_t nch, int64_t inner, const float* scale,
+                 const int32_t* zp, int64_t n_q, int32_t qmin, int32_t qmax,
+                 int round_mode, void* stream);
+
+/* out[i] = (f32)((i32)q[i] - zp) * scale */
+int dq8_dequantize(const void* q, int in_kind, float* out, int64_t outer,
+                   int64_t nch, int64_t inner, const float* scale,
+                   const int32_t* zp, int64_t n_q, void* stream);
+
+/* ---- int8 GEMM -------------------------------------------------------- */
+
+/* Bytes of device scratch dq8_qgemm needs for this problem (0 when it needs
+ * none: tp_a == 0 and tp_b == 1 and no zero points). */
+size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
+                                 int tp_b);
+
+/* out[M,N] = epilogue( sum_k A(m,k) * W(k,n) ).
+ *   A: device int8, [M,K] with row stride lda (tp_a = 0) or [K,M] with row
+ *      stride lda (tp_a = 1).
+ *   W: device int8, [N,K] row stride ldw (tp_b = 1, the GPU callers' layout) or
+ *      [K,N] row stride ldw (tp_b = 0, the CPU callers' layout).
+ *   out: device, element type per `epilogue`, row stride ldo (elements).
+ *   sx / sw / so: device f32 with n_sx / n_sw / n_so entries, each 1 or N.
+ *   zo: output zero point (REQUANT_CPU only).  Input and weight zero points must
+ *      be 0 (every reference caller is symmetric); non-zero is rejected.
+ *   workspace: device scratch of at least dq8_qgemm_workspace_bytes(), may be
+ *      NULL when that is 0.
+ * M == 0, N == 0 launch nothing and succeed; K == 0 yields epilogue(0). */
+int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
+              void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int tp_a,
+              int tp_b, int epilogue, const void* bias, int bias_kind,
+              const float* sx, int64_t n_sx, const float* sw, int64_t n_sw,
+              const float* so, int64_t n_so, int32_t zx, int32_t zw, int32_t zo,
+              void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same, forcing one kernel variant (for tests and tuning):
+ *  -1 heuristic, 0 generic scalar kernel, 1.. MFMA tile configurations
+ *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()). */
+int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
+                      const int8_t* W, int64_t ldw, void* out, int64_t ldo,
+                      int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
+                      int epilogue, const void* bias, int bias_kind,
+                      const float* sx, int64_t n_sx, const float* sw,
+                      int64_t n_sw, const float* so, int64_t n_so, int32_t zx,
+                      int32_t zw, int32_t zo, void* workspace,
+                      size_t workspace_bytes, void* stream);
+int dq8_qgemm_num_variants(void);
+const char* dq8_qgemm_variant_name(int variant);
+
+/* ---- int8 convolution (rank 4) ---------------------------------------- */
+
+/* Implicit-GEMM convolution.  Layouts are described exactly as ral_qconv's
+ * metadata vector describes them (17 host int32: input {batch,channel,h,w} dim
+ * indices, kernel {in,out,h,w}, output {batch,channel,h,w}, strides[2],
+ * dilations[2], weight_is_const) with host padding {top,bottom,left,right}.
+ * The MFMA path takes NHWC x OHWI -> NHWC with Ci % 16 == 0; every other layout
+ * runs the generic kernel.  Epilogue/bias/scales as for dq8_qgemm with N = Co. */
+int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                const int64_t w_sizes[4], const int32_t padding[4],
+                const int32_t metadata[17], void* out,
+                const int64_t out_sizes[4], int epilogue, const void* bias,
+                int bias_kind, const float* sx, const float* sw, int64_t n_sw,
+                const float* so, int32_t zo, void* stream);
+int dq8_qconv2d_variant(int variant, const int8_t* in,
+                        const int64_t in_sizes[4], const int8_t* w,
+                        const int64_t w_sizes[4], const int32_t padding[4],
+                        const int32_t metadata[17], void* out,
+                        const int64_t out_sizes[4], int epilogue,
+                        const void* bias, int bias_kind, const float* sx,
+                        const float* sw, int64_t n_sw, const float* so,
+                        int32_t zo, void* stream);
+
+/* ---- self-test hook ---------------------------------------------------- */
+
+/* Runs one v_mfma_i32_32x32x32_i8 and one v_mfma_i32_16x16x64_i8 on device
+ * buffers: a[32*32] (row i, k contiguous), b[32*32] (column j, k contiguous) ->
+ * d32[32*32] row-major; a16[16*64], b16[16*64] -> d16[16*16].  Lets a test pin
+ * the operand and result register layouts against brute force. */
+int dq8_mfma_probe(const int8_t* a, const int8_t* b, int32_t* d32,
+                   const int8_t* a16, const int8_t* b16, int32_t* d16,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DISC_Q8_H_ */
