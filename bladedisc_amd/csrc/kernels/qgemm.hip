@@ -280,6 +280,19 @@ extern "C" size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int
   return bytes;
 }
 
+extern "C" int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
+                                int64_t cols, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(rows >= 0 && cols >= 0 && ld >= cols, "dq8_transpose_s8: bad shape");
+  DQ8_REQUIRE(rows < (1LL << 31) && cols < (1LL << 31), "dq8_transpose_s8: too large");
+  if (rows == 0 || cols == 0) return 0;
+  DQ8_REQUIRE(src && dst, "dq8_transpose_s8: null pointer");
+  hipLaunchKernelGGL(transpose_s8_kernel,
+                     dim3((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(rows, 64)), dim3(256),
+                     0, (hipStream_t)stream, src, ld, dst, (int)rows, (int)cols);
+  return check_hip(hipGetLastError(), "dq8_transpose_s8 launch");
+}
+
 extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                                  const int8_t* W, int64_t ldw, void* out, int64_t ldo,
                                  int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,

@@ -1,0 +1,355 @@
+#include "mlir/ral/context/base/hip/hip_context_impl.h"
+
+#include <mutex>
+#include <sstream>
+#include <unordered_set>
+
+#include "mlir/ral/ral_helper.h"
+#include "mlir/ral/ral_logging.h"
+
+namespace tao {
+namespace ral {
+
+BaseContext::BaseContext(BaseContextOption& opt) : opt_(opt) {}
+BaseContext::~BaseContext() = default;
+
+// ------------------------------------------------------------ InternalAllocator
+InternalAllocator::InternalAllocator(alloc_t alloc_func, dealloc_t dealloc_func)
+    : alloc_func_(std::move(alloc_func)), dealloc_func_(std::move(dealloc_func)) {}
+
+InternalAllocator::~InternalAllocator() {
+  releaseAllFreeBuffers();
+  // anything still live is returned too: the context is going away
+  for (auto& kv : class_of_) dealloc_func_(kv.first);
+}
+
+size_t InternalAllocator::sizeClass(size_t bytes) {
+  constexpr size_t kMin = 256;
+  if (bytes <= kMin) return kMin;
+  size_t pow2 = kMin;
+  while (pow2 < bytes) pow2 <<= 1;        // smallest power of two >= bytes
+  const size_t quarter = pow2 >> 3;       // steps of 1/4 of the lower power
+  size_t cls = pow2 >> 1;
+  while (cls < bytes) cls += quarter;
+  return cls;
+}
+
+void InternalAllocator::releaseAllFreeBuffers() {
+  for (auto& kv : free_by_class_)
+    for (buffer_t b : kv.second) {
+      dealloc_func_(b);
+      class_of_.erase(b);
+    }
+  free_by_class_.clear();
+  pooled_bytes_ = 0;
+}
+
+buffer_t InternalAllocator::alloc(size_t bytes) {
+  const size_t cls = sizeClass(bytes);
+  auto it = free_by_class_.find(cls);
+  if (it != free_by_class_.end() && !it->second.empty()) {
+    buffer_t b = it->second.back();
+    it->second.pop_back();
+    pooled_bytes_ -= cls;
+    live_bytes_ += cls;
+    return b;
+  }
+  buffer_t b = alloc_func_(cls);
+  if (!b) {  // give the pool back to the device and retry once
+    releaseAllFreeBuffers();
+    b = alloc_func_(cls);
+    if (!b) return nullptr;
+  }
+  class_of_[b] = cls;
+  live_bytes_ += cls;
+  return b;
+}
+
+void InternalAllocator::dealloc(buffer_t buffer) {
+  auto it = class_of_.find(buffer);
+  if (it == class_of_.end()) return;  // not ours
+  free_by_class_[it->second].push_back(buffer);
+  live_bytes_ -= it->second;
+  pooled_bytes_ += it->second;
+}
+
+namespace gpu {
+
+const char* kRalBaseHipContextState = "ral_base_hip_context_state";
+
+namespace {
+
+bool hipOk(hipError_t e, ExecutionContext* ctx, const char* where) {
+  if (e == hipSuccess) return true;
+  std::ostringstream out;
+  out << "GPU failed with " << hipGetErrorString(e) << " in " << where;
+  ctx->signalError(Context::FAILURE, out.str());
+  return false;
+}
+
+struct BaseHipContextState : public Context::Resource {
+  std::mutex mu;
+  GpuStreamHandle stream = nullptr;
+  int device_ordinal = 0;
+  std::shared_ptr<Allocator> gpu_allocator;
+  bool cache_workspace_mem_across_execution = false;
+  std::unordered_set<const_buffer_t> device_persistent_buffers;
+  // code objects of compiler-generated kernels: blob -> module, (blob,name) -> fn
+  std::map<void*, hipModule_t> modules;
+  std::map<std::pair<void*, std::string>, hipFunction_t> functions;
+
+  void onExecutionFinish(ExecutionContext*) override {
+    std::lock_guard<std::mutex> guard(mu);
+    if (!cache_workspace_mem_across_execution) gpu_allocator->releaseAllFreeBuffers();
+  }
+
+  void onContextFinish(Context*) override {
+    (void)hipStreamSynchronize(stream);
+    for (const_buffer_t b : device_persistent_buffers)
+      gpu_allocator->dealloc(const_cast<buffer_t>(b));
+    device_persistent_buffers.clear();
+    for (auto& kv : modules) (void)hipModuleUnload(kv.second);
+    modules.clear();
+    functions.clear();
+    gpu_allocator->releaseAllFreeBuffers();
+  }
+};
+
+BaseHipContextState* stateOf(ExecutionContext* ctx) {
+  return ctx->getResource<BaseHipContextState>(kRalBaseHipContextState);
+}
+
+bool validStream(ExecutionContext* ctx, stream_t sidx) {
+  if (reinterpret_cast<intptr_t>(sidx) == 0) return true;
+  ctx->signalError(Context::FAILURE, "not a valid stream idx");
+  return false;
+}
+
+// ---------------------------------------------------------- driver functions
+buffer_t ral_base_hip_alloc(ExecutionContext* ctx, size_t bytes) {
+  auto* state = stateOf(ctx);
+  if (!state) return nullptr;
+  auto* exec = dynamic_cast<BaseHipExecutionContext*>(ctx);
+  if (!exec) {
+    ctx->signalError(Context::FAILURE, "alloc needs a BaseHipExecutionContext");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(state->mu);
+  void* ptr = state->gpu_allocator->alloc(bytes ? bytes : 1);
+  if (!ptr) {
+    ctx->signalError(Context::FAILURE, "device allocation of " + std::to_string(bytes) +
+                                           " bytes failed");
+    return nullptr;
+  }
+  exec->device_ptr_map[ptr] = 1;
+  return ptr;
+}
+
+buffer_t ral_base_hip_alloc_persistent(ExecutionContext* ctx, size_t bytes) {
+  auto* state = stateOf(ctx);
+  if (!state) return nullptr;
+  std::lock_guard<std::mutex> guard(state->mu);
+  void* ptr = state->gpu_allocator->alloc(bytes ? bytes : 1);
+  if (!ptr) {
+    ctx->signalError(Context::FAILURE, "persistent device allocation of " +
+                                           std::to_string(bytes) + " bytes failed");
+    return nullptr;
+  }
+  state->device_persistent_buffers.insert(ptr);
+  return ptr;
+}
+
+void ral_base_hip_dealloc(ExecutionContext* ctx, buffer_t buffer) {
+  if (!buffer) return;
+  auto* state = stateOf(ctx);
+  if (!state) return;
+  auto* exec = dynamic_cast<BaseHipExecutionContext*>(ctx);
+  std::lock_guard<std::mutex> guard(state->mu);
+  if (state->device_persistent_buffers.count(buffer)) return;
+  if (!exec) return;
+  auto it = exec->device_ptr_map.find(buffer);
+  if (it == exec->device_ptr_map.end()) {
+    TAO_VLOG(1) << "dealloc: ignoring a buffer this execution did not allocate";
+    return;
+  }
+  if (--it->second == 0) {
+    state->gpu_allocator->dealloc(buffer);
+    exec->device_ptr_map.erase(it);
+  }
+}
+
+buffer_t ral_base_hip_raw_alloc(Context* ctx, size_t bytes) {
+  auto* state = static_cast<BaseHipContextState*>(
+      ctx->getOrCreateResource(kRalBaseHipContextState, nullptr).get());
+  if (!state) return nullptr;
+  std::lock_guard<std::mutex> guard(state->mu);
+  return state->gpu_allocator->alloc(bytes ? bytes : 1);
+}
+
+void ral_base_hip_raw_dealloc(Context* ctx, buffer_t buffer) {
+  if (!buffer) return;
+  auto* state = static_cast<BaseHipContextState*>(
+      ctx->getOrCreateResource(kRalBaseHipContextState, nullptr).get());
+  if (!state) return;
+  std::lock_guard<std::mutex> guard(state->mu);
+  state->gpu_allocator->dealloc(buffer);
+}
+
+void ral_base_hip_launch(ExecutionContext* ctx, void** blobs, size_t num_blobs,
+                         const char* kernel_name, intptr_t gridX, intptr_t gridY,
+                         intptr_t gridZ, intptr_t blockX, intptr_t blockY,
+                         intptr_t blockZ, int32_t smem, void* stream_handle,
+                         int32_t /*num_args*/, void** params) {
+  if (!blockX || !blockY || !blockZ || !gridX || !gridY || !gridZ) return;  // empty
+  auto* state = stateOf(ctx);
+  if (!state || !validStream(ctx, stream_handle)) return;
+  if (num_blobs < 1 || !blobs || !blobs[0]) {
+    ctx->signalError(Context::FAILURE, "ral_kernel_launch: no code object");
+    return;
+  }
+  // a DISC build for this runtime carries one gfx950 code object per kernel
+  void* blob = blobs[0];
+  hipFunction_t fn = nullptr;
+  {
+    std::lock_guard<std::mutex> guard(state->mu);
+    auto key = std::make_pair(blob, std::string(kernel_name));
+    auto fit = state->functions.find(key);
+    if (fit == state->functions.end()) {
+      auto mit = state->modules.find(blob);
+      if (mit == state->modules.end()) {
+        hipModule_t mod = nullptr;
+        if (!hipOk(hipModuleLoadData(&mod, blob), ctx, "ModuleLoad")) return;
+        mit = state->modules.emplace(blob, mod).first;
+      }
+      if (!hipOk(hipModuleGetFunction(&fn, mit->second, kernel_name), ctx, "GetFunction"))
+        return;
+      fit = state->functions.emplace(key, fn).first;
+    }
+    fn = fit->second;
+  }
+  hipOk(hipModuleLaunchKernel(fn, (unsigned)gridX, (unsigned)gridY, (unsigned)gridZ,
+                              (unsigned)blockX, (unsigned)blockY, (unsigned)blockZ,
+                              (unsigned)smem, state->stream, params, nullptr),
+        ctx, "LaunchKernel");
+}
+
+stream_t ral_base_hip_get_stream(ExecutionContext* ctx, int32_t stream_id) {
+  if (stream_id < 0) {
+    ctx->signalError(Context::FAILURE, "not a valid stream_id");
+    return nullptr;
+  }
+  if (stream_id > 0) {
+    ctx->signalError(Context::FAILURE, "multi-stream not supported");
+    return nullptr;
+  }
+  return reinterpret_cast<stream_t>(static_cast<intptr_t>(stream_id));
+}
+
+opaque_t ral_base_hip_as_cu_stream(ExecutionContext* ctx, stream_t) {
+  auto* state = stateOf(ctx);
+  return state ? state->stream : nullptr;
+}
+
+opaque_t ral_base_hip_as_se_stream(ExecutionContext*, stream_t) { return nullptr; }
+
+void ral_base_hip_d2d(ExecutionContext* ctx, stream_t sidx, buffer_t from, buffer_t to,
+                      size_t bytes) {
+  auto* state = stateOf(ctx);
+  if (!state || !validStream(ctx, sidx) || !bytes) return;
+  hipOk(hipMemcpyAsync(to, from, bytes, hipMemcpyDeviceToDevice, state->stream), ctx, "d2d");
+}
+
+void ral_base_hip_d2h(ExecutionContext* ctx, stream_t sidx, buffer_t from, buffer_t to,
+                      size_t bytes) {
+  auto* state = stateOf(ctx);
+  if (!state || !validStream(ctx, sidx) || !bytes) return;
+  hipOk(hipMemcpyAsync(to, from, bytes, hipMemcpyDeviceToHost, state->stream), ctx, "d2h");
+}
+
+void ral_base_hip_h2d(ExecutionContext* ctx, stream_t sidx, const void* from, buffer_t to,
+                      size_t bytes) {
+  auto* state = stateOf(ctx);
+  if (!state || !validStream(ctx, sidx) || !bytes) return;
+  hipOk(hipMemcpyAsync(to, from, bytes, hipMemcpyHostToDevice, state->stream), ctx, "h2d");
+}
+
+void ral_base_hip_memset(ExecutionContext* ctx, stream_t sidx, buffer_t buffer, int value,
+                         size_t bytes) {
+  auto* state = stateOf(ctx);
+  if (!state || !validStream(ctx, sidx) || !buffer || !bytes) return;
+  hipOk(hipMemsetAsync(buffer, value, bytes, state->stream), ctx, "memset");
+}
+
+void ral_base_hip_sync_on_stream(ExecutionContext* ctx, stream_t sidx) {
+  auto* state = stateOf(ctx);
+  if (!state || !validStream(ctx, sidx)) return;
+  hipOk(hipStreamSynchronize(state->stream), ctx, "StreamSync");
+}
+
+void ral_base_hip_sync_all(ExecutionContext* ctx) {
+  hipOk(hipDeviceSynchronize(), ctx, "DeviceSync");
+}
+
+}  // namespace
+
+BaseHipExecutionContext::BaseHipExecutionContext(BaseContext* ctx)
+    : ExecutionContext(ctx) {
+  onExecutionStart();
+}
+
+BaseHipExecutionContext::~BaseHipExecutionContext() {
+  // buffers the program never handed back return to the pool with the execution
+  auto* state = getResource<BaseHipContextState>(kRalBaseHipContextState);
+  if (state) {
+    std::lock_guard<std::mutex> guard(state->mu);
+    for (auto& kv : device_ptr_map)
+      state->gpu_allocator->dealloc(const_cast<buffer_t>(kv.first));
+  }
+  device_ptr_map.clear();
+  onExecutionFinish();
+}
+
+std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
+                                                BaseHipContextOption& gpu_opt) {
+  std::unique_ptr<BaseContext> ctx(new BaseContext(opt));
+  ctx->addDriver(GPUDriver::name(), std::unique_ptr<GPUDriver>(new GPUDriver(ctx.get())));
+  ctx->getOrCreateResource(kRalBaseHipContextState, [opt, gpu_opt]() {
+    auto* state = new BaseHipContextState;
+    state->stream = gpu_opt.stream;
+    state->device_ordinal = gpu_opt.device_ordinal;
+    state->cache_workspace_mem_across_execution = opt.cache_workspace_mem_across_execution;
+    if (gpu_opt.gpu_allocator) {
+      state->gpu_allocator = gpu_opt.gpu_allocator;
+    } else {
+      state->gpu_allocator.reset(new InternalAllocator(
+          [](size_t bytes) -> buffer_t {
+            void* p = nullptr;
+            return hipMalloc(&p, bytes) == hipSuccess ? p : nullptr;
+          },
+          [](buffer_t p) { (void)hipFree(p); }));
+    }
+    return state;
+  });
+  return ctx;
+}
+
+}  // namespace gpu
+
+TAO_RAL_API(tao::ral::gpu::kRalGpuAlloc, "gpu", gpu::ral_base_hip_alloc);
+TAO_RAL_API(tao::ral::gpu::kRalGpuAllocPersistent, "gpu", gpu::ral_base_hip_alloc_persistent);
+TAO_RAL_API(tao::ral::gpu::kRalGpuDealloc, "gpu", gpu::ral_base_hip_dealloc);
+TAO_RAL_API(tao::ral::gpu::kRalGpuRawAlloc, "gpu", gpu::ral_base_hip_raw_alloc);
+TAO_RAL_API(tao::ral::gpu::kRalGpuRawDealloc, "gpu", gpu::ral_base_hip_raw_dealloc);
+TAO_RAL_API(tao::ral::gpu::kRalGpuLaunch, "gpu", gpu::ral_base_hip_launch);
+TAO_RAL_API(tao::ral::gpu::kRalGpuGetStream, "gpu", gpu::ral_base_hip_get_stream);
+TAO_RAL_API(tao::ral::gpu::kRalGpuAsCUStream, "gpu", gpu::ral_base_hip_as_cu_stream);
+TAO_RAL_API(tao::ral::gpu::kRalGpuAsSEStream, "gpu", gpu::ral_base_hip_as_se_stream);
+TAO_RAL_API(tao::ral::gpu::kRalGpuH2D, "gpu", gpu::ral_base_hip_h2d);
+TAO_RAL_API(tao::ral::gpu::kRalGpuD2H, "gpu", gpu::ral_base_hip_d2h);
+TAO_RAL_API(tao::ral::gpu::kRalGpuD2D, "gpu", gpu::ral_base_hip_d2d);
+TAO_RAL_API(tao::ral::gpu::kRalGpuSyncOnStream, "gpu", gpu::ral_base_hip_sync_on_stream);
+TAO_RAL_API(tao::ral::gpu::kRalGpuSyncAll, "gpu", gpu::ral_base_hip_sync_all);
+TAO_RAL_API(tao::ral::gpu::kRalGpuMemset, "gpu", gpu::ral_base_hip_memset);
+
+}  // namespace ral
+}  // namespace tao

@@ -1,0 +1,96 @@
+// The concrete RAL context for one AMD GPU: device memory with a size-class pool,
+// one hipStream_t for every copy and launch, and the gpu driver function set
+// registered under the names GPUDriver resolves.  Counterpart of the reference's
+// tao_compiler/mlir/ral/context/base/cuda/cuda_context_impl.{h,cc} (options :52-60,
+// driver functions :258-510, registrations :746-764) and of
+// context/base/base_context.{h,cc} (BaseContext, InternalAllocator).
+#ifndef RAL_CONTEXT_BASE_HIP_HIP_CONTEXT_IMPL_H_
+#define RAL_CONTEXT_BASE_HIP_HIP_CONTEXT_IMPL_H_
+
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "mlir/ral/device/gpu/gpu_driver.h"
+#include "mlir/ral/ral_base.h"
+#include "mlir/ral/ral_context.h"
+
+namespace tao {
+namespace ral {
+
+struct BaseContextOption {
+  // Path of the compiled program's constant store.  Empty is allowed: kernels can
+  // then be exercised without a compiled model.
+  std::string metadata_file_path;
+  bool cache_workspace_mem_across_execution = false;
+};
+
+class BaseContext : public Context {
+ public:
+  explicit BaseContext(BaseContextOption& opt);
+  ~BaseContext() override;
+  const BaseContextOption& option() const { return opt_; }
+
+ private:
+  BaseContextOption opt_;
+};
+
+// Pooling allocator on top of a raw alloc/dealloc pair.  Requests are rounded up
+// to a size class (four classes per power of two, so at most 25 % slack) and freed
+// blocks are kept per class: with a dynamic M every call asks for a different byte
+// count, and exact-size free lists would never hit.
+class InternalAllocator : public Allocator {
+ public:
+  InternalAllocator(alloc_t alloc_func, dealloc_t dealloc_func);
+  ~InternalAllocator() override;
+
+  void releaseAllFreeBuffers() override;
+  buffer_t alloc(size_t bytes) override;
+  void dealloc(buffer_t buffer) override;
+
+  static size_t sizeClass(size_t bytes);
+  size_t liveBytes() const { return live_bytes_; }
+  size_t pooledBytes() const { return pooled_bytes_; }
+
+ private:
+  alloc_t alloc_func_;
+  dealloc_t dealloc_func_;
+  std::map<size_t, std::vector<buffer_t>> free_by_class_;
+  std::unordered_map<buffer_t, size_t> class_of_;
+  size_t live_bytes_ = 0;
+  size_t pooled_bytes_ = 0;
+};
+
+namespace gpu {
+
+using GpuStreamHandle = hipStream_t;
+
+struct BaseHipContextOption {
+  GpuStreamHandle stream = nullptr;  // nullptr = the null stream
+  int device_ordinal = 0;
+  // e.g. the embedding framework's caching allocator; nullptr = hipMalloc + pool
+  std::shared_ptr<Allocator> gpu_allocator;
+};
+
+std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
+                                                BaseHipContextOption& gpu_opt);
+
+struct BaseHipExecutionContext : public ExecutionContext {
+  explicit BaseHipExecutionContext(BaseContext* ctx);
+  ~BaseHipExecutionContext() override;
+
+  // buffers handed out by `alloc` during this execution -> reference count
+  std::unordered_map<const_buffer_t, int> device_ptr_map;
+};
+
+extern const char* kRalBaseHipContextState;
+
+}  // namespace gpu
+}  // namespace ral
+}  // namespace tao
+
+#endif  // RAL_CONTEXT_BASE_HIP_HIP_CONTEXT_IMPL_H_

@@ -1,0 +1,671 @@
+// RAL entries of the quantized-inference hot path for the gpu device, backed by the
+// hand-written gfx950 kernels (include/disc_q8.h).
+//
+// Entries and the reference functions they replace (R = tao_compiler/mlir/ral/):
+//   ral_qgemm                   R context/stream_executor_based_impl.cc:427-483 (per
+//                               tensor, gpu) and the per-channel signature of
+//                               R context/common_context_impl_quantization.cc:1196-1266
+//   ral_pdll_qgemm              R context/quantized_gpu_kernel_impl.cc:329-461 (gpu
+//                               signatures: int8 / f32 bias already in output units)
+//                               and the CPU-style signatures of
+//                               R context/common_context_impl_quantization.cc:1268-1672
+//                               (f32 / s32 / no bias, per-channel weight scale)
+//   ral_pdll_qgemm_per_channel  R context/quantized_gpu_kernel_impl.cc:197-321
+//   ral_qconv                   R context/stream_executor_based_impl.cc:1831-1948
+//   ral_quantize / ral_dequantize
+//                               no runtime symbol in the reference: its compiler
+//                               expands mhlo_disc.quantize / dequantize into loops
+//                               (disc/transforms/disc_lower_quantize_and_dequantize.cc);
+//                               these entries run the same arithmetic as one kernel.
+//
+// Differences from the reference that callers can observe:
+//   * scales stay on the device: nothing here copies them to the host or
+//     synchronises the stream (the reference does both on the first or on every
+//     call); the kernels read the scale buffers themselves.
+//   * ral_qconv applies the per-channel weight scale to every channel (the
+//     reference reads element 0 only).
+//   * errors are reported through Context::signalError and the entry returns; no
+//     kernel is launched after an error.
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "disc_q8.h"
+#include "mlir/ral/context/context_util.h"
+#include "mlir/ral/context/pdll_util.h"
+#include "mlir/ral/device/gpu/gpu_driver.h"
+#include "mlir/ral/ral_context.h"
+#include "mlir/ral/ral_helper.h"
+#include "mlir/ral/ral_logging.h"
+
+namespace tao {
+namespace ral {
+namespace gpu {
+namespace q8 {
+
+namespace {
+
+void fail(ExecutionContext* ctx, const std::string& what) {
+  ctx->signalError(Context::FAILURE, what);
+}
+
+// Reports a kernel-library failure; returns true when `status` was an error.
+bool kernelFailed(ExecutionContext* ctx, int status, const char* who) {
+  if (status == 0) return false;
+  fail(ctx, std::string(who) + ": " + dq8_last_error());
+  return true;
+}
+
+GPUDriver* driverOf(ExecutionContext* ctx) {
+  auto* d = ctx->getDriver<GPUDriver>(GPUDriver::name());
+  if (!d) fail(ctx, "GPUDriver not found");
+  return d;
+}
+
+// [K,N] constant weights are turned into the kernels' [N,K] layout once and kept
+// for the life of the context, keyed by the weight buffer's address and shape.
+struct PackedWeightState : public Context::Resource {
+  struct Key {
+    const void* ptr;
+    int64_t k, n;
+    bool operator==(const Key& o) const { return ptr == o.ptr && k == o.k && n == o.n; }
+  };
+  struct Hash {
+    size_t operator()(const Key& k) const {
+      return std::hash<const void*>()(k.ptr) ^ (std::hash<int64_t>()(k.k) * 1000003u) ^
+             (std::hash<int64_t>()(k.n) * 998244353u);
+    }
+  };
+  std::mutex mu;
+  std::unordered_map<Key, int8_t*, Hash> packed;
+};
+
+const char* kPackedWeightState = "tao_ral.gpu.qgemm_packed_weight_i8";
+
+struct GemmOperands {
+  const int8_t* a = nullptr;
+  const int8_t* w = nullptr;
+  int64_t m = 0, n = 0, k = 0;
+  bool tp_a = false, tp_b = false;
+  bool weight_is_const = false;
+};
+
+struct Epilogue {
+  int mode = DQ8_EPI_REQUANT_CPU;
+  const void* bias = nullptr;
+  int bias_kind = DQ8_BIAS_NONE;
+  const float* sx = nullptr;
+  const float* sw = nullptr;
+  const float* so = nullptr;
+  int64_t n_sx = 1, n_sw = 1, n_so = 1;
+  int32_t zo = 0;
+};
+
+// Launches the GEMM, providing scratch (or the cached packed weight) for
+// operands that are not k-contiguous.
+void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const Epilogue& e,
+             int8_t* out, const char* who) {
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return;
+  void* stream = drv->asCUStream(ctx, stream_handle);
+
+  if (!op.tp_b && op.weight_is_const && op.k > 0) {
+    auto* state = ctx->getOrCreateResource<PackedWeightState>(
+        kPackedWeightState, [] { return new PackedWeightState; });
+    if (!state) return;
+    std::lock_guard<std::mutex> guard(state->mu);
+    PackedWeightState::Key key{op.w, op.k, op.n};
+    auto it = state->packed.find(key);
+    if (it == state->packed.end()) {
+      auto* nk = static_cast<int8_t*>(drv->alloc_persistent(ctx, (size_t)(op.n * op.k)));
+      if (!nk) return;
+      // [K,N] -> [N,K], once; ordered before the GEMM on the same stream
+      if (kernelFailed(ctx, dq8_transpose_s8(op.w, op.n, nk, op.k, op.n, stream), who)) return;
+      it = state->packed.emplace(key, nk).first;
+    }
+    op.w = it->second;
+    op.tp_b = true;
+  }
+
+  const int64_t lda = op.tp_a ? op.m : op.k;
+  const int64_t ldw = op.tp_b ? op.k : op.n;
+  const size_t ws_bytes = dq8_qgemm_workspace_bytes(op.m, op.n, op.k, op.tp_a, op.tp_b);
+  void* ws = nullptr;
+  if (ws_bytes) {
+    ws = drv->alloc(ctx, ws_bytes);
+    if (!ws) return;
+  }
+  int st = dq8_qgemm(op.a, lda, op.w, ldw, out, op.n, op.m, op.n, op.k, op.tp_a, op.tp_b,
+                     e.mode, e.bias, e.bias_kind, e.sx, e.n_sx, e.sw, e.n_sw, e.so, e.n_so,
+                     /*zx=*/0, /*zw=*/0, e.zo, ws, ws_bytes, stream);
+  // the pool hands `ws` out again only to later work on the same stream, which is
+  // ordered after this launch
+  if (ws) drv->dealloc(ctx, ws);
+  kernelFailed(ctx, st, who);
+}
+
+template <typename T, int N>
+bool requireContiguous(ExecutionContext* ctx, const MemRefType<T, N>& m, const char* who,
+                       const char* what) {
+  if (isContiguous(m)) return true;
+  fail(ctx, std::string(who) + ": " + what + " must be a dense row-major memref");
+  return false;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ ral_qgemm
+// result = sat8(rne(((s_x * s_w[n]) / s_o) * acc)); zero points are not read (the
+// reference gpu entry does not read them either).
+template <int WS_RANK>
+void ral_qgemm_impl(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 2> input,
+                    MemRefType<int8_t, 2> weight, MemRefType<float, 0> inputScales,
+                    MemRefType<float, WS_RANK> weightScales, MemRefType<float, 0> resultScales,
+                    MemRefType<int8_t, 2> result, bool tp_a, bool tp_b, bool weight_is_const) {
+  static const char* who = "ral_qgemm";
+  if (isEmptyMemref(input) || isEmptyMemref(weight) || isEmptyMemref(result)) {
+    TAO_VLOG(1) << "ral_qgemm: early return for empty tensor";
+    return;
+  }
+  GemmOperands op;
+  op.m = tp_a ? input.sizes[1] : input.sizes[0];
+  op.k = tp_a ? input.sizes[0] : input.sizes[1];
+  op.n = tp_b ? weight.sizes[0] : weight.sizes[1];
+  if (op.k != (tp_b ? weight.sizes[1] : weight.sizes[0])) {
+    fail(ctx, "mismatch contraction dim for ral_qgemm");
+    return;
+  }
+  if (result.sizes[0] != op.m || result.sizes[1] != op.n) {
+    fail(ctx, "ral_qgemm: result shape does not match the operands");
+    return;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight") ||
+      !requireContiguous(ctx, result, who, "result"))
+    return;
+  op.a = input.data;
+  op.w = weight.data;
+  op.tp_a = tp_a;
+  op.tp_b = tp_b;
+  op.weight_is_const = weight_is_const;
+  Epilogue e;
+  e.mode = DQ8_EPI_REQUANT_CPU;
+  e.sx = inputScales.data;
+  e.sw = weightScales.data;
+  e.so = resultScales.data;
+  if constexpr (WS_RANK == 1) {
+    e.n_sw = weightScales.sizes[0];
+    if (e.n_sw != 1 && e.n_sw != op.n) {
+      fail(ctx, "ral_qgemm: weight scale must have 1 or N entries");
+      return;
+    }
+  }
+  runGemm(ctx, stream_handle, op, e, result.data, who);
+}
+
+void ral_qgemm(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 2> input,
+               MemRefType<int8_t, 2> weight, MemRefType<float, 0> inputScales,
+               MemRefType<int32_t, 0> /*inputZeroPoints*/, MemRefType<float, 0> weightScales,
+               MemRefType<int32_t, 0> /*weightZeroPoints*/, MemRefType<float, 0> resultScales,
+               MemRefType<int32_t, 0> /*resultZeroPoints*/, MemRefType<int8_t, 2> result,
+               bool tp_a, bool tp_b, bool weight_is_const) {
+  ral_qgemm_impl<0>(ctx, stream_handle, input, weight, inputScales, weightScales, resultScales,
+                    result, tp_a, tp_b, weight_is_const);
+}
+
+void ral_qgemm_per_channel(ExecutionContext* ctx, void* stream_handle,
+                           MemRefType<int8_t, 2> input, MemRefType<int8_t, 2> weight,
+                           MemRefType<float, 0> inputScales,
+                           MemRefType<int32_t, 0> /*inputZeroPoints*/,
+                           MemRefType<float, 1> weightScales,
+                           MemRefType<int32_t, 1> /*weightZeroPoints*/,
+                           MemRefType<float, 0> resultScales,
+                           MemRefType<int32_t, 0> /*resultZeroPoints*/,
+                           MemRefType<int8_t, 2> result, bool tp_a, bool tp_b,
+                           bool weight_is_const) {
+  ral_qgemm_impl<1>(ctx, stream_handle, input, weight, inputScales, weightScales, resultScales,
+                    result, tp_a, tp_b, weight_is_const);
+}
+
+// ------------------------------------------------------------- ral_pdll_qgemm
+namespace {
+
+// Flattens the leading dims of a rank-N input into M and allocates the result
+// through the driver.  Returns false (with `result` describing a null buffer of
+// the right shape) when there is nothing to compute.
+template <int N>
+bool prepareResult(ExecutionContext* ctx, const MemRefType<int8_t, N>& input, int64_t n,
+                   int64_t* m, MemRefType<int8_t, N>* result) {
+  int64_t sizes[N];
+  *m = 1;
+  for (int i = 0; i < N - 1; ++i) {
+    *m *= input.sizes[i];
+    sizes[i] = input.sizes[i];
+  }
+  sizes[N - 1] = n;
+  if (*m == 0 || n == 0) {
+    *result = assignMemRef<int8_t, N>(nullptr, sizes);
+    return false;
+  }
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) {
+    *result = assignMemRef<int8_t, N>(nullptr, sizes);
+    return false;
+  }
+  void* data = drv->alloc(ctx, (size_t)(*m * n));
+  *result = assignMemRef<int8_t, N>(data, sizes);
+  return data != nullptr;
+}
+
+// Zero points of ral_pdll_* calls are host-resident ("s" placement in the PDLL
+// patterns); only the symmetric input/weight case has kernels.
+bool symmetricOrFail(ExecutionContext* ctx, const int32_t* zx, int64_t n_zx, const int32_t* zw,
+                     int64_t n_zw, const char* who) {
+  for (int64_t i = 0; i < n_zx; ++i)
+    if (zx && zx[i] != 0) {
+      fail(ctx, std::string(who) + ": non-zero input zero point is not supported");
+      return false;
+    }
+  for (int64_t i = 0; i < n_zw; ++i)
+    if (zw && zw[i] != 0) {
+      fail(ctx, std::string(who) + ": non-zero weight zero point is not supported");
+      return false;
+    }
+  return true;
+}
+
+}  // namespace
+
+// GPU signatures: weight [N,K], bias already in output-quantised units,
+// out = sat8(rne(((s_x*s_w)/s_o) * acc + bias[n])).
+template <int N, typename BiasT>
+MemRefType<int8_t, N> ral_pdll_qgemm_gpu(ExecutionContext* ctx, void* stream_handle,
+                                         MemRefType<int8_t, N> input,
+                                         MemRefType<int8_t, 2> weight,
+                                         MemRefType<BiasT, 1> bias,
+                                         MemRefType<float, 0> inputScales,
+                                         MemRefType<int32_t, 0> inputZeroPoints,
+                                         MemRefType<float, 0> weightScales,
+                                         MemRefType<int32_t, 0> weightZeroPoints,
+                                         MemRefType<float, 0> resultScales,
+                                         MemRefType<int32_t, 0> resultZeroPoints,
+                                         void* /*customAttrs*/) {
+  static const char* who = "ral_pdll_qgemm";
+  GemmOperands op;
+  op.n = weight.sizes[0];
+  op.k = weight.sizes[1];
+  MemRefType<int8_t, N> result;
+  if (input.sizes[N - 1] != op.k && !isEmptyMemref(input)) {
+    fail(ctx, "mismatch contraction dim for ral_pdll_qgemm");
+    int64_t zeros[N] = {0};
+    return assignMemRef<int8_t, N>(nullptr, zeros);
+  }
+  if (!prepareResult<N>(ctx, input, op.n, &op.m, &result)) return result;
+  if (!symmetricOrFail(ctx, inputZeroPoints.data, 1, weightZeroPoints.data, 1, who) ||
+      (resultZeroPoints.data && resultZeroPoints.data[0] != 0 &&
+       (fail(ctx, "ral_pdll_qgemm: non-zero result zero point is not supported"), true)))
+    return result;
+  if (bias.sizes[0] != op.n) {
+    fail(ctx, "ral_pdll_qgemm: bias must have N entries");
+    return result;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight"))
+    return result;
+  op.a = input.data;
+  op.w = weight.data;
+  op.tp_b = true;
+  Epilogue e;
+  e.mode = DQ8_EPI_REQUANT_GPU;
+  e.bias = bias.data;
+  e.bias_kind = std::is_same<BiasT, float>::value ? DQ8_BIAS_F32 : DQ8_BIAS_S8;
+  e.sx = inputScales.data;
+  e.sw = weightScales.data;
+  e.so = resultScales.data;
+  runGemm(ctx, stream_handle, op, e, result.data, who);
+  return result;
+}
+
+// Merged-QKV form: all three scales are [N] vectors, int8 bias.
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_per_channel(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<int8_t, 1> bias, MemRefType<float, 1> inputScales,
+    MemRefType<int32_t, 1> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 1> resultScales,
+    MemRefType<int32_t, 1> resultZeroPoints, void* /*customAttrs*/) {
+  static const char* who = "ral_pdll_qgemm_per_channel";
+  GemmOperands op;
+  op.n = weight.sizes[0];
+  op.k = weight.sizes[1];
+  MemRefType<int8_t, N> result;
+  if (input.sizes[N - 1] != op.k && !isEmptyMemref(input)) {
+    fail(ctx, "mismatch contraction dim for ral_pdll_qgemm_per_channel");
+    int64_t zeros[N] = {0};
+    return assignMemRef<int8_t, N>(nullptr, zeros);
+  }
+  if (!prepareResult<N>(ctx, input, op.n, &op.m, &result)) return result;
+  if (inputScales.sizes[0] != op.n || weightScales.sizes[0] != op.n ||
+      resultScales.sizes[0] != op.n || bias.sizes[0] != op.n) {
+    fail(ctx, "ral_pdll_qgemm_per_channel: scales and bias must have N entries");
+    return result;
+  }
+  if (!symmetricOrFail(ctx, inputZeroPoints.data, inputZeroPoints.sizes[0],
+                       weightZeroPoints.data, weightZeroPoints.sizes[0], who))
+    return result;
+  for (int64_t i = 0; resultZeroPoints.data && i < resultZeroPoints.sizes[0]; ++i)
+    if (resultZeroPoints.data[i] != 0) {
+      fail(ctx, "ral_pdll_qgemm_per_channel: non-zero result zero point is not supported");
+      return result;
+    }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight"))
+    return result;
+  op.a = input.data;
+  op.w = weight.data;
+  op.tp_b = true;
+  Epilogue e;
+  e.mode = DQ8_EPI_REQUANT_GPU;
+  e.bias = bias.data;
+  e.bias_kind = DQ8_BIAS_S8;
+  e.sx = inputScales.data;
+  e.sw = weightScales.data;
+  e.so = resultScales.data;
+  e.n_sx = e.n_sw = e.n_so = op.n;
+  runGemm(ctx, stream_handle, op, e, result.data, who);
+  return result;
+}
+
+// CPU-style signatures on the gpu device: per-channel weight scale, bias f32 /
+// s32 / none, weight [K,N] unless the `transpose_b` attr says otherwise,
+// out = sat8(rne((f32(acc) + b32[n]) * ((s_x*s_w[n])/s_o) + z_o)).
+namespace {
+
+struct NoBias {};
+
+template <int N>
+MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_handle,
+                                        MemRefType<int8_t, N> input,
+                                        MemRefType<int8_t, 2> weight, const void* bias,
+                                        int64_t n_bias, int bias_kind,
+                                        MemRefType<float, 0> inputScales,
+                                        MemRefType<int32_t, 0> inputZeroPoints,
+                                        MemRefType<float, 1> weightScales,
+                                        MemRefType<int32_t, 1> weightZeroPoints,
+                                        MemRefType<float, 0> resultScales,
+                                        MemRefType<int32_t, 0> resultZeroPoints,
+                                        void* customAttrs) {
+  static const char* who = "ral_pdll_qgemm";
+  int64_t zeros[N] = {0};
+  MemRefType<int8_t, N> result = assignMemRef<int8_t, N>(nullptr, zeros);
+  bool tp_a = false, tp_b = false, weight_is_const = false;
+  if (customAttrs) {
+    PDLAttr* attr = getOrParsePDLAttr(ctx, customAttrs, "ral_pdll_qgemm_gpu_cpu_style");
+    if (!attr || attr->getType() != "dict") {
+      fail(ctx, "fail to parse custom_attrs\n");
+      return result;
+    }
+    auto& dict = attr->as<DictPDLAttr>();
+    auto flag = [&](const char* key) {
+      return dict.hasKey(key) && dict.get(key).getType() == "bool" &&
+             dict.get(key).as<BoolPDLAttr>().getValue();
+    };
+    tp_a = flag("transpose_a");
+    tp_b = flag("transpose_b");
+    weight_is_const = flag("weight_is_const");
+  }
+  if (tp_a) {
+    fail(ctx, "ral_pdll_qgemm: transpose_a is not supported on gpu");
+    return result;
+  }
+  GemmOperands op;
+  op.k = tp_b ? weight.sizes[1] : weight.sizes[0];
+  op.n = tp_b ? weight.sizes[0] : weight.sizes[1];
+  if (input.sizes[N - 1] != op.k && !isEmptyMemref(input)) {
+    fail(ctx, "mismatch contraction dim for ral_pdll_qgemm");
+    return result;
+  }
+  if (!prepareResult<N>(ctx, input, op.n, &op.m, &result)) return result;
+  if (!symmetricOrFail(ctx, inputZeroPoints.data, 1, weightZeroPoints.data,
+                       weightZeroPoints.sizes[0], who))
+    return result;
+  if (weightScales.sizes[0] != 1 && weightScales.sizes[0] != op.n) {
+    fail(ctx, "ral_pdll_qgemm: weight scale must have 1 or N entries");
+    return result;
+  }
+  if (bias_kind != DQ8_BIAS_NONE && n_bias != op.n) {
+    fail(ctx, "ral_pdll_qgemm: bias must have N entries");
+    return result;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight"))
+    return result;
+  op.a = input.data;
+  op.w = weight.data;
+  op.tp_b = tp_b;
+  op.weight_is_const = weight_is_const;
+  Epilogue e;
+  e.mode = DQ8_EPI_REQUANT_CPU;
+  e.bias = bias;
+  e.bias_kind = bias_kind;
+  e.sx = inputScales.data;
+  e.sw = weightScales.data;
+  e.n_sw = weightScales.sizes[0];
+  e.so = resultScales.data;
+  e.zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
+  runGemm(ctx, stream_handle, op, e, result.data, who);
+  return result;
+}
+
+}  // namespace
+
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_f32_per_channel(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 1> bias, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, void* customAttrs) {
+  return pdllQgemmCpuStyle<N>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0],
+                              DQ8_BIAS_F32, inputScales, inputZeroPoints, weightScales,
+                              weightZeroPoints, resultScales, resultZeroPoints, customAttrs);
+}
+
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_s32_per_channel(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<int32_t, 1> bias,
+    MemRefType<float, 0> inputScales, MemRefType<int32_t, 0> inputZeroPoints,
+    MemRefType<float, 1> weightScales, MemRefType<int32_t, 1> weightZeroPoints,
+    MemRefType<float, 0> resultScales, MemRefType<int32_t, 0> resultZeroPoints,
+    void* customAttrs) {
+  return pdllQgemmCpuStyle<N>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0],
+                              DQ8_BIAS_S32, inputScales, inputZeroPoints, weightScales,
+                              weightZeroPoints, resultScales, resultZeroPoints, customAttrs);
+}
+
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_per_channel(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, void* customAttrs) {
+  return pdllQgemmCpuStyle<N>(ctx, stream_handle, input, weight, nullptr, 0, DQ8_BIAS_NONE,
+                              inputScales, inputZeroPoints, weightScales, weightZeroPoints,
+                              resultScales, resultZeroPoints, customAttrs);
+}
+
+// ------------------------------------------------------------------ ral_qconv
+// out = sat8(rne(((s_x*s_w[co])/s_o) * conv_s32(in, w))); padding and metadata are
+// host memrefs; zero points are not read.
+void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4> input,
+               MemRefType<int8_t, 4> kernel, MemRefType<int32_t, 1> padding,
+               MemRefType<float, 0> inputScales, MemRefType<int32_t, 0> /*inputZeroPoints*/,
+               MemRefType<float, 1> weightScales, MemRefType<int32_t, 1> /*weightZeroPoints*/,
+               MemRefType<float, 0> resultScales, MemRefType<int32_t, 0> /*resultZeroPoints*/,
+               MemRefType<int8_t, 4> output, MemRefType<int32_t, 1> metadata) {
+  static const char* who = "ral_qconv";
+  if (isEmptyMemref(input) || isEmptyMemref(kernel) || isEmptyMemref(output)) {
+    TAO_VLOG(1) << "ral_qconv: early return for empty tensor";
+    return;
+  }
+  if (padding.sizes[0] != 4 || metadata.sizes[0] != 17) {
+    fail(ctx, "ral_qconv: rank-4 convolution needs 4 padding and 17 metadata entries");
+    return;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, kernel, who, "kernel") ||
+      !requireContiguous(ctx, output, who, "output"))
+    return;
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return;
+  void* stream = drv->asCUStream(ctx, stream_handle);
+  int st = dq8_qconv2d(input.data, input.sizes, kernel.data, kernel.sizes, padding.data,
+                       metadata.data, output.data, output.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
+                       DQ8_BIAS_NONE, inputScales.data, weightScales.data,
+                       weightScales.sizes[0], resultScales.data, 0, stream);
+  kernelFailed(ctx, st, who);
+}
+
+// ------------------------------------------------- ral_quantize / ral_dequantize
+// axis < 0 means per tensor (rank-0 scale / zero point); otherwise the scale and
+// zero point vectors run along dimension `axis`.  Scale and zero point are device
+// buffers.
+namespace {
+
+template <int N>
+void view3(const int64_t (&sizes)[N], int64_t axis, int64_t* outer, int64_t* nch,
+           int64_t* inner) {
+  *outer = *nch = *inner = 1;
+  if (axis < 0) {
+    for (int i = 0; i < N; ++i) *inner *= sizes[i];
+    return;
+  }
+  for (int i = 0; i < N; ++i) {
+    if (i < axis) *outer *= sizes[i];
+    else if (i == axis) *nch = sizes[i];
+    else *inner *= sizes[i];
+  }
+}
+
+}  // namespace
+
+template <typename QT, int N, int SR>
+void ral_quantize(ExecutionContext* ctx, void* stream_handle, MemRefType<float, N> input,
+                  MemRefType<float, SR> scale, MemRefType<int32_t, SR> zeroPoint,
+                  MemRefType<QT, N> result, int64_t axis, int64_t quantMin, int64_t quantMax,
+                  int64_t roundMode) {
+  static const char* who = "ral_quantize";
+  if (isEmptyMemref(input)) return;
+  for (int i = 0; i < N; ++i)
+    if (input.sizes[i] != result.sizes[i]) {
+      fail(ctx, "ral_quantize: result shape differs from the input's");
+      return;
+    }
+  if ((SR == 0) != (axis < 0) || axis >= N) {
+    fail(ctx, "ral_quantize: axis does not match the rank of scale/zero_point");
+    return;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, result, who, "result"))
+    return;
+  int64_t outer, nch, inner;
+  view3<N>(input.sizes, axis, &outer, &nch, &inner);
+  int64_t n_q = 1;
+  if constexpr (SR == 1) {
+    n_q = scale.sizes[0];
+    if (n_q != nch || zeroPoint.sizes[0] != nch) {
+      fail(ctx, "ral_quantize: scale/zero_point length differs from the axis extent");
+      return;
+    }
+  }
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return;
+  int st = dq8_quantize(input.data, result.data,
+                        std::is_same<QT, int8_t>::value ? DQ8_I8 : DQ8_U8, outer, nch, inner,
+                        scale.data, zeroPoint.data, SR == 0 ? 1 : n_q, (int32_t)quantMin,
+                        (int32_t)quantMax, (int)roundMode, drv->asCUStream(ctx, stream_handle));
+  kernelFailed(ctx, st, who);
+}
+
+template <typename QT, int N, int SR>
+void ral_dequantize(ExecutionContext* ctx, void* stream_handle, MemRefType<QT, N> input,
+                    MemRefType<float, SR> scale, MemRefType<int32_t, SR> zeroPoint,
+                    MemRefType<float, N> result, int64_t axis) {
+  static const char* who = "ral_dequantize";
+  if (isEmptyMemref(input)) return;
+  for (int i = 0; i < N; ++i)
+    if (input.sizes[i] != result.sizes[i]) {
+      fail(ctx, "ral_dequantize: result shape differs from the input's");
+      return;
+    }
+  if ((SR == 0) != (axis < 0) || axis >= N) {
+    fail(ctx, "ral_dequantize: axis does not match the rank of scale/zero_point");
+    return;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, result, who, "result"))
+    return;
+  int64_t outer, nch, inner;
+  view3<N>(input.sizes, axis, &outer, &nch, &inner);
+  int64_t n_q = 1;
+  if constexpr (SR == 1) {
+    n_q = scale.sizes[0];
+    if (n_q != nch || zeroPoint.sizes[0] != nch) {
+      fail(ctx, "ral_dequantize: scale/zero_point length differs from the axis extent");
+      return;
+    }
+  }
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return;
+  int st = dq8_dequantize(input.data, std::is_same<QT, int8_t>::value ? DQ8_I8 : DQ8_U8,
+                          result.data, outer, nch, inner, scale.data, zeroPoint.data,
+                          SR == 0 ? 1 : n_q, drv->asCUStream(ctx, stream_handle));
+  kernelFailed(ctx, st, who);
+}
+
+}  // namespace q8
+}  // namespace gpu
+
+// ---------------------------------------------------------------- registration
+TAO_RAL_API("ral_qgemm", "gpu", gpu::q8::ral_qgemm);
+TAO_RAL_API("ral_qgemm", "gpu", gpu::q8::ral_qgemm_per_channel);
+
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_gpu<2, int8_t>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_gpu<3, int8_t>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_gpu<2, float>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_gpu<3, float>);
+TAO_RAL_API("ral_pdll_qgemm_per_channel", "gpu", gpu::q8::ral_pdll_qgemm_per_channel<2>);
+TAO_RAL_API("ral_pdll_qgemm_per_channel", "gpu", gpu::q8::ral_pdll_qgemm_per_channel<3>);
+
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_f32_per_channel<2>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_f32_per_channel<3>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_f32_per_channel<4>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_channel<2>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_channel<3>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_channel<4>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<2>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<3>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<4>);
+
+TAO_RAL_API("ral_qconv", "gpu", gpu::q8::ral_qconv);
+
+#define DQ8_REGISTER_QDQ(QT, N)                                              \
+  TAO_RAL_API("ral_quantize", "gpu", gpu::q8::ral_quantize<QT, N, 0>);       \
+  TAO_RAL_API("ral_quantize", "gpu", gpu::q8::ral_quantize<QT, N, 1>);       \
+  TAO_RAL_API("ral_dequantize", "gpu", gpu::q8::ral_dequantize<QT, N, 0>);   \
+  TAO_RAL_API("ral_dequantize", "gpu", gpu::q8::ral_dequantize<QT, N, 1>);
+DQ8_REGISTER_QDQ(int8_t, 1)
+DQ8_REGISTER_QDQ(int8_t, 2)
+DQ8_REGISTER_QDQ(int8_t, 3)
+DQ8_REGISTER_QDQ(int8_t, 4)
+DQ8_REGISTER_QDQ(uint8_t, 1)
+DQ8_REGISTER_QDQ(uint8_t, 2)
+DQ8_REGISTER_QDQ(uint8_t, 3)
+DQ8_REGISTER_QDQ(uint8_t, 4)
+#undef DQ8_REGISTER_QDQ
+
+}  // namespace ral
+}  // namespace tao

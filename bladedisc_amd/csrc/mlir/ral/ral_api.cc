@@ -1,0 +1,183 @@
+// C entry points of the runtime plugin ABI (include/tao_ral_api.h).
+#include "tao_ral_api.h"
+
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include <algorithm>
+#include <cstring>
+#include <sstream>
+
+#include "mlir/ral/context/base/hip/hip_context_impl.h"
+#include "mlir/ral/context/pdll_util.h"
+#include "mlir/ral/ral_context.h"
+#include "mlir/ral/ral_helper.h"
+#include "mlir/ral/ral_logging.h"
+
+namespace {
+
+// Allocator over a pair of C callbacks supplied by the embedding framework.
+class CallbackAllocator : public tao::ral::Allocator {
+ public:
+  CallbackAllocator(disc_ral_alloc_fn a, disc_ral_dealloc_fn d, void* user)
+      : alloc_(a), dealloc_(d), user_(user) {}
+  tao::ral::buffer_t alloc(size_t bytes) override { return alloc_(bytes, user_); }
+  void dealloc(tao::ral::buffer_t p) override { dealloc_(p, user_); }
+
+ private:
+  disc_ral_alloc_fn alloc_;
+  disc_ral_dealloc_fn dealloc_;
+  void* user_;
+};
+
+std::vector<std::string>& apiNames() {
+  static std::vector<std::string> names;
+  static std::once_flag once;
+  std::call_once(once, [] { names = tao::ral::TaoRalApiRegistry::Global().Names(); });
+  return names;
+}
+
+void renderJson(tao::ral::PDLAttr& a, std::ostringstream& os) {
+  using namespace tao::ral;
+  const std::string& t = a.getType();
+  auto quote = [&](const std::string& s) {
+    os << '"';
+    for (char c : s) {
+      if (c == '"' || c == '\\') os << '\\';
+      os << c;
+    }
+    os << '"';
+  };
+  if (t == "dict") {
+    auto& items = a.as<DictPDLAttr>().getValue();
+    std::vector<std::string> keys;
+    for (auto& kv : items) keys.push_back(kv.first);
+    std::sort(keys.begin(), keys.end());
+    os << '{';
+    for (size_t i = 0; i < keys.size(); ++i) {
+      if (i) os << ", ";
+      quote(keys[i]);
+      os << ": ";
+      renderJson(*items[keys[i]], os);
+    }
+    os << '}';
+  } else if (t == "str") {
+    quote(a.as<StrPDLAttr>().getValue());
+  } else if (t == "bool") {
+    os << (a.as<BoolPDLAttr>().getValue() ? "true" : "false");
+  } else if (t == "int") {
+    os << a.as<IntPDLAttr>().getValue();
+  } else if (t == "float") {
+    os.precision(17);
+    os << a.as<FloatPDLAttr>().getValue();
+  } else if (t == "intArray") {
+    auto& v = a.as<IntArrayPDLAttr>().getValue();
+    os << '[';
+    for (size_t i = 0; i < v.size(); ++i) os << (i ? ", " : "") << v[i];
+    os << ']';
+  } else if (t == "array") {
+    auto& v = a.as<ArrayPDLAttr>().getValue();
+    os << '[';
+    for (size_t i = 0; i < v.size(); ++i) {
+      if (i) os << ", ";
+      renderJson(*v[i], os);
+    }
+    os << ']';
+  } else if (t == "denseElementsAttr") {
+    auto& d = a.as<DenseElementsPDLAttr>();
+    os << "{\"dense\": ";
+    quote(d.getElementType() + std::to_string(d.getNumBits()));
+    os << ", \"shape\": [";
+    auto shape = d.getShape();
+    for (size_t i = 0; i < shape.size(); ++i) os << (i ? ", " : "") << shape[i];
+    os << "], \"bytes\": [";
+    auto& raw = d.getRawData();
+    for (size_t i = 0; i < raw.size(); ++i) os << (i ? ", " : "") << (int)raw[i];
+    os << "]}";
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* const kMlirLoweredEntry = "main";
+
+void tao_ral_call_impl(tao_ral_context_t ctx, void* name, void** args) {
+  auto* exec = static_cast<tao::ral::ExecutionContext*>(ctx);
+  TAO_VLOG(1) << "tao_ral_call: " << static_cast<const char*>(name);
+  exec->getContext()->call(static_cast<const char*>(name), args);
+}
+
+tao_ral_status_t tao_ral_last_error(tao_ral_context_t ctx, const char** err_msg) {
+  return static_cast<tao::ral::Context*>(ctx)->getLastError(err_msg);
+}
+
+void tao_ral_clear_error(tao_ral_context_t ctx) {
+  static_cast<tao::ral::Context*>(ctx)->clearError();
+}
+
+tao_ral_context_t disc_ral_context_create(void* hip_stream, int device_ordinal,
+                                          disc_ral_alloc_fn alloc,
+                                          disc_ral_dealloc_fn dealloc, void* user,
+                                          int cache_workspace) {
+  if ((alloc == nullptr) != (dealloc == nullptr)) return nullptr;
+  tao::ral::BaseContextOption opt;
+  opt.cache_workspace_mem_across_execution = cache_workspace != 0;
+  tao::ral::gpu::BaseHipContextOption gpu_opt;
+  gpu_opt.stream = static_cast<hipStream_t>(hip_stream);
+  gpu_opt.device_ordinal = device_ordinal;
+  if (alloc) gpu_opt.gpu_allocator.reset(new CallbackAllocator(alloc, dealloc, user));
+  auto ctx = tao::ral::gpu::MakeBaseHipContext(opt, gpu_opt);
+  return static_cast<tao::ral::Context*>(ctx.release());
+}
+
+void disc_ral_context_destroy(tao_ral_context_t ctx) {
+  delete static_cast<tao::ral::Context*>(ctx);
+}
+
+tao_ral_context_t disc_ral_execution_context_create(tao_ral_context_t ctx) {
+  auto* base = dynamic_cast<tao::ral::BaseContext*>(static_cast<tao::ral::Context*>(ctx));
+  if (!base) return nullptr;
+  return static_cast<tao::ral::ExecutionContext*>(
+      new tao::ral::gpu::BaseHipExecutionContext(base));
+}
+
+void disc_ral_execution_context_destroy(tao_ral_context_t exec_ctx) {
+  delete static_cast<tao::ral::ExecutionContext*>(exec_ctx);
+}
+
+tao_ral_context_t disc_ral_execution_context_get_context(tao_ral_context_t exec_ctx) {
+  return static_cast<tao::ral::ExecutionContext*>(exec_ctx)->getContext();
+}
+
+int disc_ral_api_count(void) { return static_cast<int>(apiNames().size()); }
+
+const char* disc_ral_api_name(int index) {
+  auto& names = apiNames();
+  if (index < 0 || index >= static_cast<int>(names.size())) return "";
+  return names[index].c_str();
+}
+
+int disc_ral_api_exists(const char* name) {
+  return name && tao::ral::TaoRalApiRegistry::Global().Find(name) ? 1 : 0;
+}
+
+int64_t disc_ral_attr_to_json(const uint8_t* blob, size_t size, char* out, size_t cap) {
+  if (!blob) return -1;
+  size_t used = 0;
+  auto attr = tao::ral::parsePDLAttr(blob, size, &used);
+  if (!attr) return -1;
+  std::ostringstream os;
+  renderJson(*attr, os);
+  const std::string text = os.str();
+  if (out && cap) {
+    const size_t n = std::min(cap - 1, text.size());
+    std::memcpy(out, text.data(), n);
+    out[n] = 0;
+  }
+  return static_cast<int64_t>(text.size());
+}
+
+}  // extern "C"

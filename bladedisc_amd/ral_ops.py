@@ -1,0 +1,141 @@
+"""Typed callers of the quantized RAL entries: each packs torch tensors the way the
+compiled program would and goes through ``tao_ral_call_impl`` by mangled name.
+
+Operand order of every call is the reference's (disc/transforms/
+disc_lower_to_library_call.cc:196-267 for ral_qgemm, :391-421 for ral_qconv, the
+PDLL rewrite patterns for ral_pdll_qgemm).
+"""
+import numpy as np
+import torch
+
+from . import ral
+
+
+def _zp0(a, host):
+    """A rank-0 zero point: host int32 (ral_pdll_*) or device int32."""
+    if host:
+        return a.host_array(np.zeros(1, np.int32), rank0=True)
+    z = torch.zeros(1, dtype=torch.int32, device="cuda")
+    a._keep.append(z)
+    return a.tensor(z, rank0=True)
+
+
+def qgemm(ex, x, w, sx, sw, so, out=None, tp_a=False, tp_b=True, weight_is_const=False,
+          per_channel=None):
+    """ral_qgemm: x [M,K] i8, w [N,K] (tp_b) or [K,N]; sx/so one-element device f32
+    tensors, sw one-element (per tensor, rank 0) or [N] (per channel, rank 1)."""
+    m = x.shape[1] if tp_a else x.shape[0]
+    n = w.shape[0] if tp_b else w.shape[1]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.int8, device=x.device)
+    if per_channel is None:
+        per_channel = sw.numel() > 1
+    a = ex.new_args().tensor(x).tensor(w)
+    a.tensor(sx, rank0=True)
+    _zp0(a, host=False)
+    if per_channel:
+        a.tensor(sw)
+        z = torch.zeros(sw.numel(), dtype=torch.int32, device=x.device)
+        a._keep.append(z)
+        a.tensor(z)
+    else:
+        a.tensor(sw, rank0=True)
+        _zp0(a, host=False)
+    a.tensor(so, rank0=True)
+    _zp0(a, host=False)
+    a.tensor(out)
+    a.scalar("i1", tp_a).scalar("i1", tp_b).scalar("i1", weight_is_const)
+    ex.call("ral_qgemm", "gpu", a)
+    return out
+
+
+def pdll_qgemm_gpu(ex, x, w_nk, bias, sx, sw, so):
+    """ral_pdll_qgemm, gpu signature: rank-2/3 input, weight [N,K], bias int8 or f32
+    in output-quantised units, rank-0 device scales, rank-0 host zero points.
+    Returns the callee-allocated result as a tensor view."""
+    a = ex.new_args().tensor(x).tensor(w_nk).tensor(bias)
+    for s in (sx, sw, so):
+        a.tensor(s, rank0=True)
+        _zp0(a, host=True)
+    a.blob(ral.encode_attr({}))
+    res = a.result_memref("i8", x.dim())
+    ex.call("ral_pdll_qgemm", "gpu", a)
+    return ral.memref_to_tensor(res, torch.int8)
+
+
+def pdll_qgemm_per_channel(ex, x, w_nk, bias_i8, sx_n, sw_n, so_n):
+    """ral_pdll_qgemm_per_channel (merged-QKV form): all scales are [N] vectors."""
+    n = w_nk.shape[0]
+    a = ex.new_args().tensor(x).tensor(w_nk).tensor(bias_i8)
+    for s in (sx_n, sw_n, so_n):
+        a.tensor(s)
+        a.host_array(np.zeros(n, np.int32))
+    a.blob(ral.encode_attr({}))
+    res = a.result_memref("i8", x.dim())
+    ex.call("ral_pdll_qgemm_per_channel", "gpu", a)
+    return ral.memref_to_tensor(res, torch.int8)
+
+
+def pdll_qgemm_cpu_style(ex, x, w, bias, sx, sw_n, so, zo=0, transpose_b=False,
+                         weight_is_const=True):
+    """ral_pdll_qgemm with the CPU patterns' signature on the gpu device: weight
+    [K,N] unless transpose_b, bias f32 / s32 / None, per-channel weight scale."""
+    n = w.shape[0] if transpose_b else w.shape[1]
+    a = ex.new_args().tensor(x).tensor(w)
+    if bias is not None:
+        a.tensor(bias)
+    a.tensor(sx, rank0=True)
+    _zp0(a, host=True)
+    a.tensor(sw_n)
+    a.host_array(np.zeros(sw_n.numel(), np.int32))
+    a.tensor(so, rank0=True)
+    a.host_array(np.array([zo], np.int32), rank0=True)
+    a.blob(ral.encode_attr({"transpose_a": False, "transpose_b": bool(transpose_b),
+                            "weight_is_const": bool(weight_is_const),
+                            "bias_is_const": True}))
+    res = a.result_memref("i8", x.dim())
+    ex.call("ral_pdll_qgemm", "gpu", a)
+    assert n == res.sizes[x.dim() - 1]
+    return ral.memref_to_tensor(res, torch.int8)
+
+
+def qconv(ex, x, w, padding, metadata, sx, sw_c, so, out):
+    """ral_qconv: padding [4] and metadata [17] are host int32 memrefs."""
+    a = ex.new_args().tensor(x).tensor(w)
+    a.host_array(np.asarray(padding, np.int32))
+    a.tensor(sx, rank0=True)
+    _zp0(a, host=False)
+    a.tensor(sw_c)
+    z = torch.zeros(sw_c.numel(), dtype=torch.int32, device=x.device)
+    a._keep.append(z)
+    a.tensor(z)
+    a.tensor(so, rank0=True)
+    _zp0(a, host=False)
+    a.tensor(out)
+    a.host_array(np.asarray(metadata, np.int32))
+    ex.call("ral_qconv", "gpu", a)
+    return out
+
+
+def quantize(ex, x, scale, zp, axis=None, qmin=-128, qmax=127, round_mode=1, out=None,
+             dtype=torch.int8):
+    if out is None:
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    a = ex.new_args().tensor(x)
+    a.tensor(scale, rank0=axis is None).tensor(zp, rank0=axis is None)
+    a.tensor(out)
+    a.scalar("i64", -1 if axis is None else axis).scalar("i64", qmin).scalar("i64", qmax)
+    a.scalar("i64", round_mode)
+    ex.call("ral_quantize", "gpu", a)
+    return out
+
+
+def dequantize(ex, q, scale, zp, axis=None, out=None):
+    if out is None:
+        out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    a = ex.new_args().tensor(q)
+    a.tensor(scale, rank0=axis is None).tensor(zp, rank0=axis is None)
+    a.tensor(out)
+    a.scalar("i64", -1 if axis is None else axis)
+    ex.call("ral_dequantize", "gpu", a)
+    return out

@@ -120,6 +120,13 @@ int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
 int dq8_qgemm_num_variants(void);
 const char* dq8_qgemm_variant_name(int variant);
 
+/* dst[c, r] = src[r, c] for an int8 matrix src [rows, cols] with row stride ld;
+ * dst is dense [cols, rows].  Used to put [K,N] weights into the kernels' [N,K]
+ * layout once (the reference's counterpart is oneDNN's weight pre-packing,
+ * R ral/context/common_context_impl_quantization.cc:1365-1383). */
+int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
+                     int64_t cols, void* stream);
+
 /* ---- int8 convolution (rank 4) ---------------------------------------- */
 
 /* Implicit-GEMM convolution.  Layouts are described exactly as ral_qconv's

@@ -1,0 +1,91 @@
+/*
+ * tao_ral_api.h -- the runtime-plugin C ABI that code compiled by the DISC compiler
+ * (and the TorchBlade / TF bridges) binds to, implemented for one MI355X.
+ *
+ * The first three functions and kMlirLoweredEntry are the reference's own ABI
+ * (R = alibaba/BladeDISC tao_compiler/mlir/ral/ral_api.h:37-67, ral_api.cc:29-51):
+ * a compiled program's `main` receives {ExecutionContext*, &tao_ral_call_impl} and
+ * calls every runtime service as
+ *     tao_ral_call_impl(exec_ctx, "<name>___<device>___<arg codes>___<ret codes>", args)
+ * with `args` packed as R disc/transforms/disc_to_llvm.cc:302-365 packs them.
+ *
+ * The disc_ral_* functions are a C view of what the reference exposes only as C++
+ * (MakeBaseCudaContext, R ral/context/base/cuda/cuda_context_impl.cc:168-202, and
+ * the BaseCudaExecutionContext constructor), so that hosts without a C++ binding
+ * (ctypes, cgo, JNI) can create the contexts the calls above need.
+ *
+ * Entries registered for the gpu device (query with disc_ral_api_name):
+ *   ral_qgemm, ral_pdll_qgemm, ral_pdll_qgemm_per_channel, ral_qconv,
+ *   ral_quantize, ral_dequantize, and the driver set alloc, dealloc,
+ *   ral_gpu_alloc_persistent, raw_gpu_alloc, raw_gpu_dealloc, h2d_, d2h_, d2d_,
+ *   ral_gpu_memset, ral_gpu_get_stream, sync_on_stream, ral_gpu_sync_all,
+ *   ral_gpu_as_cu_stream, ral_gpu_as_se_stream, ral_kernel_launch.
+ */
+#ifndef TAO_RAL_API_H_
+#define TAO_RAL_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* name of the entry function of a compiled program: "main" */
+extern const char* const kMlirLoweredEntry;
+
+typedef void* tao_ral_context_t;
+typedef int32_t tao_ral_status_t; /* 0 = ok */
+
+/* Calls the registered function `name` (a NUL-terminated const char*).  `ctx` is an
+ * ExecutionContext handle.  An unknown name puts the context into error state. */
+void tao_ral_call_impl(tao_ral_context_t ctx, void* name, void** args);
+
+/* Status of a Context handle since the last clear; *err_msg (if not NULL) points at
+ * a thread-local copy of the message, empty when ok. */
+tao_ral_status_t tao_ral_last_error(tao_ral_context_t ctx, const char** err_msg);
+
+/* Leaves error state.  `ctx` is a Context handle. */
+void tao_ral_clear_error(tao_ral_context_t ctx);
+
+/* ---- context lifetime -------------------------------------------------- */
+
+typedef void* (*disc_ral_alloc_fn)(size_t bytes, void* user);
+typedef void (*disc_ral_dealloc_fn)(void* ptr, void* user);
+
+/* Creates a Context for the current HIP device.  All copies and launches issued
+ * through it go to `hip_stream` (a hipStream_t; NULL = the null stream).  When
+ * `alloc`/`dealloc` are given, device memory comes from them (e.g. the embedding
+ * framework's caching allocator); otherwise from hipMalloc behind a size-class pool.
+ * `cache_workspace` != 0 keeps freed pool memory across executions.  Returns NULL on
+ * failure. */
+tao_ral_context_t disc_ral_context_create(void* hip_stream, int device_ordinal,
+                                          disc_ral_alloc_fn alloc,
+                                          disc_ral_dealloc_fn dealloc, void* user,
+                                          int cache_workspace);
+void disc_ral_context_destroy(tao_ral_context_t ctx);
+
+/* One ExecutionContext per run of a compiled program; destroying it returns every
+ * buffer the run allocated and did not hand back. */
+tao_ral_context_t disc_ral_execution_context_create(tao_ral_context_t ctx);
+void disc_ral_execution_context_destroy(tao_ral_context_t exec_ctx);
+tao_ral_context_t disc_ral_execution_context_get_context(tao_ral_context_t exec_ctx);
+
+/* ---- registry introspection ------------------------------------------- */
+
+int disc_ral_api_count(void);
+/* index in [0, count): keys in sorted order (full mangled names and bare names) */
+const char* disc_ral_api_name(int index);
+int disc_ral_api_exists(const char* name);
+
+/* Parses a serialized custom_attrs blob of `size` bytes (the last operand of every
+ * ral_pdll_* call; wire format: R disc/transforms/disc_lower_to_library_call.cc
+ * :684-848, reader R ral/context/pdll_util.cc:20-168) and renders it as JSON text
+ * into out[0..cap).  Returns the number of bytes the text needs (excluding the NUL),
+ * or -1 if the blob is malformed. */
+int64_t disc_ral_attr_to_json(const uint8_t* blob, size_t size, char* out, size_t cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TAO_RAL_API_H_ */

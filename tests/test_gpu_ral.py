@@ -1,0 +1,233 @@
+"""GPU tests of the drop-in boundary: every quantized entry is called through
+tao_ral_call_impl by its mangled name with compiler-style packed arguments and
+compared bit-for-bit with the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from bladedisc_amd import ral, ral_ops
+    ctx = ral.RalContext(stream=torch.cuda.current_stream().cuda_stream)
+    yield ctx, ral, ral_ops
+    torch.cuda.synchronize()
+    ctx.close()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def problem(seed, m, n, k):
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx = np.float32(rng.uniform(0.01, 0.03))
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40.0)
+    return rng, a, w, acc, sx, sw, so
+
+
+def f1(v):
+    return dev(np.array([v], np.float32))
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 768, 768), (1000, 3072, 768), (7, 40, 48)])
+def test_ral_qgemm_per_tensor_and_per_channel(rt, m, n, k):
+    ctx, ral, ops = rt
+    rng, a, w, acc, sx, sw, so = problem(m + n, m, n, k)
+    with ctx.execution() as ex:
+        got = ops.qgemm(ex, dev(a), dev(w), f1(sx), dev(sw), f1(so))
+        np.testing.assert_array_equal(host(got), O.requant_cpu(acc, sx, sw, so))
+        got = ops.qgemm(ex, dev(a), dev(w), f1(sx), f1(sw[0]), f1(so))
+        np.testing.assert_array_equal(host(got), O.requant_cpu(acc, sx, sw[:1], so))
+        # [K,N] weights (tp_b = false), as the CPU-style graphs pass them
+        got = ops.qgemm(ex, dev(a), dev(w.T.copy()), f1(sx), dev(sw), f1(so), tp_b=False,
+                        weight_is_const=False)   # per-call transpose through driver scratch
+        np.testing.assert_array_equal(host(got), O.requant_cpu(acc, sx, sw, so))
+
+
+def test_ral_qgemm_known_answer_gpu_case(rt, golden):
+    """The reference's (disabled) GPU test: 32x64x128, expect 128.0 after dequantize."""
+    ctx, ral, ops = rt
+    case = golden["qgemm"][1]
+    with ctx.execution() as ex:
+        x = torch.full((case["m"], case["k"]), case["x"], device="cuda")
+        z = torch.zeros(1, dtype=torch.int32, device="cuda")
+        qx = ops.quantize(ex, x, f1(case["sx"]), z)
+        w = torch.full((case["k"], case["n"]), case["w"], device="cuda")
+        qw = ops.quantize(ex, w, f1(case["sw"]), z)
+        out = ops.qgemm(ex, qx, qw, f1(case["sx"]), f1(case["sw"]), f1(case["so"]), tp_b=False)
+        f = ops.dequantize(ex, out, f1(case["so"]), z)
+        assert (host(f) == case["expect_f32"]).all()
+
+
+@pytest.mark.parametrize("rank", [2, 3])
+@pytest.mark.parametrize("bias_kind", ["s8", "f32"])
+def test_ral_pdll_qgemm_gpu_signature(rt, rank, bias_kind):
+    ctx, ral, ops = rt
+    m, n, k = 96, 256, 320
+    rng, a, w, acc, sx, sw, so = problem(rank * 10 + len(bias_kind), m, n, k)
+    if bias_kind == "s8":
+        bias = rng.integers(-128, 128, n).astype(np.int8)
+        want = O.requant_gpu(acc, sx, sw[:1], so, bias_i8=bias)
+    else:
+        bias = (rng.standard_normal(n) * 10).astype(np.float32)
+        want = O.requant_gpu(acc, sx, sw[:1], so, bias_f32=bias)
+    x = a if rank == 2 else a.reshape(4, 24, k)
+    with ctx.execution() as ex:
+        got = ops.pdll_qgemm_gpu(ex, dev(x), dev(w), dev(bias), f1(sx), f1(sw[0]), f1(so))
+        assert tuple(got.shape) == tuple(x.shape[:-1]) + (n,)
+        np.testing.assert_array_equal(host(got).reshape(m, n), want)
+
+
+def test_ral_pdll_qgemm_per_channel_merged_qkv(rt):
+    """Three per-tensor linears sharing an input, merged into one per-channel call
+    (disc_quantized_dot_merge.cc): equals the three separate results."""
+    ctx, ral, ops = rt
+    m, k, n1 = 128, 768, 768
+    rng = np.random.default_rng(99)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    ws = [rng.integers(-128, 128, (n1, k), dtype=np.int8) for _ in range(3)]
+    bs = [rng.integers(-128, 128, n1).astype(np.int8) for _ in range(3)]
+    sx = np.float32(0.02)
+    sws = [np.float32(s) for s in (0.011, 0.023, 0.017)]
+    sos = [np.float32(s) for s in (18.0, 33.0, 25.0)]
+    parts = []
+    for w, b, sw, so in zip(ws, bs, sws, sos):
+        acc, _ = O.gemm_s32_fast(a, w)
+        parts.append(O.requant_gpu(acc, sx, sw, so, bias_i8=b))
+    want = np.concatenate(parts, axis=1)
+    w_cat = np.concatenate(ws, axis=0)
+    b_cat = np.concatenate(bs)
+    sx_n = np.full(3 * n1, sx, np.float32)
+    sw_n = np.repeat(np.array(sws, np.float32), n1)
+    so_n = np.repeat(np.array(sos, np.float32), n1)
+    with ctx.execution() as ex:
+        got = ops.pdll_qgemm_per_channel(ex, dev(a), dev(w_cat), dev(b_cat), dev(sx_n),
+                                         dev(sw_n), dev(so_n))
+        np.testing.assert_array_equal(host(got), want)
+
+
+@pytest.mark.parametrize("bias_kind", ["none", "f32", "s32"])
+@pytest.mark.parametrize("rank", [2, 4])
+def test_ral_pdll_qgemm_cpu_style_signature(rt, bias_kind, rank):
+    ctx, ral, ops = rt
+    m, n, k = 64, 768, 768
+    rng, a, w, acc, sx, sw, so = problem(len(bias_kind) + rank, m, n, k)
+    bias = b32 = None
+    if bias_kind == "f32":
+        bias = (rng.standard_normal(n) * 0.01).astype(np.float32)
+        b32 = O.bias_f32_to_s32(bias, sx, sw)
+    elif bias_kind == "s32":
+        bias = b32 = rng.integers(-100000, 100000, n).astype(np.int32)
+    want = O.requant_cpu(acc, sx, sw, so, b32=b32, zo=3)
+    x = a if rank == 2 else a.reshape(2, 4, 8, k)
+    w_kn = dev(w.T.copy())
+    # constant weights are cached by address for the life of a context (as the
+    # reference caches pre-packed weights), so this test owns its context
+    ctx = ral.RalContext(stream=torch.cuda.current_stream().cuda_stream)
+    with ctx.execution() as ex:
+        for _ in range(2):   # second call hits the packed-weight cache
+            got = ops.pdll_qgemm_cpu_style(ex, dev(x), w_kn, dev(bias) if bias is not None else None,
+                                           f1(sx), dev(sw), f1(so), zo=3)
+            np.testing.assert_array_equal(host(got).reshape(m, n), want)
+        got = ops.pdll_qgemm_cpu_style(ex, dev(x), dev(w), dev(bias) if bias is not None else None,
+                                       f1(sx), dev(sw), f1(so), zo=3, transpose_b=True)
+        np.testing.assert_array_equal(host(got).reshape(m, n), want)
+    torch.cuda.synchronize()
+    ctx.close()
+
+
+def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
+    ctx, ral, ops = rt
+    with ctx.execution() as ex:
+        a = ex.new_args()
+        x = torch.zeros((4, 16), dtype=torch.int8, device="cuda")
+        w = torch.zeros((8, 16), dtype=torch.int8, device="cuda")
+        b = torch.zeros(8, dtype=torch.int8, device="cuda")
+        s = torch.ones(1, device="cuda")
+        a.tensor(x).tensor(w).tensor(b)
+        a.tensor(s, rank0=True).host_array(np.array([5], np.int32), rank0=True)
+        a.tensor(s, rank0=True).host_array(np.array([0], np.int32), rank0=True)
+        a.tensor(s, rank0=True).host_array(np.array([0], np.int32), rank0=True)
+        a.blob(ral.encode_attr({}))
+        a.result_memref("i8", 2)
+        with pytest.raises(ral.RalError, match="zero point"):
+            ex.call("ral_pdll_qgemm", "gpu", a)
+
+
+@pytest.mark.parametrize("nb,h,ci,co,k,stride,pad", [(2, 14, 64, 64, 3, 1, 1), (2, 7, 256, 128, 1, 1, 0),
+                                                      (1, 9, 32, 16, 3, 2, 1)])
+def test_ral_qconv(rt, nb, h, ci, co, k, stride, pad):
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(h + ci)
+    x = rng.integers(-128, 128, (nb, h, h, ci), dtype=np.int8)
+    w = rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8)
+    ho = (h + 2 * pad - k) // stride + 1
+    md = list(O.NHWC_OHWI_METADATA) + [stride, stride, 1, 1, 1]
+    padding = [pad] * 4
+    acc = O.conv_s32(x, w, padding, md, [nb, ho, ho, co])
+    sx = np.float32(0.02)
+    sw = rng.uniform(0.001, 0.05, co).astype(np.float32)
+    so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40.0)
+    want = O.requant_cpu(acc.reshape(-1, co), sx, sw, so).reshape(nb, ho, ho, co)
+    out = torch.empty((nb, ho, ho, co), dtype=torch.int8, device="cuda")
+    with ctx.execution() as ex:
+        ops.qconv(ex, dev(x), dev(w), padding, md, f1(sx), dev(sw), f1(so), out)
+        np.testing.assert_array_equal(host(out), want)
+
+
+@pytest.mark.parametrize("shape,axis", [((64, 768), None), ((64, 768), 1), ((768, 768), 0),
+                                        ((2, 14, 14, 64), 3)])
+def test_ral_quantize_dequantize(rt, shape, axis):
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(len(shape))
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    n = 1 if axis is None else shape[axis]
+    scale = rng.uniform(0.02, 0.08, n).astype(np.float32)
+    zp = rng.integers(-3, 4, n).astype(np.int32)
+    with ctx.execution() as ex:
+        q = ops.quantize(ex, dev(x), dev(scale), dev(zp), axis=axis)
+        want = O.quantize(x, scale, zp, axis=axis)
+        np.testing.assert_array_equal(host(q), want)
+        f = ops.dequantize(ex, q, dev(scale), dev(zp), axis=axis)
+        np.testing.assert_array_equal(host(f), O.dequantize(want, scale, zp, axis=axis))
+
+
+def test_driver_alloc_copy_roundtrip_and_pool_reuse(rt):
+    ctx, ral, ops = rt
+    import ctypes as C
+    with ctx.execution() as ex:
+        p1 = ex.alloc(1000)
+        assert p1
+        src = np.arange(250, dtype=np.int32)
+        dst = np.zeros(250, np.int32)
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0).scalar("pvoid", src.ctypes.data)
+        a.scalar("pvoid", p1).scalar("i64", 1000)
+        ex.call("h2d_", "gpu", a)
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0).scalar("pvoid", p1)
+        a.scalar("pvoid", dst.ctypes.data).scalar("i64", 1000)
+        ex.call("d2h_", "gpu", a)
+        ex.sync()
+        np.testing.assert_array_equal(dst, src)
+        ex.dealloc(p1)
+        p2 = ex.alloc(900)        # same size class (1024) -> the pooled block comes back
+        assert p2 == p1
+        ex.dealloc(p2)
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0)
+        r = a.result_scalar("pvoid")
+        ex.call("ral_gpu_as_cu_stream", "gpu", a)
+        assert (r.value or 0) == torch.cuda.current_stream().cuda_stream
+        del C
