@@ -7,6 +7,7 @@
 #include "dq8_common.h"
 #include "disc_q8.h"
 #include "qgemm_device.h"
+#include "qgemm_pipelined.h"
 
 #pragma clang fp contract(off)
 
@@ -156,7 +157,10 @@ const Variant kVariants[] = {
     {"mfma_256x256x64_w2x2", 256, 256, 64, 256},
     {"mfma_128x128x64_w2x2", 128, 128, 64, 256},
     {"mfma_64x64x64_w2x2", 64, 64, 64, 256},
+    // software-pipelined kernels (GEMM only; need K % bk == 0)
+    {"pipe_256x256x128", 256, 256, 128, 256},
 };
+constexpr int kFirstPipeVariant = 4;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
@@ -175,6 +179,26 @@ int launch_mfma(const MainParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_mfma launch");
 }
 
+template <int BM, int BN, int WM, int WN, int EPI>
+int launch_pipe(const MainParams& p, hipStream_t st) {
+  constexpr int BK = 128;
+  constexpr int lds = 2 * (BM + BN) * BK;
+  DQ8_REQUIRE(p.K >= BK && p.K % BK == 0, "pipelined qgemm needs K to be a multiple of the tile depth");
+  DQ8_REQUIRE((int64_t)BM * p.lda + p.K + 2 * BK < (1LL << 31) &&
+                  (int64_t)BN * p.ldw + p.K + 2 * BK < (1LL << 31),
+              "pipelined qgemm: row stride too large for 32-bit buffer offsets");
+  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, EPI>;
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  });
+  DQ8_HIP(attr_err);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(WM * WN * 64), lds, st, p);
+  return check_hip(hipGetLastError(), "qgemm_pipe launch");
+}
+
 template <bool CONV, int EPI>
 int launch_variant(int variant, MainParams& p, hipStream_t st) {
   const Variant& v = kVariants[variant];
@@ -185,7 +209,12 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case 2: return launch_mfma<128, 128, 64, 2, 2, CONV, EPI>(p, st);
     case 3: return launch_mfma<64, 64, 64, 2, 2, CONV, EPI>(p, st);
   }
-  return fail("unknown qgemm variant");
+  if constexpr (!CONV) {
+    switch (variant) {
+      case 4: return launch_pipe<256, 256, 2, 2, EPI>(p, st);
+    }
+  }
+  return fail("unknown or unsupported qgemm variant for this operation");
 }
 
 template <bool CONV>
@@ -204,11 +233,11 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 // smallest tile to spread the weight stream over as many CUs as possible.
 int pick_variant(int64_t M, int64_t N) {
   constexpr int64_t kCus = 256;
-  for (int v = 1; v < kNumVariants; ++v) {
+  for (int v = 1; v < kFirstPipeVariant; ++v) {
     const int64_t tiles = ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn);
     if (tiles >= kCus - kCus / 8) return v;
   }
-  return kNumVariants - 1;
+  return kFirstPipeVariant - 1;
 }
 
 int elem_size(int epilogue) {

@@ -189,6 +189,10 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
   return (bid % kXcd) * (nblocks / kXcd) + bid / kXcd;
 }
 
+template <int EPI, int FM, int FN>
+__device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
+                                              int m_base, int n_base);
+
 // LDS-tiled int8 GEMM on v_mfma_i32_32x32x32_i8.
 //   block tile BM x BN x BK, WM x WN waves, each wave a (BM/WM) x (BN/WN) tile
 //   built from 32x32 MFMA fragments; two LDS stages, global loads for stage
@@ -339,12 +343,16 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
     __syncthreads();
   }
 
-  // ---- epilogue: accumulator v of fragment (i,j) is output row
-  // m = m0 + wm*TM + i*32 + lane%32, channel n = n0 + wn*TN + j*32 + 8*(v/4) +
-  // 4*(lane/32) + v%4.
-  const EpiParams& e = p.epi;
-  const int m_base = m0 + wm * TM + (lane & 31);
-  const int n_base = n0 + wn * TN + 4 * (lane >> 5);
+  mfma_epilogue<EPI, FM, FN>(acc, p.epi, m0 + wm * TM + (lane & 31),
+                             n0 + wn * TN + 4 * (lane >> 5));
+}
+
+// Epilogue shared by the MFMA kernels.  Accumulator v of fragment (i,j) belongs to
+// output row m = m_base + i*32 (m_base already includes lane%32) and channel
+// n = n_base + j*32 + 8*(v/4) + v%4 (n_base already includes 4*(lane/32)).
+template <int EPI, int FM, int FN>
+__device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
+                                              int m_base, int n_base) {
 #pragma unroll
   for (int j = 0; j < FN; ++j) {
 #pragma unroll

@@ -1,0 +1,233 @@
+// Software-pipelined int8 MFMA GEMM for gfx950, used for the compute-bound
+// (large M) regime.  Block tile BM x BN x 128, WM x WN waves, two LDS stages.
+//
+// What shapes this kernel is the CU's vector-memory front end, not the MFMA pipe: a
+// 256x256 tile needs 64 KiB of operands per 128 of K, and the texture-address unit
+// retires a 64-lane 16-byte load at a rate set by how many cache lines each group
+// of four consecutive lanes touches.  Measured per CU (32 KiB, LDS-targeted loads):
+// 16 rows x 64 B with consecutive lanes on different rows 2150 cycles; 8 rows x
+// 128 B with consecutive lanes walking along a row 790 cycles; the 32 MFMAs that
+// consume those bytes take about 1250.  Hence:
+//  * BK = 128 and every load instruction covers 8 rows x one full 128-byte line,
+//    lanes 8r .. 8r+7 on row r;
+//  * loads write LDS directly (buffer_load_dwordx4 ... lds): no VGPR staging, no
+//    ds_write, rows past M / N and bytes past the matrix arrive as zeros;
+//  * a direct load puts lane i's 16 bytes at slot i of a 1 KiB block, so the block
+//    is 8 rows x 128 B row-major in LDS.  Read back naively, the 32 rows of an MFMA
+//    operand would hit the same banks; instead lane (r, s) fetches k-chunk
+//    c = s ^ r ^ (block & 1) of its row, i.e. chunk c of row r lives in slot
+//    c ^ r ^ (block & 1).  Any 8 consecutive rows then cover all 8 slots of a
+//    128-byte bank row and any 16 cover both halves of a 256-byte one, so the
+//    ds_read_b128 fragment reads are conflict free, while each quad of lanes still
+//    reads one contiguous 64-byte segment of global memory;
+//  * loads are issued one or two per row of four MFMAs, spread over the tile, so the
+//    wave never stalls on a full address queue, and as early as the ring allows;
+//  * fragments are double-buffered in registers; one barrier per tile.
+// Requires K % 128 == 0 and 16-byte aligned, k-contiguous operands.
+#ifndef DQ8_QGEMM_PIPELINED_H_
+#define DQ8_QGEMM_PIPELINED_H_
+
+#include "qgemm_device.h"
+
+namespace dq8 {
+
+// gfx9 raw buffer descriptor word 3: 32-bit data format, no swizzle
+constexpr int kBufferRsrcWord3 = 0x00020000;
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// 128-bit raw buffer descriptor (stride 0): base address, byte count, format word
+__device__ __forceinline__ v4i make_rsrc(const void* base, int64_t num_records) {
+  const uint64_t b = (uint64_t)base;
+  v4i r = {(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xffff), (int)num_records,
+           kBufferRsrcWord3};
+  return r;
+}
+
+// One 16-byte-per-lane buffer load whose result goes straight to LDS: lane i's
+// data lands at lds_addr + 16*i (lds_addr is wave-uniform and goes through M0).
+// Issued as inline assembly so that the wave decides itself, with an explicit
+// s_waitcnt vmcnt, when it needs the data; through the compiler builtin every LDS
+// read would first wait for all loads in flight.
+__device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, unsigned lds_addr, int voffset) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, 0 offen lds"
+      :
+      : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+      : "memory");
+}
+
+// s_waitcnt immediate for gfx9: vmcnt = n (6 bits, split), lgkmcnt = 0, expcnt = any
+constexpr int waitcnt_vm_lgkm0(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4); }
+
+template <int BM, int BN, int WM, int WN, int EPI>
+__global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParams p) {
+  // The inline assembly only assembles in the device compilation; the host pass
+  // just needs the kernel's stub.
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int BK = 128;
+  constexpr int NW = WM * WN;
+  constexpr int TM = BM / WM, TN = BN / WN;
+  constexpr int FM = TM / 32, FN = TN / 32;
+  constexpr int NKS = BK / 32;              // MFMA k-steps per tile (4)
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  // one wave-wide load instruction moves one 8-row block: 8 rows x 128 B = 1 KiB
+  constexpr int A_LD = (BM / 8) / NW;
+  constexpr int B_LD = (BN / 8) / NW;
+  constexpr int LD = A_LD + B_LD;           // load instructions per tile per wave
+  constexpr int ROWS = NKS * FM;            // rows of FN MFMAs per tile
+  static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile does not split over the waves");
+  static_assert(FM >= 1 && FN >= 1 && FN <= FM, "fragment mismatch");
+  static_assert(LD <= 63, "vmcnt is a 6-bit counter");
+  static_assert(LD <= 2 * (ROWS - FM), "not enough MFMA rows to spread the loads over");
+
+  extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int KT = p.K / BK;
+
+  // ---- buffer descriptors over the rows this block may touch
+  const int8_t* a_base = p.A + (int64_t)m0 * p.lda;
+  const int8_t* w_base = p.W + (int64_t)n0 * p.ldw;
+  const int64_t a_valid = (int64_t)(p.M - m0 - 1) * p.lda + p.K;
+  const int64_t w_valid = (int64_t)(p.N - n0 - 1) * p.ldw + p.K;
+  constexpr int64_t kMaxRecords = 0x7fffffff;
+  const v4i a_rsrc = make_rsrc(a_base, a_valid < kMaxRecords ? a_valid : kMaxRecords);
+  const v4i w_rsrc = make_rsrc(w_base, w_valid < kMaxRecords ? w_valid : kMaxRecords);
+  const unsigned lds_base = (unsigned)(size_t)(lds_void_t*)smem;
+
+  // ---- load slots.  Instruction i of this wave covers 8-row block q = wave + i*NW;
+  // lane -> row r = lane/8 of the block, LDS slot s = lane%8, global k-chunk
+  // c = s ^ r ^ (q & 1).
+  int a_off[A_LD], b_off[B_LD];      // byte offset of the lane's chunk in the block's rows
+  int a_lds[A_LD], b_lds[B_LD];      // wave-uniform LDS byte offset of the 1 KiB block
+  const int lr = lane >> 3, ls = lane & 7;
+#pragma unroll
+  for (int i = 0; i < A_LD; ++i) {
+    const int q = wave + i * NW;
+    a_off[i] = (q * 8 + lr) * (int)p.lda + ((ls ^ lr ^ (q & 1)) << 4);
+    a_lds[i] = __builtin_amdgcn_readfirstlane(q * 1024);
+  }
+#pragma unroll
+  for (int i = 0; i < B_LD; ++i) {
+    const int q = wave + i * NW;
+    b_off[i] = (q * 8 + lr) * (int)p.ldw + ((ls ^ lr ^ (q & 1)) << 4);
+    b_lds[i] = __builtin_amdgcn_readfirstlane(A_BYTES + q * 1024);
+  }
+
+  // issues load number `idx` (0 .. LD-1) of tile `kt` into stage `st`; tiles past the
+  // end of K get an out-of-range offset: zeros arrive, no memory is touched
+  auto issue_load = [&](int idx, int kt, int st) {
+    const int koff = kt < KT ? kt * BK : (int)0x80000000;
+    const unsigned base = lds_base + st * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i)
+      if (i == idx) buffer_load_lds_b128(a_rsrc, base + a_lds[i], a_off[i] + koff);
+#pragma unroll
+    for (int i = 0; i < B_LD; ++i)
+      if (A_LD + i == idx) buffer_load_lds_b128(w_rsrc, base + b_lds[i], b_off[i] + koff);
+  };
+
+  // ---- fragment addressing.  Operand row R = R0 + lane%32 sits in block R/8 at row
+  // R%8; the k-chunk c = 2*ks + lane/32 of that row is in slot c ^ (R%8) ^ (block&1).
+  // R0 is a multiple of 32, so the block parity is bit 3 of the lane.
+  const int row_in_frag = lane & 31;
+  const int swz = (lane & 7) ^ ((lane >> 3) & 1);
+  int frag_off[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks)
+    frag_off[ks] = (row_in_frag >> 3) * 1024 + (lane & 7) * 128 + (((2 * ks + (lane >> 5)) ^ swz) << 4);
+  const int a_frag0 = (wm * TM / 8) * 1024;
+  const int b_frag0 = A_BYTES + (wn * TN / 8) * 1024;
+
+  v4i fa[2][FM], fb[2][FN];
+  auto load_frag_a = [&](int set, int st, int ks, int i) {
+    fa[set][i] = *(const v4i*)(smem + st * STAGE + a_frag0 + i * 4096 + frag_off[ks]);
+  };
+  auto load_frag_b = [&](int set, int st, int ks, int j) {
+    fb[set][j] = *(const v4i*)(smem + st * STAGE + b_frag0 + j * 4096 + frag_off[ks]);
+  };
+
+  v16i acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  // Load schedule per tile: the first FM loads of tile t+1 go out right after the
+  // barrier of tile t-1 (riding on its last k-step); the rest follow, two per MFMA
+  // row, at the start of tile t.  What is left of tile t is landing time.
+  constexpr int EARLY = FM;
+
+  // ---- prologue: all of tile 0, then the early loads of tile 1
+#pragma unroll
+  for (int idx = 0; idx < LD; ++idx) issue_load(idx, 0, 0);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  __syncthreads();
+#pragma unroll
+  for (int idx = 0; idx < EARLY; ++idx) issue_load(idx, 1, 1);
+#pragma unroll
+  for (int i = 0; i < FM; ++i) load_frag_a(0, 0, 0, i);
+#pragma unroll
+  for (int j = 0; j < FN; ++j) load_frag_b(0, 0, 0, j);
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt & 1, nxt = cur ^ 1;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int fs = ks & 1, fn = fs ^ 1;
+      const bool last = ks == NKS - 1;
+      if (last) {
+        // tile kt+1 has landed for this wave, and this wave is done reading stage
+        // `cur`; after the barrier that holds for every wave
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+        __syncthreads();
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        const int row = ks * FM + i;
+        if (!last) {
+          load_frag_a(fn, cur, ks + 1, i);
+          if (i < FN) load_frag_b(fn, cur, ks + 1, i);
+          // remaining loads of tile kt+1 into the other stage, two per row
+          if (EARLY + 2 * row < LD) issue_load(EARLY + 2 * row, kt + 1, nxt);
+          if (EARLY + 2 * row + 1 < LD) issue_load(EARLY + 2 * row + 1, kt + 1, nxt);
+        } else {
+          // k-step 0 of tile kt+1, into the set the next iteration starts with
+          load_frag_a(0, nxt, 0, i);
+          if (i < FN) load_frag_b(0, nxt, 0, i);
+          // stage `cur` is free now: early loads of tile kt+2
+          if (i < EARLY) issue_load(i, kt + 2, cur);
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[fs][j], fa[fs][i], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  // nothing of this wave may still be writing LDS when the workgroup retires
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+
+  mfma_epilogue<EPI, FM, FN>(acc, p.epi, m0 + wm * TM + (lane & 31),
+                             n0 + wn * TN + 4 * (lane >> 5));
+#else
+  (void)p;
+#endif
+}
+
+}  // namespace dq8
+
+#endif  // DQ8_QGEMM_PIPELINED_H_

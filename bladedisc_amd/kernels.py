@@ -94,8 +94,11 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
     else [K,N]; scales are device f32 tensors with 1 or N entries."""
     _need_cuda(a, w, bias)
     L = _lib.lib()
-    a = a.contiguous()
-    w = w.contiguous()
+    # rows may be strided (leading dimension > row length); elements must be dense
+    if a.dim() != 2 or a.stride(1) != 1:
+        a = a.contiguous()
+    if w.dim() != 2 or w.stride(1) != 1:
+        w = w.contiguous()
     m, k = (a.shape[1], a.shape[0]) if tp_a else a.shape
     n = w.shape[0] if tp_b else w.shape[1]
     kw = w.shape[1] if tp_b else w.shape[0]
@@ -111,7 +114,8 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
     ws_bytes = L.dq8_qgemm_workspace_bytes(m, n, k, int(tp_a), int(tp_b))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     st = L.dq8_qgemm_variant(
-        variant, _ptr(a), a.shape[1], _ptr(w), w.shape[1], _ptr(out), out.stride(0) if m else n,
+        variant, _ptr(a), max(a.stride(0), a.shape[1]), _ptr(w), max(w.stride(0), w.shape[1]),
+        _ptr(out), out.stride(0) if m else n,
         m, n, k, int(tp_a), int(tp_b), epilogue, _ptr(bias), bias_kind,
         _ptr(sx), sx.numel() if sx is not None else 0,
         _ptr(sw), sw.numel() if sw is not None else 0,

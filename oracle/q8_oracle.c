@@ -248,13 +248,12 @@ void q8o_requant_cpu(const int32_t* acc, int64_t M, int64_t N,
  * and saturation (cublasLt CUDA_R_8I output with an f32 scale type). */
 void q8o_requant_gpu(const int32_t* acc, int64_t M, int64_t N,
                      const float* bias_f32, const int8_t* bias_i8,
-                     const float* sx, const float* sw, const float* so,
-                     int64_t n_s, int8_t* out) {
+                     const float* sx, int64_t n_sx, const float* sw,
+                     int64_t n_sw, const float* so, int64_t n_so, int8_t* out) {
   float* alpha = (float*)malloc(sizeof(float) * (size_t)(N > 0 ? N : 1));
   for (int64_t n = 0; n < N; ++n) {
-    int64_t i = n_s > 1 ? n : 0;
-    float t = sx[i] * sw[i];
-    alpha[n] = t / so[i];
+    float t = sx[n_sx > 1 ? n : 0] * sw[n_sw > 1 ? n : 0];
+    alpha[n] = t / so[n_so > 1 ? n : 0];
   }
 #pragma omp parallel for schedule(static)
   for (int64_t m = 0; m < M; ++m) {

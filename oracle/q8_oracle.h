@@ -88,11 +88,11 @@ void q8o_requant_cpu(const int32_t* acc, int64_t M, int64_t N,
                      int64_t n_sw, float so, int32_t zo, int8_t* out);
 
 /* E2.  Exactly one of bias_f32 / bias_i8 may be non-NULL (or none).
- * n_s is 1 (sx,sw,so rank-0) or N (all three are N-vectors). */
+ * Each of n_sx / n_sw / n_so is 1 (rank-0 scale) or N (per-channel vector). */
 void q8o_requant_gpu(const int32_t* acc, int64_t M, int64_t N,
                      const float* bias_f32, const int8_t* bias_i8,
-                     const float* sx, const float* sw, const float* so,
-                     int64_t n_s, int8_t* out);
+                     const float* sx, int64_t n_sx, const float* sw,
+                     int64_t n_sw, const float* so, int64_t n_so, int8_t* out);
 
 /* E3.  bias may be NULL. */
 void q8o_dequant_acc(const int32_t* acc, int64_t M, int64_t N, float sx,

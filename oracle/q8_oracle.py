@@ -130,13 +130,15 @@ def requant_gpu(acc, sx, sw, so, bias_f32=None, bias_i8=None):
     sx = _c(np.atleast_1d(sx), np.float32)
     sw = _c(np.atleast_1d(sw), np.float32)
     so = _c(np.atleast_1d(so), np.float32)
-    if not (sx.size == sw.size == so.size):
-        raise ValueError("E2 scales must all be rank-0 or all [N]")
+    for v in (sx, sw, so):
+        if v.size not in (1, n):
+            raise ValueError("E2 scales must have 1 or N entries")
     bf = _c(bias_f32, np.float32) if bias_f32 is not None else None
     bi = _c(bias_i8, np.int8) if bias_i8 is not None else None
     out = np.empty((m, n), np.int8)
     lib().q8o_requant_gpu(_p(acc), _i64(m), _i64(n), _p(bf), _p(bi), _p(sx),
-                          _p(sw), _p(so), _i64(sx.size), _p(out))
+                          _i64(sx.size), _p(sw), _i64(sw.size), _p(so),
+                          _i64(so.size), _p(out))
     return out
 
 
