@@ -179,14 +179,21 @@ int launch_mfma(const MainParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_mfma launch");
 }
 
+// The pipelined kernels need whole 128-deep k tiles and address each block's rows
+// with 32-bit buffer offsets.
+bool pipe_ok(int bm, int bn, int64_t K, int64_t lda, int64_t ldw) {
+  constexpr int BK = 128;
+  return K >= BK && K % BK == 0 && (int64_t)bm * lda + K + 2 * BK < (1LL << 31) &&
+         (int64_t)bn * ldw + K + 2 * BK < (1LL << 31);
+}
+
 template <int BM, int BN, int WM, int WN, int EPI>
 int launch_pipe(const MainParams& p, hipStream_t st) {
   constexpr int BK = 128;
   constexpr int lds = 2 * (BM + BN) * BK;
-  DQ8_REQUIRE(p.K >= BK && p.K % BK == 0, "pipelined qgemm needs K to be a multiple of the tile depth");
-  DQ8_REQUIRE((int64_t)BM * p.lda + p.K + 2 * BK < (1LL << 31) &&
-                  (int64_t)BN * p.ldw + p.K + 2 * BK < (1LL << 31),
-              "pipelined qgemm: row stride too large for 32-bit buffer offsets");
+  DQ8_REQUIRE(pipe_ok(BM, BN, p.K, p.lda, p.ldw),
+              "pipelined qgemm needs K to be a multiple of 128 and row strides that fit 32-bit "
+              "buffer offsets");
   auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, EPI>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
@@ -363,9 +370,11 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   e.zo = zo;
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
+  e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
 
   const bool need_generic = zx != 0 || zw != 0;
-  if (variant == -1) variant = need_generic ? 0 : pick_variant(M, N);
+  const bool auto_pick = variant == -1;
+  if (auto_pick) variant = need_generic ? 0 : pick_variant(M, N);
   if (variant == 0) {
     GenericParams g;
     g.A = A;
@@ -434,6 +443,9 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
         qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
         epilogue, g, M * N, st);
   }
+
+  // large problems whose K suits it go to the software-pipelined kernel of the same tile
+  if (auto_pick && variant == 1 && pipe_ok(256, 256, K, lda_use, ldw_use)) variant = kFirstPipeVariant;
 
   MainParams p = {};
   p.A = a_use;
@@ -524,6 +536,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   e.zo = zo;
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (Co % 4 == 0);
+  e.vec_store16 = aligned(out, 16) && (Co % 16 == 0);
 
   const bool nhwc_ohwi = ib == 0 && ic == 3 && ih == 1 && iw == 2 && ki == 3 && ko == 0 &&
                          kh == 1 && kw == 2 && ob == 0 && oc == 3 && oh == 1 && ow == 2;

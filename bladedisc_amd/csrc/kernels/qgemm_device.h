@@ -39,7 +39,8 @@ struct EpiParams {
   const float* so;
   int sx_stride, sw_stride, so_stride;  // 0 (rank-0 scale) or 1 (per channel)
   int zo;
-  int vec_store;  // 1: a group of 4 consecutive n may be stored as one 4/16-byte word
+  int vec_store;    // 1: a group of 4 consecutive n may be stored as one 4/16-byte word
+  int vec_store16;  // 1: int8 rows may be written with aligned 16-byte stores
 };
 
 // Operand description.  GEMM: A [M,K] (row stride lda), W [N,K] (row stride ldw).
@@ -108,18 +109,20 @@ __device__ __forceinline__ int sat_rne_s8(float d) {
   return (int)rintf(d);
 }
 
-// int8 result of one accumulator for the two requant modes
+// int8 result of one accumulator for the two requant modes.  The additive terms are
+// applied unconditionally (they are +0.0f when absent, which cannot change the
+// rounded integer), so the per-element code has no branches.
 template <int EPI>
 __device__ __forceinline__ int requant_one(const EpiParams& p, const ColParams& c,
                                            int acc) {
   float d = (float)acc;
   if (EPI == DQ8_EPI_REQUANT_CPU) {
-    if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
+    d = d + c.b;
     d = d * c.os;
-    if (p.zo != 0) d = d + (float)p.zo;
+    d = d + (float)p.zo;
   } else {
     d = c.os * d;
-    if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
+    d = d + c.b;
   }
   return sat_rne_s8(d);
 }
@@ -189,9 +192,10 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
   return (bid % kXcd) * (nblocks / kXcd) + bid / kXcd;
 }
 
-template <int EPI, int FM, int FN>
+template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
-                                              int m_base, int n_base);
+                                              int8_t* smem, int m_wave0, int n_wave0,
+                                              int n_blk0);
 
 // LDS-tiled int8 GEMM on v_mfma_i32_32x32x32_i8.
 //   block tile BM x BN x BK, WM x WN waves, each wave a (BM/WM) x (BN/WN) tile
@@ -343,28 +347,103 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
     __syncthreads();
   }
 
-  mfma_epilogue<EPI, FM, FN>(acc, p.epi, m0 + wm * TM + (lane & 31),
-                             n0 + wn * TN + 4 * (lane >> 5));
+  mfma_epilogue<EPI, FM, FN, NT, BN>(acc, p.epi, smem, m0 + wm * TM, n0 + wn * TN, n0);
 }
 
 // Epilogue shared by the MFMA kernels.  Accumulator v of fragment (i,j) belongs to
-// output row m = m_base + i*32 (m_base already includes lane%32) and channel
-// n = n_base + j*32 + 8*(v/4) + v%4 (n_base already includes 4*(lane/32)).
-template <int EPI, int FM, int FN>
+// output row m_wave0 + i*32 + lane%32 and channel n_wave0 + j*32 + 8*(v/4) +
+// 4*(lane/32) + v%4.
+//
+// The per-channel factors are computed once per block (thread t -> channel t) and
+// parked in LDS.  int8 results are then staged through LDS so that they leave the
+// CU as 16-byte stores with eight consecutive lanes covering one 128-byte line of
+// an output row: written straight from the accumulator layout, every store
+// instruction would touch 32 different rows with 8 bytes each.  The staging tile
+// swizzles its 16-byte chunks with the row number to keep both the dword writes
+// and the 16-byte reads spread over the banks.
+template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
-                                              int m_base, int n_base) {
+                                              int8_t* smem, int m_wave0, int n_wave0,
+                                              int n_blk0) {
+  constexpr int TM = FM * 32, TN = FN * 32;
+  constexpr int CH = TN / 16;                 // 16-byte chunks per staged row
+  constexpr int CP_BYTES = BN * 8;            // per-channel (scale, addend) pairs
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wn_off = n_wave0 - n_blk0;
+
+  __syncthreads();  // every wave is done with the operand tiles
+  float2* cp = reinterpret_cast<float2*>(smem);
+  for (int t = tid; t < BN; t += NT) {
+    const int n = n_blk0 + t;
+    const ColParams c = col_params<EPI>(e, n < e.N ? n : e.N - 1);
+    cp[t] = make_float2(c.os, c.b);
+  }
+  __syncthreads();
+
+  constexpr bool kInt8Out = EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU;
+  if (kInt8Out && e.vec_store16) {
+    int8_t* stage = smem + CP_BYTES + wave * (TM * TN);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
+        const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
+        const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
+        const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
+        const int chunk = j * 2 + (g >> 1);
+        const int dw = (2 * g + (lane >> 5)) & 3;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const int r = i * 32 + (lane & 31);
+          const int q0 = requant_one<EPI>(e, c[0], acc[i][j][4 * g + 0]);
+          const int q1 = requant_one<EPI>(e, c[1], acc[i][j][4 * g + 1]);
+          const int q2 = requant_one<EPI>(e, c[2], acc[i][j][4 * g + 2]);
+          const int q3 = requant_one<EPI>(e, c[3], acc[i][j][4 * g + 3]);
+          const uint32_t w = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) |
+                             ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
+          *reinterpret_cast<uint32_t*>(stage + r * TN + ((chunk ^ (r & (CH - 1))) << 4) + dw * 4) = w;
+        }
+      }
+    }
+    // the staging tile is private to the wave and LDS operations of one wave
+    // execute in order: no barrier needed before reading it back
+    constexpr int ROWS_PER_IT = 1024 / TN;
+    int8_t* out = static_cast<int8_t*>(e.out);
+#pragma unroll
+    for (int it = 0; it < TM / ROWS_PER_IT; ++it) {
+      const int row = it * ROWS_PER_IT + lane / CH;
+      const int chunk = lane % CH;
+      const v4i v = *reinterpret_cast<const v4i*>(stage + row * TN + ((chunk ^ (row & (CH - 1))) << 4));
+      const int m = m_wave0 + row, n = n_wave0 + chunk * 16;
+      if (m < e.M && n < e.N) {
+        int8_t* dst = out + (int64_t)m * e.ldo + n;
+        if (n + 15 < e.N) {
+          *reinterpret_cast<v4i*>(dst) = v;
+        } else {
+#pragma unroll
+          for (int b = 0; b < 16; ++b)
+            if (n + b < e.N) dst[b] = (int8_t)((uint32_t)v[b >> 2] >> (8 * (b & 3)));
+        }
+      }
+    }
+    return;
+  }
+
+  // direct stores: 4 consecutive channels of one row per accumulator quad
 #pragma unroll
   for (int j = 0; j < FN; ++j) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const int n = n_base + j * 32 + 8 * g;
+      const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
+      const int n = n_blk0 + cl;
       if (n >= e.N) continue;
-      ColParams c[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) c[q] = col_params<EPI>(e, n + q < e.N ? n + q : n);
+      const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
+      const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
+      const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        const int m = m_base + i * 32;
+        const int m = m_wave0 + i * 32 + (lane & 31);
         if (m < e.M)
           store_group4<EPI>(e, m, n, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
                             acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);

@@ -20,9 +20,16 @@
 //    128-byte bank row and any 16 cover both halves of a 256-byte one, so the
 //    ds_read_b128 fragment reads are conflict free, while each quad of lanes still
 //    reads one contiguous 64-byte segment of global memory;
-//  * loads are issued one or two per row of four MFMAs, spread over the tile, so the
-//    wave never stalls on a full address queue, and as early as the ring allows;
-//  * fragments are double-buffered in registers; one barrier per tile.
+//  * two 64 KiB stages fill the LDS.  All fragments of k-steps 2 and 3 are pulled
+//    into registers during k-step 1, so a stage is dead from k-step 2 on: it is handed
+//    back there ("stage free" barrier) and refilled while k-steps 2 and 3 still
+//    compute from registers, two loads per row of four MFMAs.  A tile's loads thus get
+//    most of a tile time to land before the "tile landed" barrier at k-step 3 of the
+//    next tile.
+// With random int8 operands and all 256 CUs busy the kernel is limited by the power
+// the matrix cores draw, not by its schedule: the shader clock, 2.4 GHz when a few
+// CUs run it, falls to 1.5-1.7 GHz (clock64 against wall_clock64), and variations of
+// the schedule that change the cycle count leave the time per tile where it is.
 // Requires K % 128 == 0 and 16-byte aligned, k-contiguous operands.
 #ifndef DQ8_QGEMM_PIPELINED_H_
 #define DQ8_QGEMM_PIPELINED_H_
@@ -82,7 +89,6 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile does not split over the waves");
   static_assert(FM >= 1 && FN >= 1 && FN <= FM, "fragment mismatch");
   static_assert(LD <= 63, "vmcnt is a 6-bit counter");
-  static_assert(LD <= 2 * (ROWS - FM), "not enough MFMA rows to spread the loads over");
 
   extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
 
@@ -150,7 +156,10 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   const int a_frag0 = (wm * TM / 8) * 1024;
   const int b_frag0 = A_BYTES + (wn * TN / 8) * 1024;
 
-  v4i fa[2][FM], fb[2][FN];
+  // Four fragment sets, one per k-step of a tile.  Set ks+1 is read one step ahead;
+  // during k-step 1 the sets for k-steps 2 AND 3 are read, so the stage is dead from
+  // k-step 2 on.
+  v4i fa[NKS][FM], fb[NKS][FN];
   auto load_frag_a = [&](int set, int st, int ks, int i) {
     fa[set][i] = *(const v4i*)(smem + st * STAGE + a_frag0 + i * 4096 + frag_off[ks]);
   };
@@ -166,18 +175,17 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-  // Load schedule per tile: the first FM loads of tile t+1 go out right after the
-  // barrier of tile t-1 (riding on its last k-step); the rest follow, two per MFMA
-  // row, at the start of tile t.  What is left of tile t is landing time.
-  constexpr int EARLY = FM;
+  // Load schedule: the LD loads of tile t+2 are issued two per row of MFMAs during
+  // k-steps 2 and 3 of tile t, into the stage tile t has just released.
+  static_assert(NKS == 4 && LD == 4 * FM, "schedule below assumes two loads per MFMA row of k-steps 2, 3");
 
-  // ---- prologue: all of tile 0, then the early loads of tile 1
+  // ---- prologue: all of tile 0, then all of tile 1
 #pragma unroll
   for (int idx = 0; idx < LD; ++idx) issue_load(idx, 0, 0);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   __syncthreads();
 #pragma unroll
-  for (int idx = 0; idx < EARLY; ++idx) issue_load(idx, 1, 1);
+  for (int idx = 0; idx < LD; ++idx) issue_load(idx, 1, 1);
 #pragma unroll
   for (int i = 0; i < FM; ++i) load_frag_a(0, 0, 0, i);
 #pragma unroll
@@ -187,33 +195,40 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
     const int cur = kt & 1, nxt = cur ^ 1;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      const int fs = ks & 1, fn = fs ^ 1;
-      const bool last = ks == NKS - 1;
-      if (last) {
-        // tile kt+1 has landed for this wave, and this wave is done reading stage
-        // `cur`; after the barrier that holds for every wave
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+      if (ks == 2) {
+        // this wave has read everything it needs from stage `cur`; once every wave
+        // has, the stage can take tile kt+2
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
+        __syncthreads();
+      }
+      if (ks == 3) {
+        // tile kt+1 (older than the 2*FM loads of tile kt+2 just issued) has landed
+        // for this wave; after the barrier, for all of them
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * FM));
         __syncthreads();
       }
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        const int row = ks * FM + i;
-        if (!last) {
-          load_frag_a(fn, cur, ks + 1, i);
-          if (i < FN) load_frag_b(fn, cur, ks + 1, i);
-          // remaining loads of tile kt+1 into the other stage, two per row
-          if (EARLY + 2 * row < LD) issue_load(EARLY + 2 * row, kt + 1, nxt);
-          if (EARLY + 2 * row + 1 < LD) issue_load(EARLY + 2 * row + 1, kt + 1, nxt);
+        if (ks == 0) {
+          load_frag_a(1, cur, 1, i);
+          if (i < FN) load_frag_b(1, cur, 1, i);
+        } else if (ks == 1) {
+          load_frag_a(2, cur, 2, i);
+          if (i < FN) load_frag_b(2, cur, 2, i);
+          load_frag_a(3, cur, 3, i);
+          if (i < FN) load_frag_b(3, cur, 3, i);
+        } else if (ks == 2) {
+          issue_load(2 * i, kt + 2, cur);
+          issue_load(2 * i + 1, kt + 2, cur);
         } else {
-          // k-step 0 of tile kt+1, into the set the next iteration starts with
           load_frag_a(0, nxt, 0, i);
           if (i < FN) load_frag_b(0, nxt, 0, i);
-          // stage `cur` is free now: early loads of tile kt+2
-          if (i < EARLY) issue_load(i, kt + 2, cur);
+          issue_load(2 * FM + 2 * i, kt + 2, cur);
+          issue_load(2 * FM + 2 * i + 1, kt + 2, cur);
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[fs][j], fa[fs][i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -221,8 +236,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   // nothing of this wave may still be writing LDS when the workgroup retires
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
 
-  mfma_epilogue<EPI, FM, FN>(acc, p.epi, m0 + wm * TM + (lane & 31),
-                             n0 + wn * TN + 4 * (lane >> 5));
+  mfma_epilogue<EPI, FM, FN, NW * 64, BN>(acc, p.epi, smem, m0 + wm * TM, n0 + wn * TN, n0);
 #else
   (void)p;
 #endif

@@ -352,5 +352,5 @@ def test_bad_arguments_fail_loudly(K):
     with pytest.raises(RuntimeError):
         K.qgemm(a, w, K.EPI_ACC_S32, variant=99)
     pipe = [i for i, n in enumerate(K.variant_names()) if n.startswith("pipe_")][0]
-    with pytest.raises(RuntimeError, match="multiple of the tile depth"):
+    with pytest.raises(RuntimeError, match="multiple of 128"):
         K.qgemm(a, w, K.EPI_ACC_S32, variant=pipe)      # K = 16
