@@ -23,6 +23,12 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, 5.0 POP/s
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, 8 TB/s
 
+# Bytes the L2s exchange with the memory side per launch of the headline kernel, from
+# two rocprofv3 --pmc passes over this script (FETCH_SIZE, WRITE_SIZE; summary and
+# commands in profiles/qgemm_4096_requant_hbm_traffic.md).  Counters cannot be read
+# from inside the run, so the figure is recorded here for the size it was measured on.
+MEASURED_TRAFFIC_BYTES = {4096: (98924 + 16384) * 1024}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -32,6 +38,14 @@ def parse():
     p.add_argument("--size", type=int, default=4096, help="M = N = K of the headline GEMM")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extra", action="store_true", help="skip the q/dq and sweep extras")
+    p.add_argument("--pattern", choices=("uniform", "ones"), default="uniform",
+                   help="operand values: 'uniform' is the benchmark's definition (integers uniform "
+                        "in [-127,127]); 'ones' is a diagnosis aid that shows how much of the time "
+                        "is the power drawn by toggling operands (same instructions, same traffic)")
+    p.add_argument("--copy-probe", action="store_true",
+                   help="also launch one plain streaming kernel of known size before the timed "
+                        "loop (dst = src + 1 over 1 GiB of int8: reads 1 GiB, writes 1 GiB), the "
+                        "yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     return p.parse_args()
 
 
@@ -62,8 +76,9 @@ class GemmCall:
         m, k = a.shape
         n = w.shape[0]
         vp = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+        cnt = lambda t: t.numel() if t is not None else 0  # noqa: E731
         self.args = (vp(a), k, vp(w), k, vp(out), n, m, n, k, 0, 1, epilogue, vp(bias),
-                     bias_kind, vp(sx), sx.numel(), vp(sw), sw.numel(), vp(so), so.numel(),
+                     bias_kind, vp(sx), cnt(sx), vp(sw), cnt(sw), vp(so), cnt(so),
                      0, 0, 0, None, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
 
     def __call__(self):
@@ -166,6 +181,22 @@ def extras(torch, steps, warmup):
             "roofline_frac": round(max(ops / us / 1e6 / PEAK_INT8_TOPS,
                                        byts / us / 1e3 / PEAK_HBM_GBPS), 4)}
     out["qgemm_bert_shapes_requant_cpu"] = sweep
+    # yardstick: the ROCm library int8 GEMM behind torch._int_mm (int32 output, no
+    # epilogue) on the headline shape and data distribution -- a library, not the reference
+    try:
+        a = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device="cuda")
+        w = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device="cuda")
+        wt = w.t()
+        _, ev = time_steps(torch, lambda: torch._int_mm(a, wt), 50, 5)
+        o32 = torch.empty((4096, 4096), dtype=torch.int32, device="cuda")
+        call = GemmCall(torch, a, w, None, None, None, None, 0, 0, o32)
+        _, ev2 = time_steps(torch, call, 50, 5)
+        out["rocm_library_int_mm_4096_s32"] = {
+            "library_us": round(ev / 50 * 1e6, 2), "library_TOPS": round(2.0 * 4096 ** 3 / (ev / 50) / 1e12, 1),
+            "dq8_qgemm_acc_s32_us": round(ev2 / 50 * 1e6, 2),
+            "dq8_qgemm_acc_s32_TOPS": round(2.0 * 4096 ** 3 / (ev2 / 50) / 1e12, 1)}
+    except Exception as exc:  # the yardstick is optional
+        out["rocm_library_int_mm_4096_s32"] = {"error": str(exc)[:200]}
     return out
 
 
@@ -183,6 +214,9 @@ def main():
 
     size = args.size
     a, w, sx, sw, so, bias_q = make_problem(torch, size)
+    if args.pattern == "ones":
+        a[:] = 1
+        w[:] = 1
     d = lambda v: torch.from_numpy(v).cuda()  # noqa: E731
     import numpy as np
     da, dw = d(a), d(w)
@@ -191,6 +225,13 @@ def main():
     out = torch.empty((size, size), dtype=torch.int8, device="cuda")
     # REQUANT_GPU epilogue (2) with an f32 bias (kind 2): out = sat8(rne(os[n]*acc + b[n]))
     call = GemmCall(torch, da, dw, dsx, dsw, dso, dbias, 2, 2, out)
+
+    if args.copy_probe:
+        src = torch.ones(1 << 30, dtype=torch.int8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     wall, ev = time_steps(torch, call, args.steps, args.warmup)
     ops = 2.0 * size * size * size
@@ -222,6 +263,8 @@ def main():
                         "f32 bias + requant to s8 (round-half-even, saturate)" % size,
             "entry": "dq8_qgemm (C ABI), epilogue REQUANT_GPU",
             "saturated_fraction": round(sat_frac, 4),
+            "operand_values": "uniform integers in [-127,127]" if args.pattern == "uniform"
+                              else "all ones (diagnosis run, not the benchmark's data)",
         },
         "roofline": {
             "bound": "mfma",
@@ -229,7 +272,8 @@ def main():
             "peak": PEAK_INT8_TOPS,
             "unit": "TOP/s",
             "frac": round(achieved / PEAK_INT8_TOPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(size) if args.pattern == "uniform" else None,
+            "algorithmic_bytes": 3 * size * size + 8 * size,
             "kernel_us": round(kernel_s * 1e6, 2),
             "ops_per_launch": ops,
         },

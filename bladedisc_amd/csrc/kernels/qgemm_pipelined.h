@@ -97,8 +97,8 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
 
-  const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  int tm, tn;
+  tile_coords(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int KT = p.K / BK;
 
