@@ -150,13 +150,23 @@ def extras(torch, steps, warmup):
     z1 = torch.zeros(1, dtype=torch.int32, device="cuda")
     sc = torch.full((cols,), 0.05, device="cuda")
     zc = torch.zeros(cols, dtype=torch.int32, device="cuda")
+    sr = torch.full((rows,), 0.05, device="cuda")
+    zr = torch.zeros(rows, dtype=torch.int32, device="cuda")
     nbytes = 5.0 * rows * cols
     reps = max(5, min(steps, 20))
-    for name, fn in (
+    cases = (
             ("quantize_per_tensor", lambda: K.quantize(x, s1, z1, out=q)),
             ("dequantize_per_tensor", lambda: K.dequantize(q, s1, z1, out=f)),
-            ("quantize_per_channel", lambda: K.quantize(x, sc, zc, axis=1, out=q)),
-            ("dequantize_per_channel", lambda: K.dequantize(q, sc, zc, axis=1, out=f))):
+            ("quantize_per_channel_last_axis", lambda: K.quantize(x, sc, zc, axis=1, out=q)),
+            ("dequantize_per_channel_last_axis", lambda: K.dequantize(q, sc, zc, axis=1, out=f)),
+            ("quantize_per_channel_axis0", lambda: K.quantize(x, sr, zr, axis=0, out=q)),
+            ("dequantize_per_channel_axis0", lambda: K.dequantize(q, sr, zr, axis=0, out=f)))
+    for _ in range(10):
+        for _, fn in cases:
+            fn()
+    for name, fn in cases:
+        # (freshly allocated device memory is slow for its first passes, hence the
+        # warm-up rounds over all cases above)
         _, ev = time_steps(torch, fn, reps, 3)
         gbps = nbytes * reps / ev / 1e9
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
