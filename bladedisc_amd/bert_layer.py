@@ -1,0 +1,154 @@
+"""Quantized BERT-base encoder layer on the quantized RAL entries.
+
+The counterpart of what the reference's post-training-quantization example produces
+for one encoder layer (examples/PyTorch/Quantization/bert_ptq.py, pytorch_blade/tests/
+quantization): the four linears (merged QKV, attention output, FFN1, FFN2) run as
+int8 GEMMs with per-tensor activation scales, per-output-channel weight scales and a
+fused bias + requantisation; ``quantize`` / ``dequantize`` sit between them and the
+fp32 LayerNorm / softmax / GELU, which PyTorch computes.  Scales come from a min/max
+calibration pass, as the reference's observers produce them.
+
+Two backends execute the quantized operators:
+  RalBackend  through ``tao_ral_call_impl`` by mangled name (what a compiled program does),
+  RawBackend  through the raw kernel C ABI (``dq8_*``), the cheaper path for timing.
+Both run the same HIP kernels.
+"""
+import math
+
+import numpy as np
+import torch
+
+from . import baseline_configs as cfg
+from . import kernels as K
+from . import ral_ops
+
+LINEARS = ("qkv", "out", "ffn1", "ffn2")
+
+
+class RawBackend:
+    name = "raw"
+
+    def __init__(self, device="cuda"):
+        self.z1 = torch.zeros(1, dtype=torch.int32, device=device)
+
+    def quantize(self, x, scale):
+        return K.quantize(x, scale, self.z1)
+
+    def dequantize(self, q, scale):
+        return K.dequantize(q, scale, self.z1)
+
+    def qlinear(self, x_q, w_q, bias, sx, sw, so):
+        """E1: sat8(rne((acc + b32) * (sx*sw/so))) with the f32 bias folded to int32."""
+        return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so, bias=bias)
+
+
+class RalBackend:
+    name = "ral"
+
+    def __init__(self, execution, device="cuda"):
+        self.ex = execution
+        self.z1 = torch.zeros(1, dtype=torch.int32, device=device)
+
+    def quantize(self, x, scale):
+        return ral_ops.quantize(self.ex, x, scale, self.z1)
+
+    def dequantize(self, q, scale):
+        return ral_ops.dequantize(self.ex, q, scale, self.z1)
+
+    def qlinear(self, x_q, w_q, bias, sx, sw, so):
+        return ral_ops.pdll_qgemm_cpu_style(self.ex, x_q, w_q, bias, sx, sw, so,
+                                            transpose_b=True, weight_is_const=True)
+
+
+def _layer_norm(x, g, b):
+    return torch.nn.functional.layer_norm(x, (x.shape[-1],), g, b, 1e-12)
+
+
+class QuantBertLayer:
+    """One encoder layer; hidden 768, 12 heads, FFN 3072 by default."""
+
+    def __init__(self, weights, backend, heads=12, device="cuda"):
+        self.be = backend
+        self.heads = heads
+        self.device = device
+        d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)  # noqa: E731
+        w = weights
+        self.f = {k: d(v) for k, v in w.items()}          # fp32 master copies
+        merged_w = np.concatenate([w["wq"], w["wk"], w["wv"]], axis=0)
+        merged_b = np.concatenate([w["bq"], w["bk"], w["bv"]], axis=0)
+        self.fw = {"qkv": merged_w, "out": w["wo"], "ffn1": w["w1"], "ffn2": w["w2"]}
+        self.fb = {"qkv": merged_b, "out": w["bo"], "ffn1": w["b1"], "ffn2": w["b2"]}
+        self.w_q, self.sw, self.bias = {}, {}, {}
+        for name in LINEARS:
+            sw = cfg.sym_scale(self.fw[name], axis=0)
+            self.w_q[name] = d(cfg.quantize_host(self.fw[name], sw, axis=0))
+            self.sw[name] = d(sw)
+            self.bias[name] = d(self.fb[name])
+        self.s_in, self.s_out = {}, {}
+
+    # ---------------------------------------------------------------- fp32 parts
+    def embed(self, tokens):
+        t = torch.as_tensor(tokens, device=self.device)
+        pos = torch.arange(t.shape[1], device=self.device)
+        h = self.f["tok_emb"][t] + self.f["pos_emb"][pos][None]
+        return _layer_norm(h, self.f["emb_ln_g"], self.f["emb_ln_b"])
+
+    def attention(self, qkv):
+        """softmax(q k^T / sqrt(d)) v in fp32.  qkv: [B, S, 3H] -> [B, S, H]."""
+        b, s, h3 = qkv.shape
+        h = h3 // 3
+        dh = h // self.heads
+        q, k, v = (t.reshape(b, s, self.heads, dh).transpose(1, 2) for t in qkv.split(h, dim=-1))
+        p = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(dh), dim=-1)
+        return (p @ v).transpose(1, 2).reshape(b, s, h)
+
+    def _linear_fp32(self, name, x):
+        return x @ torch.from_numpy(self.fw[name]).to(self.device).T + self.bias[name]
+
+    def forward_fp32(self, h, record=None):
+        """The unquantized layer; `record` collects the inputs / outputs of the linears."""
+        rec = record if record is not None else {}
+        rec["qkv_in"] = h
+        rec["qkv_out"] = self._linear_fp32("qkv", h)
+        rec["out_in"] = self.attention(rec["qkv_out"])
+        rec["out_out"] = self._linear_fp32("out", rec["out_in"])
+        rec["ffn1_in"] = _layer_norm(h + rec["out_out"], self.f["ln1_g"], self.f["ln1_b"])
+        rec["ffn1_out"] = self._linear_fp32("ffn1", rec["ffn1_in"])
+        rec["ffn2_in"] = torch.nn.functional.gelu(rec["ffn1_out"])
+        rec["ffn2_out"] = self._linear_fp32("ffn2", rec["ffn2_in"])
+        return _layer_norm(rec["ffn1_in"] + rec["ffn2_out"], self.f["ln2_g"], self.f["ln2_b"])
+
+    def calibrate(self, h):
+        """Min/max calibration: symmetric per-tensor scale max|x|/127 for the input and
+        the output of each linear, from one fp32 pass."""
+        rec = {}
+        self.forward_fp32(h, rec)
+        for name in LINEARS:
+            for which, store in (("in", self.s_in), ("out", self.s_out)):
+                amax = rec["%s_%s" % (name, which)].abs().max().clamp_min(1e-12)
+                store[name] = (amax / 127.0).reshape(1).float()
+        return rec
+
+    # ----------------------------------------------------------- quantized layer
+    def _qlinear(self, name, x, rec):
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        x_q = self.be.quantize(x2, self.s_in[name])
+        y_q = self.be.qlinear(x_q, self.w_q[name], self.bias[name], self.s_in[name],
+                              self.sw[name], self.s_out[name])
+        y = self.be.dequantize(y_q, self.s_out[name])
+        if rec is not None:
+            rec[name] = dict(x=x2, x_q=x_q, y_q=y_q, y=y)
+        return y.reshape(*shape[:-1], y.shape[-1])
+
+    def forward(self, h, record=None):
+        if not self.s_in:
+            raise RuntimeError("calibrate() first")
+        qkv = self._qlinear("qkv", h, record)
+        ctx = self.attention(qkv)
+        attn = self._qlinear("out", ctx, record)
+        h1 = _layer_norm(h + attn, self.f["ln1_g"], self.f["ln1_b"])
+        f1 = self._qlinear("ffn1", h1, record)
+        g = torch.nn.functional.gelu(f1)
+        f2 = self._qlinear("ffn2", g, record)
+        return _layer_norm(h1 + f2, self.f["ln2_g"], self.f["ln2_b"])
