@@ -49,20 +49,11 @@ def parse():
     return p.parse_args()
 
 
-def make_problem(torch, size, seed=1236):
-    """BASELINE config 3 inputs (seed = 1234 + config index)."""
-    import numpy as np
-    rng = np.random.default_rng(seed)
-    m = n = k = size
-    a = rng.integers(-127, 128, (m, k), dtype=np.int8)
-    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
-    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
-    sx = np.float32(0.02)
-    # std of an accumulator of K products of two uniform[-127,127] integers
-    std_acc = np.sqrt(k) * (127.0 * 128.0 / 3.0)
-    so = np.float32(float(sx) * float(sw.mean()) * std_acc / 40.0)
-    bias_q = (rng.standard_normal(n) * 10.0).astype(np.float32)  # bias / s_o
-    return a, w, sx, sw, so, bias_q
+def make_problem(torch, size):
+    """BASELINE config 3 inputs."""
+    from bladedisc_amd import baseline_configs as cfg
+    c = cfg.config3(size)
+    return c["a_q"], c["w_q"], c["sx"], c["sw"], c["so"], c["bias_q"]
 
 
 class GemmCall:
@@ -79,12 +70,42 @@ class GemmCall:
         cnt = lambda t: t.numel() if t is not None else 0  # noqa: E731
         self.args = (vp(a), k, vp(w), k, vp(out), n, m, n, k, 0, 1, epilogue, vp(bias),
                      bias_kind, vp(sx), cnt(sx), vp(sw), cnt(sw), vp(so), cnt(so),
-                     0, 0, 0, None, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+                     0, 0, 0, None, 0)
+        self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def __call__(self):
-        st = self.L.dq8_qgemm(*self.args)
+        st = self.L.dq8_qgemm(*self.args, self.stream)
         if st != 0:
             raise RuntimeError(self.L.dq8_last_error().decode())
+
+
+def time_graph(torch, calls, launches=20, replays=10):
+    """GPU time per pass over `calls` (objects with a .stream attribute and __call__)
+    with the launches captured into a HIP graph, so that short kernels are timed back to
+    back instead of at the rate Python can launch them.  Returns seconds per pass."""
+    side = torch.cuda.Stream()
+    saved = [c.stream for c in calls]
+    graph = torch.cuda.CUDAGraph()
+    try:
+        with torch.cuda.graph(graph, stream=side):
+            handle = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for c in calls:
+                c.stream = handle
+            for _ in range(launches):
+                for c in calls:
+                    c()
+    finally:
+        for c, st in zip(calls, saved):
+            c.stream = st
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / (launches * replays)
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -137,9 +158,195 @@ def cpu_baseline(a, w, sx, sw, so, bias_q, budget_s=12.0):
                       % (reps, rows, a.shape[0], a.shape[0], n, k, dt)}
 
 
+class FnCall:
+    """Adapter so that time_graph can drive any launcher that uses torch's current
+    stream."""
+    stream = None
+
+    def __init__(self, fn):
+        self.fn = fn
+
+    def __call__(self):
+        self.fn()
+
+
+def cpu_time(fn, min_time=0.3, max_reps=10):
+    """Best wall time of fn over a few repetitions (at least min_time in total)."""
+    fn()
+    best, total, reps = float("inf"), 0.0, 0
+    while reps < max_reps and (total < min_time or reps < 2):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best, total, reps = min(best, dt), total + dt, reps + 1
+    return best
+
+
+def roof(ops, byts, seconds):
+    """TOP/s, GB/s and the larger of the two roofline fractions."""
+    tops, gbps = ops / seconds / 1e12, byts / seconds / 1e9
+    return {"us": round(seconds * 1e6, 2), "TOPS": round(tops, 2), "GB/s": round(gbps, 1),
+            "roofline_frac": round(max(tops / PEAK_INT8_TOPS, gbps / PEAK_HBM_GBPS), 4)}
+
+
+def config_reports(torch, K):
+    """All five benchmark configurations: GPU time of the quantized operators (launches
+    captured in a HIP graph, inputs resident) next to the CPU oracle on the host cores.
+    Parity of exactly these inputs is what tests/test_gpu_configs.py checks."""
+    import numpy as np
+    import oracle as O
+    from bladedisc_amd import baseline_configs as cfg
+    dev = lambda v: torch.from_numpy(np.ascontiguousarray(v)).cuda()  # noqa: E731
+    f1 = lambda v: dev(np.array([v], np.float32))                     # noqa: E731
+    z1 = torch.zeros(1, dtype=torch.int32, device="cuda")
+    rep = {}
+
+    # ---- 1: single quantized linear, f32 in -> f32 out
+    c = cfg.config1()
+    x, wq, bias = dev(c["x"]), dev(c["w_q"]), dev(c["bias"])
+    sx, sw, so = f1(c["sx"]), dev(c["sw"]), f1(c["so"])
+    xq = torch.empty((64, 768), dtype=torch.int8, device="cuda")
+    yq = torch.empty((64, 768), dtype=torch.int8, device="cuda")
+    y = torch.empty((64, 768), device="cuda")
+    chain = [FnCall(lambda: K.quantize(x, sx, z1, out=xq)),
+             FnCall(lambda: K.qgemm(xq, wq, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so, bias=bias, out=yq)),
+             FnCall(lambda: K.dequantize(yq, so, z1, out=y))]
+    gpu_s = time_graph(torch, chain)
+
+    def cpu1():
+        q = O.quantize(c["x"], c["sx"], 0)
+        acc, _ = O.gemm_s32_fast(q, c["w_q"])
+        b32 = O.bias_f32_to_s32(c["bias"], float(c["sx"]), c["sw"])
+        O.dequantize(O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]), b32=b32), c["so"], 0)
+    cpu_s = cpu_time(cpu1)
+    rep["1_single_linear_64x768x768_q_gemm_dq"] = {
+        "gpu_us": round(gpu_s * 1e6, 2), "cpu_us": round(cpu_s * 1e6, 1),
+        "gpu_over_cpu": round(cpu_s / gpu_s, 1)}
+
+    # ---- 2: dynamic-M sweep, E1 requant, int8 out
+    sweep = {}
+    for (k, n) in cfg.BERT_LINEARS:
+        for m in cfg.SWEEP_M:
+            c = cfg.config2(m, k, n)
+            a, w = dev(c["a_q"]), dev(c["w_q"])
+            sx, sw, so = f1(c["sx"]), dev(c["sw"]), f1(c["so"])
+            o = torch.empty((m, n), dtype=torch.int8, device="cuda")
+            call = GemmCall(torch, a, w, sx, sw, so, None, 1, 0, o)
+            gpu_s = time_graph(torch, [call])
+
+            def cpu2():
+                acc, _ = O.gemm_s32_fast(c["a_q"], c["w_q"])
+                O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]))
+            cpu_s = cpu_time(cpu2, min_time=0.05, max_reps=5)
+            r = roof(2.0 * m * n * k, m * k + n * k + m * n + 4 * n, gpu_s)
+            r["cpu_us"] = round(cpu_s * 1e6, 1)
+            sweep["M%d_K%d_N%d" % (m, k, n)] = r
+    rep["2_dynamic_m_sweep_requant"] = sweep
+
+    # ---- 3: 8192^3 next to the headline 4096^3
+    c = cfg.config3(8192)
+    a, w = dev(c["a_q"]), dev(c["w_q"])
+    o = torch.empty((8192, 8192), dtype=torch.int8, device="cuda")
+    call = GemmCall(torch, a, w, f1(c["sx"]), dev(c["sw"]), f1(c["so"]), dev(c["bias_q"]), 2, 2, o)
+    _, ev = time_steps(torch, call, 20, 3)
+    r = roof(2.0 * 8192 ** 3, 3 * 8192 ** 2 + 8 * 8192, ev / 20)
+
+    def cpu3():
+        acc, _ = O.gemm_s32_fast(c["a_q"], c["w_q"])
+        O.requant_gpu(acc, c["sx"], c["sw"], c["so"], bias_f32=c["bias_q"])
+    r["cpu_us"] = round(cpu_time(cpu3, min_time=0.0, max_reps=2) * 1e6, 1)
+    rep["3_large_square_8192_fused_bias_requant"] = r
+    del a, w, o, call
+
+    # ---- 4: int8 NHWC convolutions
+    convs = {}
+    for conv in cfg.RESNET_CONVS:
+        c = cfg.config4(conv)
+        nb, h, w_, ci, co, k = (conv[t] for t in ("nb", "h", "w", "ci", "co", "k"))
+        pad4, md, osh = O.conv_attrs((nb, h, w_, ci), (co, k, k, ci), "NHWC", [1, 1, 1, 1],
+                                     [1, 1, 1, 1], "EXPLICIT",
+                                     explicit_paddings=[0, 0, conv["pad"], conv["pad"],
+                                                        conv["pad"], conv["pad"], 0, 0])
+        md[:12] = O.NHWC_OHWI_METADATA
+        xq, wq = dev(c["x_q"]), dev(c["w_q"])
+        sx, sw, so = f1(c["sx"]), dev(c["sw"]), f1(c["so"])
+        o = torch.empty(tuple(osh), dtype=torch.int8, device="cuda")
+        gpu_s = time_graph(torch, [FnCall(lambda: K.qconv2d(xq, wq, pad4, md, osh, K.EPI_REQUANT_CPU,
+                                                            sx=sx, sw=sw, so=so, out=o))])
+        mg, kg = nb * osh[1] * osh[2], k * k * ci
+        r = roof(2.0 * mg * co * kg, nb * h * w_ * ci + co * kg + mg * co + 4 * co, gpu_s)
+        # CPU: the GEMM the convolution reduces to (im2col done beforehand, not timed)
+        cols = np.ascontiguousarray(np.lib.stride_tricks.sliding_window_view(
+            np.pad(c["x_q"], ((0, 0), (conv["pad"],) * 2, (conv["pad"],) * 2, (0, 0))),
+            (k, k), axis=(1, 2)).transpose(0, 1, 2, 4, 5, 3).reshape(mg, kg))
+        wmat = c["w_q"].reshape(co, kg)
+
+        def cpu4():
+            acc, _ = O.gemm_s32_fast(cols, wmat)
+            O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]))
+        r["cpu_us"] = round(cpu_time(cpu4, min_time=0.05, max_reps=5) * 1e6, 1)
+        r["cpu_note"] = "int8 GEMM of the pre-built im2col matrix + requant"
+        convs[conv["name"]] = r
+        del cols
+    rep["4_resnet_convs_requant"] = convs
+
+    # ---- 5: quantized BERT-base encoder layer, batch 8
+    from bladedisc_amd import bert_layer as B
+    weights = cfg.config5_weights()
+    layer = B.QuantBertLayer(weights, B.RawBackend())
+    bert = {}
+    for seq in cfg.BERT_SEQ_LENS:
+        h = layer.embed(cfg.config5_tokens(8, seq))
+        layer.calibrate(h)
+        rec = {}
+        layer.forward(h, rec)
+        torch.cuda.synchronize()
+        per, gpu_sum, cpu_sum = {}, 0.0, 0.0
+        for name in B.LINEARS:
+            r = rec[name]
+            xin, xq, yq, yf = r["x"].contiguous(), r["x_q"], r["y_q"], r["y"]
+            sx, sw, so = layer.s_in[name], layer.sw[name], layer.s_out[name]
+            wq, bias = layer.w_q[name], layer.bias[name]
+            chain = [FnCall(lambda: K.quantize(xin, sx, z1, out=xq)),
+                     FnCall(lambda: K.qgemm(xq, wq, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so,
+                                            bias=bias, out=yq)),
+                     FnCall(lambda: K.dequantize(yq, so, z1, out=yf))]
+            gpu_s = time_graph(torch, chain)
+            hx, hw, hb = xin.cpu().numpy(), wq.cpu().numpy(), layer.fb[name]
+            fsx, fso, hsw = float(sx.cpu()[0]), float(so.cpu()[0]), sw.cpu().numpy()
+
+            def cpu5():
+                q = O.quantize(hx, fsx, 0)
+                acc, _ = O.gemm_s32_fast(q, hw)
+                b32 = O.bias_f32_to_s32(hb, fsx, hsw)
+                O.dequantize(O.requant_cpu(acc, fsx, hsw, fso, b32=b32), fso, 0)
+            cpu_s = cpu_time(cpu5, min_time=0.05, max_reps=5)
+            m, kk = xin.shape
+            n = wq.shape[0]
+            per[name] = {"shape_MxKxN": [m, kk, n], "gpu_us": round(gpu_s * 1e6, 2),
+                         "cpu_us": round(cpu_s * 1e6, 1)}
+            gpu_sum += gpu_s
+            cpu_sum += cpu_s
+        # the whole layer (quantized operators + fp32 attention / LayerNorm / GELU in
+        # PyTorch), eager launches from Python
+        for _ in range(3):
+            layer.forward(h)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            layer.forward(h)
+        torch.cuda.synchronize()
+        bert["seq%d" % seq] = {"linears_q_gemm_dq": per,
+                               "quantized_ops_gpu_us": round(gpu_sum * 1e6, 2),
+                               "quantized_ops_cpu_us": round(cpu_sum * 1e6, 1),
+                               "layer_eager_wall_us": round((time.perf_counter() - t0) / 10 * 1e6, 1)}
+    rep["5_bert_base_layer_batch8"] = bert
+    return rep
+
+
 def extras(torch, steps, warmup):
-    """q/dq bandwidth on a tensor larger than the 256 MB last-level cache, and a few
-    BERT-shaped GEMMs (dynamic M)."""
+    """q/dq bandwidth on a tensor larger than the 256 MB last-level cache, the five
+    benchmark configurations against the CPU oracle, and a library yardstick."""
     from bladedisc_amd import kernels as K
     out = {}
     rows, cols = 65536, 4096
@@ -172,25 +379,7 @@ def extras(torch, steps, warmup):
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 5}
     del x, q, f
-    sweep = {}
-    for (m, n, k) in ((16, 768, 768), (128, 768, 768), (1000, 3072, 768), (4096, 768, 3072),
-                      (16384, 768, 768)):
-        a = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
-        w = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
-        sx = torch.tensor([0.02], device="cuda")
-        sw = torch.rand(n, device="cuda") * 0.049 + 0.001
-        so = torch.tensor([20.0], device="cuda")
-        o = torch.empty((m, n), dtype=torch.int8, device="cuda")
-        call = GemmCall(torch, a, w, sx, sw, so, None, 1, 0, o)
-        _, ev = time_steps(torch, call, 50, 5)
-        us = ev / 50 * 1e6
-        ops, byts = 2.0 * m * n * k, m * k + n * k + m * n + 4 * n
-        sweep["%dx%dx%d" % (m, n, k)] = {
-            "us": round(us, 2), "TOPS": round(ops / us / 1e6, 2),
-            "GB/s": round(byts / us / 1e3, 1),
-            "roofline_frac": round(max(ops / us / 1e6 / PEAK_INT8_TOPS,
-                                       byts / us / 1e3 / PEAK_HBM_GBPS), 4)}
-    out["qgemm_bert_shapes_requant_cpu"] = sweep
+    out["configs"] = config_reports(torch, K)
     # yardstick: the ROCm library int8 GEMM behind torch._int_mm (int32 output, no
     # epilogue) on the headline shape and data distribution -- a library, not the reference
     try:

@@ -8,6 +8,7 @@
 #include "disc_q8.h"
 #include "qgemm_device.h"
 #include "qgemm_pipelined.h"
+#include "qgemm_skinny.h"
 
 #pragma clang fp contract(off)
 
@@ -157,10 +158,18 @@ const Variant kVariants[] = {
     {"mfma_256x256x64_w2x2", 256, 256, 64, 256},
     {"mfma_128x128x64_w2x2", 128, 128, 64, 256},
     {"mfma_64x64x64_w2x2", 64, 64, 64, 256},
-    // software-pipelined kernels (GEMM only; need K % bk == 0)
+    // software-pipelined kernels, operands loaded straight into LDS
     {"pipe_256x256x128", 256, 256, 128, 256},
+    {"pipe_128x128x128", 128, 128, 128, 256},
+    {"pipe_64x64x128", 64, 64, 128, 256},
+    {"pipe_256x64x128", 256, 64, 128, 256},
+    // small-M kernel: 16 output channels per workgroup, K split over the waves (GEMM only)
+    {"skinny_16", 16, 16, 64, 512},
 };
-constexpr int kFirstPipeVariant = 4;
+constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
+constexpr int kSkinnyVariant = 8;
+// largest M the heuristic hands to the small-M kernel
+constexpr int64_t kSkinnyMaxM = 32;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
@@ -179,22 +188,23 @@ int launch_mfma(const MainParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_mfma launch");
 }
 
-// The pipelined kernels need whole 128-deep k tiles and address each block's rows
-// with 32-bit buffer offsets.
-bool pipe_ok(int bm, int bn, int64_t K, int64_t lda, int64_t ldw) {
+// The pipelined kernels address each block's rows (GEMM) or the whole image
+// (convolution) with 32-bit buffer offsets.
+bool pipe_ok(int bm, int bn, const MainParams& p, bool conv) {
   constexpr int BK = 128;
-  return K >= BK && K % BK == 0 && (int64_t)bm * lda + K + 2 * BK < (1LL << 31) &&
-         (int64_t)bn * ldw + K + 2 * BK < (1LL << 31);
+  if (p.K < 16 || p.K % 16 != 0) return false;
+  if ((int64_t)bn * p.ldw + p.K + 2 * BK >= (1LL << 31)) return false;
+  if (conv) return p.conv_bytes < (1LL << 31) && p.Ci % 16 == 0;
+  return (int64_t)bm * p.lda + p.K + 2 * BK < (1LL << 31);
 }
 
-template <int BM, int BN, int WM, int WN, int EPI>
+template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
 int launch_pipe(const MainParams& p, hipStream_t st) {
   constexpr int BK = 128;
   constexpr int lds = 2 * (BM + BN) * BK;
-  DQ8_REQUIRE(pipe_ok(BM, BN, p.K, p.lda, p.ldw),
-              "pipelined qgemm needs K to be a multiple of 128 and row strides that fit 32-bit "
-              "buffer offsets");
-  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, EPI>;
+  DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
+              "pipelined qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
+  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, CONV, EPI>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -206,6 +216,23 @@ int launch_pipe(const MainParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_pipe launch");
 }
 
+template <int NW, int MT, int EPI>
+int launch_skinny_t(const MainParams& p, hipStream_t st) {
+  const dim3 grid((unsigned)ceil_div(p.N, 16), (unsigned)ceil_div(p.M, 16 * MT));
+  DQ8_REQUIRE(grid.y <= 65535, "small-M qgemm: M too large for this variant");
+  hipLaunchKernelGGL((qgemm_skinny_kernel<NW, MT, EPI>), grid, dim3(NW * 64), 0, st, p);
+  return check_hip(hipGetLastError(), "qgemm_skinny launch");
+}
+
+// rows per workgroup grow with M (fewer passes over W), waves with the depth of K
+template <int EPI>
+int launch_skinny(const MainParams& p, hipStream_t st) {
+  const bool deep = p.K >= 1024;
+  if (p.M <= 16) return deep ? launch_skinny_t<8, 1, EPI>(p, st) : launch_skinny_t<4, 1, EPI>(p, st);
+  if (p.M <= 32) return deep ? launch_skinny_t<8, 2, EPI>(p, st) : launch_skinny_t<4, 2, EPI>(p, st);
+  return deep ? launch_skinny_t<8, 4, EPI>(p, st) : launch_skinny_t<4, 4, EPI>(p, st);
+}
+
 template <bool CONV, int EPI>
 int launch_variant(int variant, MainParams& p, hipStream_t st) {
   const Variant& v = kVariants[variant];
@@ -215,11 +242,13 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case 1: return launch_mfma<256, 256, 64, 2, 2, CONV, EPI>(p, st);
     case 2: return launch_mfma<128, 128, 64, 2, 2, CONV, EPI>(p, st);
     case 3: return launch_mfma<64, 64, 64, 2, 2, CONV, EPI>(p, st);
+    case kPipe256: return launch_pipe<256, 256, 2, 2, CONV, EPI>(p, st);
+    case kPipe128: return launch_pipe<128, 128, 2, 2, CONV, EPI>(p, st);
+    case kPipe64: return launch_pipe<64, 64, 2, 2, CONV, EPI>(p, st);
+    case kPipe256x64: return launch_pipe<256, 64, 4, 1, CONV, EPI>(p, st);
   }
   if constexpr (!CONV) {
-    switch (variant) {
-      case 4: return launch_pipe<256, 256, 2, 2, EPI>(p, st);
-    }
+    if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
   }
   return fail("unknown or unsupported qgemm variant for this operation");
 }
@@ -235,16 +264,23 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
   return fail("unknown epilogue");
 }
 
-// Picks the MFMA tile from the dynamic problem size: the largest tile that still
-// yields at least about one workgroup per compute unit; small problems take the
-// smallest tile to spread the weight stream over as many CUs as possible.
-int pick_variant(int64_t M, int64_t N) {
-  constexpr int64_t kCus = 256;
-  for (int v = 1; v < kFirstPipeVariant; ++v) {
-    const int64_t tiles = ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn);
-    if (tiles >= kCus - kCus / 8) return v;
+// Picks the kernel from the dynamic problem size.  `pipe` says whether the pipelined
+// kernels can take the operands.  Measured on BERT-shaped and square problems: the
+// 256x256 tile pays once it fills the chip (>= ~240 tiles), the 128x128 tile from about
+// 120 tiles on, below that the 64x64 tile spreads the weight stream over more CUs; narrow
+// outputs (N <= 64) take the 256x64 tile.
+int pick_variant(int64_t M, int64_t N, bool pipe) {
+  auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
+  if (pipe) {
+    if (N <= 64 && M >= 256 * 64) return kPipe256x64;
+    if (tiles(kPipe256) >= 240) return kPipe256;
+    if (tiles(kPipe128) >= 120) return kPipe128;
+    return kPipe64;
   }
-  return kFirstPipeVariant - 1;
+  constexpr int64_t kCus = 256;
+  for (int v = 1; v <= 3; ++v)
+    if (tiles(v) >= kCus - kCus / 8) return v;
+  return 3;
 }
 
 int elem_size(int epilogue) {
@@ -374,7 +410,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
 
   const bool need_generic = zx != 0 || zw != 0;
   const bool auto_pick = variant == -1;
-  if (auto_pick) variant = need_generic ? 0 : pick_variant(M, N);
+  if (auto_pick && need_generic) variant = 0;
   if (variant == 0) {
     GenericParams g;
     g.A = A;
@@ -444,9 +480,6 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
         epilogue, g, M * N, st);
   }
 
-  // large problems whose K suits it go to the software-pipelined kernel of the same tile
-  if (auto_pick && variant == 1 && pipe_ok(256, 256, K, lda_use, ldw_use)) variant = kFirstPipeVariant;
-
   MainParams p = {};
   p.A = a_use;
   p.W = w_use;
@@ -456,6 +489,8 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.N = (int)N;
   p.K = (int)K;
   p.epi = e;
+  if (auto_pick)
+    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, pipe_ok(256, 256, p, false));
   return launch_epi<false>(variant, p, epilogue, st);
 }
 
@@ -541,7 +576,8 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   const bool nhwc_ohwi = ib == 0 && ic == 3 && ih == 1 && iw == 2 && ki == 3 && ko == 0 &&
                          kh == 1 && kw == 2 && ob == 0 && oc == 3 && oh == 1 && ow == 2;
   const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16);
-  if (variant == -1) variant = fast_ok ? pick_variant(Mg, Co) : 0;
+  const bool auto_pick = variant == -1;
+  if (auto_pick && !fast_ok) variant = 0;
   if (variant != 0)
     DQ8_REQUIRE(fast_ok, "dq8_qconv2d: the MFMA variants need NHWC x OHWI, Ci % 16 == 0 and "
                          "16-byte aligned tensors");
@@ -583,7 +619,9 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   p.Kh = (int)Kh; p.Kw = (int)Kw;
   p.pad_t = padding[0]; p.pad_l = padding[2];
   p.sh = sh; p.sw_ = sw_; p.dh = dh; p.dw = dw;
+  p.conv_bytes = NB * H * Wd * Ci;
   p.epi = e;
+  if (auto_pick) variant = pick_variant(Mg, Co, pipe_ok(256, 256, p, true));
   return launch_epi<true>(variant, p, epilogue, st);
 }
 

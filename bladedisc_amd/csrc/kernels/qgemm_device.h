@@ -53,6 +53,7 @@ struct MainParams {
   // convolution geometry (unused by the plain GEMM)
   int H, Wd, Ci, Ho, Wo, Kh, Kw;
   int pad_t, pad_l, sh, sw_, dh, dw;
+  int64_t conv_bytes;   // size of the NHWC image tensor in bytes
   int tiles_m, tiles_n;
   EpiParams epi;
 };

@@ -30,7 +30,11 @@
 // the matrix cores draw, not by its schedule: the shader clock, 2.4 GHz when a few
 // CUs run it, falls to 1.5-1.7 GHz (clock64 against wall_clock64), and variations of
 // the schedule that change the cycle count leave the time per tile where it is.
-// Requires K % 128 == 0 and 16-byte aligned, k-contiguous operands.
+// Requires K % 16 == 0 and 16-byte aligned, k-contiguous operands; the last k tile is
+// completed with zeros (chunks at k >= K are given an out-of-range offset).
+// CONV: the A operand is an NHWC image read in place as the im2col matrix (row m =
+// (batch, ho, wo), k = (kh, kw, ci), Ci % 16 == 0); a lane recomputes the tap of its
+// 16-byte chunk once per k tile, and taps that fall into the padding load zeros.
 #ifndef DQ8_QGEMM_PIPELINED_H_
 #define DQ8_QGEMM_PIPELINED_H_
 
@@ -69,7 +73,7 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, unsigned lds_addr
 // s_waitcnt immediate for gfx9: vmcnt = n (6 bits, split), lgkmcnt = 0, expcnt = any
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4); }
 
-template <int BM, int BN, int WM, int WN, int EPI>
+template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
 __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParams p) {
   // The inline assembly only assembles in the device compilation; the host pass
   // just needs the kernel's stub.
@@ -89,6 +93,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile does not split over the waves");
   static_assert(FM >= 1 && FN >= 1 && FN <= FM, "fragment mismatch");
   static_assert(LD <= 63, "vmcnt is a 6-bit counter");
+  static_assert(NW % 2 == 0, "the chunk a lane loads must not depend on the load slot");
 
   extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
 
@@ -100,48 +105,94 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   int tm, tn;
   tile_coords(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  const int KT = p.K / BK;
+  const int KT = (p.K + BK - 1) / BK;
 
-  // ---- buffer descriptors over the rows this block may touch
-  const int8_t* a_base = p.A + (int64_t)m0 * p.lda;
-  const int8_t* w_base = p.W + (int64_t)n0 * p.ldw;
-  const int64_t a_valid = (int64_t)(p.M - m0 - 1) * p.lda + p.K;
-  const int64_t w_valid = (int64_t)(p.N - n0 - 1) * p.ldw + p.K;
+  // ---- buffer descriptors over the rows this block may touch (GEMM) or the whole
+  // image (convolution)
   constexpr int64_t kMaxRecords = 0x7fffffff;
+  constexpr int kOutOfRange = (int)0x80000000;
+  const int8_t* a_base = CONV ? p.A : p.A + (int64_t)m0 * p.lda;
+  const int8_t* w_base = p.W + (int64_t)n0 * p.ldw;
+  const int64_t a_valid = CONV ? p.conv_bytes : (int64_t)(p.M - m0 - 1) * p.lda + p.K;
+  const int64_t w_valid = (int64_t)(p.N - n0 - 1) * p.ldw + p.K;
   const v4i a_rsrc = make_rsrc(a_base, a_valid < kMaxRecords ? a_valid : kMaxRecords);
   const v4i w_rsrc = make_rsrc(w_base, w_valid < kMaxRecords ? w_valid : kMaxRecords);
   const unsigned lds_base = (unsigned)(size_t)(lds_void_t*)smem;
 
   // ---- load slots.  Instruction i of this wave covers 8-row block q = wave + i*NW;
   // lane -> row r = lane/8 of the block, LDS slot s = lane%8, global k-chunk
-  // c = s ^ r ^ (q & 1).
-  int a_off[A_LD], b_off[B_LD];      // byte offset of the lane's chunk in the block's rows
-  int a_lds[A_LD], b_lds[B_LD];      // wave-uniform LDS byte offset of the 1 KiB block
+  // c = s ^ r ^ (q & 1).  NW is even, so q & 1 = wave & 1 and the lane loads the same
+  // chunk c in every slot.
   const int lr = lane >> 3, ls = lane & 7;
+  const int kc = (ls ^ lr ^ (wave & 1)) << 4;   // byte offset of the lane's chunk in a k tile
+  int a_off[A_LD], b_off[B_LD];      // GEMM: byte offset of the lane's chunk in row 0 of the tile
+  int a_lds[A_LD], b_lds[B_LD];      // wave-uniform LDS byte offset of the 1 KiB block
+  int a_h[CONV ? A_LD : 1], a_w[CONV ? A_LD : 1], a_n[CONV ? A_LD : 1];   // conv: row geometry
 #pragma unroll
   for (int i = 0; i < A_LD; ++i) {
     const int q = wave + i * NW;
-    a_off[i] = (q * 8 + lr) * (int)p.lda + ((ls ^ lr ^ (q & 1)) << 4);
     a_lds[i] = __builtin_amdgcn_readfirstlane(q * 1024);
+    if (CONV) {
+      const int m = m0 + q * 8 + lr;
+      const int hw = p.Ho * p.Wo;
+      const int n_img = m / hw, rem = m - n_img * hw;
+      const int ho = rem / p.Wo, wo = rem - ho * p.Wo;
+      // rows past M get a coordinate no tap can bring back into the image
+      a_h[i] = m < p.M ? ho * p.sh - p.pad_t : -(1 << 24);
+      a_w[i] = wo * p.sw_ - p.pad_l;
+      a_n[i] = n_img * p.H * p.Wd;
+      a_off[i] = 0;
+    } else {
+      a_off[i] = (q * 8 + lr) * (int)p.lda + kc;
+    }
   }
 #pragma unroll
   for (int i = 0; i < B_LD; ++i) {
     const int q = wave + i * NW;
-    b_off[i] = (q * 8 + lr) * (int)p.ldw + ((ls ^ lr ^ (q & 1)) << 4);
+    b_off[i] = (q * 8 + lr) * (int)p.ldw + kc;
     b_lds[i] = __builtin_amdgcn_readfirstlane(A_BYTES + q * 1024);
   }
 
-  // issues load number `idx` (0 .. LD-1) of tile `kt` into stage `st`; tiles past the
-  // end of K get an out-of-range offset: zeros arrive, no memory is touched
-  auto issue_load = [&](int idx, int kt, int st) {
-    const int koff = kt < KT ? kt * BK : (int)0x80000000;
+  // Per k tile: is the lane's chunk inside K, and (conv) which tap does it belong to.
+  // tile_setup(kt) precedes the issue_load calls of tile kt.
+  int t_koff = kOutOfRange, t_dh = 0, t_dw = 0, t_ci = 0;
+  auto tile_setup = [&](int kt) {
+    const int k = kt * BK + kc;
+    const bool in = kt < KT && k < p.K;
+    t_koff = in ? kt * BK : kOutOfRange;
+    if (CONV) {
+      const unsigned tap = (unsigned)k / (unsigned)p.Ci;
+      t_ci = k - (int)tap * p.Ci;
+      const unsigned kh = tap / (unsigned)p.Kw;
+      t_dh = (int)kh * p.dh;
+      t_dw = (int)(tap - kh * p.Kw) * p.dw;
+    }
+  };
+
+  // issues load number `idx` (0 .. LD-1) of tile `kt` into stage `st`; chunks past the
+  // end of K (and conv taps in the padding) get an out-of-range offset: zeros arrive,
+  // no memory is touched
+  auto issue_load = [&](int idx, int st) {
     const unsigned base = lds_base + st * STAGE;
 #pragma unroll
     for (int i = 0; i < A_LD; ++i)
-      if (i == idx) buffer_load_lds_b128(a_rsrc, base + a_lds[i], a_off[i] + koff);
+      if (i == idx) {
+        int voff;
+        if (CONV) {
+          const int hi = a_h[i] + t_dh, wi = a_w[i] + t_dw;
+          const bool ok = t_koff != kOutOfRange && (unsigned)hi < (unsigned)p.H &&
+                          (unsigned)wi < (unsigned)p.Wd;
+          voff = ok ? (a_n[i] + hi * p.Wd + wi) * p.Ci + t_ci : kOutOfRange;
+        } else {
+          voff = t_koff != kOutOfRange ? a_off[i] + t_koff : kOutOfRange;
+        }
+        buffer_load_lds_b128(a_rsrc, base + a_lds[i], voff);
+      }
 #pragma unroll
     for (int i = 0; i < B_LD; ++i)
-      if (A_LD + i == idx) buffer_load_lds_b128(w_rsrc, base + b_lds[i], b_off[i] + koff);
+      if (A_LD + i == idx)
+        buffer_load_lds_b128(w_rsrc, base + b_lds[i],
+                             t_koff != kOutOfRange ? b_off[i] + t_koff : kOutOfRange);
   };
 
   // ---- fragment addressing.  Operand row R = R0 + lane%32 sits in block R/8 at row
@@ -175,17 +226,21 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-  // Load schedule: the LD loads of tile t+2 are issued two per row of MFMAs during
-  // k-steps 2 and 3 of tile t, into the stage tile t has just released.
-  static_assert(NKS == 4 && LD == 4 * FM, "schedule below assumes two loads per MFMA row of k-steps 2, 3");
+  // Load schedule: the LD loads of tile t+2 are issued during k-steps 2 and 3 of tile
+  // t, LPR per row of MFMAs, into the stage tile t has just released.
+  static_assert(NKS == 4, "schedule below assumes four k-steps per tile");
+  constexpr int LPR = (LD + 2 * FM - 1) / (2 * FM);          // loads per MFMA row
+  constexpr int LD_KS2 = FM * LPR < LD ? FM * LPR : LD;       // loads issued during k-step 2
 
   // ---- prologue: all of tile 0, then all of tile 1
+  tile_setup(0);
 #pragma unroll
-  for (int idx = 0; idx < LD; ++idx) issue_load(idx, 0, 0);
+  for (int idx = 0; idx < LD; ++idx) issue_load(idx, 0);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   __syncthreads();
+  tile_setup(1);
 #pragma unroll
-  for (int idx = 0; idx < LD; ++idx) issue_load(idx, 1, 1);
+  for (int idx = 0; idx < LD; ++idx) issue_load(idx, 1);
 #pragma unroll
   for (int i = 0; i < FM; ++i) load_frag_a(0, 0, 0, i);
 #pragma unroll
@@ -200,11 +255,12 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
         // has, the stage can take tile kt+2
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(63));
         __syncthreads();
+        tile_setup(kt + 2);
       }
       if (ks == 3) {
-        // tile kt+1 (older than the 2*FM loads of tile kt+2 just issued) has landed
+        // tile kt+1 (older than the LD_KS2 loads of tile kt+2 just issued) has landed
         // for this wave; after the barrier, for all of them
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(2 * FM));
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(LD_KS2));
         __syncthreads();
       }
 #pragma unroll
@@ -218,13 +274,13 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
           load_frag_a(3, cur, 3, i);
           if (i < FN) load_frag_b(3, cur, 3, i);
         } else if (ks == 2) {
-          issue_load(2 * i, kt + 2, cur);
-          issue_load(2 * i + 1, kt + 2, cur);
+#pragma unroll
+          for (int l = 0; l < LPR; ++l) issue_load(i * LPR + l, cur);
         } else {
           load_frag_a(0, nxt, 0, i);
           if (i < FN) load_frag_b(0, nxt, 0, i);
-          issue_load(2 * FM + 2 * i, kt + 2, cur);
-          issue_load(2 * FM + 2 * i + 1, kt + 2, cur);
+#pragma unroll
+          for (int l = 0; l < LPR; ++l) issue_load((FM + i) * LPR + l, cur);
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j)

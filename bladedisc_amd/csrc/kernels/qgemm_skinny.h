@@ -1,0 +1,93 @@
+// int8 GEMM for small M (a handful of tokens): the work is streaming W once, so the
+// kernel is organised around memory parallelism, not MFMA utilisation.
+//
+//  * one workgroup per 16 output channels x (16 * MT) rows; N / 16 workgroups spread the
+//    weight stream over the CUs;
+//  * the K loop is split over the NW waves of the workgroup (wave w takes 64-deep
+//    k-steps w, w + NW, ...) and every wave keeps U steps of loads in flight, so a
+//    3072-deep reduction is 6 dependent steps instead of 48; partial sums meet in LDS;
+//  * operands go straight from global memory into v_mfma_i32_16x16x64_i8 operand
+//    layout (lane l: row l % 16, 16 k-bytes of group l / 16); W is the row operand, so
+//    the 4 accumulator registers of a lane are 4 consecutive output channels.
+// Needs K % 16 == 0 and 16-byte aligned, k-contiguous rows, like the other MFMA kernels.
+#ifndef DQ8_QGEMM_SKINNY_H_
+#define DQ8_QGEMM_SKINNY_H_
+
+#include "qgemm_device.h"
+
+namespace dq8 {
+
+template <int NW, int MT, int EPI>
+__global__ void __launch_bounds__(NW * 64) qgemm_skinny_kernel(const MainParams p) {
+  constexpr int U = 4;  // k-steps in flight per wave
+  __shared__ int red[NW][MT][256];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int m0 = blockIdx.y * 16 * MT;
+  const int KS = (p.K + 63) / 64;
+
+  const bool w_ok = n0 + r < p.N;
+  const int8_t* wp = p.W + (int64_t)(w_ok ? n0 + r : 0) * p.ldw + g * 16;
+  const int8_t* ap[MT];
+  bool a_ok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    a_ok[t] = m0 + t * 16 + r < p.M;
+    ap[t] = p.A + (int64_t)(a_ok[t] ? m0 + t * 16 + r : 0) * p.lda + g * 16;
+  }
+
+  v4i acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (v4i){0, 0, 0, 0};
+
+  const v4i zero = {0, 0, 0, 0};
+  for (int ks0 = wave; ks0 < KS; ks0 += NW * U) {
+    v4i wf[U], af[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (ks0 + u * NW) * 64;
+      // K % 16 == 0: a lane's 16-byte chunk is entirely inside or outside the row
+      const bool in = k + g * 16 < p.K;
+      wf[u] = (in && w_ok) ? *(const v4i*)(wp + k) : zero;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) af[u][t] = (in && a_ok[t]) ? *(const v4i*)(ap[t] + k) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], af[u][t], acc[t], 0, 0, 0);
+  }
+
+  // D: register v of lane (r, g) is output channel 4g + v of row r
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][t][r * 16 + 4 * g + v] = acc[t][v];
+  __syncthreads();
+
+  for (int idx = threadIdx.x; idx < MT * 256; idx += NW * 64) {
+    const int t = idx >> 8, e = idx & 255;
+    const int m = m0 + t * 16 + (e >> 4), n = n0 + (e & 15);
+    if (m >= p.M || n >= p.N) continue;
+    int sum = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += red[w][t][e];
+    const EpiParams& ep = p.epi;
+    const ColParams c = col_params<EPI>(ep, n);
+    const int64_t off = (int64_t)m * ep.ldo + n;
+    if (EPI == DQ8_EPI_ACC_S32)
+      ((int32_t*)ep.out)[off] = sum;
+    else if (EPI == DQ8_EPI_DEQUANT_F32)
+      ((float*)ep.out)[off] = dequant_one(ep, c, sum);
+    else
+      ((int8_t*)ep.out)[off] = (int8_t)requant_one<EPI>(ep, c, sum);
+  }
+}
+
+}  // namespace dq8
+
+#endif  // DQ8_QGEMM_SKINNY_H_

@@ -318,3 +318,32 @@ def test_conv_nchw_oihw_layout_via_metadata():
     md = [0, 1, 2, 3, 1, 0, 2, 3, 0, 1, 2, 3, 1, 1, 1, 1, 1]
     got = O.conv_s32(x2, w2, [1, 1, 1, 1], md, [2, 3, 6, 6])
     np.testing.assert_array_equal(got.transpose(0, 2, 3, 1), ref)
+
+
+def test_requant_cpu_tie_margin_audit():
+    """E1's order of float operations lives in a library that is absent from the
+    reference checkout.  This audit bounds what a different order could change: on
+    the single-linear benchmark inputs, the alternative evaluation orders differ from
+    E1 only where the pre-rounding value sits next to a .5 tie."""
+    from bladedisc_amd import baseline_configs as C
+    c = C.config1()
+    x_q = O.quantize(c["x"], c["sx"], 0)
+    acc = O.gemm_s32(x_q, c["w_q"], tp_b=True)
+    sx, sw, so, bias = np.float32(c["sx"]), c["sw"], np.float32(c["so"]), c["bias"]
+    b32 = O.bias_f32_to_s32(bias, float(sx), sw)
+    base = O.requant_cpu(acc, float(sx), sw, float(so), b32=b32).astype(np.int32)
+    f = np.float32
+    os_ = ((sx * sw).astype(f) / so).astype(f)
+    pre = ((acc.astype(f) + b32.astype(f)).astype(f) * os_).astype(f)
+    assert np.array_equal(np.clip(np.rint(pre), -128, 127).astype(np.int32), base)
+    dist_to_tie = np.abs(np.abs(pre - np.floor(pre)) - 0.5)
+    # (a) distribute the scale over the sum: acc*os + b32*os
+    alt_a = ((acc.astype(f) * os_).astype(f) + (b32.astype(f) * os_).astype(f)).astype(f)
+    # (b) dequantize first, add the real-valued bias, divide by the output scale
+    alt_b = (((acc.astype(f) * (sx * sw).astype(f)).astype(f) + bias).astype(f) / so).astype(f)
+    for alt, margin in ((alt_a, 2.0 ** -10), (alt_b, 2.0 ** -10 + float(os_.max()))):
+        q = np.clip(np.rint(alt), -128, 127).astype(np.int32)
+        differs = q != base
+        assert np.abs(q - base).max() <= 1
+        assert np.all(dist_to_tie[differs] < margin)
+        assert differs.mean() < 0.01
