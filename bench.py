@@ -170,11 +170,13 @@ class FnCall:
         self.fn()
 
 
-def cpu_time(fn, min_time=0.3, max_reps=10):
-    """Best wall time of fn over a few repetitions (at least min_time in total)."""
+def cpu_time(fn, min_time=0.3, max_reps=10, min_reps=5):
+    """Best wall time of fn over a few repetitions (at least min_reps, and at least
+    min_time in total unless max_reps comes first); the minimum filters the scheduler
+    stalls of a shared host."""
     fn()
     best, total, reps = float("inf"), 0.0, 0
-    while reps < max_reps and (total < min_time or reps < 2):
+    while reps < max_reps and (total < min_time or reps < min_reps):
         t0 = time.perf_counter()
         fn()
         dt = time.perf_counter() - t0
@@ -237,7 +239,7 @@ def config_reports(torch, K):
             def cpu2():
                 acc, _ = O.gemm_s32_fast(c["a_q"], c["w_q"])
                 O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]))
-            cpu_s = cpu_time(cpu2, min_time=0.05, max_reps=5)
+            cpu_s = cpu_time(cpu2, min_time=0.05, max_reps=8)
             r = roof(2.0 * m * n * k, m * k + n * k + m * n + 4 * n, gpu_s)
             r["cpu_us"] = round(cpu_s * 1e6, 1)
             sweep["M%d_K%d_N%d" % (m, k, n)] = r
@@ -254,7 +256,7 @@ def config_reports(torch, K):
     def cpu3():
         acc, _ = O.gemm_s32_fast(c["a_q"], c["w_q"])
         O.requant_gpu(acc, c["sx"], c["sw"], c["so"], bias_f32=c["bias_q"])
-    r["cpu_us"] = round(cpu_time(cpu3, min_time=0.0, max_reps=2) * 1e6, 1)
+    r["cpu_us"] = round(cpu_time(cpu3, min_time=0.0, max_reps=2, min_reps=2) * 1e6, 1)
     rep["3_large_square_8192_fused_bias_requant"] = r
     del a, w, o, call
 
@@ -284,7 +286,7 @@ def config_reports(torch, K):
         def cpu4():
             acc, _ = O.gemm_s32_fast(cols, wmat)
             O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]))
-        r["cpu_us"] = round(cpu_time(cpu4, min_time=0.05, max_reps=5) * 1e6, 1)
+        r["cpu_us"] = round(cpu_time(cpu4, min_time=0.05, max_reps=8) * 1e6, 1)
         r["cpu_note"] = "int8 GEMM of the pre-built im2col matrix + requant"
         convs[conv["name"]] = r
         del cols
@@ -320,7 +322,7 @@ def config_reports(torch, K):
                 acc, _ = O.gemm_s32_fast(q, hw)
                 b32 = O.bias_f32_to_s32(hb, fsx, hsw)
                 O.dequantize(O.requant_cpu(acc, fsx, hsw, fso, b32=b32), fso, 0)
-            cpu_s = cpu_time(cpu5, min_time=0.05, max_reps=5)
+            cpu_s = cpu_time(cpu5, min_time=0.05, max_reps=8)
             m, kk = xin.shape
             n = wq.shape[0]
             per[name] = {"shape_MxKxN": [m, kk, n], "gpu_us": round(gpu_s * 1e6, 2),

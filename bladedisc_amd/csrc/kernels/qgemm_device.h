@@ -128,6 +128,35 @@ __device__ __forceinline__ int requant_one(const EpiParams& p, const ColParams& 
   return sat_rne_s8(d);
 }
 
+// Four requantised results packed into one word (byte e = result of accumulator e).
+// Same arithmetic as requant_one; rounding and conversion are done by adding
+// 1.5 * 2^23: for |d| <= 128 the sum is rounded to an integer by the addition itself
+// (round-to-nearest-even) and its low mantissa byte is the two's-complement int8.
+template <int EPI>
+__device__ __forceinline__ uint32_t requant_pack4(const EpiParams& p, const ColParams (&c)[4],
+                                                  int a0, int a1, int a2, int a3) {
+  const int acc[4] = {a0, a1, a2, a3};
+  uint32_t bits[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float d = (float)acc[e];
+    if (EPI == DQ8_EPI_REQUANT_CPU) {
+      d = d + c[e].b;
+      d = d * c[e].os;
+      d = d + (float)p.zo;
+    } else {
+      d = c[e].os * d;
+      d = d + c[e].b;
+    }
+    d = fminf(fmaxf(d, -128.0f), 127.0f);  // NaN -> -128, like the CPU path
+    d = d + 12582912.0f;
+    bits[e] = __float_as_uint(d);
+  }
+  const uint32_t lo = __builtin_amdgcn_perm(bits[1], bits[0], 0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm(bits[3], bits[2], 0x04000c0cu);
+  return lo | hi;
+}
+
 __device__ __forceinline__ float dequant_one(const EpiParams& p, const ColParams& c,
                                              int acc) {
   float d = (float)acc * c.os;
@@ -145,17 +174,13 @@ __device__ __forceinline__ void store_group4(const EpiParams& p, int m, int n,
   const bool full = n + 3 < p.N;
   if (EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU) {
     int8_t* out = (int8_t*)p.out;
-    int q[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) q[e] = requant_one<EPI>(p, c[e], acc[e]);
+    const uint32_t w = requant_pack4<EPI>(p, c, a0, a1, a2, a3);
     if (full && p.vec_store) {
-      uint32_t w = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) |
-                   ((uint32_t)(q[2] & 0xff) << 16) | ((uint32_t)(q[3] & 0xff) << 24);
       *(uint32_t*)(out + off) = w;
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        if (n + e < p.N) out[off + e] = (int8_t)q[e];
+        if (n + e < p.N) out[off + e] = (int8_t)(w >> (8 * e));
     }
   } else if (EPI == DQ8_EPI_ACC_S32) {
     int32_t* out = (int32_t*)p.out;
@@ -414,12 +439,8 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           const int r = i * 32 + (lane & 31);
-          const int q0 = requant_one<EPI>(e, c[0], acc[i][j][4 * g + 0]);
-          const int q1 = requant_one<EPI>(e, c[1], acc[i][j][4 * g + 1]);
-          const int q2 = requant_one<EPI>(e, c[2], acc[i][j][4 * g + 2]);
-          const int q3 = requant_one<EPI>(e, c[3], acc[i][j][4 * g + 3]);
-          const uint32_t w = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) |
-                             ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
+          const uint32_t w = requant_pack4<EPI>(e, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
+                                                acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
           *reinterpret_cast<uint32_t*>(stage + r * TN + ((chunk ^ (r & (CH - 1))) << 4) + dw * 4) = w;
         }
       }

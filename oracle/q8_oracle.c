@@ -304,23 +304,21 @@ void q8o_quantize_f32(const float* x, int64_t outer, int64_t nch, int64_t inner,
                       int64_t qmin, int64_t qmax, int round_mode, int out_kind,
                       void* out) {
   const float fmin = (float)qmin, fmax = (float)qmax;
-  for (int64_t o = 0; o < outer; ++o)
-    for (int64_t c = 0; c < nch; ++c) {
-      int64_t qi = n_q > 1 ? c : 0;
-      float s = scale[qi];
-      float z = (float)zp[qi];
-      for (int64_t i = 0; i < inner; ++i) {
-        int64_t idx = (o * nch + c) * inner + i;
-        float t0 = x[idx] / s;
-        float t1 = t0 + z;
-        float t2 = round_mode == Q8O_ROUND_HALF_TO_EVEN ? rne_f32(t1)
-                                                        : roundf(t1);
-        /* mhlo.clamp(min, x, max) = min(max(x, lo), hi) */
-        float t3 = t2 < fmin ? fmin : t2;
-        t3 = t3 > fmax ? fmax : t3;
-        store_q(out, idx, out_kind, (double)t3);
-      }
-    }
+  const int64_t total = outer * nch * inner;
+  /* elements are independent: split the flat index range over the threads */
+#pragma omp parallel for schedule(static) if (total > 65536)
+  for (int64_t idx = 0; idx < total; ++idx) {
+    const int64_t qi = n_q > 1 ? (idx / inner) % nch : 0;
+    const float s = scale[qi];
+    const float z = (float)zp[qi];
+    float t0 = x[idx] / s;
+    float t1 = t0 + z;
+    float t2 = round_mode == Q8O_ROUND_HALF_TO_EVEN ? rne_f32(t1) : roundf(t1);
+    /* mhlo.clamp(min, x, max) = min(max(x, lo), hi) */
+    float t3 = t2 < fmin ? fmin : t2;
+    t3 = t3 > fmax ? fmax : t3;
+    store_q(out, idx, out_kind, (double)t3);
+  }
 }
 
 /* R: hlo_disc_ops.cc:286-309 -- double: x/scale + zp, nearbyint narrowed through
@@ -356,23 +354,21 @@ void q8o_quantize_fold(const float* x, int64_t outer, int64_t nch,
 void q8o_dequantize(const void* q, int in_kind, int64_t outer, int64_t nch,
                     int64_t inner, const float* scale, const int32_t* zp,
                     int64_t n_q, float* out) {
-  for (int64_t o = 0; o < outer; ++o)
-    for (int64_t c = 0; c < nch; ++c) {
-      int64_t qi = n_q > 1 ? c : 0;
-      for (int64_t i = 0; i < inner; ++i) {
-        int64_t idx = (o * nch + c) * inner + i;
-        int32_t v;
-        switch (in_kind) {
-          case Q8O_I8: v = ((const int8_t*)q)[idx]; break;
-          case Q8O_U8: v = ((const uint8_t*)q)[idx]; break;
-          case Q8O_I16: v = ((const int16_t*)q)[idx]; break;
-          case Q8O_U16: v = ((const uint16_t*)q)[idx]; break;
-          default: v = ((const int32_t*)q)[idx]; break;
-        }
-        int32_t t0 = v - zp[qi];
-        out[idx] = (float)t0 * scale[qi];
-      }
+  const int64_t total = outer * nch * inner;
+#pragma omp parallel for schedule(static) if (total > 65536)
+  for (int64_t idx = 0; idx < total; ++idx) {
+    const int64_t qi = n_q > 1 ? (idx / inner) % nch : 0;
+    int32_t v;
+    switch (in_kind) {
+      case Q8O_I8: v = ((const int8_t*)q)[idx]; break;
+      case Q8O_U8: v = ((const uint8_t*)q)[idx]; break;
+      case Q8O_I16: v = ((const int16_t*)q)[idx]; break;
+      case Q8O_U16: v = ((const uint16_t*)q)[idx]; break;
+      default: v = ((const int32_t*)q)[idx]; break;
     }
+    int32_t t0 = v - zp[qi];
+    out[idx] = (float)t0 * scale[qi];
+  }
 }
 
 /* ------------------------------------------------------------------------ */
