@@ -12,6 +12,9 @@
 //                               (f32 / s32 / no bias, per-channel weight scale)
 //   ral_pdll_qgemm_per_channel  R context/quantized_gpu_kernel_impl.cc:197-321
 //   ral_qconv                   R context/stream_executor_based_impl.cc:1831-1948
+//   ral_pdll_qconv2d            R context/common_context_impl_quantization.cc:352-607
+//                               (registered there for cpu only, :1685; same signature
+//                               and attributes here for gpu)
 //   ral_quantize / ral_dequantize
 //                               no runtime symbol in the reference: its compiler
 //                               expands mhlo_disc.quantize / dequantize into loops
@@ -33,6 +36,7 @@
 
 #include "disc_q8.h"
 #include "mlir/ral/context/context_util.h"
+#include "mlir/ral/context/conv_attr_util.h"
 #include "mlir/ral/context/pdll_util.h"
 #include "mlir/ral/device/gpu/gpu_driver.h"
 #include "mlir/ral/ral_context.h"
@@ -529,6 +533,89 @@ void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4>
   kernelFailed(ctx, st, who);
 }
 
+// ----------------------------------------------------------- ral_pdll_qconv2d
+// The attribute-driven convolution entry: data_format / strides / dilations / padding
+// come as custom attributes, the result is allocated here.  Weights are
+// [out_channels, filter_h, filter_w, in_channels].
+//   out = sat8(rne(f32(conv_s32(in, w)) * ((s_x*s_w[co])/s_o) + z_o))
+MemRefType<int8_t, 4> ral_pdll_qconv2d(ExecutionContext* ctx, void* stream_handle,
+                                       MemRefType<int8_t, 4> input,
+                                       MemRefType<int8_t, 4> weight,
+                                       MemRefType<float, 0> inputScales,
+                                       MemRefType<int32_t, 0> inputZeroPoints,
+                                       MemRefType<float, 1> weightScales,
+                                       MemRefType<int32_t, 1> weightZeroPoints,
+                                       MemRefType<float, 0> resultScales,
+                                       MemRefType<int32_t, 0> resultZeroPoints,
+                                       void* customAttrs) {
+  static const char* who = "ral_pdll_qconv2d";
+  int64_t zeros[4] = {0, 0, 0, 0};
+  MemRefType<int8_t, 4> result = assignMemRef<int8_t, 4>(nullptr, zeros);
+  if (isEmptyMemref(input) || isEmptyMemref(weight)) {
+    TAO_VLOG(1) << who << ": early return for empty tensor";
+    return result;
+  }
+  PDLAttr* attr = customAttrs ? getOrParsePDLAttr(ctx, customAttrs, who) : nullptr;
+  if (!attr || attr->getType() != "dict") {
+    fail(ctx, "fail to parse custom_attrs\n");
+    return result;
+  }
+  auto& dict = attr->as<DictPDLAttr>();
+  auto has = [&](const char* key, const char* type) {
+    return dict.hasKey(key) && dict.get(key).getType() == type;
+  };
+  if (!has("data_format", "str") || !has("padding", "str") || !has("strides", "intArray") ||
+      !has("dilations", "intArray")) {
+    fail(ctx, std::string(who) + ": data_format, padding, strides and dilations are required");
+    return result;
+  }
+  std::vector<int64_t> explicit_paddings;
+  if (has("explicit_paddings", "intArray"))
+    explicit_paddings = dict.get("explicit_paddings").as<IntArrayPDLAttr>().getValue();
+  const bool weight_is_const = has("weight_is_const", "bool") &&
+                               dict.get("weight_is_const").as<BoolPDLAttr>().getValue();
+  Conv2dPlan plan;
+  const std::string err =
+      planConv2d(dict.get("data_format").as<StrPDLAttr>().getValue(),
+                 dict.get("strides").as<IntArrayPDLAttr>().getValue(),
+                 dict.get("dilations").as<IntArrayPDLAttr>().getValue(),
+                 dict.get("padding").as<StrPDLAttr>().getValue(), explicit_paddings,
+                 weight_is_const, input.sizes, weight.sizes, &plan);
+  if (!err.empty()) {
+    fail(ctx, std::string(who) + ": " + err);
+    return result;
+  }
+  if (!symmetricOrFail(ctx, inputZeroPoints.data, 1, weightZeroPoints.data,
+                       weightZeroPoints.sizes[0], who))
+    return result;
+  if (weightScales.sizes[0] != 1 && weightScales.sizes[0] != weight.sizes[0]) {
+    fail(ctx, std::string(who) + ": weight scale must have 1 or out_channels entries");
+    return result;
+  }
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight"))
+    return result;
+  int64_t total = 1;
+  for (int i = 0; i < 4; ++i) {
+    if (plan.result_sizes[i] < 0) plan.result_sizes[i] = 0;
+    total *= plan.result_sizes[i];
+  }
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return result;
+  if (total == 0) return assignMemRef<int8_t, 4>(nullptr, plan.result_sizes);
+  auto* data = static_cast<int8_t*>(drv->alloc(ctx, (size_t)total));
+  if (!data) return result;
+  result = assignMemRef<int8_t, 4>(data, plan.result_sizes);
+  void* stream = drv->asCUStream(ctx, stream_handle);
+  const int32_t zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
+  int st = dq8_qconv2d(input.data, input.sizes, weight.data, weight.sizes, plan.padding,
+                       plan.metadata, result.data, result.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
+                       DQ8_BIAS_NONE, inputScales.data, weightScales.data,
+                       weightScales.sizes[0], resultScales.data, zo, stream);
+  kernelFailed(ctx, st, who);
+  return result;
+}
+
 // ------------------------------------------------- ral_quantize / ral_dequantize
 // axis < 0 means per tensor (rank-0 scale / zero point); otherwise the scale and
 // zero point vectors run along dimension `axis`.  Scale and zero point are device
@@ -651,6 +738,7 @@ TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channe
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<4>);
 
 TAO_RAL_API("ral_qconv", "gpu", gpu::q8::ral_qconv);
+TAO_RAL_API("ral_pdll_qconv2d", "gpu", gpu::q8::ral_pdll_qconv2d);
 
 #define DQ8_REGISTER_QDQ(QT, N)                                              \
   TAO_RAL_API("ral_quantize", "gpu", gpu::q8::ral_quantize<QT, N, 0>);       \

@@ -10,6 +10,7 @@
 #include <sstream>
 
 #include "mlir/ral/context/base/hip/hip_context_impl.h"
+#include "mlir/ral/context/conv_attr_util.h"
 #include "mlir/ral/context/pdll_util.h"
 #include "mlir/ral/ral_context.h"
 #include "mlir/ral/ral_helper.h"
@@ -162,6 +163,28 @@ const char* disc_ral_api_name(int index) {
 
 int disc_ral_api_exists(const char* name) {
   return name && tao::ral::TaoRalApiRegistry::Global().Find(name) ? 1 : 0;
+}
+
+int disc_ral_conv2d_plan(const char* data_format, const int64_t* strides, int n_strides,
+                         const int64_t* dilations, int n_dilations, const char* padding,
+                         const int64_t* explicit_paddings, int n_explicit,
+                         int weight_is_const, const int64_t in_sizes[4],
+                         const int64_t w_sizes[4], int32_t padding_out[4],
+                         int32_t metadata_out[17], int64_t result_sizes_out[4]) {
+  if (!data_format || !padding || !in_sizes || !w_sizes || !padding_out || !metadata_out ||
+      !result_sizes_out || n_strides < 0 || n_dilations < 0 || n_explicit < 0)
+    return 1;
+  tao::ral::Conv2dPlan plan;
+  const std::string err = tao::ral::planConv2d(
+      data_format, std::vector<int64_t>(strides, strides + n_strides),
+      std::vector<int64_t>(dilations, dilations + n_dilations), padding,
+      std::vector<int64_t>(explicit_paddings, explicit_paddings + n_explicit),
+      weight_is_const != 0, in_sizes, w_sizes, &plan);
+  if (!err.empty()) return 1;
+  std::memcpy(padding_out, plan.padding, sizeof(plan.padding));
+  std::memcpy(metadata_out, plan.metadata, sizeof(plan.metadata));
+  std::memcpy(result_sizes_out, plan.result_sizes, sizeof(plan.result_sizes));
+  return 0;
 }
 
 int64_t disc_ral_attr_to_json(const uint8_t* blob, size_t size, char* out, size_t cap) {

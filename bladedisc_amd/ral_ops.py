@@ -117,6 +117,44 @@ def qconv(ex, x, w, padding, metadata, sx, sw_c, so, out):
     return out
 
 
+def pdll_qconv2d(ex, x, w_ohwi, sx, sw_c, so, data_format="NHWC", strides=(1, 1, 1, 1),
+                 dilations=(1, 1, 1, 1), padding="SAME", explicit_paddings=(),
+                 weight_is_const=True, zo=0):
+    """ral_pdll_qconv2d: TensorFlow-style attributes, callee-allocated result."""
+    a = ex.new_args().tensor(x).tensor(w_ohwi)
+    a.tensor(sx, rank0=True)
+    _zp0(a, host=True)
+    a.tensor(sw_c)
+    a.host_array(np.zeros(sw_c.numel(), np.int32))
+    a.tensor(so, rank0=True)
+    a.host_array(np.array([zo], np.int32), rank0=True)
+    a.blob(ral.encode_attr({"data_format": data_format, "strides": [int(v) for v in strides],
+                            "dilations": [int(v) for v in dilations], "padding": padding,
+                            "explicit_paddings": [int(v) for v in explicit_paddings],
+                            "weight_is_const": bool(weight_is_const)}))
+    res = a.result_memref("i8", 4)
+    ex.call("ral_pdll_qconv2d", "gpu", a)
+    return ral.memref_to_tensor(res, torch.int8)
+
+
+def conv2d_plan(in_shape, w_shape, data_format, strides, dilations, padding,
+                explicit_paddings=(), weight_is_const=True):
+    """(padding[4], metadata[17], result_shape[4]) as ral_pdll_qconv2d derives them;
+    raises ValueError for malformed attributes.  Host only."""
+    import ctypes as C
+    L = ral.lib()
+    i64 = lambda v: (C.c_int64 * max(len(v), 1))(*[int(t) for t in v])  # noqa: E731
+    pad, md, out = (C.c_int32 * 4)(), (C.c_int32 * 17)(), (C.c_int64 * 4)()
+    L.disc_ral_conv2d_plan.restype = C.c_int
+    rc = L.disc_ral_conv2d_plan(data_format.encode(), i64(strides), len(strides),
+                                i64(dilations), len(dilations), padding.encode(),
+                                i64(explicit_paddings), len(explicit_paddings),
+                                int(weight_is_const), i64(in_shape), i64(w_shape), pad, md, out)
+    if rc != 0:
+        raise ValueError("malformed convolution attributes")
+    return list(pad), list(md), list(out)
+
+
 def quantize(ex, x, scale, zp, axis=None, qmin=-128, qmax=127, round_mode=1, out=None,
              dtype=torch.int8):
     if out is None:

@@ -78,6 +78,19 @@ int disc_ral_api_count(void);
 const char* disc_ral_api_name(int index);
 int disc_ral_api_exists(const char* name);
 
+/* Diagnostic: what ral_pdll_qconv2d derives from its TensorFlow-style attributes
+ * (the rules of tao_compiler/mlir/ral/context/common_context_impl_quantization.h:27-206):
+ * padding {lo0,hi0,lo1,hi1}, the 17-entry ral_qconv metadata vector and the result
+ * shape.  Weights are [out_channels, filter_h, filter_w, in_channels].  Returns 0, or 1
+ * when the attributes are malformed.  Host only; no counterpart in the reference's C
+ * ABI. */
+int disc_ral_conv2d_plan(const char* data_format, const int64_t* strides, int n_strides,
+                         const int64_t* dilations, int n_dilations, const char* padding,
+                         const int64_t* explicit_paddings, int n_explicit,
+                         int weight_is_const, const int64_t in_sizes[4],
+                         const int64_t w_sizes[4], int32_t padding_out[4],
+                         int32_t metadata_out[17], int64_t result_sizes_out[4]);
+
 /* Parses a serialized custom_attrs blob of `size` bytes (the last operand of every
  * ral_pdll_* call; wire format: R disc/transforms/disc_lower_to_library_call.cc
  * :684-848, reader R ral/context/pdll_util.cc:20-168) and renders it as JSON text

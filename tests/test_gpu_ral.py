@@ -189,6 +189,50 @@ def test_ral_qconv(rt, nb, h, ci, co, k, stride, pad):
         np.testing.assert_array_equal(host(out), want)
 
 
+@pytest.mark.parametrize("fmt,padding,k,stride,dil", [("NHWC", "SAME", 3, 1, 1), ("NHWC", "VALID", 3, 2, 2),
+                                                      ("NHWC", "SAME", 1, 1, 1), ("NCHW", "SAME", 3, 1, 1),
+                                                      ("NHWC", "EXPLICIT", 3, 1, 1)])
+def test_ral_pdll_qconv2d(rt, fmt, padding, k, stride, dil):
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(k * 10 + stride + len(padding))
+    nb, h, w_, ci, co = 2, 14, 12, 32, 48
+    x = rng.integers(-128, 128, (nb, h, w_, ci) if fmt == "NHWC" else (nb, ci, h, w_), dtype=np.int8)
+    wt = rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8)
+    explicit = [0, 0, 1, 2, 2, 0, 0, 0] if padding == "EXPLICIT" else []
+    sp = [1, stride, stride, 1] if fmt == "NHWC" else [1, 1, stride, stride]
+    dl = [1, dil, dil, 1] if fmt == "NHWC" else [1, 1, dil, dil]
+    pad4, md, out_shape = O.conv_attrs(x.shape, wt.shape, fmt, sp, dl, padding,
+                                       explicit_paddings=explicit)
+    acc = O.conv_s32(x, wt, pad4, md, out_shape)
+    sx = np.float32(0.02)
+    sw = rng.uniform(0.001, 0.05, co).astype(np.float32)
+    so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40.0)
+    ch_axis = 3 if fmt == "NHWC" else 1
+    acc2 = np.ascontiguousarray(np.moveaxis(acc, ch_axis, -1))
+    want = np.moveaxis(O.requant_cpu(acc2.reshape(-1, co), sx, sw, so, zo=3).reshape(acc2.shape),
+                       -1, ch_axis)
+    with ctx.execution() as ex:
+        got = ops.pdll_qconv2d(ex, dev(x), dev(wt), f1(sx), dev(sw), f1(so), data_format=fmt,
+                               strides=sp, dilations=dl, padding=padding,
+                               explicit_paddings=explicit, zo=3)
+        assert list(got.shape) == list(out_shape)
+        np.testing.assert_array_equal(host(got), want)
+
+
+def test_ral_pdll_qconv2d_rejects_bad_attrs(rt):
+    ctx, ral, ops = rt
+    x = torch.zeros((1, 4, 4, 16), dtype=torch.int8, device="cuda")
+    w = torch.zeros((16, 3, 3, 16), dtype=torch.int8, device="cuda")
+    own = ral.RalContext()
+    try:
+        with own.execution() as ex:
+            with pytest.raises(ral.RalError, match="padding must be"):
+                ops.pdll_qconv2d(ex, x, w, f1(1.0), dev(np.ones(16, np.float32)), f1(1.0),
+                                 padding="FULL")
+    finally:
+        own.close()
+
+
 @pytest.mark.parametrize("shape,axis", [((64, 768), None), ((64, 768), 1), ((768, 768), 0),
                                         ((2, 14, 14, 64), 3)])
 def test_ral_quantize_dequantize(rt, shape, axis):

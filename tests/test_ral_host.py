@@ -193,3 +193,60 @@ def test_size_class_pool_is_exposed_through_raw_alloc_names():
         c = size_class(b)
         assert c >= b and c <= max(256, b * 1.25 + 1) and c >= prev
         prev = c
+
+
+def test_conv2d_plan_matches_oracle():
+    """The attribute -> padding / metadata / result-shape rules of ral_pdll_qconv2d,
+    against the oracle's restatement of the reference helpers
+    (common_context_impl_quantization.h:27-206), over the attribute forms the reference
+    accepts."""
+    import itertools
+    import oracle as O
+    from bladedisc_amd import ral_ops
+    cases = 0
+    for fmt, pad, (kh, kw), nstr, stride, dil in itertools.product(
+            ("NHWC", "NCHW"), ("SAME", "VALID", "EXPLICIT4", "EXPLICIT8"), ((1, 1), (3, 3), (5, 2)),
+            (1, 2, 4), (1, 2, 3), (1, 2)):
+        h, w, ci, co = 13, 10, 8, 6
+        in_shape = (2, h, w, ci) if fmt == "NHWC" else (2, ci, h, w)
+        w_shape = (co, kh, kw, ci)
+        sp = (1, 2) if fmt == "NHWC" else (2, 3)
+        def attr(v):
+            if nstr == 1:
+                return [v]
+            if nstr == 2:
+                return [v, v + 1]
+            full = [1, 1, 1, 1]
+            full[sp[0]], full[sp[1]] = v, v + 1
+            return full
+        strides, dilations = attr(stride), attr(dil)
+        explicit = []
+        padding = pad
+        if pad == "EXPLICIT4":
+            padding, explicit = "EXPLICIT", [1, 2, 0, 3]
+        elif pad == "EXPLICIT8":
+            padding = "EXPLICIT"
+            explicit = [0] * 8
+            explicit[2 * sp[0]:2 * sp[0] + 2] = [2, 1]
+            explicit[2 * sp[1]:2 * sp[1] + 2] = [0, 1]
+        want = O.conv_attrs(in_shape, w_shape, fmt, strides, dilations, padding,
+                            explicit_paddings=explicit, weight_is_const=bool(cases & 1))
+        got = ral_ops.conv2d_plan(in_shape, w_shape, fmt, strides, dilations, padding,
+                                  explicit_paddings=explicit, weight_is_const=bool(cases & 1))
+        assert got == tuple(want) or list(got) == [list(want[0]), list(want[1]), list(want[2])], \
+            (fmt, pad, kh, kw, strides, dilations, got, want)
+        cases += 1
+    assert cases == 2 * 4 * 3 * 3 * 3 * 2
+    # the closed forms of the reference's own conv tests: 1x1 SAME keeps the size,
+    # 3x3 VALID loses two, stride 2 + dilation 2 on 7 -> 2
+    assert ral_ops.conv2d_plan((1, 5, 5, 4), (3, 1, 1, 4), "NHWC", [1], [1], "SAME")[2] == [1, 5, 5, 3]
+    assert ral_ops.conv2d_plan((1, 5, 5, 4), (3, 3, 3, 4), "NHWC", [1], [1], "VALID")[2] == [1, 3, 3, 3]
+    assert ral_ops.conv2d_plan((1, 7, 7, 4), (3, 3, 3, 4), "NHWC", [2], [2], "VALID")[2] == [1, 2, 2, 3]
+    for bad in (dict(data_format="NHW"), dict(data_format="ABCD"), dict(padding="FULL"),
+                dict(strides=[1, 1, 1]), dict(strides=[0]), dict(explicit_paddings=[1, 2, 3],
+                                                                 padding="EXPLICIT")):
+        kw = dict(data_format="NHWC", strides=[1], dilations=[1], padding="SAME",
+                  explicit_paddings=[])
+        kw.update(bad)
+        with pytest.raises(ValueError):
+            ral_ops.conv2d_plan((1, 5, 5, 4), (3, 3, 3, 4), **kw)
