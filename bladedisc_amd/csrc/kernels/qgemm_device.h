@@ -238,7 +238,23 @@ __device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, i
 template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
-                                              int n_blk0);
+                                              int n_blk0, const ColParams* early = nullptr);
+
+// The per-channel factors of the channels thread t is responsible for in the epilogue
+// (t, t + NT, ...), fetched at the start of a kernel so that the cold loads of scales
+// and bias and the division are off the critical path when the main loop ends.
+template <int EPI, int NT, int BN>
+struct EarlyColParams {
+  static constexpr int kPerThread = (BN + NT - 1) / NT;
+  ColParams c[kPerThread];
+  __device__ __forceinline__ void fetch(const EpiParams& e, int n_blk0) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int n = n_blk0 + (int)threadIdx.x + i * NT;
+      c[i] = col_params<EPI>(e, n < e.N ? n : e.N - 1);
+    }
+  }
+};
 
 // LDS-tiled int8 GEMM on v_mfma_i32_32x32x32_i8.
 //   block tile BM x BN x BK, WM x WN waves, each wave a (BM/WM) x (BN/WN) tile
@@ -407,7 +423,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
 template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
-                                              int n_blk0) {
+                                              int n_blk0, const ColParams* early) {
   constexpr int TM = FM * 32, TN = FN * 32;
   constexpr int CH = TN / 16;                 // 16-byte chunks per staged row
   constexpr int CP_BYTES = BN * 8;            // per-channel (scale, addend) pairs
@@ -416,10 +432,18 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
 
   __syncthreads();  // every wave is done with the operand tiles
   float2* cp = reinterpret_cast<float2*>(smem);
-  for (int t = tid; t < BN; t += NT) {
-    const int n = n_blk0 + t;
-    const ColParams c = col_params<EPI>(e, n < e.N ? n : e.N - 1);
-    cp[t] = make_float2(c.os, c.b);
+  if (early) {
+#pragma unroll
+    for (int i = 0; i < (BN + NT - 1) / NT; ++i) {
+      const int t = tid + i * NT;
+      if (t < BN) cp[t] = make_float2(early[i].os, early[i].b);
+    }
+  } else {
+    for (int t = tid; t < BN; t += NT) {
+      const int n = n_blk0 + t;
+      const ColParams c = col_params<EPI>(e, n < e.N ? n : e.N - 1);
+      cp[t] = make_float2(c.os, c.b);
+    }
   }
   __syncthreads();
 

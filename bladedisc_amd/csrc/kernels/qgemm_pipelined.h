@@ -232,10 +232,17 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   constexpr int LPR = (LD + 2 * FM - 1) / (2 * FM);          // loads per MFMA row
   constexpr int LD_KS2 = FM * LPR < LD ? FM * LPR : LD;       // loads issued during k-step 2
 
-  // ---- prologue: all of tile 0, then all of tile 1
+  // ---- prologue: all of tile 0, then all of tile 1.  The per-channel epilogue factors
+  // are fetched behind tile 0: their cold loads and the division overlap its flight
+  // instead of sitting between the main loop and the stores.  (Sending tile 1 out before
+  // tile 0 has landed was measured and loses: every CU then pulls 128 KiB before the
+  // first MFMA, and at full occupancy that start-up burst costs more than the one
+  // exposed latency it saves.)
   tile_setup(0);
 #pragma unroll
   for (int idx = 0; idx < LD; ++idx) issue_load(idx, 0);
+  EarlyColParams<EPI, NW * 64, BN> early;
+  early.fetch(p.epi, n0);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   __syncthreads();
   tile_setup(1);
@@ -292,7 +299,8 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   // nothing of this wave may still be writing LDS when the workgroup retires
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
 
-  mfma_epilogue<EPI, FM, FN, NW * 64, BN>(acc, p.epi, smem, m0 + wm * TM, n0 + wn * TN, n0);
+  mfma_epilogue<EPI, FM, FN, NW * 64, BN>(acc, p.epi, smem, m0 + wm * TM, n0 + wn * TN, n0,
+                                          early.c);
 #else
   (void)p;
 #endif
