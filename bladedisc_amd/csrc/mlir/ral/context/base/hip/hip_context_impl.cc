@@ -76,6 +76,7 @@ void InternalAllocator::dealloc(buffer_t buffer) {
 namespace gpu {
 
 const char* kRalBaseHipContextState = "ral_base_hip_context_state";
+const char* kRalGlobalConstantState = "ral_global_constant_state";
 
 namespace {
 
@@ -297,6 +298,48 @@ BaseHipExecutionContext::BaseHipExecutionContext(BaseContext* ctx)
   onExecutionStart();
 }
 
+void BaseHipExecutionContext::bindInput(int input_idx, buffer_t buffer,
+                                        const buffer_shape_t& shape) {
+  Tensor t;
+  t.buffer = buffer;
+  t.shape = shape;
+  inputs[input_idx] = std::move(t);
+  input_ptr_set.insert(buffer);
+}
+
+void BaseHipExecutionContext::bindOutput(int output_idx,
+                                         std::unique_ptr<OutputBufferWrapper>* output) {
+  auto it = outputs.find(output_idx);
+  if (it == outputs.end()) {
+    signalError(Context::FAILURE, "output not found");
+    return;
+  }
+  auto* wrapper = new BaseOutputBufferWrapper(it->second.buffer, it->second.shape);
+  output->reset(wrapper);
+  const_buffer_t buffer = it->second.buffer;
+  // a buffer seen as an output before already has its deleter; a forwarded input or a
+  // persistent buffer (a constant) is not the program's to free
+  if (!output_ptr_set.insert(buffer).second) return;
+  if (input_ptr_set.count(buffer)) return;
+  auto* state = getResource<BaseHipContextState>(kRalBaseHipContextState);
+  if (!state) return;
+  std::lock_guard<std::mutex> guard(state->mu);
+  if (state->device_persistent_buffers.count(buffer)) return;
+  auto dit = device_ptr_map.find(buffer);
+  if (dit == device_ptr_map.end()) return;
+  if (--dit->second == 0) {
+    // the last reference leaves with the output: the wrapper returns it to the pool
+    std::shared_ptr<Allocator> allocator = state->gpu_allocator;
+    std::mutex* mu = &state->mu;
+    wrapper->set_deleter([allocator, mu](buffer_t data) {
+      std::lock_guard<std::mutex> g(*mu);
+      allocator->dealloc(data);
+    });
+    device_ptr_map.erase(dit);
+  }
+  if (outputSharedOrder[buffer] == 1) wrapper->markOwned();
+}
+
 BaseHipExecutionContext::~BaseHipExecutionContext() {
   // buffers the program never handed back return to the pool with the execution
   auto* state = getResource<BaseHipContextState>(kRalBaseHipContextState);
@@ -309,9 +352,29 @@ BaseHipExecutionContext::~BaseHipExecutionContext() {
   onExecutionFinish();
 }
 
+bool isPersistentDeviceBuffer(ExecutionContext* ctx, const_buffer_t buffer) {
+  auto* state = ctx->getResource<BaseHipContextState>(kRalBaseHipContextState);
+  if (!state) return false;
+  std::lock_guard<std::mutex> guard(state->mu);
+  return state->device_persistent_buffers.count(buffer) != 0;
+}
+
+void RalGlobalConstantState::onContextFinish(Context*) {
+  // device constants come from alloc_persistent and go with the context state
+  for (auto& kv : host_constants) ::operator delete(kv.second.first);
+  host_constants.clear();
+  device_constants.clear();
+}
+
 std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
                                                 BaseHipContextOption& gpu_opt) {
   std::unique_ptr<BaseContext> ctx(new BaseContext(opt));
+  ctx->getOrCreateResource(kRalGlobalConstantState, [opt]() {
+    auto* state = new RalGlobalConstantState;
+    if (!opt.metadata_file_path.empty())
+      state->metadata = MetadataFile::loadFromFile(opt.metadata_file_path);
+    return state;
+  });
   ctx->addDriver(GPUDriver::name(), std::unique_ptr<GPUDriver>(new GPUDriver(ctx.get())));
   ctx->getOrCreateResource(kRalBaseHipContextState, [opt, gpu_opt]() {
     auto* state = new BaseHipContextState;

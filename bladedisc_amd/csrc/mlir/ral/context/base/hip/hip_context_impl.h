@@ -12,12 +12,16 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <mutex>
 #include <unordered_map>
+#include <unordered_set>
+#include <utility>
 #include <vector>
 
 #include "mlir/ral/device/gpu/gpu_driver.h"
 #include "mlir/ral/ral_base.h"
 #include "mlir/ral/ral_context.h"
+#include "mlir/ral/ral_metadata.h"
 
 namespace tao {
 namespace ral {
@@ -79,15 +83,75 @@ struct BaseHipContextOption {
 std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
                                                 BaseHipContextOption& gpu_opt);
 
+// A program output as handed to the embedding framework.  When the wrapper owns the
+// buffer (the program allocated it and nothing else refers to it) its destructor
+// returns the buffer to the context's allocator, unless release() was called first.
+class BaseOutputBufferWrapper : public OutputBufferWrapper {
+ public:
+  using Deleter = std::function<void(buffer_t)>;
+  BaseOutputBufferWrapper(buffer_t data, buffer_shape_t shape)
+      : data_(data), shape_(std::move(shape)) {}
+  ~BaseOutputBufferWrapper() override {
+    if (deleter_) deleter_(data_);
+  }
+  const_buffer_t data() override { return data_; }
+  const buffer_shape_t& shape() override { return shape_; }
+  void set_deleter(Deleter deleter) { deleter_ = std::move(deleter); }
+  bool owned() const override { return owned_; }
+  void markOwned() override { owned_ = true; }
+  void release() override {
+    deleter_ = nullptr;
+    owned_ = false;
+  }
+
+ private:
+  buffer_t data_;
+  buffer_shape_t shape_;
+  Deleter deleter_;
+  bool owned_ = false;
+};
+
+struct Tensor {
+  buffer_t buffer = nullptr;
+  buffer_shape_t shape;
+};
+
+// One run of a compiled program: its input / output bindings and the buffers it
+// allocated.  Counterpart of BaseExecutionContext + BaseCudaExecutionContext
+// (context/base/base_context.cc:63-95, context/base/cuda/cuda_context_impl.cc:219-252).
 struct BaseHipExecutionContext : public ExecutionContext {
   explicit BaseHipExecutionContext(BaseContext* ctx);
   ~BaseHipExecutionContext() override;
 
+  void bindInput(int input_idx, buffer_t buffer, const buffer_shape_t& shape) override;
+  void bindOutput(int output_idx, std::unique_ptr<OutputBufferWrapper>* output) override;
+
   // buffers handed out by `alloc` during this execution -> reference count
   std::unordered_map<const_buffer_t, int> device_ptr_map;
+  std::unordered_map<int32_t, Tensor> inputs;
+  std::unordered_map<int32_t, Tensor> outputs;
+  std::unordered_set<const_buffer_t> input_ptr_set;
+  std::unordered_set<const_buffer_t> output_ptr_set;
+  // how many outputs share one underlying buffer
+  std::unordered_map<const_buffer_t, int32_t> outputSharedOrder;
 };
 
 extern const char* kRalBaseHipContextState;
+
+// Context-level store of the program's constants (ral_const): loaded lazily from the
+// metadata file named in BaseContextOption, kept for the life of the context.
+struct RalGlobalConstantState : public Context::Resource {
+  using Item = std::pair<buffer_t, buffer_shape_t>;
+  std::mutex mu;
+  std::unordered_map<std::string, Item> host_constants;
+  std::unordered_map<std::string, Item> device_constants;
+  std::unique_ptr<MetadataFile> metadata;
+  void onContextFinish(Context* ctx) override;
+};
+extern const char* kRalGlobalConstantState;
+
+// device buffers that outlive executions (alloc_persistent): true if `buffer` is one
+bool isPersistentDeviceBuffer(ExecutionContext* ctx, const_buffer_t buffer);
 
 }  // namespace gpu
 }  // namespace ral

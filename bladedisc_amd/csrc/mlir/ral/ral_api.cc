@@ -15,6 +15,7 @@
 #include "mlir/ral/ral_context.h"
 #include "mlir/ral/ral_helper.h"
 #include "mlir/ral/ral_logging.h"
+#include "mlir/ral/ral_metadata.h"
 
 namespace {
 
@@ -123,8 +124,18 @@ tao_ral_context_t disc_ral_context_create(void* hip_stream, int device_ordinal,
                                           disc_ral_alloc_fn alloc,
                                           disc_ral_dealloc_fn dealloc, void* user,
                                           int cache_workspace) {
+  return disc_ral_context_create_for_program(hip_stream, device_ordinal, alloc, dealloc, user,
+                                             cache_workspace, nullptr);
+}
+
+tao_ral_context_t disc_ral_context_create_for_program(void* hip_stream, int device_ordinal,
+                                                      disc_ral_alloc_fn alloc,
+                                                      disc_ral_dealloc_fn dealloc, void* user,
+                                                      int cache_workspace,
+                                                      const char* metadata_file_path) {
   if ((alloc == nullptr) != (dealloc == nullptr)) return nullptr;
   tao::ral::BaseContextOption opt;
+  if (metadata_file_path) opt.metadata_file_path = metadata_file_path;
   opt.cache_workspace_mem_across_execution = cache_workspace != 0;
   tao::ral::gpu::BaseHipContextOption gpu_opt;
   gpu_opt.stream = static_cast<hipStream_t>(hip_stream);
@@ -151,6 +162,77 @@ void disc_ral_execution_context_destroy(tao_ral_context_t exec_ctx) {
 
 tao_ral_context_t disc_ral_execution_context_get_context(tao_ral_context_t exec_ctx) {
   return static_cast<tao::ral::ExecutionContext*>(exec_ctx)->getContext();
+}
+
+int disc_ral_execution_bind_input(tao_ral_context_t exec_ctx, int input_idx, void* buffer,
+                                  const int64_t* shape, int rank) {
+  auto* exec = static_cast<tao::ral::ExecutionContext*>(exec_ctx);
+  if (!exec || rank < 0 || (rank > 0 && !shape)) return 1;
+  exec->bindInput(input_idx, buffer, tao::ral::buffer_shape_t(shape, shape + rank));
+  return 0;
+}
+
+disc_ral_output_t disc_ral_execution_take_output(tao_ral_context_t exec_ctx, int output_idx) {
+  auto* exec = static_cast<tao::ral::ExecutionContext*>(exec_ctx);
+  if (!exec) return nullptr;
+  std::unique_ptr<tao::ral::OutputBufferWrapper> out;
+  exec->bindOutput(output_idx, &out);
+  return out.release();
+}
+
+const void* disc_ral_output_data(disc_ral_output_t output) {
+  return output ? static_cast<tao::ral::OutputBufferWrapper*>(output)->data() : nullptr;
+}
+
+int disc_ral_output_rank(disc_ral_output_t output) {
+  return output ? (int)static_cast<tao::ral::OutputBufferWrapper*>(output)->shape().size() : -1;
+}
+
+int64_t disc_ral_output_dim(disc_ral_output_t output, int i) {
+  if (!output) return -1;
+  const auto& shape = static_cast<tao::ral::OutputBufferWrapper*>(output)->shape();
+  return i >= 0 && i < (int)shape.size() ? shape[i] : -1;
+}
+
+int disc_ral_output_owned(disc_ral_output_t output) {
+  return output && static_cast<tao::ral::OutputBufferWrapper*>(output)->owned() ? 1 : 0;
+}
+
+void disc_ral_output_release(disc_ral_output_t output) {
+  if (output) static_cast<tao::ral::OutputBufferWrapper*>(output)->release();
+}
+
+void disc_ral_output_destroy(disc_ral_output_t output) {
+  delete static_cast<tao::ral::OutputBufferWrapper*>(output);
+}
+
+int disc_ral_metadata_emit(const char* path, int count, const uint8_t* is_host,
+                           const char* const* names, const char* const* hex_values) {
+  if (!path || count < 0 || (count > 0 && (!is_host || !names || !hex_values))) return 1;
+  tao::ral::MetadataFileEmitter emitter(path);
+  if (!emitter.emitHeader()) return 1;
+  for (int i = 0; i < count; ++i) {
+    if (!names[i] || !hex_values[i]) return 1;
+    const bool ok = is_host[i] ? emitter.emitHostConstant(names[i], hex_values[i])
+                               : emitter.emitDeviceConstant(names[i], hex_values[i]);
+    if (!ok) return 1;
+  }
+  return emitter.emitTailer() ? 0 : 1;
+}
+
+int disc_ral_metadata_count(const char* path, int* host_constants, int* device_constants,
+                            const char* const* probe_names, int n_probe) {
+  auto file = path ? tao::ral::MetadataFile::loadFromFile(path) : nullptr;
+  if (!file) return 1;
+  int h = 0, d = 0;
+  for (int i = 0; i < n_probe; ++i) {
+    const std::string* data = nullptr;
+    if (probe_names[i] && file->getHostConstant(probe_names[i], data)) ++h;
+    if (probe_names[i] && file->getDeviceConstant(probe_names[i], data)) ++d;
+  }
+  if (host_constants) *host_constants = h;
+  if (device_constants) *device_constants = d;
+  return 0;
 }
 
 int disc_ral_api_count(void) { return static_cast<int>(apiNames().size()); }

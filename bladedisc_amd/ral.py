@@ -307,6 +307,20 @@ def encode_attr(value):
     raise TypeError("cannot serialise %r" % (value,))
 
 
+def device_view(ptr, shape, dtype, device="cuda"):
+    """A torch tensor over `ptr` (device memory owned by someone else), no copy."""
+    import torch
+    typestr = {torch.int8: "|i1", torch.uint8: "|u1", torch.float32: "<f4", torch.int32: "<i4"}[dtype]
+
+    class _Holder:
+        pass
+
+    h = _Holder()
+    h.__cuda_array_interface__ = {"shape": tuple(int(s) for s in shape), "typestr": typestr,
+                                  "data": (int(ptr), False), "version": 2}
+    return torch.as_tensor(h, device=device)
+
+
 def memref_to_tensor(st, dtype, device="cuda"):
     """Wraps a result memref (callee-allocated device buffer) as a torch tensor
     without copying.  The buffer stays owned by the execution context."""

@@ -63,6 +63,15 @@ tao_ral_context_t disc_ral_context_create(void* hip_stream, int device_ordinal,
                                           disc_ral_alloc_fn alloc,
                                           disc_ral_dealloc_fn dealloc, void* user,
                                           int cache_workspace);
+/* Same, for running a whole compiled program: `metadata_file_path` names the program's
+ * constant store (the side file the compiler writes, ral/ral_metadata.cc:60-200), from
+ * which ral_const serves constants by name; NULL = no constants.  Counterpart of
+ * BaseContextOption::metadata_file_path (context/base/base_context.h:29-34). */
+tao_ral_context_t disc_ral_context_create_for_program(void* hip_stream, int device_ordinal,
+                                                      disc_ral_alloc_fn alloc,
+                                                      disc_ral_dealloc_fn dealloc, void* user,
+                                                      int cache_workspace,
+                                                      const char* metadata_file_path);
 void disc_ral_context_destroy(tao_ral_context_t ctx);
 
 /* One ExecutionContext per run of a compiled program; destroying it returns every
@@ -70,6 +79,35 @@ void disc_ral_context_destroy(tao_ral_context_t ctx);
 tao_ral_context_t disc_ral_execution_context_create(tao_ral_context_t ctx);
 void disc_ral_execution_context_destroy(tao_ral_context_t exec_ctx);
 tao_ral_context_t disc_ral_execution_context_get_context(tao_ral_context_t exec_ctx);
+
+/* Program inputs and outputs: C face of ExecutionContext::bindInput / bindOutput
+ * (ral/ral_context.h:164-167; context/base/base_context.cc:63-95).  Inputs are borrowed.
+ * An output handle owns its buffer when the program allocated it and nothing else
+ * refers to it (disc_ral_output_owned): destroying the handle then returns the buffer to
+ * the context's allocator, unless disc_ral_output_release was called first, which
+ * leaves the buffer to the caller.  Outputs that alias an input or a constant are never
+ * freed by the handle.  bind_input returns 0 on success. */
+typedef void* disc_ral_output_t;
+int disc_ral_execution_bind_input(tao_ral_context_t exec_ctx, int input_idx, void* buffer,
+                                  const int64_t* shape, int rank);
+disc_ral_output_t disc_ral_execution_take_output(tao_ral_context_t exec_ctx, int output_idx);
+const void* disc_ral_output_data(disc_ral_output_t output);
+int disc_ral_output_rank(disc_ral_output_t output);
+int64_t disc_ral_output_dim(disc_ral_output_t output, int i);
+int disc_ral_output_owned(disc_ral_output_t output);
+void disc_ral_output_release(disc_ral_output_t output);
+void disc_ral_output_destroy(disc_ral_output_t output);
+
+/* Writes / inspects a constant store in the reference's metadata-file format
+ * (ral/ral_metadata.cc:60-200): names[i] -> hex_values[i] (the constant's bytes as a
+ * hexadecimal string), a host constant where is_host[i] != 0, else a device constant.
+ * A constant's name is "<id>_<element type>_<d0xd1...>", e.g. "w0_i8_768x768".
+ * disc_ral_metadata_count loads a file and counts how many of the probe names it holds
+ * as host and as device constants.  Both return 0 on success.  Host only. */
+int disc_ral_metadata_emit(const char* path, int count, const uint8_t* is_host,
+                           const char* const* names, const char* const* hex_values);
+int disc_ral_metadata_count(const char* path, int* host_constants, int* device_constants,
+                            const char* const* probe_names, int n_probe);
 
 /* ---- registry introspection ------------------------------------------- */
 

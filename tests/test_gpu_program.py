@@ -1,0 +1,121 @@
+"""A whole compiled program on the runtime: a C stand-in for a DISC-generated `main`
+(tests/programs/qlinear_program.c) fetches its input, materialises its constants from
+a metadata file, runs quantize -> ral_pdll_qgemm -> dequantize and hands back its
+output, all through tao_ral_call_impl.  Checked against the CPU oracle."""
+import ctypes as C
+import os
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+import oracle as O  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def hexstr(a):
+    return np.ascontiguousarray(a).tobytes().hex()
+
+
+@pytest.fixture(scope="module")
+def program(tmp_path_factory):
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc is needed to build the stand-in program")
+    from bladedisc_amd import ral
+    d = tmp_path_factory.mktemp("program")
+    blob = ral.encode_attr({"transpose_a": False, "transpose_b": True, "weight_is_const": True,
+                            "bias_is_const": True})
+    with open(d / "attrs.c", "w") as f:
+        f.write("const unsigned char kQgemmAttrs[] = {%s, 0};\n" % ", ".join(str(b) for b in blob))
+    so = str(d / "libqlinear_program.so")
+    subprocess.check_call(["gcc", "-O1", "-shared", "-fPIC", "-o", so,
+                           os.path.join(HERE, "programs", "qlinear_program.c"), str(d / "attrs.c")])
+    return C.CDLL(so), d
+
+
+def test_compiled_program_runs_on_the_runtime(program):
+    lib, d = program
+    from bladedisc_amd import baseline_configs as cfg
+    from bladedisc_amd import ral
+    L = ral.lib()
+    c = cfg.config1()
+    names = ["w0_i8_768x768", "b0_f32_768", "sw0_f32_768", "sx0_f32_", "so0_f32_", "z0_i32_"]
+    values = [hexstr(c["w_q"]), hexstr(c["bias"]), hexstr(c["sw"]),
+              hexstr(np.array([c["sx"]], np.float32)), hexstr(np.array([c["so"]], np.float32)),
+              hexstr(np.array([0], np.int32))]
+    meta = str(d / "program.metadata").encode()
+    n = len(names)
+    L.disc_ral_metadata_emit.restype = C.c_int
+    rc = L.disc_ral_metadata_emit(meta, n, (C.c_uint8 * n)(*([0] * n)),
+                                  (C.c_char_p * n)(*[s.encode() for s in names]),
+                                  (C.c_char_p * n)(*[v.encode() for v in values]))
+    assert rc == 0
+
+    L.disc_ral_context_create_for_program.restype = C.c_void_p
+    L.disc_ral_execution_take_output.restype = C.c_void_p
+    L.disc_ral_output_data.restype = C.c_void_p
+    L.disc_ral_output_dim.restype = C.c_int64
+    stream = torch.cuda.current_stream().cuda_stream
+    ctx = L.disc_ral_context_create_for_program(C.c_void_p(stream), 0, None, None, None, 1, meta)
+    assert ctx
+    call_impl = C.cast(L.tao_ral_call_impl, C.c_void_p).value
+    try:
+        for m in (64, 5):                       # two executions, a dynamic M, cached constants
+            x = torch.from_numpy(np.ascontiguousarray(c["x"][:m])).cuda()
+            ex = L.disc_ral_execution_context_create(C.c_void_p(ctx))
+            assert L.disc_ral_execution_bind_input(C.c_void_p(ex), 0, C.c_void_p(x.data_ptr()),
+                                                   (C.c_int64 * 2)(m, 768), 2) == 0
+            ctx_struct = (C.c_void_p * 2)(ex, call_impl)
+            lib.disc_program_main(ctx_struct)
+            msg = C.c_char_p()
+            assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) == 0, msg.value
+            out = L.disc_ral_execution_take_output(C.c_void_p(ex), 0)
+            fwd = L.disc_ral_execution_take_output(C.c_void_p(ex), 1)
+            assert out and fwd
+            assert L.disc_ral_output_rank(C.c_void_p(out)) == 2
+            assert [L.disc_ral_output_dim(C.c_void_p(out), i) for i in range(2)] == [m, 768]
+            # output 0 was allocated by the program: the handle owns it; output 1 is the
+            # input buffer handed back and stays the caller's
+            assert L.disc_ral_output_owned(C.c_void_p(out)) == 1
+            assert L.disc_ral_output_owned(C.c_void_p(fwd)) == 0
+            assert L.disc_ral_output_data(C.c_void_p(fwd)) == x.data_ptr()
+            torch.cuda.synchronize()
+            y = ral.device_view(L.disc_ral_output_data(C.c_void_p(out)), (m, 768),
+                                torch.float32).cpu().numpy()
+            # oracle: the same chain on the host
+            xq = O.quantize(c["x"][:m], c["sx"], 0)
+            acc = O.gemm_s32(xq, c["w_q"], tp_b=True)
+            b32 = O.bias_f32_to_s32(c["bias"], float(c["sx"]), c["sw"])
+            yq = O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]), b32=b32)
+            np.testing.assert_array_equal(y, O.dequantize(yq, c["so"], 0))
+            L.disc_ral_output_destroy(C.c_void_p(out))
+            L.disc_ral_output_destroy(C.c_void_p(fwd))
+            L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+    finally:
+        torch.cuda.synchronize()
+        L.disc_ral_context_destroy(C.c_void_p(ctx))
+
+
+def test_missing_constant_is_reported(program):
+    lib, d = program
+    from bladedisc_amd import ral
+    L = ral.lib()
+    L.disc_ral_context_create_for_program.restype = C.c_void_p
+    meta = str(d / "empty.metadata").encode()
+    assert L.disc_ral_metadata_emit(meta, 0, None, None, None) == 0
+    ctx = L.disc_ral_context_create_for_program(None, 0, None, None, None, 1, meta)
+    x = torch.zeros((4, 768), device="cuda")
+    ex = L.disc_ral_execution_context_create(C.c_void_p(ctx))
+    L.disc_ral_execution_bind_input(C.c_void_p(ex), 0, C.c_void_p(x.data_ptr()), (C.c_int64 * 2)(4, 768), 2)
+    call_impl = C.cast(L.tao_ral_call_impl, C.c_void_p).value
+    lib.disc_program_main((C.c_void_p * 2)(ex, call_impl))
+    msg = C.c_char_p()
+    assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) != 0
+    assert b"not found in metadata file" in msg.value
+    L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+    torch.cuda.synchronize()
+    L.disc_ral_context_destroy(C.c_void_p(ctx))

@@ -250,3 +250,80 @@ def test_conv2d_plan_matches_oracle():
         kw.update(bad)
         with pytest.raises(ValueError):
             ral_ops.conv2d_plan((1, 5, 5, 4), (3, 3, 3, 4), **kw)
+
+
+def test_metadata_file_round_trip(tmp_path):
+    """Constant store in the reference's metadata-file layout: written, read back,
+    duplicate names refused, a damaged file rejected."""
+    import struct
+    L = ral.lib()
+    path = str(tmp_path / "m.metadata").encode()
+    names = [b"w0_i8_2x2", b"h0_f32_", b"w1_f32_3"]
+    vals = [b"01ff7f80", b"0000803f", b"00"]
+    flags = (C.c_uint8 * 3)(0, 1, 0)
+    assert L.disc_ral_metadata_emit(path, 3, flags, (C.c_char_p * 3)(*names),
+                                    (C.c_char_p * 3)(*vals)) == 0
+    raw = open(path, "rb").read()
+    # layout: magic, records {is_host u8, len-prefixed key, len-prefixed value}, count
+    assert struct.unpack_from("<Q", raw, 0)[0] == 0x1234567890ABCDEF
+    assert struct.unpack_from("<Q", raw, len(raw) - 8)[0] == 3
+    assert raw[8] == 0 and struct.unpack_from("<Q", raw, 9)[0] == len(names[0])
+    assert raw[17:17 + len(names[0])] == names[0]
+    h, d = C.c_int(), C.c_int()
+    probes = (C.c_char_p * 4)(*(names + [b"absent_i8_1"]))
+    assert L.disc_ral_metadata_count(path, C.byref(h), C.byref(d), probes, 4) == 0
+    assert (h.value, d.value) == (1, 2)
+    # duplicate device constant
+    dup = str(tmp_path / "dup.metadata").encode()
+    assert L.disc_ral_metadata_emit(dup, 2, (C.c_uint8 * 2)(0, 0), (C.c_char_p * 2)(b"a_i8_1", b"a_i8_1"),
+                                    (C.c_char_p * 2)(b"00", b"01")) != 0
+    # truncated and wrong-magic files
+    bad = str(tmp_path / "bad.metadata")
+    open(bad, "wb").write(raw[:-12])
+    assert L.disc_ral_metadata_count(bad.encode(), None, None, probes, 4) != 0
+    open(bad, "wb").write(b"\x00" * 8 + raw[8:])
+    assert L.disc_ral_metadata_count(bad.encode(), None, None, probes, 4) != 0
+    assert L.disc_ral_metadata_count(str(tmp_path / "nope").encode(), None, None, probes, 4) != 0
+
+
+def test_program_io_bindings_on_host_memory():
+    """ral_recv_input / ral_send_output / take_output with plain host buffers: inputs are
+    found by index and rank, an output that is an input is forwarded, unknown indices
+    are errors."""
+    L = ral.lib()
+    L.disc_ral_execution_take_output.restype = C.c_void_p
+    L.disc_ral_output_data.restype = C.c_void_p
+    L.disc_ral_output_dim.restype = C.c_int64
+    ctx = ral.RalContext()
+    try:
+        with ctx.execution() as ex:
+            buf = np.arange(12, dtype=np.float32)
+            assert L.disc_ral_execution_bind_input(C.c_void_p(ex.handle), 3,
+                                                   C.c_void_p(buf.ctypes.data),
+                                                   (C.c_int64 * 2)(3, 4), 2) == 0
+            a = ral.Args().ctx(ex.handle)
+            a.scalar("i64", 3)
+            res = a.result_memref("f32", 2)
+            ex.call("ral_recv_input", "cpu", a)
+            assert res.data == buf.ctypes.data and list(res.sizes) == [3, 4]
+            assert list(res.strides) == [4, 1]
+            # send it back as output 0
+            a = ral.Args().ctx(ex.handle)
+            a.scalar("i64", 0)
+            a.memref("f32", buf.ctypes.data, [3, 4])
+            ex.call("ral_send_output", "cpu", a)
+            out = L.disc_ral_execution_take_output(C.c_void_p(ex.handle), 0)
+            assert out and L.disc_ral_output_data(C.c_void_p(out)) == buf.ctypes.data
+            assert L.disc_ral_output_owned(C.c_void_p(out)) == 0
+            assert [L.disc_ral_output_dim(C.c_void_p(out), i) for i in range(2)] == [3, 4]
+            L.disc_ral_output_destroy(C.c_void_p(out))
+        own = ral.RalContext()
+        with own.execution() as ex:
+            a = ral.Args().ctx(ex.handle)
+            a.scalar("i64", 7)
+            a.result_memref("f32", 2)
+            with pytest.raises(ral.RalError, match="invalid input index"):
+                ex.call("ral_recv_input", "cpu", a)
+        own.close()
+    finally:
+        ctx.close()
