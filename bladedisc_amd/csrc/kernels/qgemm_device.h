@@ -148,7 +148,9 @@ __device__ __forceinline__ uint32_t requant_pack4(const EpiParams& p, const ColP
       d = c[e].os * d;
       d = d + c[e].b;
     }
-    d = fminf(fmaxf(d, -128.0f), 127.0f);  // NaN -> -128, like the CPU path
+    // v_med3_f32: one instruction for the clamp; with a NaN operand it returns the
+    // minimum of the other two, so NaN -> -128 like the CPU path
+    d = __builtin_amdgcn_fmed3f(d, -128.0f, 127.0f);
     d = d + 12582912.0f;
     bits[e] = __float_as_uint(d);
   }
@@ -482,7 +484,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
       if (m < e.M && n < e.N) {
         int8_t* dst = out + (int64_t)m * e.ldo + n;
         if (n + 15 < e.N) {
-          *reinterpret_cast<v4i*>(dst) = v;
+          __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
         } else {
 #pragma unroll
           for (int b = 0; b < 16; ++b)

@@ -40,6 +40,14 @@
 
 #include "qgemm_device.h"
 
+// Timeline hook for profiling builds: a harness may define DQ8_TRACE_POINT(i) before
+// including this header to record when a workgroup passes stage i (0 entry, 1 first
+// tile landed, 2 main loop done, 3 results computed and stored).  Expands to nothing in
+// the library.
+#ifndef DQ8_TRACE_POINT
+#define DQ8_TRACE_POINT(i)
+#endif
+
 namespace dq8 {
 
 // gfx9 raw buffer descriptor word 3: 32-bit data format, no swizzle
@@ -96,6 +104,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   static_assert(NW % 2 == 0, "the chunk a lane loads must not depend on the load slot");
 
   extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+  DQ8_TRACE_POINT(0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -245,6 +254,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   early.fetch(p.epi, n0);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   __syncthreads();
+  DQ8_TRACE_POINT(1);
   tile_setup(1);
 #pragma unroll
   for (int idx = 0; idx < LD; ++idx) issue_load(idx, 1);
@@ -298,9 +308,11 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   }
   // nothing of this wave may still be writing LDS when the workgroup retires
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  DQ8_TRACE_POINT(2);
 
   mfma_epilogue<EPI, FM, FN, NW * 64, BN>(acc, p.epi, smem, m0 + wm * TM, n0 + wn * TN, n0,
                                           early.c);
+  DQ8_TRACE_POINT(3);
 #else
   (void)p;
 #endif

@@ -338,6 +338,34 @@ def test_qconv_known_answers(K, golden):
             assert (out.astype(np.float32) * case["so"] == case["expect_f32"]).all(), case["src"]
 
 
+def test_requant_nan_and_inf_scales_saturate_like_the_oracle(K):
+    """A NaN or infinite per-channel factor: NaN results go to -128, infinities
+    saturate by sign, on every kernel family and both requant epilogues."""
+    rng = np.random.default_rng(11)
+    m, n, k = 130, 256, 256
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx = np.float32(0.02)
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    sw[3] = np.nan
+    sw[7] = np.inf
+    sw[200] = -np.inf
+    so = np.float32(2.0)
+    bias = rng.standard_normal(n).astype(np.float32)
+    with np.errstate(all="ignore"):
+        want_gpu = O.requant_gpu(acc, sx, sw, so, bias_f32=bias)
+        want_cpu = O.requant_cpu(acc, sx, sw, so)
+    assert (want_gpu[:, 3] == -128).all()
+    for v in gemm_variants(K, k):
+        got = host(K.qgemm(dev(a), dev(w), K.EPI_REQUANT_GPU, sx=dev(np.array([sx])), sw=dev(sw),
+                           so=dev(np.array([so])), bias=dev(bias), variant=v))
+        np.testing.assert_array_equal(got, want_gpu, err_msg="variant %d" % v)
+        got = host(K.qgemm(dev(a), dev(w), K.EPI_REQUANT_CPU, sx=dev(np.array([sx])), sw=dev(sw),
+                           so=dev(np.array([so])), variant=v))
+        np.testing.assert_array_equal(got, want_cpu, err_msg="variant %d" % v)
+
+
 def test_bad_arguments_fail_loudly(K):
     a = torch.zeros((4, 16), dtype=torch.int8, device="cuda")
     w = torch.zeros((4, 32), dtype=torch.int8, device="cuda")
