@@ -7,8 +7,9 @@ int8 values uniform in [-127,127], per-channel weight scales uniform in
 (round-half-to-even, saturate).  One "step" is one such GEMM; inputs are resident
 in HBM before the timed region.  Prints ONE JSON line.
 
-Extra (same line, under "extra"): quantize / dequantize GB/s on a 1 GiB f32 tensor
-and the other BASELINE configs at a glance.
+Extra (same line, under "extra"): quantize / dequantize GB/s on a 1 GiB f32 tensor,
+all five benchmark configurations next to the CPU oracle, and the ROCm library int8
+GEMM as a yardstick.
 """
 import argparse
 import ctypes as C
