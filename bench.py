@@ -38,7 +38,9 @@ def parse():
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--size", type=int, default=4096, help="M = N = K of the headline GEMM")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    p.add_argument("--no-extra", action="store_true", help="skip the q/dq and sweep extras")
+    p.add_argument("--no-extra", action="store_true", help="skip the extras")
+    p.add_argument("--extras", choices=("all", "qdq"), default="all",
+                   help="'qdq': only the quantize / dequantize bandwidth cases (for profiling)")
     p.add_argument("--pattern", choices=("uniform", "ones"), default="uniform",
                    help="operand values: 'uniform' is the benchmark's definition (integers uniform "
                         "in [-127,127]); 'ones' is a diagnosis aid that shows how much of the time "
@@ -347,7 +349,7 @@ def config_reports(torch, K):
     return rep
 
 
-def extras(torch, steps, warmup):
+def extras(torch, steps, warmup, which="all"):
     """q/dq bandwidth on a tensor larger than the 256 MB last-level cache, the five
     benchmark configurations against the CPU oracle, and a library yardstick."""
     from bladedisc_amd import kernels as K
@@ -382,6 +384,8 @@ def extras(torch, steps, warmup):
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 5}
     del x, q, f
+    if which == "qdq":
+        return out
     out["configs"] = config_reports(torch, K)
     # yardstick: the ROCm library int8 GEMM behind torch._int_mm (int32 output, no
     # epilogue) on the headline shape and data distribution -- a library, not the reference
@@ -485,7 +489,7 @@ def main():
     else:
         result["cpu_baseline"] = None
     if not args.no_extra:
-        result["extra"] = extras(torch, args.steps, args.warmup)
+        result["extra"] = extras(torch, args.steps, args.warmup, args.extras)
     print(json.dumps(result))
 
 
