@@ -338,6 +338,28 @@ def test_qconv_known_answers(K, golden):
             assert (out.astype(np.float32) * case["so"] == case["expect_f32"]).all(), case["src"]
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(300, 200, 256, 64), (17, 48, 1040, 16), (1000, 768, 768, 128)])
+def test_qgemm_strided_rows_all_variants(K, m, n, k, pad):
+    """Operands and output that are column slices of wider buffers (row stride > row
+    length): the kernels must neither read the gap as data nor write into it."""
+    rng = np.random.default_rng(m + n + k)
+    a_full = rng.integers(-128, 128, (m, k + pad), dtype=np.int8)
+    w_full = rng.integers(-128, 128, (n, k + 2 * pad), dtype=np.int8)
+    a, w = a_full[:, :k], w_full[:, pad:pad + k]
+    acc, _ = O.gemm_s32_fast(np.ascontiguousarray(a), np.ascontiguousarray(w))
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    want = O.requant_cpu(acc, sx, sw, so)
+    da, dw = dev(a_full)[:, :k], dev(w_full)[:, pad:pad + k]
+    for v in [-1] + gemm_variants(K, k):
+        out_full = torch.full((m, n + pad), 77, dtype=torch.int8, device="cuda")
+        K.qgemm(da, dw, K.EPI_REQUANT_CPU, sx=dev(np.array([sx])), sw=dev(sw),
+                so=dev(np.array([so])), out=out_full[:, :n], variant=v)
+        got = host(out_full)
+        np.testing.assert_array_equal(got[:, :n], want, err_msg="variant %d" % v)
+        assert (got[:, n:] == 77).all(), "variant %d wrote past the row" % v
+
+
 def test_requant_nan_and_inf_scales_saturate_like_the_oracle(K):
     """A NaN or infinite per-channel factor: NaN results go to -128, infinities
     saturate by sign, on every kernel family and both requant epilogues."""
@@ -376,3 +398,15 @@ def test_bad_arguments_fail_loudly(K):
         K.qgemm(a, w, K.EPI_REQUANT_CPU)          # scales missing
     with pytest.raises(RuntimeError):
         K.qgemm(a, w, K.EPI_ACC_S32, variant=99)
+    # limits are checked before any pointer is touched
+    from bladedisc_amd import _lib
+    L = _lib.lib()
+    import ctypes as C
+    big = C.c_int64(1 << 31)
+    one = C.c_int64(1)
+    st = L.dq8_qgemm(None, one, None, one, None, big, one, big, one, 0, 1, 0, None, 0, None, one,
+                     None, one, None, one, 0, 0, 0, None, C.c_size_t(0), None)
+    assert st != 0 and b"2^31" in L.dq8_last_error()
+    st = L.dq8_qgemm(None, one, None, one, None, one, C.c_int64(-1), one, one, 0, 1, 0, None, 0,
+                     None, one, None, one, None, one, 0, 0, 0, None, C.c_size_t(0), None)
+    assert st != 0 and b"negative" in L.dq8_last_error()
