@@ -341,10 +341,26 @@ def config_reports(torch, K):
         for _ in range(10):
             layer.forward(h)
         torch.cuda.synchronize()
+        eager_us = (time.perf_counter() - t0) / 10 * 1e6
+        # the same layer replayed from a HIP graph
+        graph_us = None
+        try:
+            replay, _, _ = layer.capture(h)
+            for _ in range(3):
+                replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(20):
+                replay()
+            torch.cuda.synchronize()
+            graph_us = round((time.perf_counter() - t0) / 20 * 1e6, 1)
+        except Exception as exc:  # capture is an optimisation, not the path under test
+            graph_us = "capture failed: %s" % str(exc)[:100]
         bert["seq%d" % seq] = {"linears_q_gemm_dq": per,
                                "quantized_ops_gpu_us": round(gpu_sum * 1e6, 2),
                                "quantized_ops_cpu_us": round(cpu_sum * 1e6, 1),
-                               "layer_eager_wall_us": round((time.perf_counter() - t0) / 10 * 1e6, 1)}
+                               "layer_eager_wall_us": round(eager_us, 1),
+                               "layer_graph_replay_us": graph_us}
     rep["5_bert_base_layer_batch8"] = bert
     return rep
 

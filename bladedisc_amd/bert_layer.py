@@ -141,6 +141,27 @@ class QuantBertLayer:
             rec[name] = dict(x=x2, x_q=x_q, y_q=y_q, y=y)
         return y.reshape(*shape[:-1], y.shape[-1])
 
+    def capture(self, h):
+        """Records one forward pass on `h`'s shape into a HIP graph and returns
+        (replay, static_input, static_output): copy new activations into static_input,
+        call replay(), read static_output.  A BERT layer at small batch x seq is a few
+        dozen short kernels, and launching them one by one from the host takes longer
+        than running them; a graph replays them back to back.  Only the raw backend can be
+        captured (its kernels take preallocated outputs; the RAL entries allocate theirs)."""
+        if not isinstance(self.be, RawBackend):
+            raise RuntimeError("graph capture needs the raw backend")
+        static_in = h.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):        # warm-up on the capture stream
+            for _ in range(2):
+                self.forward(static_in)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            static_out = self.forward(static_in)
+        return graph.replay, static_in, static_out
+
     def forward(self, h, record=None):
         if not self.s_in:
             raise RuntimeError("calibrate() first")

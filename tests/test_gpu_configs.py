@@ -178,3 +178,22 @@ def test_config5_bert_layer(C, seq, backend):
         if ex is not None:
             ex.close()
             ctx.close()
+
+
+def test_config5_bert_layer_graph_replays_match_eager(C):
+    """The captured layer against eager execution: several replays, with eager work and
+    synchronisations in between, each compared bit for bit."""
+    from bladedisc_amd import bert_layer as B
+    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend())
+    h0 = layer.embed(C.config5_tokens(8, 32))
+    layer.calibrate(h0)
+    replay, static_in, static_out = layer.capture(h0)
+    for i in range(4):
+        h = layer.embed(C.config5_tokens(8, 32) if i == 0 else
+                        np.roll(C.config5_tokens(8, 32), i, axis=1))
+        want = layer.forward(h)                       # eager work between the replays
+        torch.cuda.synchronize()
+        static_in.copy_(h)
+        replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, want), "replay %d differs from eager" % i
