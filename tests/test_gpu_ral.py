@@ -275,3 +275,45 @@ def test_driver_alloc_copy_roundtrip_and_pool_reuse(rt):
         ex.call("ral_gpu_as_cu_stream", "gpu", a)
         assert (r.value or 0) == torch.cuda.current_stream().cuda_stream
         del C
+
+
+def test_concurrent_executions_on_one_context(rt):
+    """One Context serves several ExecutionContexts from different threads
+    (ral/ral_context.h:52-58 in the reference): registry lookups, the attribute cache,
+    the packed-weight cache and the allocator are shared.  Every thread checks its own
+    results against the oracle."""
+    import threading
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(99)
+    k, n = 256, 192
+    w_kn = rng.integers(-128, 128, (k, n), dtype=np.int8)           # [K,N]: goes through the pack cache
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    sx, so = np.float32(0.02), np.float32(0.5)
+    d_w, d_sw, d_bias = dev(w_kn), dev(sw), dev(bias)
+    b32 = O.bias_f32_to_s32(bias, float(sx), sw)
+    errors = []
+
+    def worker(tid):
+        try:
+            r = np.random.default_rng(tid)
+            for it in range(12):
+                m = int(r.integers(1, 300))
+                a = r.integers(-128, 128, (m, k), dtype=np.int8)
+                with ctx.execution() as ex:
+                    got = ops.pdll_qgemm_cpu_style(ex, dev(a), d_w, d_bias, f1(sx), d_sw, f1(so),
+                                                   transpose_b=False, weight_is_const=True)
+                    torch.cuda.synchronize()
+                    acc = O.gemm_s32(a, w_kn)
+                    want = O.requant_cpu(acc, float(sx), sw, float(so), b32=b32)
+                    if not np.array_equal(got.cpu().numpy(), want):
+                        errors.append("thread %d iteration %d (m=%d) differs" % (tid, it, m))
+        except Exception as exc:  # noqa: BLE001
+            errors.append("thread %d: %r" % (tid, exc))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
