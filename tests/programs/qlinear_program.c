@@ -13,6 +13,7 @@
  * Test fixture only; compiled with gcc by tests/test_gpu_program.py. */
 #include <stdint.h>
 #include <string.h>
+#include <time.h>
 
 typedef void (*ral_call_t)(void* exec, void* name, void** args);
 
@@ -116,4 +117,46 @@ void disc_program_main(void** ctx_struct) {
     call(exec, (void*)"ral_send_output___cpu___pvoid_i64_m2df32___void", args); }
   { int64_t idx = 1; void* args[16]; int n = 0; args[n++] = &exec; args[n++] = &idx; n = push2(args, n, &x);
     call(exec, (void*)"ral_send_output___cpu___pvoid_i64_m2df32___void", args); }
+}
+
+/* Host cost of the dispatch path: `n` back-to-back ral_pdll_qgemm calls on M rows of
+ * uninitialised int8 data (each call allocates its result, which is freed at once), one
+ * stream synchronisation at the end.  Returns microseconds per call. */
+double disc_program_qgemm_loop(void** ctx_struct, int64_t M, int n) {
+  void* exec = ctx_struct[0];
+  ral_call_t call = (ral_call_t)ctx_struct[1];
+  void* stream = 0;
+  MemRef2 w; MemRef1 bias, sw; MemRef0 sx, so;
+  const_call(call, exec, "ral_const___gpu___pvoid_pvoid_pvoid_i32___m2di8", "w0_i8_768x768", 0, &w);
+  const_call(call, exec, "ral_const___gpu___pvoid_pvoid_pvoid_i32___m1df32", "b0_f32_768", 1, &bias);
+  const_call(call, exec, "ral_const___gpu___pvoid_pvoid_pvoid_i32___m1df32", "sw0_f32_768", 2, &sw);
+  const_call(call, exec, "ral_const___gpu___pvoid_pvoid_pvoid_i32___m0df32", "sx0_f32_", 3, &sx);
+  const_call(call, exec, "ral_const___gpu___pvoid_pvoid_pvoid_i32___m0df32", "so0_f32_", 4, &so);
+  const int64_t N = w.sizes[0], K = w.sizes[1];
+  MemRef2 xq = {0};
+  xq.base = xq.data = gpu_alloc(call, exec, M * K);
+  xq.sizes[0] = M; xq.sizes[1] = K; xq.strides[0] = K; xq.strides[1] = 1;
+  int32_t zx = 0, zo = 0; int32_t zw_data[768]; memset(zw_data, 0, sizeof(zw_data));
+  MemRef0 zx_m = {&zx, &zx, 0}, zo_m = {&zo, &zo, 0};
+  MemRef1 zw_m = {zw_data, zw_data, 0, {N}, {1}};
+  const void* attrs = kQgemmAttrs;
+  struct timespec t0, t1;
+  clock_gettime(CLOCK_MONOTONIC, &t0);
+  for (int it = 0; it < n; ++it) {
+    MemRef2 yq;
+    void* args[64]; int k = 0;
+    args[k++] = &exec; args[k++] = &stream;
+    k = push2(args, k, &xq); k = push2(args, k, &w); k = push1(args, k, &bias);
+    k = push0(args, k, &sx); k = push0(args, k, &zx_m);
+    k = push1(args, k, &sw); k = push1(args, k, &zw_m);
+    k = push0(args, k, &so); k = push0(args, k, &zo_m);
+    args[k++] = &attrs; args[k++] = &yq;
+    call(exec, (void*)"ral_pdll_qgemm___gpu___pvoid_pvoid_m2di8_m2di8_m1df32_m0df32_m0di32_m1df32_m1di32_m0df32_m0di32_pvoid___m2di8", args);
+    gpu_dealloc(call, exec, yq.data);
+  }
+  { void* args[2] = {&exec, &stream};
+    call(exec, (void*)"sync_on_stream___gpu___pvoid_pvoid___void", args); }
+  clock_gettime(CLOCK_MONOTONIC, &t1);
+  gpu_dealloc(call, exec, xq.data);
+  return ((t1.tv_sec - t0.tv_sec) * 1e6 + (t1.tv_nsec - t0.tv_nsec) * 1e-3) / n;
 }

@@ -119,3 +119,45 @@ def test_missing_constant_is_reported(program):
     L.disc_ral_execution_context_destroy(C.c_void_p(ex))
     torch.cuda.synchronize()
     L.disc_ral_context_destroy(C.c_void_p(ctx))
+
+
+def test_dispatch_path_cost_per_call(program, capsys):
+    """Whole path of one ral_pdll_qgemm call from compiled code (name lookup, argument
+    unpacking, cached attributes, pooled allocation, launch): it must stay in the range of
+    the kernel it launches, far from the reference's copy-scales-to-host-and-synchronise
+    per call."""
+    lib, d = program
+    from bladedisc_amd import baseline_configs as cfg
+    from bladedisc_amd import ral
+    L = ral.lib()
+    c = cfg.config1()
+    names = ["w0_i8_768x768", "b0_f32_768", "sw0_f32_768", "sx0_f32_", "so0_f32_"]
+    values = [hexstr(c["w_q"]), hexstr(c["bias"]), hexstr(c["sw"]),
+              hexstr(np.array([c["sx"]], np.float32)), hexstr(np.array([c["so"]], np.float32))]
+    meta = str(d / "loop.metadata").encode()
+    n = len(names)
+    assert L.disc_ral_metadata_emit(meta, n, (C.c_uint8 * n)(*([0] * n)),
+                                    (C.c_char_p * n)(*[s.encode() for s in names]),
+                                    (C.c_char_p * n)(*[v.encode() for v in values])) == 0
+    L.disc_ral_context_create_for_program.restype = C.c_void_p
+    ctx = L.disc_ral_context_create_for_program(None, 0, None, None, None, 1, meta)
+    ex = L.disc_ral_execution_context_create(C.c_void_p(ctx))
+    call_impl = C.cast(L.tao_ral_call_impl, C.c_void_p).value
+    lib.disc_program_qgemm_loop.restype = C.c_double
+    lib.disc_program_qgemm_loop.argtypes = [C.c_void_p, C.c_int64, C.c_int]
+    ctx_struct = (C.c_void_p * 2)(ex, call_impl)
+    try:
+        report = {}
+        for m in (1, 16, 256, 4096):
+            lib.disc_program_qgemm_loop(ctx_struct, m, 50)            # warm the caches
+            report[m] = lib.disc_program_qgemm_loop(ctx_struct, m, 2000)
+        msg = C.c_char_p()
+        assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) == 0, msg.value
+        with capsys.disabled():
+            print("\nral_pdll_qgemm from compiled code, us per call (768x768 weights):",
+                  {m: round(v, 2) for m, v in report.items()})
+        assert report[1] < 25 and report[16] < 25
+    finally:
+        L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+        torch.cuda.synchronize()
+        L.disc_ral_context_destroy(C.c_void_p(ctx))
