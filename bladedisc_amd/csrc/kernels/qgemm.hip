@@ -163,11 +163,14 @@ const Variant kVariants[] = {
     {"pipe_128x128x128", 128, 128, 128, 256},
     {"pipe_64x64x128", 64, 64, 128, 256},
     {"pipe_256x64x128", 256, 64, 128, 256},
+    // the same with the k tiles split over 2 groups of waves inside the workgroup
+    {"pipe_64x64x128_k2", 64, 64, 128, 512},
     // small-M kernel: 16 output channels per workgroup, K split over the waves (GEMM only)
     {"skinny_16", 16, 16, 64, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
-constexpr int kSkinnyVariant = 8;
+constexpr int kPipe64k2 = 8;
+constexpr int kSkinnyVariant = 9;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -198,13 +201,13 @@ bool pipe_ok(int bm, int bn, const MainParams& p, bool conv) {
   return (int64_t)bm * p.lda + p.K + 2 * BK < (1LL << 31);
 }
 
-template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
+template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI>
 int launch_pipe(const MainParams& p, hipStream_t st) {
   constexpr int BK = 128;
-  constexpr int lds = 2 * (BM + BN) * BK;
+  constexpr int lds = KSPLIT * 2 * (BM + BN) * BK;
   DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
               "pipelined qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
-  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, CONV, EPI>;
+  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, KSPLIT, CONV, EPI>;
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [&] {
@@ -212,7 +215,7 @@ int launch_pipe(const MainParams& p, hipStream_t st) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   });
   DQ8_HIP(attr_err);
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(WM * WN * 64), lds, st, p);
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(WM * WN * KSPLIT * 64), lds, st, p);
   return check_hip(hipGetLastError(), "qgemm_pipe launch");
 }
 
@@ -242,10 +245,11 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case 1: return launch_mfma<256, 256, 64, 2, 2, CONV, EPI>(p, st);
     case 2: return launch_mfma<128, 128, 64, 2, 2, CONV, EPI>(p, st);
     case 3: return launch_mfma<64, 64, 64, 2, 2, CONV, EPI>(p, st);
-    case kPipe256: return launch_pipe<256, 256, 2, 2, CONV, EPI>(p, st);
-    case kPipe128: return launch_pipe<128, 128, 2, 2, CONV, EPI>(p, st);
-    case kPipe64: return launch_pipe<64, 64, 2, 2, CONV, EPI>(p, st);
-    case kPipe256x64: return launch_pipe<256, 64, 4, 1, CONV, EPI>(p, st);
+    case kPipe256: return launch_pipe<256, 256, 2, 2, 1, CONV, EPI>(p, st);
+    case kPipe128: return launch_pipe<128, 128, 2, 2, 1, CONV, EPI>(p, st);
+    case kPipe64: return launch_pipe<64, 64, 2, 2, 1, CONV, EPI>(p, st);
+    case kPipe256x64: return launch_pipe<256, 64, 4, 1, 1, CONV, EPI>(p, st);
+    case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, CONV, EPI>(p, st);
   }
   if constexpr (!CONV) {
     if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
@@ -268,14 +272,17 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 // kernels can take the operands.  Measured on BERT-shaped and square problems: the
 // 256x256 tile pays once it fills the chip (>= ~240 tiles), the 128x128 tile from about
 // 120 tiles on, below that the 64x64 tile spreads the weight stream over more CUs; narrow
-// outputs (N <= 64) take the 256x64 tile.
-int pick_variant(int64_t M, int64_t N, bool pipe) {
+// outputs (N <= 64) take the 256x64 tile.  With 64x64 tiles a CU's operand loads, not its
+// MFMAs, set the pace (16 KiB per 128 of k against 128 MFMA cycles per SIMD); when few
+// CUs are busy and K is deep, splitting K over two wave groups of the workgroup still
+// shortens the chain of dependent k tiles (about 10 % at K = 3072).
+int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe) {
   auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
   if (pipe) {
     if (N <= 64 && M >= 256 * 64) return kPipe256x64;
     if (tiles(kPipe256) >= 240) return kPipe256;
     if (tiles(kPipe128) >= 120) return kPipe128;
-    return kPipe64;
+    return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
   constexpr int64_t kCus = 256;
   for (int v = 1; v <= 3; ++v)
@@ -490,7 +497,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.K = (int)K;
   p.epi = e;
   if (auto_pick)
-    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, pipe_ok(256, 256, p, false));
+    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false));
   return launch_epi<false>(variant, p, epilogue, st);
 }
 
@@ -621,7 +628,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   p.sh = sh; p.sw_ = sw_; p.dh = dh; p.dw = dw;
   p.conv_bytes = NB * H * Wd * Ci;
   p.epi = e;
-  if (auto_pick) variant = pick_variant(Mg, Co, pipe_ok(256, 256, p, true));
+  if (auto_pick) variant = pick_variant(Mg, Co, Kg, pipe_ok(256, 256, p, true));
   return launch_epi<true>(variant, p, epilogue, st);
 }
 

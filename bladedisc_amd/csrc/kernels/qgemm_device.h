@@ -240,7 +240,8 @@ __device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, i
 template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
-                                              int n_blk0, const ColParams* early = nullptr);
+                                              int n_blk0, const ColParams* early = nullptr,
+                                              int wave_slot = -1, bool active = true);
 
 // The per-channel factors of the channels thread t is responsible for in the epilogue
 // (t, t + NT, ...), fetched at the start of a kernel so that the cold loads of scales
@@ -425,11 +426,15 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
 template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
-                                              int n_blk0, const ColParams* early) {
+                                              int n_blk0, const ColParams* early,
+                                              int wave_slot, bool active) {
+  // `wave_slot`: which per-wave staging tile this wave uses (default: its index in the
+  // workgroup); waves with `active` false only take part in the barriers.
   constexpr int TM = FM * 32, TN = FN * 32;
   constexpr int CH = TN / 16;                 // 16-byte chunks per staged row
   constexpr int CP_BYTES = BN * 8;            // per-channel (scale, addend) pairs
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = wave_slot >= 0 ? wave_slot : tid >> 6;
   const int wn_off = n_wave0 - n_blk0;
 
   __syncthreads();  // every wave is done with the operand tiles
@@ -448,6 +453,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     }
   }
   __syncthreads();
+  if (!active) return;
 
   constexpr bool kInt8Out = EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU;
   if (kInt8Out && e.vec_store16) {

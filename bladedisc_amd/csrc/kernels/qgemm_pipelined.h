@@ -30,6 +30,12 @@
 // the matrix cores draw, not by its schedule: the shader clock, 2.4 GHz when a few
 // CUs run it, falls to 1.5-1.7 GHz (clock64 against wall_clock64), and variations of
 // the schedule that change the cycle count leave the time per tile where it is.
+// KSPLIT > 1: the workgroup has KSPLIT groups of WM x WN waves; group g runs the same
+// pipeline, with LDS stages of its own, over k tiles [g * ceil(KT / KSPLIT), ...), and the
+// groups' accumulators are added through LDS before group 0 runs the epilogue.  For
+// problems with few output tiles and a deep K this puts KSPLIT times as many waves on the
+// dependent chain of k tiles (a 3072-deep reduction on 64 x 64 tiles is 6 steps instead of
+// 24) without a second kernel or global atomics.
 // Requires K % 16 == 0 and 16-byte aligned, k-contiguous operands; the last k tile is
 // completed with zeros (chunks at k >= K are given an out-of-range offset).
 // CONV: the A operand is an NHWC image read in place as the im2col matrix (row m =
@@ -81,13 +87,14 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, unsigned lds_addr
 // s_waitcnt immediate for gfx9: vmcnt = n (6 bits, split), lgkmcnt = 0, expcnt = any
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4); }
 
-template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
-__global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParams p) {
+template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI>
+__global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const MainParams p) {
   // The inline assembly only assembles in the device compilation; the host pass
   // just needs the kernel's stub.
 #if defined(__HIP_DEVICE_COMPILE__)
   constexpr int BK = 128;
-  constexpr int NW = WM * WN;
+  constexpr int NW = WM * WN;               // waves of one k group
+  constexpr int NT = NW * KSPLIT * 64;      // threads of the workgroup
   constexpr int TM = BM / WM, TN = BN / WN;
   constexpr int FM = TM / 32, FN = TN / 32;
   constexpr int NKS = BK / 32;              // MFMA k-steps per tile (4)
@@ -103,18 +110,22 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   static_assert(LD <= 63, "vmcnt is a 6-bit counter");
   static_assert(NW % 2 == 0, "the chunk a lane loads must not depend on the load slot");
 
-  extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+  extern __shared__ __attribute__((aligned(1024))) int8_t smem_all[];
   DQ8_TRACE_POINT(0);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int kg = (tid >> 6) / NW;           // k group of this wave
+  const int wave = (tid >> 6) % NW;         // wave index inside the group
   const int wm = wave / WN, wn = wave % WN;
+  int8_t* smem = smem_all + kg * (2 * STAGE);
 
   int tm, tn;
   tile_coords(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  const int KT = (p.K + BK - 1) / BK;
+  const int KT_ALL = (p.K + BK - 1) / BK;
+  const int KT = (KT_ALL + KSPLIT - 1) / KSPLIT;   // k tiles per group
+  const int kt0 = kg * KT;                          // first k tile of this group
 
   // ---- buffer descriptors over the rows this block may touch (GEMM) or the whole
   // image (convolution)
@@ -126,7 +137,9 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   const int64_t w_valid = (int64_t)(p.N - n0 - 1) * p.ldw + p.K;
   const v4i a_rsrc = make_rsrc(a_base, a_valid < kMaxRecords ? a_valid : kMaxRecords);
   const v4i w_rsrc = make_rsrc(w_base, w_valid < kMaxRecords ? w_valid : kMaxRecords);
-  const unsigned lds_base = (unsigned)(size_t)(lds_void_t*)smem;
+  // wave-uniform (it depends on the wave's k group only): keep it in a scalar register
+  const unsigned lds_base =
+      (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(size_t)(lds_void_t*)smem);
 
   // ---- load slots.  Instruction i of this wave covers 8-row block q = wave + i*NW;
   // lane -> row r = lane/8 of the block, LDS slot s = lane%8, global k-chunk
@@ -166,9 +179,9 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   // tile_setup(kt) precedes the issue_load calls of tile kt.
   int t_koff = kOutOfRange, t_dh = 0, t_dw = 0, t_ci = 0;
   auto tile_setup = [&](int kt) {
-    const int k = kt * BK + kc;
+    const int k = (kt0 + kt) * BK + kc;
     const bool in = kt < KT && k < p.K;
-    t_koff = in ? kt * BK : kOutOfRange;
+    t_koff = in ? (kt0 + kt) * BK : kOutOfRange;
     if (CONV) {
       const unsigned tap = (unsigned)k / (unsigned)p.Ci;
       t_ci = k - (int)tap * p.Ci;
@@ -250,7 +263,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   tile_setup(0);
 #pragma unroll
   for (int idx = 0; idx < LD; ++idx) issue_load(idx, 0);
-  EarlyColParams<EPI, NW * 64, BN> early;
+  EarlyColParams<EPI, NT, BN> early;
   early.fetch(p.epi, n0);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   __syncthreads();
@@ -310,8 +323,38 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_pipe_kernel(const MainParam
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   DQ8_TRACE_POINT(2);
 
-  mfma_epilogue<EPI, FM, FN, NW * 64, BN>(acc, p.epi, smem, m0 + wm * TM, n0 + wn * TN, n0,
-                                          early.c);
+  if (KSPLIT > 1) {
+    // add the groups' partial sums: groups 1.. park their accumulators in LDS (lane-major,
+    // conflict free), group 0 collects them
+    constexpr int PER_WAVE = FM * FN * 16 * 64;   // ints
+    int* red = reinterpret_cast<int*>(smem_all);
+    __syncthreads();   // every group is done with its operand stages
+    if (kg > 0) {
+      int* mine = red + ((kg - 1) * NW + wave) * PER_WAVE + lane;
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) mine[((i * FN + j) * 16 + v) * 64] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (kg == 0) {
+#pragma unroll
+      for (int g = 1; g < KSPLIT; ++g) {
+        const int* theirs = red + ((g - 1) * NW + wave) * PER_WAVE + lane;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] += theirs[((i * FN + j) * 16 + v) * 64];
+      }
+    }
+  }
+
+  mfma_epilogue<EPI, FM, FN, NT, BN>(acc, p.epi, smem_all, m0 + wm * TM, n0 + wn * TN, n0,
+                                     early.c, wave, kg == 0);
   DQ8_TRACE_POINT(3);
 #else
   (void)p;
