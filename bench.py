@@ -400,6 +400,28 @@ def extras(torch, steps, warmup, which="all"):
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 5}
     del x, q, f
+    # smaller activations (they fit the 256 MB last-level cache; launches captured in a graph)
+    small = {}
+    for shape in ((16, 768), (1000, 768), (4096, 768), (16384, 768), (32, 56, 56, 64),
+                  (4096, 4096), (16384, 4096)):
+        n = 1
+        for d in shape:
+            n *= d
+        xs = torch.randn(shape, device="cuda")
+        qs = torch.empty(shape, dtype=torch.int8, device="cuda")
+        fs = torch.empty(shape, device="cuda")
+        cs = torch.full((shape[-1],), 0.05, device="cuda")
+        czs = torch.zeros(shape[-1], dtype=torch.int32, device="cuda")
+        ax = len(shape) - 1
+        row = {}
+        for name, fn in (("q_tensor", lambda: K.quantize(xs, s1, z1, out=qs)),
+                         ("dq_tensor", lambda: K.dequantize(qs, s1, z1, out=fs)),
+                         ("q_last_axis", lambda: K.quantize(xs, cs, czs, axis=ax, out=qs)),
+                         ("dq_last_axis", lambda: K.dequantize(qs, cs, czs, axis=ax, out=fs))):
+            t = time_graph(torch, [FnCall(fn)], launches=20, replays=5)
+            row[name] = {"us": round(t * 1e6, 2), "GB/s": round(5.0 * n / t / 1e9, 1)}
+        small["x".join(str(d) for d in shape)] = row
+    out["quantize_dequantize_shapes"] = small
     if which == "qdq":
         return out
     out["configs"] = config_reports(torch, K)

@@ -108,8 +108,9 @@ dequantize_tensor_v8(const uint2* __restrict__ q, float4* __restrict__ out,
 }
 
 // ------------------------------------------- per channel, channel = last axis
-// x: [rows, nch], nch % 4 == 0.  blockIdx.x tiles channels (4 per thread),
-// blockIdx.y tiles rows; each block walks rows_per_block rows.
+// x: [rows, nch], nch % 4 == 0.  threadIdx.x / blockIdx.x tile channels (4 per thread),
+// threadIdx.y / blockIdx.y tile rows: each block walks rows_per_block rows, blockDim.y at
+// a time (tensors with few channels put several rows side by side in one workgroup).
 template <int ROUND>
 __global__ void __launch_bounds__(kThreads)
 quantize_lastaxis_v4(const float4* __restrict__ x, uint32_t* __restrict__ out,
@@ -121,27 +122,25 @@ quantize_lastaxis_v4(const float4* __restrict__ x, uint32_t* __restrict__ out,
   const float4 s = scale[c4];
   const int4 zi = zp[c4];
   const float4 z = make_float4((float)zi.x, (float)zi.y, (float)zi.z, (float)zi.w);
-  int64_t r = (int64_t)blockIdx.y * rows_per_block;
-  const int64_t r_end = r + rows_per_block < rows ? r + rows_per_block : rows;
+  const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end = r_begin + rows_per_block < rows ? r_begin + rows_per_block : rows;
+  const int64_t step = blockDim.y;               // rows between two rows of this thread
+  const int64_t hop = step * nch4;               // the same in units
+  int64_t r = r_begin + threadIdx.y;
   const float4* px = x + r * nch4 + c4;
   uint32_t* po = out + r * nch4 + c4;
-  for (; r + 3 < r_end; r += 4, px += 4 * (int64_t)nch4, po += 4 * (int64_t)nch4) {
-    float4 v0 = px[0], v1 = px[nch4], v2 = px[2 * (int64_t)nch4],
-           v3 = px[3 * (int64_t)nch4];
-    po[0] = pack4(quant_one<ROUND>(v0.x, s.x, z.x, lo, hi), quant_one<ROUND>(v0.y, s.y, z.y, lo, hi),
-                  quant_one<ROUND>(v0.z, s.z, z.z, lo, hi), quant_one<ROUND>(v0.w, s.w, z.w, lo, hi));
-    po[nch4] = pack4(quant_one<ROUND>(v1.x, s.x, z.x, lo, hi), quant_one<ROUND>(v1.y, s.y, z.y, lo, hi),
-                     quant_one<ROUND>(v1.z, s.z, z.z, lo, hi), quant_one<ROUND>(v1.w, s.w, z.w, lo, hi));
-    po[2 * (int64_t)nch4] = pack4(quant_one<ROUND>(v2.x, s.x, z.x, lo, hi), quant_one<ROUND>(v2.y, s.y, z.y, lo, hi),
-                                  quant_one<ROUND>(v2.z, s.z, z.z, lo, hi), quant_one<ROUND>(v2.w, s.w, z.w, lo, hi));
-    po[3 * (int64_t)nch4] = pack4(quant_one<ROUND>(v3.x, s.x, z.x, lo, hi), quant_one<ROUND>(v3.y, s.y, z.y, lo, hi),
-                                  quant_one<ROUND>(v3.z, s.z, z.z, lo, hi), quant_one<ROUND>(v3.w, s.w, z.w, lo, hi));
+  auto one = [&](const float4& v) {
+    return pack4(quant_one<ROUND>(v.x, s.x, z.x, lo, hi), quant_one<ROUND>(v.y, s.y, z.y, lo, hi),
+                 quant_one<ROUND>(v.z, s.z, z.z, lo, hi), quant_one<ROUND>(v.w, s.w, z.w, lo, hi));
+  };
+  for (; r + 3 * step < r_end; r += 4 * step, px += 4 * hop, po += 4 * hop) {
+    const float4 v0 = px[0], v1 = px[hop], v2 = px[2 * hop], v3 = px[3 * hop];
+    po[0] = one(v0);
+    po[hop] = one(v1);
+    po[2 * hop] = one(v2);
+    po[3 * hop] = one(v3);
   }
-  for (; r < r_end; ++r, px += nch4, po += nch4) {
-    float4 v = px[0];
-    po[0] = pack4(quant_one<ROUND>(v.x, s.x, z.x, lo, hi), quant_one<ROUND>(v.y, s.y, z.y, lo, hi),
-                  quant_one<ROUND>(v.z, s.z, z.z, lo, hi), quant_one<ROUND>(v.w, s.w, z.w, lo, hi));
-  }
+  for (; r < r_end; r += step, px += hop, po += hop) po[0] = one(px[0]);
 }
 
 template <bool SIGNED>
@@ -154,19 +153,21 @@ dequantize_lastaxis_v4(const uint32_t* __restrict__ q, float4* __restrict__ out,
   if (c4 >= nch4) return;
   const float4 s = scale[c4];
   const int4 z = zp[c4];
-  int64_t r = (int64_t)blockIdx.y * rows_per_block;
-  const int64_t r_end = r + rows_per_block < rows ? r + rows_per_block : rows;
+  const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end = r_begin + rows_per_block < rows ? r_begin + rows_per_block : rows;
+  const int64_t step = blockDim.y;
+  const int64_t hop = step * nch4;
+  int64_t r = r_begin + threadIdx.y;
   const uint32_t* pq = q + r * nch4 + c4;
   float4* po = out + r * nch4 + c4;
-  for (; r + 3 < r_end; r += 4, pq += 4 * (int64_t)nch4, po += 4 * (int64_t)nch4) {
-    const uint32_t w0 = pq[0], w1 = pq[nch4], w2 = pq[2 * (int64_t)nch4],
-                   w3 = pq[3 * (int64_t)nch4];
+  for (; r + 3 * step < r_end; r += 4 * step, pq += 4 * hop, po += 4 * hop) {
+    const uint32_t w0 = pq[0], w1 = pq[hop], w2 = pq[2 * hop], w3 = pq[3 * hop];
     po[0] = dequant_word4<SIGNED>(w0, z, s);
-    po[nch4] = dequant_word4<SIGNED>(w1, z, s);
-    po[2 * (int64_t)nch4] = dequant_word4<SIGNED>(w2, z, s);
-    po[3 * (int64_t)nch4] = dequant_word4<SIGNED>(w3, z, s);
+    po[hop] = dequant_word4<SIGNED>(w1, z, s);
+    po[2 * hop] = dequant_word4<SIGNED>(w2, z, s);
+    po[3 * hop] = dequant_word4<SIGNED>(w3, z, s);
   }
-  for (; r < r_end; ++r, pq += nch4, po += nch4) po[0] = dequant_word4<SIGNED>(pq[0], z, s);
+  for (; r < r_end; r += step, pq += hop, po += hop) po[0] = dequant_word4<SIGNED>(pq[0], z, s);
 }
 
 // ------------------------------------- per channel, inner % 4 == 0 (any axis)
@@ -259,15 +260,23 @@ int grid_for(int64_t work_items, int per_thread) {
 // along rows; about 64 Ki workgroups (a sweep, as for the per-tensor kernels) of at
 // least 4 rows each so the per-channel parameters in registers are reused.
 struct LastAxisPlan {
-  int bx, gx, gy, rows_per_block;
+  int bx, by, gx, gy, rows_per_block;
 };
 LastAxisPlan plan_last_axis(int64_t rows, int units) {
   LastAxisPlan p;
-  p.bx = units >= kThreads ? kThreads : (int)(dq8::ceil_div(units, 64) * 64);
+  if (units >= kThreads) {
+    p.bx = kThreads;
+  } else {   // few channels: the next power of two, the rest of the workgroup goes to rows
+    p.bx = 1;
+    while (p.bx < units) p.bx *= 2;
+  }
+  p.by = kThreads / p.bx;
   p.gx = (int)dq8::ceil_div(units, p.bx);
+  // each thread walks at least four of its rows; rows_per_block is a multiple of by
   int64_t rpb = dq8::ceil_div(rows * p.gx, 65536);
-  if (rpb < 4) rpb = 4;
-  if (dq8::ceil_div(rows, rpb) > 65535) rpb = dq8::ceil_div(rows, 65535);
+  if (rpb < 4 * p.by) rpb = 4 * p.by;
+  rpb = dq8::ceil_div(rpb, p.by) * p.by;
+  if (dq8::ceil_div(rows, rpb) > 65535) rpb = dq8::ceil_div(dq8::ceil_div(rows, 65535), p.by) * p.by;
   p.rows_per_block = (int)rpb;
   p.gy = (int)dq8::ceil_div(rows, rpb);
   return p;
@@ -331,7 +340,7 @@ extern "C" int dq8_quantize(const float* x, void* out, int out_kind,
              dq8::aligned(scale, 16) && dq8::aligned(zp, 16)) {
     const int nch4 = (int)(nch / 4);
     const LastAxisPlan lp = plan_last_axis(outer, nch4);
-    LAUNCH_RND(quantize_lastaxis_v4, dim3(lp.gx, lp.gy), dim3(lp.bx), (const float4*)x,
+    LAUNCH_RND(quantize_lastaxis_v4, dim3(lp.gx, lp.gy), dim3(lp.bx, lp.by), (const float4*)x,
                (uint32_t*)out, outer, nch4, lp.rows_per_block, (const float4*)scale,
                (const int4*)zp, lo, hi);
   } else if (vec_ok && inner % 4 == 0 && outer * nch < (1LL << 31)) {
@@ -389,7 +398,7 @@ extern "C" int dq8_dequantize(const void* q, int in_kind, float* out,
     const int nch4 = (int)(nch / 4);
     const LastAxisPlan lp = plan_last_axis(outer, nch4);
     auto k = is_signed ? dequantize_lastaxis_v4<true> : dequantize_lastaxis_v4<false>;
-    hipLaunchKernelGGL(k, dim3(lp.gx, lp.gy), dim3(lp.bx), 0, st, (const uint32_t*)q,
+    hipLaunchKernelGGL(k, dim3(lp.gx, lp.gy), dim3(lp.bx, lp.by), 0, st, (const uint32_t*)q,
                        (float4*)out, outer, nch4, lp.rows_per_block, (const float4*)scale,
                        (const int4*)zp);
   } else if (vec_ok && inner % 4 == 0 && outer * nch < (1LL << 31)) {
