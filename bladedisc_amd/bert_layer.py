@@ -80,9 +80,11 @@ class QuantBertLayer:
         self.fb = {"qkv": merged_b, "out": w["bo"], "ffn1": w["b1"], "ffn2": w["b2"]}
         self.w_q, self.sw, self.bias = {}, {}, {}
         for name in LINEARS:
-            sw = cfg.sym_scale(self.fw[name], axis=0)
-            self.w_q[name] = d(cfg.quantize_host(self.fw[name], sw, axis=0))
-            self.sw[name] = d(sw)
+            # per-output-channel symmetric weight scales; the weights are quantized by
+            # the same GPU kernel that serves mhlo_disc.quantize
+            self.sw[name] = d(cfg.sym_scale(self.fw[name], axis=0))
+            zeros = torch.zeros(self.sw[name].numel(), dtype=torch.int32, device=device)
+            self.w_q[name] = K.quantize(d(self.fw[name]), self.sw[name], zeros, axis=0)
             self.bias[name] = d(self.fb[name])
         self.s_in, self.s_out = {}, {}
 
