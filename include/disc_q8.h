@@ -94,8 +94,10 @@ size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
  *      [K,N] row stride ldw (tp_b = 0, the CPU callers' layout).
  *   out: device, element type per `epilogue`, row stride ldo (elements).
  *   sx / sw / so: device f32 with n_sx / n_sw / n_so entries, each 1 or N.
- *   zo: output zero point (REQUANT_CPU only).  Input and weight zero points must
- *      be 0 (every reference caller is symmetric); non-zero is rejected.
+ *   zx / zw: input and weight zero points, acc = sum (A - zx) * (W - zw).  Every
+ *      reference caller is symmetric (0); non-zero values are computed by the generic
+ *      scalar kernel, not the MFMA kernels.
+ *   zo: output zero point (REQUANT_CPU only).
  *   workspace: device scratch of at least dq8_qgemm_workspace_bytes(), may be
  *      NULL when that is 0.
  * M == 0, N == 0 launch nothing and succeed; K == 0 yields epilogue(0). */
@@ -108,7 +110,9 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
 
 /* Same, forcing one kernel variant (for tests and tuning):
  *  -1 heuristic, 0 generic scalar kernel, 1.. MFMA tile configurations
- *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()). */
+ *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()).  A problem
+ *  an MFMA variant cannot take (K % 16 != 0, unaligned rows, zero points) runs on the
+ *  generic kernel whatever the variant. */
 int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                       const int8_t* W, int64_t ldw, void* out, int64_t ldo,
                       int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
