@@ -111,8 +111,8 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
 /* Same, forcing one kernel variant (for tests and tuning):
  *  -1 heuristic, 0 generic scalar kernel, 1.. MFMA tile configurations
  *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()).  A problem
- *  an MFMA variant cannot take (K % 16 != 0, unaligned rows, zero points) runs on the
- *  generic kernel whatever the variant. */
+ *  an MFMA variant cannot take (K % 16 != 0, unaligned rows) runs on the generic
+ *  kernel whatever the variant; non-zero zx / zw with a forced MFMA variant is an error. */
 int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                       const int8_t* W, int64_t ldw, void* out, int64_t ldo,
                       int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
