@@ -360,6 +360,55 @@ def test_qgemm_strided_rows_all_variants(K, m, n, k, pad):
         assert (got[:, n:] == 77).all(), "variant %d wrote past the row" % v
 
 
+def test_qgemm_random_shapes_epilogues_variants(K):
+    """Seeded sweep over ragged shapes, every epilogue / bias kind and every kernel
+    variant (heuristic included), bit-exact against the oracle."""
+    rng = np.random.default_rng(20240611)
+    nvar = len(K.variant_names())
+    for case in range(80):
+        m = int(rng.choice([1, 2, 7, 16, 31, 33, 64, 100, 129, 255, 300, 513, 1000]))
+        n = int(rng.choice([1, 3, 16, 17, 48, 64, 65, 130, 256, 300, 768]))
+        k = int(rng.choice([16, 32, 48, 64, 112, 128, 144, 256, 400, 768, 1040]))
+        a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+        w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        acc, _ = O.gemm_s32_fast(a, w)
+        sx, sw = make_scales(rng, n, per_channel=bool(rng.integers(0, 2)))
+        so = pick_so(acc, sx, np.broadcast_to(sw, (n,)))
+        v = int(rng.integers(-1, nvar))
+        epi = int(rng.integers(0, 4))
+        tag = "case %d: %dx%dx%d variant %d epilogue %d" % (case, m, n, k, v, epi)
+        da, dw = dev(a), dev(w)
+        dsx, dsw, dso = dev(np.array([sx])), dev(sw), dev(np.array([so]))
+        if epi == 0:
+            got = host(K.qgemm(da, dw, K.EPI_ACC_S32, variant=v))
+            np.testing.assert_array_equal(got, acc, err_msg=tag)
+        elif epi == 1:
+            kind = int(rng.integers(0, 3))
+            bias = [None, rng.integers(-5000, 5000, n).astype(np.int32),
+                    rng.standard_normal(n).astype(np.float32)][kind]
+            b32 = bias if kind != 2 else O.bias_f32_to_s32(bias, float(sx), np.broadcast_to(sw, (n,)))
+            zo = int(rng.integers(-5, 6))
+            want = O.requant_cpu(acc, float(sx), sw, float(so), b32=b32, zo=zo)
+            got = host(K.qgemm(da, dw, K.EPI_REQUANT_CPU, sx=dsx, sw=dsw, so=dso,
+                               bias=None if bias is None else dev(bias), zo=zo, variant=v))
+            np.testing.assert_array_equal(got, want, err_msg=tag)
+        elif epi == 2:
+            kind = int(rng.integers(0, 3))
+            bias = [None, rng.standard_normal(n).astype(np.float32) * 5,
+                    rng.integers(-128, 128, n, dtype=np.int8)][kind]
+            want = O.requant_gpu(acc, sx, sw, so, bias_f32=bias if kind == 1 else None,
+                                 bias_i8=bias if kind == 2 else None)
+            got = host(K.qgemm(da, dw, K.EPI_REQUANT_GPU, sx=dsx, sw=dsw, so=dso,
+                               bias=None if bias is None else dev(bias), variant=v))
+            np.testing.assert_array_equal(got, want, err_msg=tag)
+        else:
+            bias = rng.standard_normal(n).astype(np.float32) if rng.integers(0, 2) else None
+            want = O.dequant_acc(acc, float(sx), sw, bias=bias)
+            got = host(K.qgemm(da, dw, K.EPI_DEQUANT_F32, sx=dsx, sw=dsw,
+                               bias=None if bias is None else dev(bias), variant=v))
+            np.testing.assert_array_equal(got, want, err_msg=tag)
+
+
 def test_requant_nan_and_inf_scales_saturate_like_the_oracle(K):
     """A NaN or infinite per-channel factor: NaN results go to -128, infinities
     saturate by sign, on every kernel family and both requant epilogues."""
