@@ -28,3 +28,16 @@ def test_variant_table_and_version():
     from bladedisc_amd import kernels
     names = kernels.variant_names()
     assert names[0] == "generic" and len(names) >= 4
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No CPU fallback: without the built library every operator raises."""
+    import pytest
+    from bladedisc_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libdisc_q8_ral.so"))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.lib()
+    from bladedisc_amd import kernels
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        kernels.variant_names()
