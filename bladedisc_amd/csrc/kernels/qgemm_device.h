@@ -501,6 +501,55 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     return;
   }
 
+  if (!kInt8Out && e.vec_store) {
+    // int32 / f32 results: one 32 x 32 fragment (4 KiB) at a time through a per-wave LDS
+    // tile, 128-byte rows with the 16-byte chunks swizzled by the row, then out as full
+    // 128-byte row segments (8 lanes per row) instead of 32-byte pieces of 32 rows.
+    int8_t* stage = smem + CP_BYTES + wave * 4096;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int r = lane & 31;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
+          const int chunk = 2 * g + (lane >> 5);
+          v4i w;
+          if (EPI == DQ8_EPI_ACC_S32) {
+            w = (v4i){acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2],
+                      acc[i][j][4 * g + 3]};
+          } else {
+            const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
+            const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
+            const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              w[q] = __float_as_int(dequant_one(e, c[q], acc[i][j][4 * g + q]));
+          }
+          *reinterpret_cast<v4i*>(stage + r * 128 + ((chunk ^ (r & 7)) << 4)) = w;
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int row = it * 8 + (lane >> 3), chunk = lane & 7;
+          const v4i v = *reinterpret_cast<const v4i*>(stage + row * 128 + ((chunk ^ (row & 7)) << 4));
+          const int m = m_wave0 + i * 32 + row, n = n_wave0 + j * 32 + chunk * 4;
+          if (m < e.M && n < e.N) {
+            int32_t* dst = static_cast<int32_t*>(e.out) + (int64_t)m * e.ldo + n;
+            if (n + 3 < e.N) {
+              __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
+            } else {
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                if (n + q < e.N) dst[q] = v[q];
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
+
   // direct stores: 4 consecutive channels of one row per accumulator quad
 #pragma unroll
   for (int j = 0; j < FN; ++j) {
