@@ -9,6 +9,7 @@
 #include "qgemm_device.h"
 #include "qgemm_pipelined.h"
 #include "qgemm_skinny.h"
+#include "qconv_direct.h"
 
 #pragma clang fp contract(off)
 
@@ -167,10 +168,14 @@ const Variant kVariants[] = {
     {"pipe_64x64x128_k2", 64, 64, 128, 512},
     // small-M kernel: 16 output channels per workgroup, K split over the waves (GEMM only)
     {"skinny_16", 16, 16, 64, 512},
+    // 3x3 stride-1 convolution with the input patch resident in LDS (convolution only)
+    {"direct3x3_256x64", 256, 64, 128, 256},
+    {"direct3x3_128x64", 128, 64, 128, 256},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
 constexpr int kSkinnyVariant = 9;
+constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct variants
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -288,6 +293,19 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe) {
   for (int v = 1; v <= 3; ++v)
     if (tiles(v) >= kCus - kCus / 8) return v;
   return 3;
+}
+
+// Whether a 3x3 stride-1 convolution goes to the kernel that keeps the input patch in LDS
+// (and with which tile), or to the implicit GEMM.  Measured on ResNet / VGG shaped layers
+// with batch 1 .. 128: with at most 64 input and output channels the implicit GEMM is bound
+// by its operand loads (each input pixel is fetched nine times) and the direct kernel wins
+// by 12-30 % once its 256-pixel tiles fill the chip; with more channels the implicit GEMM's
+// larger tiles are as fast or faster.  Returns the configuration or -1.
+int pick_direct_conv(int64_t images, int64_t pixels_per_image, int64_t Ci, int64_t Co) {
+  if (Ci > 64 || Co > 64) return -1;
+  int bm, bn;
+  direct_conv_tile(0, &bm, &bn);
+  return images * ceil_div(pixels_per_image, bm) * ceil_div(Co, bn) >= 256 ? 0 : -1;
 }
 
 int elem_size(int epilogue) {
@@ -628,7 +646,28 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   p.sh = sh; p.sw_ = sw_; p.dh = dh; p.dw = dw;
   p.conv_bytes = NB * H * Wd * Ci;
   p.epi = e;
-  if (auto_pick) variant = pick_variant(Mg, Co, Kg, pipe_ok(256, 256, p, true));
+
+  DirectConvParams d = {};
+  d.in = in;
+  d.w = w;
+  d.NB = (int)NB; d.H = (int)H; d.Wd = (int)Wd; d.Ci = (int)Ci; d.Co = (int)Co;
+  d.Ho = (int)Ho; d.Wo = (int)Wo;
+  d.pad_t = padding[0]; d.pad_l = padding[2];
+  d.epi = e;
+  const bool direct_shape = Kh == 3 && Kw == 3 && sh == 1 && sw_ == 1 && dh == 1 && dw == 1;
+  if (variant >= kDirectConv0) {
+    DQ8_REQUIRE(direct_shape && direct_conv_plan(variant - kDirectConv0, &d),
+                "dq8_qconv2d: the direct variants need a 3x3 filter with stride and dilation "
+                "1, Ci in {32, 64, 128, 256} and a patch that fits the LDS");
+    return launch_direct_conv(variant - kDirectConv0, epilogue, d, st);
+  }
+  if (auto_pick) {
+    if (direct_shape) {
+      const int c = pick_direct_conv(NB, Ho * Wo, Ci, Co);
+      if (c >= 0 && direct_conv_plan(c, &d)) return launch_direct_conv(c, epilogue, d, st);
+    }
+    variant = pick_variant(Mg, Co, Kg, pipe_ok(256, 256, p, true));
+  }
   return launch_epi<true>(variant, p, epilogue, st);
 }
 

@@ -241,7 +241,8 @@ template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
                                               int n_blk0, const ColParams* early = nullptr,
-                                              int wave_slot = -1, bool active = true);
+                                              int wave_slot = -1, bool active = true,
+                                              int m_limit = -1);
 
 // The per-channel factors of the channels thread t is responsible for in the epilogue
 // (t, t + NT, ...), fetched at the start of a kernel so that the cold loads of scales
@@ -253,6 +254,9 @@ struct EarlyColParams {
   __device__ __forceinline__ void fetch(const EpiParams& e, int n_blk0) {
 #pragma unroll
     for (int i = 0; i < kPerThread; ++i) {
+      // (a wave whose channels all lie past the block's BN has nothing to fetch)
+      c[i] = ColParams{0.f, 0.f};
+      if ((int)(threadIdx.x & ~63u) + i * NT >= BN) continue;
       const int n = n_blk0 + (int)threadIdx.x + i * NT;
       c[i] = col_params<EPI>(e, n < e.N ? n : e.N - 1);
     }
@@ -427,9 +431,11 @@ template <int EPI, int FM, int FN, int NT, int BN>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
                                               int n_blk0, const ColParams* early,
-                                              int wave_slot, bool active) {
+                                              int wave_slot, bool active, int m_limit) {
   // `wave_slot`: which per-wave staging tile this wave uses (default: its index in the
-  // workgroup); waves with `active` false only take part in the barriers.
+  // workgroup); waves with `active` false only take part in the barriers; rows at or
+  // past `m_limit` (default: M) are not stored.
+  const int m_end = m_limit >= 0 ? m_limit : e.M;
   constexpr int TM = FM * 32, TN = FN * 32;
   constexpr int CH = TN / 16;                 // 16-byte chunks per staged row
   constexpr int CP_BYTES = BN * 8;            // per-channel (scale, addend) pairs
@@ -487,7 +493,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
       const int chunk = lane % CH;
       const v4i v = *reinterpret_cast<const v4i*>(stage + row * TN + ((chunk ^ (row & (CH - 1))) << 4));
       const int m = m_wave0 + row, n = n_wave0 + chunk * 16;
-      if (m < e.M && n < e.N) {
+      if (m < m_end && n < e.N) {
         int8_t* dst = out + (int64_t)m * e.ldo + n;
         if (n + 15 < e.N) {
           __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
@@ -534,7 +540,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
           const int row = it * 8 + (lane >> 3), chunk = lane & 7;
           const v4i v = *reinterpret_cast<const v4i*>(stage + row * 128 + ((chunk ^ (row & 7)) << 4));
           const int m = m_wave0 + i * 32 + row, n = n_wave0 + j * 32 + chunk * 4;
-          if (m < e.M && n < e.N) {
+          if (m < m_end && n < e.N) {
             int32_t* dst = static_cast<int32_t*>(e.out) + (int64_t)m * e.ldo + n;
             if (n + 3 < e.N) {
               __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
@@ -564,7 +570,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
         const int m = m_wave0 + i * 32 + (lane & 31);
-        if (m < e.M)
+        if (m < m_end)
           store_group4<EPI>(e, m, n, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
                             acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
       }

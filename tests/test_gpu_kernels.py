@@ -27,7 +27,7 @@ def host(t):
 def gemm_variants(K, k):
     """All variant ids.  (With a contraction length that is not a multiple of 16 the MFMA
     variants hand the problem to the generic kernel.)"""
-    return list(range(len(K.variant_names())))
+    return [i for i, nm in enumerate(K.variant_names()) if not nm.startswith("direct3x3_")]
 
 
 def make_scales(rng, n, per_channel=True):
@@ -280,6 +280,13 @@ CONVS = [  # nb, h, w, ci, co, k, stride, pad, dil
     (2, 6, 6, 5, 6, 3, 1, 1, 1),      # Ci % 16 != 0 -> generic kernel
     (4, 28, 28, 64, 64, 3, 1, 1, 1),  # K = 576: a partial last k tile, several tiles of rows
     (2, 15, 13, 48, 80, 3, 2, 1, 2),  # ragged everything, K = 432
+    # the direct 3x3 kernels: every channel count they take, images of one tile and of
+    # several with a ragged last one, ragged Co, no / one / two pixels of padding
+    (3, 20, 18, 32, 40, 3, 1, 1, 1),
+    (2, 30, 30, 128, 136, 3, 1, 1, 1),
+    (2, 12, 10, 256, 64, 3, 1, 0, 1),
+    (1, 33, 17, 64, 200, 3, 1, 2, 1),
+    (1, 36, 36, 256, 64, 3, 1, 1, 1),  # a patch of 107 KiB: LDS addresses beyond 128 KiB
 ]
 
 
@@ -297,6 +304,8 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
     names = K.variant_names()
     variants = [-1, 0] + ([i for i, nm in enumerate(names) if nm.startswith(("mfma_", "pipe_"))]
                           if ci % 16 == 0 else [])
+    if k == 3 and stride == 1 and dil == 1 and ci in (32, 64, 128, 256):
+        variants += [i for i, nm in enumerate(names) if nm.startswith("direct3x3_")]
     for v in variants:
         got = host(K.qconv2d(dev(x), dev(wt), padding, md, out_shape, K.EPI_ACC_S32, variant=v))
         np.testing.assert_array_equal(got, acc, err_msg="variant %d" % v)
@@ -307,6 +316,35 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
         got = host(K.qconv2d(dev(x), dev(wt), padding, md, out_shape, K.EPI_REQUANT_CPU,
                              sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])), variant=v))
         np.testing.assert_array_equal(got, want, err_msg="variant %d" % v)
+
+
+def test_qconv_direct_variants_refuse_what_they_cannot_run(K):
+    """A named direct-convolution variant fails with an error, not a wrong result, on a
+    filter that is not 3x3 stride 1, on a channel count it has no layout for, and on an image
+    row too wide for its patch to fit the LDS; the automatic choice runs all of them."""
+    names = K.variant_names()
+    direct = [i for i, nm in enumerate(names) if nm.startswith("direct3x3_")]
+    assert direct
+    rng = np.random.default_rng(5)
+    cases = [  # nb, h, w, ci, co, k, stride
+        (1, 8, 8, 64, 64, 1, 1),
+        (1, 9, 9, 64, 64, 3, 2),
+        (1, 8, 8, 48, 64, 3, 1),
+        (1, 4, 300, 256, 64, 3, 1),
+    ]
+    for nb, h, w_, ci, co, k, stride in cases:
+        pad = k // 2
+        x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8)
+        ho = (h + 2 * pad - k) // stride + 1
+        wo = (w_ + 2 * pad - k) // stride + 1
+        md = list(O.NHWC_OHWI_METADATA) + [stride, stride, 1, 1, 1]
+        out_shape = [nb, ho, wo, co]
+        for v in direct:
+            with pytest.raises(RuntimeError, match="direct variants"):
+                K.qconv2d(dev(x), dev(wt), [pad] * 4, md, out_shape, K.EPI_ACC_S32, variant=v)
+        got = host(K.qconv2d(dev(x), dev(wt), [pad] * 4, md, out_shape, K.EPI_ACC_S32))
+        np.testing.assert_array_equal(got, O.conv_s32(x, wt, [pad] * 4, md, out_shape))
 
 
 def test_qconv_nchw_oihw_generic(K):
@@ -364,7 +402,7 @@ def test_qgemm_random_shapes_epilogues_variants(K):
     """Seeded sweep over ragged shapes, every epilogue / bias kind and every kernel
     variant (heuristic included), bit-exact against the oracle."""
     rng = np.random.default_rng(20240611)
-    nvar = len(K.variant_names())
+    nvar = len(gemm_variants(K, 16))     # ids 0 .. nvar-1: the GEMM kernels
     for case in range(80):
         m = int(rng.choice([1, 2, 7, 16, 31, 33, 64, 100, 129, 255, 300, 513, 1000]))
         n = int(rng.choice([1, 3, 16, 17, 48, 64, 65, 130, 256, 300, 768]))
