@@ -104,7 +104,6 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   constexpr int A_LD = (BM / 8) / NW;
   constexpr int B_LD = (BN / 8) / NW;
   constexpr int LD = A_LD + B_LD;           // load instructions per tile per wave
-  constexpr int ROWS = NKS * FM;            // rows of FN MFMAs per tile
   static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile does not split over the waves");
   static_assert(FM >= 1 && FN >= 1 && FN <= FM, "fragment mismatch");
   static_assert(LD <= 63, "vmcnt is a 6-bit counter");
