@@ -93,12 +93,12 @@ void run(int NB, int H, int Ci, int Co) {
     printf("   %-16s %6.2f %6.2f %6.2f\n", names[i], v.front(), v[grid / 2], v.back());
   }
   printf("  us a workgroup spends in each stage (min / median / max):\n");
-  const char* stages[3] = {"entry -> patch", "k loop", "requant + store"};
+  const char* stage_names[3] = {"entry -> patch", "k loop", "requant + store"};
   for (int i = 1; i < 4; ++i) {
     std::vector<double> v;
     for (int b = 0; b < grid; ++b) v.push_back((t[4 * b + i] - t[4 * b + i - 1]) / 100.0);
     std::sort(v.begin(), v.end());
-    printf("   %-16s %6.2f %6.2f %6.2f\n", stages[i - 1], v.front(), v[grid / 2], v.back());
+    printf("   %-16s %6.2f %6.2f %6.2f\n", stage_names[i - 1], v.front(), v[grid / 2], v.back());
   }
   CK(hipFree(in)); CK(hipFree(w)); CK(hipFree(out));
   CK(hipFree(sx)); CK(hipFree(sw)); CK(hipFree(so)); CK(hipFree(bias));

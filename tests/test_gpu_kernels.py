@@ -287,6 +287,7 @@ CONVS = [  # nb, h, w, ci, co, k, stride, pad, dil
     (2, 12, 10, 256, 64, 3, 1, 0, 1),
     (1, 33, 17, 64, 200, 3, 1, 2, 1),
     (1, 36, 36, 256, 64, 3, 1, 1, 1),  # a patch of 107 KiB: LDS addresses beyond 128 KiB
+    (1, 6, 150, 64, 64, 3, 1, 1, 1),   # a wide image: tiles of 256 pixels span 2-3 rows
 ]
 
 
