@@ -171,11 +171,14 @@ const Variant kVariants[] = {
     // 3x3 stride-1 convolution with the input patch resident in LDS (convolution only)
     {"direct3x3_256x64", 256, 64, 128, 256},
     {"direct3x3_128x64", 128, 64, 128, 256},
+    // 256x256 tile on eight waves (two per SIMD), wave tile 128x64
+    {"pipe_256x256x128_w8", 256, 256, 128, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
 constexpr int kSkinnyVariant = 9;
 constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct variants
+constexpr int kPipe256w8 = 12;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -255,6 +258,7 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case kPipe64: return launch_pipe<64, 64, 2, 2, 1, CONV, EPI>(p, st);
     case kPipe256x64: return launch_pipe<256, 64, 4, 1, 1, CONV, EPI>(p, st);
     case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, CONV, EPI>(p, st);
+    case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, CONV, EPI>(p, st);
   }
   if constexpr (!CONV) {
     if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
@@ -274,18 +278,25 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 }
 
 // Picks the kernel from the dynamic problem size.  `pipe` says whether the pipelined
-// kernels can take the operands.  Measured on BERT-shaped and square problems: the
-// 256x256 tile pays once it fills the chip (>= ~240 tiles), the 128x128 tile from about
-// 120 tiles on, below that the 64x64 tile spreads the weight stream over more CUs; narrow
-// outputs (N <= 64) take the 256x64 tile.  With 64x64 tiles a CU's operand loads, not its
-// MFMAs, set the pace (16 KiB per 128 of k against 128 MFMA cycles per SIMD); when few
-// CUs are busy and K is deep, splitting K over two wave groups of the workgroup still
-// shortens the chain of dependent k tiles (about 10 % at K = 3072).
+// kernels can take the operands.  Measured on BERT-shaped and square problems (M 256 ..
+// 16384, N 768 .. 4096, K 768 .. 4096):
+//  * the 256x256 tile runs on eight waves (two per SIMD, wave tile 128x64): against four
+//    waves of 128x128 the epilogue's chain of VALU instructions per wave halves (5.7 -> 3.1
+//    us) and a wave's LDS waits are covered by its neighbour, 3 % at 4096^3 and 10-25 % at
+//    K = 768; it pays once its tiles fill about 55 % of the CUs and, past one round of 256
+//    tiles, when the last round is not mostly empty (288 tiles = 2 rounds lose to 128x128);
+//  * the 128x128 tile from about 120 tiles on, below that the 64x64 tile spreads the weight
+//    stream over more CUs; narrow outputs (N <= 64) take the 256x64 tile.  With 64x64 tiles a
+//    CU's operand loads, not its MFMAs, set the pace (16 KiB per 128 of k against 128 MFMA
+//    cycles per SIMD); when few CUs are busy and K is deep, splitting K over two wave groups
+//    of the workgroup still shortens the chain of dependent k tiles (about 10 % at K = 3072).
 int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe) {
   auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
   if (pipe) {
     if (N <= 64 && M >= 256 * 64) return kPipe256x64;
-    if (tiles(kPipe256) >= 240) return kPipe256;
+    const int64_t t256 = tiles(kPipe256w8);
+    const int64_t rounds = ceil_div(t256, 256);
+    if (t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * 256 * rounds)) return kPipe256w8;
     if (tiles(kPipe128) >= 120) return kPipe128;
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
@@ -655,7 +666,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   d.pad_t = padding[0]; d.pad_l = padding[2];
   d.epi = e;
   const bool direct_shape = Kh == 3 && Kw == 3 && sh == 1 && sw_ == 1 && dh == 1 && dw == 1;
-  if (variant >= kDirectConv0) {
+  if (variant >= kDirectConv0 && variant < kDirectConv0 + kNumDirectConvConfigs) {
     DQ8_REQUIRE(direct_shape && direct_conv_plan(variant - kDirectConv0, &d),
                 "dq8_qconv2d: the direct variants need a 3x3 filter with stride and dilation "
                 "1, Ci in {32, 64, 128, 256} and a patch that fits the LDS");

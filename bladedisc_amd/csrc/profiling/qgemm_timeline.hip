@@ -2,8 +2,8 @@
 // first k tile land, finish the main loop and finish storing?  A standalone profiling
 // program (not part of the library): it instantiates the kernel from the library's own
 // header with the DQ8_TRACE_POINT hook defined, launches it on M = N = 4096 with three
-// depths of K, and prints the stage times over all workgroups next to the hipEvent time
-// of the launch.
+// depths of K, once with four and once with eight waves per workgroup, and prints the
+// stage times over all workgroups next to the hipEvent time of the launch.
 //
 // Build and run (bladedisc_amd/build.py: build_profiling_tools()):
 //   hipcc -O3 -std=c++17 --offload-arch=gfx950 -ffp-contract=off \
@@ -21,9 +21,13 @@ __device__ long long g_trace[4 * 4096];
 #include "qgemm_pipelined.h"
 #define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e)); exit(1);} } while (0)
 using namespace dq8;
-int main(int argc, char** argv) {
+// WM x WN waves on the 256x256 tile: 2 x 2 (one wave per SIMD, wave tile 128x128) or 2 x 4
+// (two per SIMD, wave tile 128x64)
+template <int WM, int WN>
+void run() {
   const int M = 4096, N = 4096;
-  for (int K : {128, 1024, 4096}) {
+  printf("---- %d waves per workgroup\n", WM * WN);
+  for (int K : {128, 768, 4096}) {
     int8_t *A, *W, *out; float *sx, *sw, *so, *bias;
     CK(hipMalloc(&A, (size_t)M * K)); CK(hipMalloc(&W, (size_t)N * K)); CK(hipMalloc(&out, (size_t)M * N));
     CK(hipMalloc(&sx, 4)); CK(hipMalloc(&sw, 4 * N)); CK(hipMalloc(&so, 4)); CK(hipMalloc(&bias, 4 * N));
@@ -36,13 +40,13 @@ int main(int argc, char** argv) {
     p.epi.out = out; p.epi.ldo = N; p.epi.M = M; p.epi.N = N; p.epi.bias = bias; p.epi.bias_kind = DQ8_BIAS_F32;
     p.epi.sx = sx; p.epi.sw = sw; p.epi.so = so; p.epi.sx_stride = 0; p.epi.sw_stride = 1; p.epi.so_stride = 0; p.epi.zo = 0;
     p.epi.vec_store = 1; p.epi.vec_store16 = 1;
-    auto kern = qgemm_pipe_kernel<256, 256, 2, 2, 1, false, DQ8_EPI_REQUANT_GPU>;
+    auto kern = qgemm_pipe_kernel<256, 256, WM, WN, 1, false, DQ8_EPI_REQUANT_GPU>;
     CK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 131072));
     hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
-    for (int r = 0; r < 3; ++r) hipLaunchKernelGGL(kern, dim3(256), dim3(256), 131072, 0, p);
+    for (int r = 0; r < 3; ++r) hipLaunchKernelGGL(kern, dim3(256), dim3(WM * WN * 64), 131072, 0, p);
     CK(hipDeviceSynchronize());
     CK(hipEventRecord(e0));
-    hipLaunchKernelGGL(kern, dim3(256), dim3(256), 131072, 0, p);
+    hipLaunchKernelGGL(kern, dim3(256), dim3(WM * WN * 64), 131072, 0, p);
     CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
     float ms; CK(hipEventElapsedTime(&ms, e0, e1));
     std::vector<long long> t(4 * 256);
@@ -59,5 +63,10 @@ int main(int argc, char** argv) {
     for (int i = 0; i < 4; ++i) printf("   %-16s %6.2f %6.2f %6.2f\n", names[i], st[i][0], st[i][1], st[i][2]);
     CK(hipFree(A)); CK(hipFree(W)); CK(hipFree(out));
   }
+}
+
+int main() {
+  run<2, 2>();
+  run<2, 4>();
   return 0;
 }

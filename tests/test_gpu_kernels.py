@@ -403,7 +403,7 @@ def test_qgemm_random_shapes_epilogues_variants(K):
     """Seeded sweep over ragged shapes, every epilogue / bias kind and every kernel
     variant (heuristic included), bit-exact against the oracle."""
     rng = np.random.default_rng(20240611)
-    nvar = len(gemm_variants(K, 16))     # ids 0 .. nvar-1: the GEMM kernels
+    choices = [-1] + gemm_variants(K, 16)
     for case in range(80):
         m = int(rng.choice([1, 2, 7, 16, 31, 33, 64, 100, 129, 255, 300, 513, 1000]))
         n = int(rng.choice([1, 3, 16, 17, 48, 64, 65, 130, 256, 300, 768]))
@@ -413,7 +413,7 @@ def test_qgemm_random_shapes_epilogues_variants(K):
         acc, _ = O.gemm_s32_fast(a, w)
         sx, sw = make_scales(rng, n, per_channel=bool(rng.integers(0, 2)))
         so = pick_so(acc, sx, np.broadcast_to(sw, (n,)))
-        v = int(rng.integers(-1, nvar))
+        v = choices[int(rng.integers(0, len(choices)))]
         epi = int(rng.integers(0, 4))
         tag = "case %d: %dx%dx%d variant %d epilogue %d" % (case, m, n, k, v, epi)
         da, dw = dev(a), dev(w)
