@@ -28,7 +28,7 @@ PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, 8 TB/s
 # two rocprofv3 --pmc passes over this script (FETCH_SIZE, WRITE_SIZE; summary and
 # commands in profiles/qgemm_4096_requant_hbm_traffic.md).  Counters cannot be read
 # from inside the run, so the figure is recorded here for the size it was measured on.
-MEASURED_TRAFFIC_BYTES = {4096: (98924 + 16384) * 1024}
+MEASURED_TRAFFIC_BYTES = {4096: (98660 + 23150) * 1024}
 
 
 def parse():
@@ -41,6 +41,9 @@ def parse():
     p.add_argument("--size", type=int, default=4096, help="M = N = K of the headline GEMM")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extra", action="store_true", help="skip the extras")
+    p.add_argument("--no-two-stream", action="store_true",
+                   help="skip the two-stream throughput leg (profiling runs: its overlapping "
+                        "launches would blur per-kernel durations and counters)")
     p.add_argument("--extras", choices=("all", "qdq"), default="all",
                    help="'qdq': only the quantize / dequantize bandwidth cases (for profiling)")
     p.add_argument("--pattern", choices=("uniform", "ones"), default="uniform",
@@ -450,6 +453,26 @@ def extras(torch, steps, warmup, which="all"):
     return out
 
 
+def two_stream(torch, args, ops, da, dw, dsx, dsw, dso, dbias, out):
+    side = [torch.cuda.Stream(), torch.cuda.Stream()]
+    out2 = torch.empty_like(out)
+    calls2 = []
+    for st, o in zip(side, (out, out2)):
+        with torch.cuda.stream(st):
+            calls2.append(GemmCall(torch, da, dw, dsx, dsw, dso, dbias, 2, 2, o))
+    for i in range(2 * args.warmup):
+        calls2[i % 2]()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        calls2[i % 2]()
+    torch.cuda.synchronize()
+    wall2 = time.perf_counter() - t0
+    return {"value": round(ops * args.steps / wall2 / 1e12, 2), "unit": "TOPS",
+            "ms_per_step": round(wall2 / args.steps * 1e3, 5),
+            "note": "same GEMM, launches alternating over two HIP streams"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -532,24 +555,8 @@ def main():
     # over two streams (two output buffers) the tail of one GEMM (epilogue, write-back,
     # completion) overlaps the head of the next.  Reported next to the headline, which
     # stays the single-stream figure.
-    side = [torch.cuda.Stream(), torch.cuda.Stream()]
-    out2 = torch.empty_like(out)
-    calls2 = []
-    for st, o in zip(side, (out, out2)):
-        with torch.cuda.stream(st):
-            calls2.append(GemmCall(torch, da, dw, dsx, dsw, dso, dbias, 2, 2, o))
-    for i in range(2 * args.warmup):
-        calls2[i % 2]()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        calls2[i % 2]()
-    torch.cuda.synchronize()
-    wall2 = time.perf_counter() - t0
-    result["two_stream_throughput"] = {
-        "value": round(ops * args.steps / wall2 / 1e12, 2), "unit": "TOPS",
-        "ms_per_step": round(wall2 / args.steps * 1e3, 5),
-        "note": "same GEMM, launches alternating over two HIP streams"}
+    if not args.no_two_stream:
+        result["two_stream_throughput"] = two_stream(torch, args, ops, da, dw, dsx, dsw, dso, dbias, out)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(a, w, sx, sw, so, bias_q)
