@@ -171,14 +171,16 @@ const Variant kVariants[] = {
     // 3x3 stride-1 convolution with the input patch resident in LDS (convolution only)
     {"direct3x3_256x64", 256, 64, 128, 256},
     {"direct3x3_128x64", 128, 64, 128, 256},
-    // 256x256 tile on eight waves (two per SIMD), wave tile 128x64
+    // eight waves per workgroup: 256x256 with wave tile 128x64 (two waves per SIMD), 128x128
+    // with wave tile 64x32 (two workgroups per CU: four waves per SIMD)
     {"pipe_256x256x128_w8", 256, 256, 128, 512},
+    {"pipe_128x128x128_w8", 128, 128, 128, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
 constexpr int kSkinnyVariant = 9;
 constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct variants
-constexpr int kPipe256w8 = 12;
+constexpr int kPipe256w8 = 12, kPipe128w8 = 13;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -259,6 +261,7 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case kPipe256x64: return launch_pipe<256, 64, 4, 1, 1, CONV, EPI>(p, st);
     case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, CONV, EPI>(p, st);
     case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, CONV, EPI>(p, st);
+    case kPipe128w8: return launch_pipe<128, 128, 2, 4, 1, CONV, EPI>(p, st);
   }
   if constexpr (!CONV) {
     if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
@@ -285,7 +288,8 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 //    us) and a wave's LDS waits are covered by its neighbour, 3 % at 4096^3 and 10-25 % at
 //    K = 768; it pays once its tiles fill about 55 % of the CUs and, past one round of 256
 //    tiles, when the last round is not mostly empty (288 tiles = 2 rounds lose to 128x128);
-//  * the 128x128 tile from about 120 tiles on, below that the 64x64 tile spreads the weight
+//  * the 128x128 tile from about 120 tiles on -- on eight waves (wave tile 64x32) while
+//    K < 4096: 3-20 % faster at K = 768 .. 3072, 2 % slower at K = 4096 --, below that the 64x64 tile spreads the weight
 //    stream over more CUs; narrow outputs (N <= 64) take the 256x64 tile.  With 64x64 tiles a
 //    CU's operand loads, not its MFMAs, set the pace (16 KiB per 128 of k against 128 MFMA
 //    cycles per SIMD); when few CUs are busy and K is deep, splitting K over two wave groups
@@ -297,7 +301,7 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe) {
     const int64_t t256 = tiles(kPipe256w8);
     const int64_t rounds = ceil_div(t256, 256);
     if (t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * 256 * rounds)) return kPipe256w8;
-    if (tiles(kPipe128) >= 120) return kPipe128;
+    if (tiles(kPipe128) >= 120) return K < 4096 ? kPipe128w8 : kPipe128;
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
   constexpr int64_t kCus = 256;
