@@ -647,6 +647,24 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
         epilogue, g, Mg * Co, st);
   }
 
+  // A 1x1 filter with stride 1 and no padding is a plain GEMM over the pixels: the GEMM
+  // instantiations load their rows without the per-tap address arithmetic.
+  if (auto_pick && Kh == 1 && Kw == 1 && sh == 1 && sw_ == 1 && padding[0] == 0 &&
+      padding[1] == 0 && padding[2] == 0 && padding[3] == 0) {
+    MainParams g = {};
+    g.A = in;
+    g.W = w;
+    g.lda = Ci;
+    g.ldw = Ci;
+    g.M = (int)Mg;
+    g.N = (int)Co;
+    g.K = (int)Ci;
+    g.epi = e;
+    const int v = Mg <= kSkinnyMaxM ? kSkinnyVariant
+                                    : pick_variant(Mg, Co, Ci, pipe_ok(256, 256, g, false));
+    return launch_epi<false>(v, g, epilogue, st);
+  }
+
   MainParams p = {};
   p.A = in;
   p.W = w;
