@@ -71,9 +71,10 @@ PDLAttrPtr parseDense(Reader& r, const std::string& tag) {
     if (d != 0 && count > kMaxCount / d) return nullptr;
     count *= d;
   }
-  bool splat = false;
+  uint8_t splat_byte = 0;   // read as a byte: any non-zero value means "splat"
   std::string raw;
-  if (!r.pod(&splat) || !r.str(&raw)) return nullptr;
+  if (!r.pod(&splat_byte) || !r.str(&raw)) return nullptr;
+  const bool splat = splat_byte != 0;
   std::vector<uint8_t> data(raw.begin(), raw.end());
   if (splat) {
     // one element stored; expand it to the full shape
