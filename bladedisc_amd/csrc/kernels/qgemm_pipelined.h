@@ -30,6 +30,11 @@
 // the matrix cores draw, not by its schedule: the shader clock, 2.4 GHz when a few
 // CUs run it, falls to 1.5-1.7 GHz (clock64 against wall_clock64), and variations of
 // the schedule that change the cycle count leave the time per tile where it is.
+// Waves per workgroup: the 256x256 tile runs on WM x WN = 2 x 4 waves, two per SIMD with a
+// 128x64 wave tile.  Against 2 x 2 waves of 128x128 the requantisation of the epilogue -- a
+// chain of VALU instructions of which a wave issues about one per 5 cycles -- is half as long
+// per wave (5.7 -> 3.1 us), the accumulators fit ordinary VGPRs, and one wave's LDS and
+// barrier waits are covered by the other's MFMAs.
 // KSPLIT > 1: the workgroup has KSPLIT groups of WM x WN waves; group g runs the same
 // pipeline, with LDS stages of its own, over k tiles [g * ceil(KT / KSPLIT), ...), and the
 // groups' accumulators are added through LDS before group 0 runs the epilogue.  For
