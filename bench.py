@@ -28,7 +28,7 @@ PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, 8 TB/s
 # two rocprofv3 --pmc passes over this script (FETCH_SIZE, WRITE_SIZE; summary and
 # commands in profiles/qgemm_4096_requant_hbm_traffic.md).  Counters cannot be read
 # from inside the run, so the figure is recorded here for the size it was measured on.
-MEASURED_TRAFFIC_BYTES = {4096: (98660 + 23150) * 1024}
+MEASURED_TRAFFIC_BYTES = {4096: (98660 + 16384) * 1024}
 
 
 def parse():

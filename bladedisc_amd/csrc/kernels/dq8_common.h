@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <string>
@@ -25,6 +26,22 @@ inline bool aligned(const void* p, size_t a) {
 }
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Dynamic LDS above the default limit has to be allowed per kernel and per device.  `done`
+// is the kernel's bit set of devices (by ordinal) on which that has happened; two threads
+// racing on the first launch both set the attribute, which is harmless.
+inline int allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>* done) {
+  int dev = 0;
+  if (int s = check_hip(hipGetDevice(&dev), "hipGetDevice")) return s;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done->load(std::memory_order_acquire) & bit) return 0;
+  if (int s = check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            bytes),
+                        "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
+    return s;
+  done->fetch_or(bit, std::memory_order_release);
+  return 0;
+}
 
 }  // namespace dq8
 

@@ -2,7 +2,6 @@
 #include "qconv_direct.h"
 
 #include <algorithm>
-#include <mutex>
 
 #include "dq8_common.h"
 #include "disc_q8.h"
@@ -24,13 +23,8 @@ template <int BM, int BN, int WM, int WN, int EPI>
 int launch_t(const DirectConvParams& p, hipStream_t st) {
   const int lds = p.patch_bytes + kStages * BN * 128;
   auto kern = qconv3x3_direct_kernel<BM, BN, WM, WN, kStages, EPI>;
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
-  std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  });
-  DQ8_HIP(attr_err);
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLdsBytes, &lds_allowed)) return s;
   const int64_t grid = (int64_t)p.NB * p.tiles_per_image * p.tiles_n;
   DQ8_REQUIRE(grid < (1LL << 31), "direct convolution: too many tiles");
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WM * WN * 64), lds, st, p);

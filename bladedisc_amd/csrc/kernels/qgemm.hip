@@ -2,7 +2,6 @@
 // (any layout, any alignment, zero points) scalar kernels, and the MFMA layout
 // probe.  The tile shape is chosen at run time from the dynamic M.
 #include <algorithm>
-#include <mutex>
 
 #include "dq8_common.h"
 #include "disc_q8.h"
@@ -189,13 +188,8 @@ template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
 int launch_mfma(const MainParams& p, hipStream_t st) {
   constexpr int lds = 2 * (BM + BN) * (BK + 16);
   auto kern = qgemm_mfma_kernel<BM, BN, BK, WM, WN, CONV, EPI>;
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
-  std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-  });
-  DQ8_HIP(attr_err);
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
   const int grid = p.tiles_m * p.tiles_n;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, st, p);
   return check_hip(hipGetLastError(), "qgemm_mfma launch");
@@ -218,13 +212,8 @@ int launch_pipe(const MainParams& p, hipStream_t st) {
   DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
               "pipelined qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
   auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, KSPLIT, CONV, EPI>;
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
-  std::call_once(once, [&] {
-    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-  });
-  DQ8_HIP(attr_err);
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(WM * WN * KSPLIT * 64), lds, st, p);
   return check_hip(hipGetLastError(), "qgemm_pipe launch");
 }
