@@ -84,6 +84,23 @@ def build_profiling_tools():
     return built
 
 
+def build_test_code_objects():
+    """Device code objects the GPU tests hand to ral_kernel_launch (tests/programs/*.hip ->
+    *.hsaco next to the source), as a compiled program would carry them."""
+    progs = os.path.join(ROOT, "tests", "programs")
+    built = []
+    for f in sorted(os.listdir(progs)):
+        if not f.endswith(".hip"):
+            continue
+        out = os.path.join(progs, f[:-4] + ".hsaco")
+        cmd = [HIPCC, "-O3", "-std=c++17", "--genco"] + DEVICE + ["-o", out, os.path.join(progs, f)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for %s:\n%s" % (f, r.stdout + r.stderr))
+        built.append(out)
+    return built
+
+
 def build(force=False, verbose=False, jobs=8):
     os.makedirs(OBJ, exist_ok=True)
     srcs = sources()
@@ -106,4 +123,5 @@ def build(force=False, verbose=False, jobs=8):
 
 if __name__ == "__main__":
     path = build(force="--force" in sys.argv, verbose=True)
+    build_test_code_objects()
     print("built", path)

@@ -18,6 +18,9 @@ void clear_error();
 
 inline int check_hip(hipError_t e, const char* what) {
   if (e == hipSuccess) return 0;
+  // reported through the status; do not leave it in the thread's HIP error state as well,
+  // where the caller's framework would find it at its next GPU call
+  (void)hipGetLastError();
   return fail(std::string(what) + ": " + hipGetErrorString(e));
 }
 

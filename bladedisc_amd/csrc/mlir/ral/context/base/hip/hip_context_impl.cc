@@ -82,6 +82,9 @@ namespace {
 
 bool hipOk(hipError_t e, ExecutionContext* ctx, const char* where) {
   if (e == hipSuccess) return true;
+  // The error is reported through the context; take it off the thread's HIP error state so
+  // that the framework sharing this thread does not trip over it at its next GPU call.
+  (void)hipGetLastError();
   std::ostringstream out;
   out << "GPU failed with " << hipGetErrorString(e) << " in " << where;
   ctx->signalError(Context::FAILURE, out.str());

@@ -13,6 +13,7 @@ from . import _lib
 _SCALAR_CODES = {
     "i1": C.c_bool, "i8": C.c_int8, "ui8": C.c_uint8, "i32": C.c_int32,
     "i64": C.c_int64, "f32": C.c_float, "f64": C.c_double, "pvoid": C.c_void_p,
+    "ppvoid": C.c_void_p,
 }
 
 _TORCH_CODES = None

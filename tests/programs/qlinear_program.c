@@ -53,7 +53,14 @@ static void gpu_dealloc(ral_call_t call, void* exec, void* ptr) {
   call(exec, (void*)"dealloc___gpu___pvoid_pvoid___void", args);
 }
 
-void disc_program_main(void** ctx_struct) {
+/* input -> constants -> quantize -> ral_pdll_qgemm: the part both programs share */
+typedef struct {
+  void* exec; ral_call_t call; void* stream;
+  MemRef2 x, yq; MemRef0 so, zero;
+  int64_t M, N;
+} Front;
+
+static void run_front(void** ctx_struct, Front* f) {
   void* exec = ctx_struct[0];
   ral_call_t call = (ral_call_t)ctx_struct[1];
   void* stream = 0;   /* stream index 0 */
@@ -101,6 +108,23 @@ void disc_program_main(void** ctx_struct) {
     call(exec, (void*)"ral_pdll_qgemm___gpu___pvoid_pvoid_m2di8_m2di8_m1df32_m0df32_m0di32_m1df32_m1di32_m0df32_m0di32_pvoid___m2di8", args); }
   gpu_dealloc(call, exec, xq.data);
 
+  f->exec = exec; f->call = call; f->stream = stream;
+  f->x = x; f->yq = yq; f->so = so; f->zero = zero; f->M = M; f->N = N;
+}
+
+static void send_outputs(Front* f, MemRef2* y) {
+  void* exec = f->exec; ral_call_t call = f->call;
+  /* ---- output 0 = y; output 1 = x (an input forwarded unchanged) */
+  { int64_t idx = 0; void* args[16]; int n = 0; args[n++] = &exec; args[n++] = &idx; n = push2(args, n, y);
+    call(exec, (void*)"ral_send_output___cpu___pvoid_i64_m2df32___void", args); }
+  { int64_t idx = 1; void* args[16]; int n = 0; args[n++] = &exec; args[n++] = &idx; n = push2(args, n, &f->x);
+    call(exec, (void*)"ral_send_output___cpu___pvoid_i64_m2df32___void", args); }
+}
+
+void disc_program_main(void** ctx_struct) {
+  Front f; run_front(ctx_struct, &f);
+  void* exec = f.exec; ral_call_t call = f.call; void* stream = f.stream;
+  MemRef2 yq = f.yq; MemRef0 so = f.so, zero = f.zero; const int64_t M = f.M, N = f.N;
   /* ---- y = dequantize(yq) */
   MemRef2 y = {0};
   y.base = y.data = gpu_alloc(call, exec, M * N * 4);
@@ -112,11 +136,34 @@ void disc_program_main(void** ctx_struct) {
     call(exec, (void*)"ral_dequantize___gpu___pvoid_pvoid_m2di8_m0df32_m0di32_m2df32_i64___void", args); }
   gpu_dealloc(call, exec, yq.data);
 
-  /* ---- output 0 = y; output 1 = x (an input forwarded unchanged) */
-  { int64_t idx = 0; void* args[16]; int n = 0; args[n++] = &exec; args[n++] = &idx; n = push2(args, n, &y);
-    call(exec, (void*)"ral_send_output___cpu___pvoid_i64_m2df32___void", args); }
-  { int64_t idx = 1; void* args[16]; int n = 0; args[n++] = &exec; args[n++] = &idx; n = push2(args, n, &x);
-    call(exec, (void*)"ral_send_output___cpu___pvoid_i64_m2df32___void", args); }
+  send_outputs(&f, &y);
+}
+
+/* The same program with the dequantize replaced by a fused elementwise kernel that the
+ * compiler would have generated and embedded as a code object:
+ * y = relu(dequantize(yq)) + x, launched through ral_kernel_launch (N must equal K). */
+static const void* g_code_object = 0;
+void disc_program_set_code_object(const void* blob) { g_code_object = blob; }
+
+void disc_program_main_fused(void** ctx_struct) {
+  Front f; run_front(ctx_struct, &f);
+  void* exec = f.exec; ral_call_t call = f.call; void* stream = f.stream;
+  const int64_t M = f.M, N = f.N;
+  MemRef2 y = {0};
+  y.base = y.data = gpu_alloc(call, exec, M * N * 4);
+  y.sizes[0] = M; y.sizes[1] = N; y.strides[0] = N; y.strides[1] = 1;
+  { void* blobs[1] = {(void*)g_code_object}; void** blobs_p = blobs; int64_t num_blobs = 1;
+    const char* name = "fused_dequant_relu_residual";
+    int64_t total = M * N;
+    int64_t gx = (total + 255) / 256, gy = 1, gz = 1, bx = 256, by = 1, bz = 1;
+    int32_t smem = 0, num_args = 5;
+    void* params[5] = {&f.yq.data, &f.so.data, &f.x.data, &y.data, &total};
+    void** params_p = params;
+    void* args[14] = {&exec, &blobs_p, &num_blobs, &name, &gx, &gy, &gz, &bx, &by, &bz, &smem,
+                      &stream, &num_args, &params_p};
+    call(exec, (void*)"ral_kernel_launch___gpu___pvoid_ppvoid_i64_pvoid_i64_i64_i64_i64_i64_i64_i32_pvoid_i32_ppvoid___void", args); }
+  gpu_dealloc(call, exec, f.yq.data);
+  send_outputs(&f, &y);
 }
 
 /* Host cost of the dispatch path: `n` back-to-back ral_pdll_qgemm calls on M rows of

@@ -100,6 +100,81 @@ def test_compiled_program_runs_on_the_runtime(program):
         L.disc_ral_context_destroy(C.c_void_p(ctx))
 
 
+def test_program_with_an_embedded_code_object(program):
+    """The same program with its dequantize replaced by a fused elementwise kernel that
+    travels as a gfx950 code object, the way the compiler ships its generated kernels, and
+    is launched through ral_kernel_launch: y = relu(dequantize(qgemm(...))) + x.  Two
+    executions (the second finds the loaded module cached), checked bit for bit."""
+    lib, d = program
+    hsaco = os.path.join(HERE, "programs", "fused_dequant_relu_residual.hsaco")
+    assert os.path.exists(hsaco), "run __graft_entry__.build() first: it compiles the code object"
+    blob = open(hsaco, "rb").read()
+    blob_buf = C.create_string_buffer(blob, len(blob))      # lives as long as the context
+    lib.disc_program_set_code_object(C.cast(blob_buf, C.c_void_p))
+    from bladedisc_amd import baseline_configs as cfg
+    from bladedisc_amd import ral
+    L = ral.lib()
+    c = cfg.config1()
+    names = ["w0_i8_768x768", "b0_f32_768", "sw0_f32_768", "sx0_f32_", "so0_f32_", "z0_i32_"]
+    values = [hexstr(c["w_q"]), hexstr(c["bias"]), hexstr(c["sw"]),
+              hexstr(np.array([c["sx"]], np.float32)), hexstr(np.array([c["so"]], np.float32)),
+              hexstr(np.array([0], np.int32))]
+    meta = str(d / "fused.metadata").encode()
+    n = len(names)
+    L.disc_ral_metadata_emit.restype = C.c_int
+    assert L.disc_ral_metadata_emit(meta, n, (C.c_uint8 * n)(*([0] * n)),
+                                    (C.c_char_p * n)(*[s.encode() for s in names]),
+                                    (C.c_char_p * n)(*[v.encode() for v in values])) == 0
+    L.disc_ral_context_create_for_program.restype = C.c_void_p
+    L.disc_ral_execution_take_output.restype = C.c_void_p
+    L.disc_ral_output_data.restype = C.c_void_p
+    stream = torch.cuda.current_stream().cuda_stream
+    ctx = L.disc_ral_context_create_for_program(C.c_void_p(stream), 0, None, None, None, 1, meta)
+    assert ctx
+    call_impl = C.cast(L.tao_ral_call_impl, C.c_void_p).value
+    try:
+        for m in (64, 7):
+            x = torch.from_numpy(np.ascontiguousarray(c["x"][:m])).cuda()
+            ex = L.disc_ral_execution_context_create(C.c_void_p(ctx))
+            assert L.disc_ral_execution_bind_input(C.c_void_p(ex), 0, C.c_void_p(x.data_ptr()),
+                                                   (C.c_int64 * 2)(m, 768), 2) == 0
+            lib.disc_program_main_fused((C.c_void_p * 2)(ex, call_impl))
+            msg = C.c_char_p()
+            assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) == 0, msg.value
+            out = L.disc_ral_execution_take_output(C.c_void_p(ex), 0)
+            assert out
+            torch.cuda.synchronize()
+            y = ral.device_view(L.disc_ral_output_data(C.c_void_p(out)), (m, 768),
+                                torch.float32).cpu().numpy()
+            xq = O.quantize(c["x"][:m], c["sx"], 0)
+            acc = O.gemm_s32(xq, c["w_q"], tp_b=True)
+            b32 = O.bias_f32_to_s32(c["bias"], float(c["sx"]), c["sw"])
+            yq = O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]), b32=b32)
+            deq = yq.astype(np.float32) * np.float32(c["so"])
+            want = np.maximum(deq, np.float32(0)) + c["x"][:m].astype(np.float32)
+            np.testing.assert_array_equal(y, want)
+            L.disc_ral_output_destroy(C.c_void_p(out))
+            L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+        # a kernel name the code object does not hold is an error, not a crash
+        ex = L.disc_ral_execution_context_create(C.c_void_p(ctx))
+        a = ral.Args().ctx(ex)
+        blobs = (C.c_void_p * 1)(C.cast(blob_buf, C.c_void_p).value)
+        a.scalar("ppvoid", C.cast(blobs, C.c_void_p).value).scalar("i64", 1)
+        a.scalar("pvoid", C.cast(C.c_char_p(b"no_such_kernel"), C.c_void_p).value)
+        for v in (1, 1, 1, 64, 1, 1):
+            a.scalar("i64", v)
+        a.scalar("i32", 0).scalar("pvoid", None).scalar("i32", 0).scalar("ppvoid", None)
+        L.tao_ral_call_impl(C.c_void_p(ex), ral.mangle("ral_kernel_launch", "gpu", a.arg_codes).encode(),
+                            a.pack())
+        msg = C.c_char_p()
+        assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) != 0
+        assert b"GetFunction" in msg.value
+        L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+    finally:
+        torch.cuda.synchronize()
+        L.disc_ral_context_destroy(C.c_void_p(ctx))
+
+
 def test_missing_constant_is_reported(program):
     lib, d = program
     from bladedisc_amd import ral
