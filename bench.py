@@ -404,6 +404,18 @@ def extras(torch, steps, warmup, which="all"):
         gbps = nbytes * reps / ev / 1e9
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 5}
+    # calibration statistic (running min / max): 4 bytes read per element
+    lo1, hi1 = torch.full((1,), float("inf"), device="cuda"), torch.full((1,), float("-inf"), device="cuda")
+    loc, hic = torch.full((cols,), float("inf"), device="cuda"), torch.full((cols,), float("-inf"), device="cuda")
+    lor, hir = torch.full((rows,), float("inf"), device="cuda"), torch.full((rows,), float("-inf"), device="cuda")
+    ws = torch.empty(1 << 24, dtype=torch.uint8, device="cuda")
+    for name, fn in (("minmax_per_tensor", lambda: K.minmax(x, lo1, hi1, workspace=ws)),
+                     ("minmax_per_channel_last_axis", lambda: K.minmax(x, loc, hic, axis=1, workspace=ws)),
+                     ("minmax_per_channel_axis0", lambda: K.minmax(x, lor, hir, axis=0, workspace=ws))):
+        _, ev = time_steps(torch, fn, reps, 3)
+        gbps = 4.0 * rows * cols * reps / ev / 1e9
+        out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
+                     "shape": [rows, cols], "bytes_per_elem": 4}
     del x, q, f
     # smaller activations (they fit the 256 MB last-level cache; launches captured in a graph)
     small = {}

@@ -74,6 +74,27 @@ def quantize(x, scale, zero_point, axis=None, qmin=-128, qmax=127,
     return out
 
 
+def minmax(x, min_io, max_io, axis=None, workspace=None):
+    """Folds the minimum and maximum of `x` (device f32), per tensor (axis None) or per
+    slice along `axis`, into the running values min_io / max_io (device f32, one entry or
+    one per channel).  Returns (min_io, max_io)."""
+    _need_cuda(x, min_io, max_io)
+    if x.dtype != torch.float32 or min_io.dtype != torch.float32 or max_io.dtype != torch.float32:
+        raise TypeError("minmax takes float32 tensors")
+    x = x.contiguous()
+    outer, nch, inner = _view3(tuple(x.shape), axis)
+    if min_io.numel() != nch or max_io.numel() != nch:
+        raise ValueError("min / max state must have one entry per channel (%d)" % nch)
+    L = _lib.lib()
+    need = L.dq8_minmax_workspace_bytes(outer, nch, inner)
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    st = L.dq8_minmax(_ptr(x), outer, nch, inner, _ptr(min_io), _ptr(max_io), _ptr(workspace),
+                      workspace.numel() * workspace.element_size(), _stream())
+    _lib.check(st, "dq8_minmax")
+    return min_io, max_io
+
+
 def dequantize(q, scale, zero_point, axis=None, out=None):
     _need_cuda(q, scale, zero_point)
     q = q.contiguous()

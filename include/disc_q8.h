@@ -17,6 +17,8 @@
  *                     (R ral/context/common_context_impl_quantization.cc:1196-1672).
  *   dq8_qconv2d    -> the fused int8 convolution behind ral_qconv
  *                     (R ral/context/stream_executor_based_impl.cc:1506-1588, 1831-1948).
+ *   dq8_minmax     -> torch.aminmax in the calibration observers
+ *                     (R tools/torch_quant/torch_quant/observer.py:236-241, 261-281).
  *   dq8_quantize / dq8_dequantize
  *                  -> the loops the compiler generates from mhlo_disc.quantize /
  *                     mhlo_disc.dequantize
@@ -64,6 +66,23 @@ int dq8_version(void);
 /* Number of compute units / LDS bytes / clock the library sees on the current
  * device; fills what it can, returns 0 on success. */
 int dq8_device_info(int* compute_units, int* lds_bytes_per_cu, int* clock_khz);
+
+/* ---- calibration statistics -------------------------------------------- */
+
+/* Running minimum and maximum of a float tensor, per tensor or per channel: what the
+ * reference's calibration observers accumulate before they derive scales and zero points
+ * (R tools/torch_quant/torch_quant/observer.py:236-241 MinMaxObserver via torch.aminmax,
+ * :261-281 PerChannelMinMaxObserver).  x (device, f32) is viewed as [outer, channels, inner];
+ * for every channel c
+ *     min_io[c] = min(min_io[c], min over o, i of x[o, c, i])
+ *     max_io[c] = max(max_io[c], max ...)
+ * so the caller keeps the observer's state in min_io / max_io (device f32, `channels`
+ * entries, +inf / -inf before anything has been observed).  A NaN in a channel's data makes
+ * both of its values NaN, as torch.aminmax does.  An empty tensor leaves the state as it is.
+ * `workspace` (device) must hold dq8_minmax_workspace_bytes(...) bytes. */
+size_t dq8_minmax_workspace_bytes(int64_t outer, int64_t channels, int64_t inner);
+int dq8_minmax(const float* x, int64_t outer, int64_t channels, int64_t inner, float* min_io,
+               float* max_io, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- quantize / dequantize -------------------------------------------- */
 
