@@ -117,6 +117,68 @@ transpose_s8_kernel(const int8_t* __restrict__ src, int64_t ld, int8_t* __restri
   }
 }
 
+// out[r] = mul * sum_k X[r, k] + add for an int8 matrix whose rows are 16-byte aligned and a
+// multiple of 16 long: the zero-point corrections of a GEMM.  One wave per row.
+__global__ void __launch_bounds__(256)
+rowsum_s8_kernel(const int8_t* __restrict__ X, int64_t ld, int rows, int K, int mul, int add,
+                 int32_t* __restrict__ out) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const v4i* p = reinterpret_cast<const v4i*>(X + (int64_t)row * ld);
+  int s = 0;
+  for (int c = lane; c < K / 16; c += 64) {
+    const v4i v = p[c];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int x = v[w];
+      s += (int)(int8_t)x + (int)(int8_t)(x >> 8) + (int)(int8_t)(x >> 16) + (x >> 24);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (lane == 0) out[row] = mul * s + add;
+}
+
+// Second pass of a GEMM with zero points: the symmetric MFMA kernels have left
+// sum_k A W in `acc` ([M, N] int32, dense); with SA[m] and SW[n] the row sums,
+//   sum_k (A - zx)(W - zw) = acc - zx SW[n] - zw SA[m] + K zx zw
+// (corr_n[n] = -zx SW[n] + K zx zw, corr_m[m] = -zw SA[m]; int32 arithmetic wraps exactly
+// like the direct sum), then the epilogue.
+// A thread owns one output channel (its scale, bias and column correction are computed
+// once) and walks `rows` rows, four loads in flight; consecutive threads read and write
+// consecutive addresses.
+template <int EPI>
+__global__ void __launch_bounds__(256)
+zero_point_epilogue_kernel(const int32_t* __restrict__ acc, const int32_t* __restrict__ corr_n,
+                           const int32_t* __restrict__ corr_m, int rows, const EpiParams e) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= e.N) return;
+  const ColParams c = col_params<EPI>(e, n);
+  const unsigned cn = (unsigned)corr_n[n];
+  const int m_begin = blockIdx.y * rows;
+  const int m_end = m_begin + rows < e.M ? m_begin + rows : e.M;
+  auto finish = [&](int m, int raw) {
+    const unsigned a = (unsigned)raw + cn + (corr_m ? (unsigned)corr_m[m] : 0u);
+    const int64_t off = (int64_t)m * e.ldo + n;
+    if (EPI == DQ8_EPI_ACC_S32)
+      ((int32_t*)e.out)[off] = (int)a;
+    else if (EPI == DQ8_EPI_DEQUANT_F32)
+      ((float*)e.out)[off] = dequant_one(e, c, (int)a);
+    else
+      ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, (int)a);
+  };
+  int m = m_begin;
+  for (; m + 3 < m_end; m += 4) {
+    int raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) raw[u] = acc[(int64_t)(m + u) * e.N + n];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) finish(m + u, raw[u]);
+  }
+  for (; m < m_end; ++m) finish(m, acc[(int64_t)m * e.N + n]);
+}
+
 // one MFMA of each shape, operands straight from global memory
 __global__ void __launch_bounds__(64)
 mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* a16,
@@ -381,6 +443,16 @@ extern "C" size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int
   return bytes;
 }
 
+extern "C" size_t dq8_qgemm_workspace_bytes_zp(int64_t M, int64_t N, int64_t K, int tp_a,
+                                               int tp_b, int32_t zx, int32_t zw) {
+  size_t bytes = dq8_qgemm_workspace_bytes(M, N, K, tp_a, tp_b);
+  if (zx != 0 || zw != 0) {
+    auto pad = [](int64_t v) { return (size_t)((v + 255) / 256 * 256); };
+    bytes += pad(M * N * 4) + pad(N * 4) + pad(M * 4);
+  }
+  return bytes;
+}
+
 extern "C" int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
                                 int64_t cols, void* stream) {
   clear_error();
@@ -437,9 +509,16 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
 
-  const bool need_generic = zx != 0 || zw != 0;
+  // Zero points: the MFMA kernels are symmetric.  With scratch for an int32 [M, N]
+  // intermediate the heuristic runs them and corrects the sums in a second pass; without it
+  // (or for operands they cannot take) the generic kernel subtracts the zero points itself.
+  const bool has_zp = zx != 0 || zw != 0;
   const bool auto_pick = variant == -1;
-  if (auto_pick && need_generic) variant = 0;
+  const bool zp_two_pass =
+      has_zp && auto_pick && K > 0 && K % 16 == 0 && workspace != nullptr && aligned(workspace, 256) &&
+      workspace_bytes >= dq8_qgemm_workspace_bytes_zp(M, N, K, tp_a, tp_b, zx, zw) &&
+      (tp_a || (aligned(A, 16) && lda % 16 == 0)) && (!tp_b || (aligned(W, 16) && ldw % 16 == 0));
+  if (auto_pick && has_zp && !zp_two_pass) variant = 0;
   if (variant == 0) {
     GenericParams g;
     g.A = A;
@@ -457,8 +536,9 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
         qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
         epilogue, g, M * N, st);
   }
-  DQ8_REQUIRE(!need_generic,
-              "dq8_qgemm: input/weight zero points are only supported by the generic variant");
+  DQ8_REQUIRE(!has_zp || zp_two_pass,
+              "dq8_qgemm: input/weight zero points need the heuristic (variant -1) or the "
+              "generic variant");
 
   // MFMA path wants A [M,K] and W [N,K], both k-contiguous: transpose the others
   // into the workspace.
@@ -485,6 +565,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                          dim3(256), 0, st, W, ldw, dst, (int)K, (int)N);
       w_use = dst;
       ldw_use = K;
+      ws_off += pad(N * K);
     }
     DQ8_HIP(hipGetLastError());
   }
@@ -500,8 +581,8 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
     g.w_sn = ldw_use;
     g.w_sk = 1;
     g.K = (int)K;
-    g.zx = 0;
-    g.zw = 0;
+    g.zx = zx;
+    g.zw = zw;
     g.epi = e;
     return launch_generic_epi<GenericParams>(
         qgemm_generic_kernel<DQ8_EPI_ACC_S32>, qgemm_generic_kernel<DQ8_EPI_REQUANT_CPU>,
@@ -520,7 +601,54 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.epi = e;
   if (auto_pick)
     variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false));
-  return launch_epi<false>(variant, p, epilogue, st);
+  if (!zp_two_pass) return launch_epi<false>(variant, p, epilogue, st);
+
+  // ---- zero points: raw sums into scratch, row-sum corrections, then the epilogue
+  int32_t* acc = reinterpret_cast<int32_t*>((int8_t*)workspace + ws_off);
+  int32_t* corr_n = reinterpret_cast<int32_t*>((int8_t*)acc + pad(M * N * 4));
+  int32_t* corr_m = reinterpret_cast<int32_t*>((int8_t*)corr_n + pad(N * 4));
+  EpiParams raw = {};
+  raw.out = acc;
+  raw.ldo = N;
+  raw.M = (int)M;
+  raw.N = (int)N;
+  raw.bias_kind = DQ8_BIAS_NONE;
+  raw.vec_store = N % 4 == 0;
+  raw.vec_store16 = N % 4 == 0;
+  p.epi = raw;
+  if (int s = launch_epi<false>(variant, p, DQ8_EPI_ACC_S32, st)) return s;
+  // (wrapping int32 arithmetic on purpose, as in the kernels)
+  const int kzz = (int)((uint32_t)K * (uint32_t)zx * (uint32_t)zw);
+  hipLaunchKernelGGL(rowsum_s8_kernel, dim3((unsigned)ceil_div(N, 4)), dim3(256), 0, st, w_use,
+                     ldw_use, (int)N, (int)K, -zx, kzz, corr_n);
+  if (zw != 0)
+    hipLaunchKernelGGL(rowsum_s8_kernel, dim3((unsigned)ceil_div(M, 4)), dim3(256), 0, st, a_use,
+                       lda_use, (int)M, (int)K, -zw, 0, corr_m);
+  DQ8_HIP(hipGetLastError());
+  const int32_t* cm = zw != 0 ? corr_m : nullptr;
+  // rows per workgroup: 64 for large outputs, fewer while that leaves under ~2048 workgroups
+  const int64_t col_blocks = ceil_div(N, 256);
+  const int zp_rows = (int)std::min<int64_t>(64, std::max<int64_t>(4, M * col_blocks / 2048));
+  const dim3 blocks((unsigned)col_blocks, (unsigned)ceil_div(M, zp_rows));
+  DQ8_REQUIRE(blocks.y <= 65535u, "dq8_qgemm: too many rows for the zero-point pass");
+  switch (epilogue) {
+    case DQ8_EPI_ACC_S32:
+      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_ACC_S32>, blocks, dim3(256), 0,
+                         st, acc, corr_n, cm, zp_rows, e);
+      break;
+    case DQ8_EPI_REQUANT_CPU:
+      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_REQUANT_CPU>, blocks, dim3(256),
+                         0, st, acc, corr_n, cm, zp_rows, e);
+      break;
+    case DQ8_EPI_REQUANT_GPU:
+      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_REQUANT_GPU>, blocks, dim3(256),
+                         0, st, acc, corr_n, cm, zp_rows, e);
+      break;
+    default:
+      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_DEQUANT_F32>, blocks, dim3(256),
+                         0, st, acc, corr_n, cm, zp_rows, e);
+  }
+  return check_hip(hipGetLastError(), "zero_point_epilogue launch");
 }
 
 extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,

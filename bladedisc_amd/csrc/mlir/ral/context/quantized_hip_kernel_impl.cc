@@ -93,6 +93,7 @@ struct GemmOperands {
   int64_t m = 0, n = 0, k = 0;
   bool tp_a = false, tp_b = false;
   bool weight_is_const = false;
+  int32_t zx = 0, zw = 0;   // input / weight zero point: acc = sum (a - zx)(w - zw)
 };
 
 struct Epilogue {
@@ -134,7 +135,10 @@ void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const 
 
   const int64_t lda = op.tp_a ? op.m : op.k;
   const int64_t ldw = op.tp_b ? op.k : op.n;
-  const size_t ws_bytes = dq8_qgemm_workspace_bytes(op.m, op.n, op.k, op.tp_a, op.tp_b);
+  // (with a zero point: room for the int32 intermediate that keeps the problem on the MFMA
+  // kernels)
+  const size_t ws_bytes =
+      dq8_qgemm_workspace_bytes_zp(op.m, op.n, op.k, op.tp_a, op.tp_b, op.zx, op.zw);
   void* ws = nullptr;
   if (ws_bytes) {
     ws = drv->alloc(ctx, ws_bytes);
@@ -142,7 +146,7 @@ void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const 
   }
   int st = dq8_qgemm(op.a, lda, op.w, ldw, out, op.n, op.m, op.n, op.k, op.tp_a, op.tp_b,
                      e.mode, e.bias, e.bias_kind, e.sx, e.n_sx, e.sw, e.n_sw, e.so, e.n_so,
-                     /*zx=*/0, /*zw=*/0, e.zo, ws, ws_bytes, stream);
+                     op.zx, op.zw, e.zo, ws, ws_bytes, stream);
   // the pool hands `ws` out again only to later work on the same stream, which is
   // ordered after this launch
   if (ws) drv->dealloc(ctx, ws);
@@ -263,7 +267,8 @@ bool prepareResult(ExecutionContext* ctx, const MemRefType<int8_t, N>& input, in
 }
 
 // Zero points of ral_pdll_* calls are host-resident ("s" placement in the PDLL
-// patterns); only the symmetric input/weight case has kernels.
+// patterns).  The entries with the reference's gpu signatures are symmetric, as the
+// reference's are (its gpu kernels never read the zero points).
 bool symmetricOrFail(ExecutionContext* ctx, const int32_t* zx, int64_t n_zx, const int32_t* zw,
                      int64_t n_zw, const char* who) {
   for (int64_t i = 0; i < n_zx; ++i)
@@ -431,9 +436,16 @@ MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_hand
     return result;
   }
   if (!prepareResult<N>(ctx, input, op.n, &op.m, &result)) return result;
-  if (!symmetricOrFail(ctx, inputZeroPoints.data, 1, weightZeroPoints.data,
-                       weightZeroPoints.sizes[0], who))
-    return result;
+  // One input zero point and one weight zero point, as oneDNN takes them from the
+  // reference's CPU entries (ideep matmul.hpp:516-517, 548-549; the reference silently uses
+  // element 0 of a weight zero-point vector -- a vector that is not uniform is refused here).
+  op.zx = inputZeroPoints.data ? inputZeroPoints.data[0] : 0;
+  op.zw = weightZeroPoints.data && weightZeroPoints.sizes[0] > 0 ? weightZeroPoints.data[0] : 0;
+  for (int64_t i = 1; weightZeroPoints.data && i < weightZeroPoints.sizes[0]; ++i)
+    if (weightZeroPoints.data[i] != op.zw) {
+      fail(ctx, "ral_pdll_qgemm: per-channel weight zero points are not supported");
+      return result;
+    }
   if (weightScales.sizes[0] != 1 && weightScales.sizes[0] != op.n) {
     fail(ctx, "ral_pdll_qgemm: weight scale must have 1 or N entries");
     return result;

@@ -132,7 +132,10 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
     sw = _scale(sw, dev) if sw is not None else None
     so = _scale(so, dev) if so is not None else None
     bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
-    ws_bytes = L.dq8_qgemm_workspace_bytes(m, n, k, int(tp_a), int(tp_b))
+    # with zero points and the heuristic this includes the int32 intermediate of the
+    # two-pass path; a forced generic variant (0) needs none of it
+    ws_bytes = (L.dq8_qgemm_workspace_bytes_zp(m, n, k, int(tp_a), int(tp_b), zx, zw)
+                if variant == -1 else L.dq8_qgemm_workspace_bytes(m, n, k, int(tp_a), int(tp_b)))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     st = L.dq8_qgemm_variant(
         variant, _ptr(a), max(a.stride(0), a.shape[1]), _ptr(w), max(w.stride(0), w.shape[1]),

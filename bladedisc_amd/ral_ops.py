@@ -77,17 +77,18 @@ def pdll_qgemm_per_channel(ex, x, w_nk, bias_i8, sx_n, sw_n, so_n):
 
 
 def pdll_qgemm_cpu_style(ex, x, w, bias, sx, sw_n, so, zo=0, transpose_b=False,
-                         weight_is_const=True):
+                         weight_is_const=True, zx=0, zw=0):
     """ral_pdll_qgemm with the CPU patterns' signature on the gpu device: weight
-    [K,N] unless transpose_b, bias f32 / s32 / None, per-channel weight scale."""
+    [K,N] unless transpose_b, bias f32 / s32 / None, per-channel weight scale; zx: input
+    zero point, zw: weight zero point(s), a value or one per channel (host values)."""
     n = w.shape[0] if transpose_b else w.shape[1]
     a = ex.new_args().tensor(x).tensor(w)
     if bias is not None:
         a.tensor(bias)
     a.tensor(sx, rank0=True)
-    _zp0(a, host=True)
+    a.host_array(np.array([zx], np.int32), rank0=True)
     a.tensor(sw_n)
-    a.host_array(np.zeros(sw_n.numel(), np.int32))
+    a.host_array(np.broadcast_to(np.asarray(zw, np.int32), (sw_n.numel(),)).copy())
     a.tensor(so, rank0=True)
     a.host_array(np.array([zo], np.int32), rank0=True)
     a.blob(ral.encode_attr({"transpose_a": False, "transpose_b": bool(transpose_b),

@@ -101,10 +101,16 @@ int dq8_dequantize(const void* q, int in_kind, float* out, int64_t outer,
 
 /* ---- int8 GEMM -------------------------------------------------------- */
 
-/* Bytes of device scratch dq8_qgemm needs for this problem (0 when it needs
- * none: tp_a == 0 and tp_b == 1 and no zero points). */
+/* Bytes of device scratch dq8_qgemm needs for this problem with zx == zw == 0 (0 when it
+ * needs none: tp_a == 0 and tp_b == 1). */
 size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
                                  int tp_b);
+/* The same for given input / weight zero points: with a non-zero one it adds an int32
+ * [M, N] intermediate and two correction vectors, which lets dq8_qgemm keep such a problem
+ * on the MFMA kernels.  A caller that passes less (but at least
+ * dq8_qgemm_workspace_bytes()) still gets the right result, from the generic kernel. */
+size_t dq8_qgemm_workspace_bytes_zp(int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
+                                    int32_t zx, int32_t zw);
 
 /* out[M,N] = epilogue( sum_k A(m,k) * W(k,n) ).
  *   A: device int8, [M,K] with row stride lda (tp_a = 0) or [K,M] with row
@@ -113,9 +119,13 @@ size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
  *      [K,N] row stride ldw (tp_b = 0, the CPU callers' layout).
  *   out: device, element type per `epilogue`, row stride ldo (elements).
  *   sx / sw / so: device f32 with n_sx / n_sw / n_so entries, each 1 or N.
- *   zx / zw: input and weight zero points, acc = sum (A - zx) * (W - zw).  Every
- *      reference caller is symmetric (0); non-zero values are computed by the generic
- *      scalar kernel, not the MFMA kernels.
+ *   zx / zw: input and weight zero points, acc = sum (A - zx) * (W - zw) (what oneDNN
+ *      computes for the reference's CPU entries, R ral/context/mkldnn/ideep/ideep/
+ *      operators/matmul.hpp:516-549: one source zero point, the first weight zero point).
+ *      With scratch of dq8_qgemm_workspace_bytes_zp() the symmetric MFMA kernels compute
+ *      sum A W into an int32 intermediate and a second pass applies
+ *      - zx sum_k W - zw sum_k A + K zx zw and the epilogue; with less scratch, or
+ *      operands the MFMA kernels cannot take, the generic scalar kernel is used.
  *   zo: output zero point (REQUANT_CPU only).
  *   workspace: device scratch of at least dq8_qgemm_workspace_bytes(), may be
  *      NULL when that is 0.
@@ -131,7 +141,8 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
  *  -1 heuristic, 0 generic scalar kernel, 1.. MFMA tile configurations
  *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()).  A problem
  *  an MFMA variant cannot take (K % 16 != 0, unaligned rows) runs on the generic
- *  kernel whatever the variant; non-zero zx / zw with a forced MFMA variant is an error. */
+ *  kernel whatever the variant; non-zero zx / zw with a forced MFMA variant is an error
+ *  (they need the heuristic or the generic variant). */
 int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                       const int8_t* W, int64_t ldw, void* out, int64_t ldo,
                       int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,

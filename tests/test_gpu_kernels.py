@@ -169,6 +169,58 @@ def test_qgemm_zero_points_generic(K):
         K.qgemm(dev(a), dev(w), K.EPI_ACC_S32, zx=3, variant=2)
 
 
+@pytest.mark.parametrize("m,n,k,tp_a,tp_b,zx,zw", [
+    (64, 768, 768, 0, 1, 7, 0), (300, 130, 400, 0, 1, -128, 0), (33, 48, 64, 0, 1, 5, -3),
+    (256, 512, 1040, 0, 0, 100, 0), (100, 96, 128, 1, 1, 127, 2), (1, 768, 3072, 0, 1, 11, 0),
+    (1000, 768, 768, 0, 1, -77, 9),
+])
+def test_qgemm_zero_points_on_the_mfma_path(K, m, n, k, tp_a, tp_b, zx, zw):
+    """Asymmetric operands stay on the MFMA kernels when the caller provides the scratch for
+    the two-pass scheme: every epilogue equals the oracle's direct sum of (a - zx)(w - zw);
+    without the scratch the generic kernel gives the same result."""
+    rng = np.random.default_rng(m + n + k + zx)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc = O.gemm_s32(a, w, tp_b=True, zx=zx, zw=zw)
+    a_in = np.ascontiguousarray(a.T) if tp_a else a
+    w_in = w if tp_b else np.ascontiguousarray(w.T)
+    kw = dict(tp_a=bool(tp_a), tp_b=bool(tp_b), zx=zx, zw=zw)
+    got = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_ACC_S32, **kw))
+    np.testing.assert_array_equal(got, acc)
+    got0 = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_ACC_S32, variant=0, **kw))   # generic
+    np.testing.assert_array_equal(got0, acc)
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    bias = (rng.standard_normal(n) * 3).astype(np.float32)
+    dsx, dsw, dso = dev(np.array([sx])), dev(sw), dev(np.array([so]))
+    b32 = O.bias_f32_to_s32(bias, sx, sw)
+    want = O.requant_cpu(acc, sx, sw, so, b32=b32, zo=5)
+    got = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_REQUANT_CPU, sx=dsx, sw=dsw, so=dso,
+                       bias=dev(bias), zo=5, **kw))
+    np.testing.assert_array_equal(got, want)
+    want = O.requant_gpu(acc, sx, sw, so, bias_f32=bias)
+    got = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_REQUANT_GPU, sx=dsx, sw=dsw, so=dso,
+                       bias=dev(bias), **kw))
+    np.testing.assert_array_equal(got, want)
+    want = O.dequant_acc(acc, sx, sw, bias=bias)
+    got = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_DEQUANT_F32, sx=dsx, sw=dsw, bias=dev(bias), **kw))
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_qgemm_zero_points_full_size_property(K):
+    """4096^3 with an input zero point: the two-pass result equals the symmetric result of
+    the shifted problem computed another way -- acc(a - zx, w) = acc(a, w) - zx * colsum(w)
+    -- with both sides from the GPU in int32 and the column sums from numpy."""
+    n = 4096
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda", generator=g)
+    w = torch.randint(-128, 128, (n, n), dtype=torch.int8, device="cuda", generator=g)
+    sym = K.qgemm(a, w, K.EPI_ACC_S32)
+    asym = K.qgemm(a, w, K.EPI_ACC_S32, zx=37)
+    colsum = w.to(torch.int32).sum(dim=1)
+    assert torch.equal(asym, sym - 37 * colsum[None, :])
+
+
 def test_qgemm_known_answers(K, golden):
     for case in golden["qgemm"]:
         m, k, n = case["m"], case["k"], case["n"]

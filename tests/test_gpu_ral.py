@@ -150,6 +150,39 @@ def test_ral_pdll_qgemm_cpu_style_signature(rt, bias_kind, rank):
     ctx.close()
 
 
+def test_ral_pdll_qgemm_cpu_style_zero_points(rt):
+    """Asymmetric input (one zero point) and a uniform weight zero point through the
+    CPU-signature entry: acc = sum (a - z_x)(w - z_w), the oneDNN semantics of the
+    reference's CPU entries; a weight zero-point vector that is not uniform is refused."""
+    ctx, ral, ops = rt
+    m, n, k = 200, 768, 768
+    rng = np.random.default_rng(91)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    sx = np.float32(0.02)
+    sw = rng.uniform(0.001, 0.02, n).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.5).astype(np.float32)
+    ctx = ral.RalContext(stream=torch.cuda.current_stream().cuda_stream)
+    with ctx.execution() as ex:
+        for zx, zw in ((17, 0), (-100, 4)):
+            acc = O.gemm_s32(a, w, tp_b=True, zx=zx, zw=zw)
+            so = np.float32(np.std(acc * (sx * sw.mean())) / 40)
+            want = O.requant_cpu(acc, sx, sw, so, b32=O.bias_f32_to_s32(bias, sx, sw), zo=-6)
+            got = ops.pdll_qgemm_cpu_style(ex, dev(a), dev(w), dev(bias), f1(sx), dev(sw), f1(so),
+                                           zo=-6, transpose_b=True, zx=zx, zw=zw)
+            np.testing.assert_array_equal(host(got), want)
+            got = ops.pdll_qgemm_cpu_style(ex, dev(a), dev(w.T.copy()), dev(bias), f1(sx), dev(sw),
+                                           f1(so), zo=-6, transpose_b=False, zx=zx, zw=zw)
+            np.testing.assert_array_equal(host(got), want)
+        zw_vec = np.zeros(n, np.int32)
+        zw_vec[5] = 1
+        with pytest.raises(ral.RalError, match="per-channel weight zero points"):
+            ops.pdll_qgemm_cpu_style(ex, dev(a), dev(w), dev(bias), f1(sx), dev(sw), f1(np.float32(1)),
+                                     transpose_b=True, zw=zw_vec)
+    torch.cuda.synchronize()
+    ctx.close()
+
+
 def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
     ctx, ral, ops = rt
     with ctx.execution() as ex:
