@@ -371,6 +371,41 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
         np.testing.assert_array_equal(got, want, err_msg="variant %d" % v)
 
 
+def test_qconv_direct_random_shapes(K):
+    """Seeded sweep for the kernels that keep the input patch in LDS: image sizes that make
+    tiles start and end anywhere in a row, every channel count, ragged output channels,
+    asymmetric padding, both tile shapes, two epilogues -- bit-exact against the oracle."""
+    rng = np.random.default_rng(20250117)
+    names = K.variant_names()
+    direct = [i for i, nm in enumerate(names) if nm.startswith("direct3x3_")]
+    for case in range(24):
+        nb = int(rng.integers(1, 4))
+        h = int(rng.integers(3, 40))
+        w_ = int(rng.integers(3, 70))
+        ci = int(rng.choice([32, 64, 128, 256]))
+        co = int(rng.choice([8, 17, 64, 72, 130]))
+        pad = [int(v) for v in rng.integers(0, 3, 4)]          # top, bottom, left, right
+        ho, wo = h + pad[0] + pad[1] - 2, w_ + pad[2] + pad[3] - 2
+        if ho < 1 or wo < 1 or (ho + 10) * (wo + 2) * ci > 120 * 1024:
+            continue
+        x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, 3, 3, ci), dtype=np.int8)
+        md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+        out_shape = [nb, ho, wo, co]
+        acc = O.conv_s32(x, wt, pad, md, out_shape)
+        sx, sw = make_scales(rng, co)
+        so = pick_so(acc, sx, sw)
+        want = O.requant_cpu(acc.reshape(-1, co), sx, sw, so).reshape(out_shape)
+        tag = "case %d: %dx%dx%dx%d -> %d pad %s" % (case, nb, h, w_, ci, co, pad)
+        for v in direct:
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_ACC_S32, variant=v))
+            np.testing.assert_array_equal(got, acc, err_msg=tag + " variant %d" % v)
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU,
+                                 sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])),
+                                 variant=v))
+            np.testing.assert_array_equal(got, want, err_msg=tag + " variant %d" % v)
+
+
 def test_qconv_direct_variants_refuse_what_they_cannot_run(K):
     """A named direct-convolution variant fails with an error, not a wrong result, on a
     filter that is not 3x3 stride 1, on a channel count it has no layout for, and on an image
