@@ -38,6 +38,7 @@ _PROTOS = {
                                    C.POINTER(_I64), _INT, _VP, _INT, _VP, _VP, _I64,
                                    _VP, _I32, _VP]),
     "dq8_mfma_probe": (_INT, [_VP] * 7),
+    "dq8_lut8": (_INT, [_VP, _VP, _I64, _VP, _VP]),
     "dq8_minmax_workspace_bytes": (_SZ, [_I64, _I64, _I64]),
     "dq8_minmax": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP, _SZ, _VP]),
 }

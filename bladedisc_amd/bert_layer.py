@@ -41,6 +41,9 @@ class RawBackend:
         """E1: sat8(rne((acc + b32) * (sx*sw/so))) with the f32 bias folded to int32."""
         return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so, bias=bias)
 
+    def lut8(self, q, table):
+        return K.lut8(q, table)
+
 
 class RalBackend:
     name = "ral"
@@ -59,6 +62,11 @@ class RalBackend:
         return ral_ops.pdll_qgemm_cpu_style(self.ex, x_q, w_q, bias, sx, sw, so,
                                             transpose_b=True, weight_is_const=True)
 
+    def lut8(self, q, table):
+        # a compiled program would carry this as one of its own generated kernels; the
+        # runtime has no entry for it
+        return K.lut8(q, table)
+
 
 def _layer_norm(x, g, b):
     return torch.nn.functional.layer_norm(x, (x.shape[-1],), g, b, 1e-12)
@@ -67,7 +75,13 @@ def _layer_norm(x, g, b):
 class QuantBertLayer:
     """One encoder layer; hidden 768, 12 heads, FFN 3072 by default."""
 
-    def __init__(self, weights, backend, heads=12, device="cuda"):
+    def __init__(self, weights, backend, heads=12, device="cuda", fuse_gelu=False):
+        """fuse_gelu: run dequantize -> GELU -> quantize between the two FFN linears as one
+        256-entry table lookup on the int8 tensor (what the compiler's fusion of those three
+        elementwise operators amounts to); the result is bit-identical to the three separate
+        operators because the table is built by running exactly them on all 256 inputs."""
+        self.fuse_gelu = fuse_gelu
+        self.gelu_table = None
         self.be = backend
         self.heads = heads
         self.device = device
@@ -129,19 +143,38 @@ class QuantBertLayer:
             for which, store in (("in", self.s_in), ("out", self.s_out)):
                 amax = rec["%s_%s" % (name, which)].abs().max().clamp_min(1e-12)
                 store[name] = (amax / 127.0).reshape(1).float()
+        self.gelu_table = K.activation_table(torch.nn.functional.gelu, self.s_out["ffn1"],
+                                             self.be.z1, self.s_in["ffn2"], self.be.z1)
         return rec
 
     # ----------------------------------------------------------- quantized layer
+    def _gemm(self, name, x_q):
+        return self.be.qlinear(x_q, self.w_q[name], self.bias[name], self.s_in[name],
+                               self.sw[name], self.s_out[name])
+
     def _qlinear(self, name, x, rec):
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         x_q = self.be.quantize(x2, self.s_in[name])
-        y_q = self.be.qlinear(x_q, self.w_q[name], self.bias[name], self.s_in[name],
-                              self.sw[name], self.s_out[name])
+        y_q = self._gemm(name, x_q)
         y = self.be.dequantize(y_q, self.s_out[name])
         if rec is not None:
             rec[name] = dict(x=x2, x_q=x_q, y_q=y_q, y=y)
         return y.reshape(*shape[:-1], y.shape[-1])
+
+    def _ffn_fused(self, h1, rec):
+        """quantize -> ffn1 -> [table: dequantize, GELU, quantize] -> ffn2 -> dequantize."""
+        shape = h1.shape
+        x2 = h1.reshape(-1, shape[-1])
+        x_q = self.be.quantize(x2, self.s_in["ffn1"])
+        y1_q = self._gemm("ffn1", x_q)
+        x2_q = self.be.lut8(y1_q, self.gelu_table)
+        y2_q = self._gemm("ffn2", x2_q)
+        y2 = self.be.dequantize(y2_q, self.s_out["ffn2"])
+        if rec is not None:
+            rec["ffn1"] = dict(x=x2, x_q=x_q, y_q=y1_q)
+            rec["ffn2"] = dict(x_q=x2_q, y_q=y2_q, y=y2)
+        return y2.reshape(*shape[:-1], y2.shape[-1])
 
     def capture(self, h):
         """Records one forward pass on `h`'s shape into a HIP graph and returns
@@ -171,7 +204,10 @@ class QuantBertLayer:
         ctx = self.attention(qkv)
         attn = self._qlinear("out", ctx, record)
         h1 = _layer_norm(h + attn, self.f["ln1_g"], self.f["ln1_b"])
-        f1 = self._qlinear("ffn1", h1, record)
-        g = torch.nn.functional.gelu(f1)
-        f2 = self._qlinear("ffn2", g, record)
+        if self.fuse_gelu:
+            f2 = self._ffn_fused(h1, record)
+        else:
+            f1 = self._qlinear("ffn1", h1, record)
+            g = torch.nn.functional.gelu(f1)
+            f2 = self._qlinear("ffn2", g, record)
         return _layer_norm(h1 + f2, self.f["ln2_g"], self.f["ln2_b"])

@@ -95,6 +95,34 @@ def minmax(x, min_io, max_io, axis=None, workspace=None):
     return min_io, max_io
 
 
+def lut8(q, table, out=None):
+    """out[i] = table[bit pattern of q[i]] for an int8 / uint8 device tensor; `table` is a
+    256-entry device tensor of the output's 8-bit type."""
+    _need_cuda(q, table)
+    if q.element_size() != 1 or table.element_size() != 1 or table.numel() != 256:
+        raise TypeError("lut8 takes 8-bit tensors and a 256-entry table")
+    q = q.contiguous()
+    if out is None:
+        out = torch.empty(q.shape, dtype=table.dtype, device=q.device)
+    st = _lib.lib().dq8_lut8(_ptr(q), _ptr(out), q.numel(), _ptr(table), _stream())
+    _lib.check(st, "dq8_lut8")
+    return out
+
+
+def activation_table(fn, s_in, z_in, s_out, z_out, in_dtype=torch.int8, out_dtype=torch.int8,
+                     device="cuda"):
+    """The table of  q -> quantize(fn(dequantize(q, s_in, z_in)), s_out, z_out)  for every
+    8-bit q, built with the same dequantize / quantize kernels a chain of separate operators
+    would run, so that  lut8(q, table)  equals that chain bit for bit.  s_*: one-element
+    device f32 tensors, z_*: one-element device i32 tensors; fn: a torch elementwise function.
+    Entry i belongs to the input whose bit pattern is i."""
+    bits = torch.arange(256, dtype=torch.int16, device=device).to(torch.uint8)
+    q = bits.view(in_dtype) if in_dtype != torch.uint8 else bits
+    y = fn(dequantize(q, s_in, z_in))
+    qmin, qmax = (-128, 127) if out_dtype == torch.int8 else (0, 255)
+    return quantize(y, s_out, z_out, qmin=qmin, qmax=qmax, dtype=out_dtype)
+
+
 def dequantize(q, scale, zero_point, axis=None, out=None):
     _need_cuda(q, scale, zero_point)
     q = q.contiguous()

@@ -99,6 +99,16 @@ int dq8_dequantize(const void* q, int in_kind, float* out, int64_t outer,
                    int64_t nch, int64_t inner, const float* scale,
                    const int32_t* zp, int64_t n_q, void* stream);
 
+/* ---- elementwise function between two quantized tensors ----------------- */
+
+/* out[i] = table[in[i]] over n bytes (device; in == out allowed), `table` = 256 device bytes
+ * indexed by the input byte's bit pattern (for int8 data: index (uint8_t)q).  The compiler
+ * fuses dequantize -> activation -> quantize chains between two quantized operators into one
+ * generated kernel (R disc/transforms/disc_lower_quantize_and_dequantize.cc lowers both ends
+ * to elementwise ops that the fusion pass merges with the activation); since the chain's
+ * input takes at most 256 values, its result is exactly a table, whatever the activation. */
+int dq8_lut8(const void* in, void* out, int64_t n, const void* table, void* stream);
+
 /* ---- int8 GEMM -------------------------------------------------------- */
 
 /* Bytes of device scratch dq8_qgemm needs for this problem with zx == zw == 0 (0 when it

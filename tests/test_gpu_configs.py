@@ -180,6 +180,27 @@ def test_config5_bert_layer(C, seq, backend):
             ctx.close()
 
 
+@pytest.mark.parametrize("seq", [32, 384])
+def test_config5_bert_layer_gelu_as_table_is_bit_identical(C, seq):
+    """dequantize -> GELU -> quantize between the two FFN linears as one table lookup on the
+    int8 tensor: same int8 input to the second linear, same layer output, bit for bit."""
+    from bladedisc_amd import bert_layer as B
+    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend())
+    h = layer.embed(C.config5_tokens(8, seq))
+    layer.calibrate(h)
+    rec_a, rec_b = {}, {}
+    want = layer.forward(h, rec_a)
+    layer.fuse_gelu = True
+    got = layer.forward(h, rec_b)
+    torch.cuda.synchronize()
+    assert torch.equal(rec_b["ffn1"]["y_q"], rec_a["ffn1"]["y_q"])
+    assert torch.equal(rec_b["ffn2"]["x_q"], rec_a["ffn2"]["x_q"])
+    assert torch.equal(got, want)
+    # the table really bends the values (GELU is not the identity on this range)
+    t = layer.gelu_table.cpu().numpy().astype(np.int32)
+    assert t.min() <= 0 and t.max() > 50 and (t[128:] <= 0).all()     # negatives map near 0-
+
+
 def test_config5_bert_layer_graph_replays_match_eager(C):
     """The captured layer against eager execution: several replays, with eager work and
     synchronisations in between, each compared bit for bit."""

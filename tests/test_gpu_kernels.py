@@ -323,6 +323,46 @@ def test_quantize_empty(K):
     assert K.quantize(x, s, z).shape == (0, 8)
 
 
+# ------------------------------------------------------------------------- table
+@pytest.mark.parametrize("n", [0, 1, 15, 16, 17, 4099, 1 << 20])
+def test_lut8_matches_numpy_take(K, n):
+    rng = np.random.default_rng(n)
+    table = rng.integers(-128, 128, 256, dtype=np.int8)
+    q = rng.integers(-128, 128, n, dtype=np.int8)
+    want = table[q.view(np.uint8)]
+    got = K.lut8(dev(q), dev(table))
+    np.testing.assert_array_equal(host(got), want)
+    if n > 20:
+        base = dev(np.concatenate([[0], q]).astype(np.int8))
+        view = base[1:]                                      # 1-byte aligned only
+        np.testing.assert_array_equal(host(K.lut8(view, dev(table))), want)
+        buf = dev(q)
+        K.lut8(buf, dev(table), out=buf)                     # in place
+        np.testing.assert_array_equal(host(buf), want)
+    u = rng.integers(0, 256, max(n, 1), dtype=np.uint8)
+    tu = rng.integers(0, 256, 256, dtype=np.uint8)
+    np.testing.assert_array_equal(host(K.lut8(dev(u), dev(tu))), tu[u])
+
+
+def test_activation_table_equals_the_operator_chain(K):
+    """table[q] = quantize(f(dequantize(q))) built from the kernels themselves: a lookup
+    equals running the three operators, for an asymmetric input and output."""
+    rng = np.random.default_rng(2)
+    q = dev(rng.integers(-128, 128, (300, 77), dtype=np.int8))
+    s_in, z_in = dev(np.array([0.037], np.float32)), dev(np.array([-11], np.int32))
+    s_out, z_out = dev(np.array([0.021], np.float32)), dev(np.array([7], np.int32))
+    for fn in (torch.nn.functional.gelu, torch.tanh, torch.relu):
+        table = K.activation_table(fn, s_in, z_in, s_out, z_out)
+        chain = K.quantize(fn(K.dequantize(q, s_in, z_in)), s_out, z_out)
+        assert torch.equal(K.lut8(q, table), chain)
+        # and the oracle's view of it for one function with exact float32 semantics
+    table = host(K.activation_table(torch.relu, s_in, z_in, s_out, z_out))
+    allq = np.arange(256, dtype=np.uint8).view(np.int8)
+    deq = O.dequantize(allq, np.float32(0.037), np.array([-11], np.int32))
+    want = O.quantize(np.maximum(deq, 0), np.float32(0.021), np.array([7], np.int32))
+    np.testing.assert_array_equal(table, want)
+
+
 # ------------------------------------------------------------------------- conv
 CONVS = [  # nb, h, w, ci, co, k, stride, pad, dil
     (2, 14, 14, 64, 64, 3, 1, 1, 1),
