@@ -435,6 +435,22 @@ def extras(torch, steps, warmup, which="all"):
         gbps = 4.0 * rows * cols * reps / ev / 1e9
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 4}
+    # tf.QuantizeV2 / tf.Dequantize (mode SCALED), ranges as device operands; the wrappers
+    # allocate their results, from torch's caching allocator after the first call
+    from bladedisc_amd import tf_quant as TQ
+    mn1, mx1 = torch.full((), -4.0, device="cuda"), torch.full((), 4.0, device="cuda")
+    mnc, mxc = torch.full((cols,), -4.0, device="cuda"), torch.full((cols,), 4.0, device="cuda")
+    tf_cases = (("tf_quantize_v2_scaled_per_tensor", lambda: TQ.quantize_v2(x, mn1, mx1, mode="SCALED")),
+                ("tf_quantize_v2_scaled_last_axis", lambda: TQ.quantize_v2(x, mnc, mxc, mode="SCALED", axis=1)),
+                ("tf_dequantize_scaled_per_tensor", lambda: TQ.dequantize(q, mn1, mx1, mode="SCALED")))
+    for _, fn in tf_cases:
+        for _ in range(3):
+            fn()
+    for name, fn in tf_cases:
+        _, ev = time_steps(torch, fn, reps, 3)
+        gbps = nbytes * reps / ev / 1e9
+        out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
+                     "shape": [rows, cols], "bytes_per_elem": 5}
     del x, q, f
     # smaller activations (they fit the 256 MB last-level cache; launches captured in a graph)
     small = {}

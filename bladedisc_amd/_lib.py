@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_PKG, "libdisc_q8_ral.so")
 _lib = None
 
 _I64, _I32, _INT, _VP, _SZ = C.c_int64, C.c_int32, C.c_int, C.c_void_p, C.c_size_t
+_F32 = C.c_float
 
 # name -> (restype, argtypes); mirrors include/disc_q8.h
 _PROTOS = {
@@ -39,6 +40,11 @@ _PROTOS = {
                                    _VP, _I32, _VP]),
     "dq8_mfma_probe": (_INT, [_VP] * 7),
     "dq8_lut8": (_INT, [_VP, _VP, _I64, _VP, _VP]),
+    "dq8_tf_params_bytes": (_SZ, [_I64]),
+    "dq8_tf_quantize_v2": (_INT, [_VP, _VP, _INT, _I64, _I64, _I64, _VP, _VP, _INT, _INT, _F32,
+                                  _VP, _VP, _VP, _SZ, _VP]),
+    "dq8_tf_dequantize": (_INT, [_VP, _INT, _VP, _I64, _I64, _I64, _VP, _VP, _INT, _VP, _SZ,
+                                 _VP]),
     "dq8_minmax_workspace_bytes": (_SZ, [_I64, _I64, _I64]),
     "dq8_minmax": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP, _SZ, _VP]),
 }

@@ -1,0 +1,83 @@
+// Pieces shared by the bandwidth-bound elementwise kernels (quantize / dequantize in their
+// mhlo_disc and TensorFlow forms): byte packing and the launch shapes of the three access
+// patterns -- a linear sweep, [rows, channels] tiles with the channel on the last axis, and
+// one (outer, channel) row per blockIdx.y.
+#pragma once
+#include <algorithm>
+#include <cstdint>
+
+#include "dq8_common.h"
+
+namespace dq8 {
+namespace elementwise {
+
+constexpr int kThreads = 256;
+
+// A zero the compiler cannot see through.  Adding it to a workgroup-uniform index
+// turns the parameter fetch into a vector load, which is issued together with the
+// data load; as a scalar load it would be waited for (a cold miss, one per row) before
+// the data load even starts.
+__device__ __forceinline__ unsigned opaque_zero() {
+  unsigned z;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+  return z;
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+  return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) |
+         ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+
+template <bool SIGNED>
+__device__ __forceinline__ int4 unpack4(uint32_t w) {
+  if (SIGNED)
+    return make_int4((int8_t)(w & 0xff), (int8_t)((w >> 8) & 0xff), (int8_t)((w >> 16) & 0xff),
+                     (int8_t)(w >> 24));
+  return make_int4(w & 0xff, (w >> 8) & 0xff, (w >> 16) & 0xff, w >> 24);
+}
+
+inline int grid_for(int64_t work_items, int per_thread) {
+  // enough blocks to cover the work with `per_thread` items per thread, capped at
+  // 16 blocks per CU (256 CUs) so the grid-stride loops keep loads in flight
+  int64_t blocks = dq8::ceil_div(work_items, (int64_t)kThreads * per_thread);
+  if (blocks < 1) blocks = 1;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  return (int)blocks;
+}
+
+// Launch shape of the last-axis kernels: threads along the channel units, blockIdx.y
+// along rows; about 64 Ki workgroups (a sweep, as for the per-tensor kernels) of at
+// least 4 rows each so the per-channel parameters in registers are reused.
+struct LastAxisPlan {
+  int bx, by, gx, gy, rows_per_block;
+};
+inline LastAxisPlan plan_last_axis(int64_t rows, int units) {
+  LastAxisPlan p;
+  if (units >= kThreads) {
+    p.bx = kThreads;
+  } else {   // few channels: the next power of two, the rest of the workgroup goes to rows
+    p.bx = 1;
+    while (p.bx < units) p.bx *= 2;
+  }
+  p.by = kThreads / p.bx;
+  p.gx = (int)dq8::ceil_div(units, p.bx);
+  // each thread walks at least four of its rows; rows_per_block is a multiple of by
+  int64_t rpb = dq8::ceil_div(rows * p.gx, 65536);
+  if (rpb < 4 * p.by) rpb = 4 * p.by;
+  rpb = dq8::ceil_div(rpb, p.by) * p.by;
+  if (dq8::ceil_div(rows, rpb) > 65535) rpb = dq8::ceil_div(dq8::ceil_div(rows, 65535), p.by) * p.by;
+  p.rows_per_block = (int)rpb;
+  p.gy = (int)dq8::ceil_div(rows, rpb);
+  return p;
+}
+
+// one thread per unit, the whole tensor in one sweep
+inline unsigned sweep_grid(int64_t units) {
+  int64_t blocks = dq8::ceil_div(units, (int64_t)kThreads);
+  if (blocks < 1) blocks = 1;
+  if (blocks > (1LL << 22)) blocks = 1LL << 22;
+  return (unsigned)blocks;
+}
+
+}  // namespace elementwise
+}  // namespace dq8

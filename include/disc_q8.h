@@ -23,6 +23,9 @@
  *                  -> the loops the compiler generates from mhlo_disc.quantize /
  *                     mhlo_disc.dequantize
  *                     (R disc/transforms/disc_lower_quantize_and_dequantize.cc:36-139, 141-215).
+ *   dq8_tf_quantize_v2 / dq8_tf_dequantize
+ *                  -> the loops the compiler generates from tf.QuantizeV2 / tf.Dequantize
+ *                     (R disc/transforms/lower_tf.cc:307-560, 562-654).
  */
 #ifndef DISC_Q8_H_
 #define DISC_Q8_H_
@@ -57,6 +60,10 @@ extern "C" {
 /* mhlo_disc round_mode (R disc/IR/hlo_disc_enums.td) */
 #define DQ8_ROUND_HALF_AWAY_FROM_ZERO 0
 #define DQ8_ROUND_HALF_TO_EVEN 1
+
+/* tf.QuantizeV2 modes */
+#define DQ8_TF_SCALED 0
+#define DQ8_TF_MIN_FIRST 1
 
 /* ---- library ---------------------------------------------------------- */
 
@@ -108,6 +115,41 @@ int dq8_dequantize(const void* q, int in_kind, float* out, int64_t outer,
  * to elementwise ops that the fusion pass merges with the activation); since the chain's
  * input takes at most 256 values, its result is exactly a table, whatever the activation. */
 int dq8_lut8(const void* in, void* out, int64_t n, const void* table, void* stream);
+
+/* ---- TensorFlow's QuantizeV2 / Dequantize ------------------------------ */
+
+/* tf.QuantizeV2 as the reference lowers it (R disc/transforms/lower_tf.cc:307-560): x
+ * (device, f32) is viewed as [outer, channels, inner]; min_range / max_range (device f32)
+ * hold `channels` entries (1 = per tensor, the op's axis = -1).  For every channel the range
+ * is first adjusted (R :365-393: extended to contain zero and to be at least
+ * ensure_minimum_range * max(|min|, |max|, 1) wide), then
+ *   DQ8_TF_SCALED    (R :453-560)  f = min(min_q / min', max_q / max') over the sides whose
+ *                    product with the bound is positive, min_q = lowest + narrow_range;
+ *                    q = (T) round(clamp(x, min_q / f, max_q / f) * f);
+ *                    out_min / out_max = min_q / f, max_q / f
+ *   DQ8_TF_MIN_FIRST (R :395-451, channels = 1 only) r = (max' - min') / 255;
+ *                    q = (T) clamp(round(x r) - (round(min' r) - lowest), lowest, highest);
+ *                    out_min / out_max = min', max'
+ * Every step is a separately rounded f32 operation; round is tf.Round (half to even), the
+ * only rounding the reference's pattern accepts (it refuses round_mode HALF_TO_EVEN, whose
+ * TF kernel differs, and mode MIN_COMBINED).  out_min / out_max (device f32, `channels`
+ * entries) are the op's second and third results.  `params` (device, 16-byte aligned,
+ * dq8_tf_params_bytes(channels) bytes) is working storage; after the call its float
+ * [4 c + 2] is the factor channel c was multiplied by. */
+size_t dq8_tf_params_bytes(int64_t channels);
+int dq8_tf_quantize_v2(const float* x, void* out, int out_kind, int64_t outer, int64_t channels,
+                       int64_t inner, const float* min_range, const float* max_range, int mode,
+                       int narrow_range, float ensure_minimum_range, float* out_min,
+                       float* out_max, void* params, size_t params_bytes, void* stream);
+
+/* tf.Dequantize, mode SCALED (R disc/transforms/lower_tf.cc:562-654):
+ *   out = f[c] * (float) q,   f = max(min / min_q, max / highest) for int8 input,
+ *                             f = max / 255 for uint8 input.
+ * Same view and range operands as above; `params` as above (after the call its first
+ * `channels` floats are f). */
+int dq8_tf_dequantize(const void* q, int in_kind, float* out, int64_t outer, int64_t channels,
+                      int64_t inner, const float* min_range, const float* max_range,
+                      int narrow_range, void* params, size_t params_bytes, void* stream);
 
 /* ---- int8 GEMM -------------------------------------------------------- */
 
