@@ -41,6 +41,10 @@ class RawBackend:
         """E1: sat8(rne((acc + b32) * (sx*sw/so))) with the f32 bias folded to int32."""
         return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so, bias=bias)
 
+    def qlinear_dequantized(self, x_q, w_q, bias, sx, sw, so):
+        """qlinear followed by dequantize(., so), in the GEMM's epilogue: f32 out."""
+        return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU_DEQUANT_F32, sx=sx, sw=sw, so=so, bias=bias)
+
     def lut8(self, q, table):
         return K.lut8(q, table)
 
@@ -75,12 +79,16 @@ def _layer_norm(x, g, b):
 class QuantBertLayer:
     """One encoder layer; hidden 768, 12 heads, FFN 3072 by default."""
 
-    def __init__(self, weights, backend, heads=12, device="cuda", fuse_gelu=False):
-        """fuse_gelu: run dequantize -> GELU -> quantize between the two FFN linears as one
+    def __init__(self, weights, backend, heads=12, device="cuda", fuse_gelu=False,
+                 fuse_dequant=False):
+        """fuse_dequant (raw backend): a linear whose int8 result is only dequantized writes
+        the dequantized f32 from the GEMM's epilogue (same bits, no int8 round trip).
+        fuse_gelu: run dequantize -> GELU -> quantize between the two FFN linears as one
         256-entry table lookup on the int8 tensor (what the compiler's fusion of those three
         elementwise operators amounts to); the result is bit-identical to the three separate
         operators because the table is built by running exactly them on all 256 inputs."""
         self.fuse_gelu = fuse_gelu
+        self.fuse_dequant = fuse_dequant
         self.gelu_table = None
         self.be = backend
         self.heads = heads
@@ -152,12 +160,20 @@ class QuantBertLayer:
         return self.be.qlinear(x_q, self.w_q[name], self.bias[name], self.s_in[name],
                                self.sw[name], self.s_out[name])
 
+    def _gemm_dequantized(self, name, x_q):
+        """(y_q or None, y): the linear's int8 result and its dequantized form."""
+        if self.fuse_dequant:
+            return None, self.be.qlinear_dequantized(x_q, self.w_q[name], self.bias[name],
+                                                     self.s_in[name], self.sw[name],
+                                                     self.s_out[name])
+        y_q = self._gemm(name, x_q)
+        return y_q, self.be.dequantize(y_q, self.s_out[name])
+
     def _qlinear(self, name, x, rec):
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
         x_q = self.be.quantize(x2, self.s_in[name])
-        y_q = self._gemm(name, x_q)
-        y = self.be.dequantize(y_q, self.s_out[name])
+        y_q, y = self._gemm_dequantized(name, x_q)
         if rec is not None:
             rec[name] = dict(x=x2, x_q=x_q, y_q=y_q, y=y)
         return y.reshape(*shape[:-1], y.shape[-1])
@@ -169,8 +185,7 @@ class QuantBertLayer:
         x_q = self.be.quantize(x2, self.s_in["ffn1"])
         y1_q = self._gemm("ffn1", x_q)
         x2_q = self.be.lut8(y1_q, self.gelu_table)
-        y2_q = self._gemm("ffn2", x2_q)
-        y2 = self.be.dequantize(y2_q, self.s_out["ffn2"])
+        y2_q, y2 = self._gemm_dequantized("ffn2", x2_q)
         if rec is not None:
             rec["ffn1"] = dict(x=x2, x_q=x_q, y_q=y1_q)
             rec["ffn2"] = dict(x_q=x2_q, y_q=y2_q, y=y2)

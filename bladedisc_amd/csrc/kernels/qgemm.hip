@@ -33,7 +33,7 @@ __device__ __forceinline__ void store_one(const EpiParams& e, int m, int n, int 
   if (EPI == DQ8_EPI_ACC_S32)
     ((int32_t*)e.out)[off] = acc;
   else if (EPI == DQ8_EPI_DEQUANT_F32)
-    ((float*)e.out)[off] = dequant_one(e, c, acc);
+    ((float*)e.out)[off] = dequant_one(e, c, acc, dequant_so(e));
   else
     ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, acc);
 }
@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(256) qconv_generic_kernel(const GenericConvPar
     if (EPI == DQ8_EPI_ACC_S32)
       ((int32_t*)p.epi.out)[off] = acc;
     else if (EPI == DQ8_EPI_DEQUANT_F32)
-      ((float*)p.epi.out)[off] = dequant_one(p.epi, c, acc);
+      ((float*)p.epi.out)[off] = dequant_one(p.epi, c, acc, dequant_so(p.epi));
     else
       ((int8_t*)p.epi.out)[off] = (int8_t)requant_one<EPI>(p.epi, c, acc);
   }
@@ -155,6 +155,7 @@ zero_point_epilogue_kernel(const int32_t* __restrict__ acc, const int32_t* __res
   const int n = blockIdx.x * 256 + threadIdx.x;
   if (n >= e.N) return;
   const ColParams c = col_params<EPI>(e, n);
+  const float so_val = EPI == DQ8_EPI_DEQUANT_F32 ? dequant_so(e) : 0.0f;
   const unsigned cn = (unsigned)corr_n[n];
   const int m_begin = blockIdx.y * rows;
   const int m_end = m_begin + rows < e.M ? m_begin + rows : e.M;
@@ -164,7 +165,7 @@ zero_point_epilogue_kernel(const int32_t* __restrict__ acc, const int32_t* __res
     if (EPI == DQ8_EPI_ACC_S32)
       ((int32_t*)e.out)[off] = (int)a;
     else if (EPI == DQ8_EPI_DEQUANT_F32)
-      ((float*)e.out)[off] = dequant_one(e, c, (int)a);
+      ((float*)e.out)[off] = dequant_one(e, c, (int)a, so_val);
     else
       ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, (int)a);
   };
@@ -345,13 +346,19 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 //    CU's operand loads, not its MFMAs, set the pace (16 KiB per 128 of k against 128 MFMA
 //    cycles per SIMD); when few CUs are busy and K is deep, splitting K over two wave groups
 //    of the workgroup still shortens the chain of dependent k tiles (about 10 % at K = 3072).
-int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe) {
+//  * 4-byte outputs (int32 sums, f32): the epilogue writes four times as much and, with one
+//    256x256 tile per CU, all of it at the very end; while the main loop is short (K < 2048)
+//    128x128 tiles, several per CU, write under each other's main loops instead
+//    (3072 x 3072 x 768 to f32: 21.8 us against 26.1).
+int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) {
   auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
   if (pipe) {
     if (N <= 64 && M >= 256 * 64) return kPipe256x64;
     const int64_t t256 = tiles(kPipe256w8);
     const int64_t rounds = ceil_div(t256, 256);
-    if (t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * 256 * rounds)) return kPipe256w8;
+    if (t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * 256 * rounds) &&
+        (out_bytes == 1 || K >= 2048))
+      return kPipe256w8;
     if (tiles(kPipe128) >= 120) return K < 4096 ? kPipe128w8 : kPipe128;
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
@@ -479,19 +486,29 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   DQ8_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
               "dq8_qgemm: dimension exceeds 2^31-1");
   DQ8_REQUIRE(variant >= -1 && variant < kNumVariants, "dq8_qgemm: unknown variant");
+  // requant -> dequantize in one epilogue: validated as the requant form it starts with,
+  // run by the f32-output kernels
+  int requant = 0;
+  if (epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || epilogue == DQ8_EPI_REQUANT_GPU_DEQUANT_F32) {
+    requant = epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 ? 1 : 2;
+    DQ8_REQUIRE(n_so == 1, "dq8_qgemm: the requant -> dequantize epilogues take a per-tensor "
+                           "output scale");
+    epilogue = requant == 1 ? DQ8_EPI_REQUANT_CPU : DQ8_EPI_REQUANT_GPU;
+  }
   if (int s = check_epilogue("dq8_qgemm", epilogue, bias, bias_kind, sx, sw, so, n_sx,
                              n_sw, n_so, N))
     return s;
+  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
+              "dq8_qgemm: an output zero point needs the REQUANT_CPU epilogue");
+  if (requant) epilogue = DQ8_EPI_DEQUANT_F32;
   if (M == 0 || N == 0) return 0;
   DQ8_REQUIRE(out != nullptr, "dq8_qgemm: null output");
   DQ8_REQUIRE(K == 0 || (A && W), "dq8_qgemm: null operand");
   DQ8_REQUIRE(lda >= (tp_a ? M : K) && ldw >= (tp_b ? K : N) && ldo >= N,
               "dq8_qgemm: leading dimension smaller than the row length");
-  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
-              "dq8_qgemm: an output zero point needs the REQUANT_CPU epilogue");
   hipStream_t st = (hipStream_t)stream;
 
-  EpiParams e;
+  EpiParams e = {};
   e.out = out;
   e.ldo = ldo;
   e.M = (int)M;
@@ -505,6 +522,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   e.sw_stride = n_sw > 1;
   e.so_stride = n_so > 1;
   e.zo = zo;
+  e.requant = requant;
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
@@ -600,7 +618,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.K = (int)K;
   p.epi = e;
   if (auto_pick)
-    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false));
+    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false), zp_two_pass ? 4 : es);
   if (!zp_two_pass) return launch_epi<false>(variant, p, epilogue, st);
 
   // ---- zero points: raw sums into scratch, row-sum corrections, then the epilogue
@@ -712,7 +730,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
               "dq8_qconv2d: an output zero point needs the REQUANT_CPU epilogue");
   hipStream_t st = (hipStream_t)stream;
 
-  EpiParams e;
+  EpiParams e = {};
   e.out = out;
   e.ldo = Co;
   e.M = (int)Mg;
@@ -778,7 +796,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
     g.K = (int)Ci;
     g.epi = e;
     const int v = Mg <= kSkinnyMaxM ? kSkinnyVariant
-                                    : pick_variant(Mg, Co, Ci, pipe_ok(256, 256, g, false));
+                                    : pick_variant(Mg, Co, Ci, pipe_ok(256, 256, g, false), es);
     return launch_epi<false>(v, g, epilogue, st);
   }
 
@@ -816,7 +834,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
       const int c = pick_direct_conv(NB, Ho * Wo, Ci, Co);
       if (c >= 0 && direct_conv_plan(c, &d)) return launch_direct_conv(c, epilogue, d, st);
     }
-    variant = pick_variant(Mg, Co, Kg, pipe_ok(256, 256, p, true));
+    variant = pick_variant(Mg, Co, Kg, pipe_ok(256, 256, p, true), es);
   }
   return launch_epi<true>(variant, p, epilogue, st);
 }

@@ -39,6 +39,9 @@ struct EpiParams {
   const float* so;
   int sx_stride, sw_stride, so_stride;  // 0 (rank-0 scale) or 1 (per channel)
   int zo;
+  // DEQUANT_F32 only.  0: out = f32(acc) * (sx sw) + bias.  1 / 2: the REQUANT_CPU /
+  // REQUANT_GPU result q, dequantized in place: out = (float)(q - zo) * so[0].
+  int requant;
   int vec_store;    // 1: a group of 4 consecutive n may be stored as one 4/16-byte word
   int vec_store16;  // 1: int8 rows may be written with aligned 16-byte stores
 };
@@ -81,13 +84,18 @@ __device__ __forceinline__ ColParams col_params(const EpiParams& p, int n) {
   const float sx = p.sx[(int64_t)n * p.sx_stride];
   const float sw = p.sw[(int64_t)n * p.sw_stride];
   const float prod = sx * sw;
-  if (EPI == DQ8_EPI_DEQUANT_F32) {
+  // the arithmetic the factors are for: a compile-time constant except under DEQUANT_F32
+  const int mode = EPI != DQ8_EPI_DEQUANT_F32 ? EPI
+                   : p.requant == 1           ? DQ8_EPI_REQUANT_CPU
+                   : p.requant == 2           ? DQ8_EPI_REQUANT_GPU
+                                              : DQ8_EPI_DEQUANT_F32;
+  if (mode == DQ8_EPI_DEQUANT_F32) {
     c.os = prod;
     if (p.bias_kind == DQ8_BIAS_F32) c.b = ((const float*)p.bias)[n];
     return c;
   }
   const float so = p.so[(int64_t)n * p.so_stride];
-  if (EPI == DQ8_EPI_REQUANT_CPU) {
+  if (mode == DQ8_EPI_REQUANT_CPU) {
     c.os = prod / (1.0f * so);
     if (p.bias_kind == DQ8_BIAS_S32) {
       c.b = (float)((const int32_t*)p.bias)[n];
@@ -159,8 +167,31 @@ __device__ __forceinline__ uint32_t requant_pack4(const EpiParams& p, const ColP
   return lo | hi;
 }
 
+// The output scale the fused requant -> dequantize forms multiply by (one load per kernel;
+// unused otherwise).
+__device__ __forceinline__ float dequant_so(const EpiParams& p) {
+  return p.requant ? p.so[0] : 0.0f;
+}
+
 __device__ __forceinline__ float dequant_one(const EpiParams& p, const ColParams& c,
-                                             int acc) {
+                                             int acc, float so_val) {
+  if (p.requant) {
+    // requant_one's arithmetic, then dequantize's: (float)((int)q - zo) * so
+    float d = (float)acc;
+    if (p.requant == 1) {
+      d = d + c.b;
+      d = d * c.os;
+      d = d + (float)p.zo;
+    } else {
+      d = c.os * d;
+      d = d + c.b;
+    }
+    d = rintf(__builtin_amdgcn_fmed3f(d, -128.0f, 127.0f));
+    // (added, not subtracted: a rounded -0.0 becomes the +0.0 that the integer
+    // subtraction of dequantize yields)
+    d = d + (float)(-p.zo);
+    return d * so_val;
+  }
   float d = (float)acc * c.os;
   if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
   return d;
@@ -197,8 +228,9 @@ __device__ __forceinline__ void store_group4(const EpiParams& p, int m, int n,
   } else {
     float* out = (float*)p.out;
     float f[4];
+    const float so_val = dequant_so(p);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) f[e] = dequant_one(p, c[e], acc[e]);
+    for (int e = 0; e < 4; ++e) f[e] = dequant_one(p, c[e], acc[e], so_val);
     if (full && p.vec_store) {
       v4f w = {f[0], f[1], f[2], f[3]};
       *(v4f*)(out + off) = w;
@@ -519,6 +551,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     // tile, 128-byte rows with the 16-byte chunks swizzled by the row, then out as full
     // 128-byte row segments (8 lanes per row) instead of 32-byte pieces of 32 rows.
     int8_t* stage = smem + CP_BYTES + wave * 4096;
+    const float so_val = EPI == DQ8_EPI_DEQUANT_F32 ? dequant_so(e) : 0.0f;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
 #pragma unroll
@@ -538,7 +571,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
             const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-              w[q] = __float_as_int(dequant_one(e, c[q], acc[i][j][4 * g + q]));
+              w[q] = __float_as_int(dequant_one(e, c[q], acc[i][j][4 * g + q], so_val));
           }
           *reinterpret_cast<v4i*>(stage + r * 128 + ((chunk ^ (r & 7)) << 4)) = w;
         }

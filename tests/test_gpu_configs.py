@@ -201,6 +201,26 @@ def test_config5_bert_layer_gelu_as_table_is_bit_identical(C, seq):
     assert t.min() <= 0 and t.max() > 50 and (t[128:] <= 0).all()     # negatives map near 0-
 
 
+@pytest.mark.parametrize("seq", [32, 384])
+@pytest.mark.parametrize("fuse_gelu", [False, True])
+def test_config5_bert_layer_dequantize_in_the_gemm_epilogue_is_bit_identical(C, seq, fuse_gelu):
+    """Each linear whose int8 result is only dequantized writes the dequantized f32 from its
+    epilogue: the f32 tensors and the layer output keep their bits."""
+    from bladedisc_amd import bert_layer as B
+    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend(), fuse_gelu=fuse_gelu)
+    h = layer.embed(C.config5_tokens(8, seq))
+    layer.calibrate(h)
+    rec_a, rec_b = {}, {}
+    want = layer.forward(h, rec_a)
+    layer.fuse_dequant = True
+    got = layer.forward(h, rec_b)
+    torch.cuda.synchronize()
+    for name in ("qkv", "out", "ffn2"):
+        assert rec_b[name]["y_q"] is None
+        assert torch.equal(rec_b[name]["y"].view(torch.int32), rec_a[name]["y"].view(torch.int32))
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+
+
 def test_config5_bert_layer_graph_replays_match_eager(C):
     """The captured layer against eager execution: several replays, with eager work and
     synchronisations in between, each compared bit for bit."""

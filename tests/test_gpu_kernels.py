@@ -124,6 +124,52 @@ def test_qgemm_requant_gpu(K, per_channel, bias):
         np.testing.assert_array_equal(got, want, err_msg="variant %d" % v)
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 768, 768), (1000, 768, 3072), (257, 130, 64), (3072, 3072, 768),
+                                   (5, 130, 784)])
+@pytest.mark.parametrize("form", ["cpu_f32", "cpu_s32_zo", "gpu_s8", "gpu_none"])
+def test_qgemm_requant_then_dequantize_in_one_epilogue(K, m, n, k, form):
+    """Epilogues 4 / 5: the f32 result must equal, bit for bit, dequantize applied to the int8
+    result of the requant epilogue -- against the oracle's two functions and against the two
+    separate GPU kernels."""
+    rng = np.random.default_rng(m * 7 + n + k + len(form))
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    zo = 0
+    t = lambda v: dev(np.array([v], np.float32))
+    if form.startswith("cpu"):
+        epi, fused = K.EPI_REQUANT_CPU, K.EPI_REQUANT_CPU_DEQUANT_F32
+        if form == "cpu_f32":
+            bf = (rng.standard_normal(n) * 10 * so).astype(np.float32)
+            bias_t, b32 = dev(bf), O.bias_f32_to_s32(bf, sx, sw)
+        else:
+            b32 = rng.integers(-200000, 200000, n).astype(np.int32)
+            bias_t, zo = dev(b32), 5
+        q_want = O.requant_cpu(acc, sx, sw, so, b32=b32, zo=zo)
+    else:
+        epi, fused = K.EPI_REQUANT_GPU, K.EPI_REQUANT_GPU_DEQUANT_F32
+        bi = rng.integers(-128, 128, n).astype(np.int8) if form == "gpu_s8" else None
+        bias_t = dev(bi) if bi is not None else None
+        q_want = O.requant_gpu(acc, np.array([sx], np.float32), sw, np.array([so], np.float32),
+                               bias_i8=bi)
+    want = O.dequantize(q_want, np.array([so], np.float32), np.array([zo], np.int32))
+    sov, zov = t(so), dev(np.array([zo], np.int32))
+    for v in [-1] + gemm_variants(K, k):
+        got = K.qgemm(dev(a), dev(w), fused, sx=t(sx), sw=dev(sw), so=sov, bias=bias_t, zo=zo,
+                      variant=v)
+        assert got.dtype == torch.float32
+        two = K.dequantize(K.qgemm(dev(a), dev(w), epi, sx=t(sx), sw=dev(sw), so=sov, bias=bias_t,
+                                   zo=zo, variant=v), sov, zov)
+        assert torch.equal(got, two), "variant %d" % v
+        assert np.array_equal(host(got).view(np.uint32), want.view(np.uint32)), "variant %d" % v
+    # a per-channel output scale is refused
+    with pytest.raises(RuntimeError, match="per-tensor"):
+        K.qgemm(dev(a), dev(w), fused, sx=t(sx), sw=dev(sw), so=dev(np.full(n, so, np.float32)),
+                bias=bias_t, zo=zo)
+
+
 def test_qgemm_dequant_f32(K):
     m, n, k = 64, 768, 768
     rng = np.random.default_rng(5)
