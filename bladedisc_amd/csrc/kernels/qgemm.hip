@@ -33,7 +33,7 @@ __device__ __forceinline__ void store_one(const EpiParams& e, int m, int n, int 
   if (EPI == DQ8_EPI_ACC_S32)
     ((int32_t*)e.out)[off] = acc;
   else if (EPI == DQ8_EPI_DEQUANT_F32)
-    ((float*)e.out)[off] = dequant_one(e, c, acc, dequant_so(e));
+    ((float*)e.out)[off] = dequant_one_any(e, c, acc, dequant_so(e));
   else
     ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, acc);
 }
@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(256) qconv_generic_kernel(const GenericConvPar
     if (EPI == DQ8_EPI_ACC_S32)
       ((int32_t*)p.epi.out)[off] = acc;
     else if (EPI == DQ8_EPI_DEQUANT_F32)
-      ((float*)p.epi.out)[off] = dequant_one(p.epi, c, acc, dequant_so(p.epi));
+      ((float*)p.epi.out)[off] = dequant_one_any(p.epi, c, acc, dequant_so(p.epi));
     else
       ((int8_t*)p.epi.out)[off] = (int8_t)requant_one<EPI>(p.epi, c, acc);
   }
@@ -159,25 +159,32 @@ zero_point_epilogue_kernel(const int32_t* __restrict__ acc, const int32_t* __res
   const unsigned cn = (unsigned)corr_n[n];
   const int m_begin = blockIdx.y * rows;
   const int m_end = m_begin + rows < e.M ? m_begin + rows : e.M;
-  auto finish = [&](int m, int raw) {
-    const unsigned a = (unsigned)raw + cn + (corr_m ? (unsigned)corr_m[m] : 0u);
-    const int64_t off = (int64_t)m * e.ldo + n;
-    if (EPI == DQ8_EPI_ACC_S32)
-      ((int32_t*)e.out)[off] = (int)a;
-    else if (EPI == DQ8_EPI_DEQUANT_F32)
-      ((float*)e.out)[off] = dequant_one(e, c, (int)a, so_val);
-    else
-      ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, (int)a);
+  auto walk = [&](auto form) {
+    constexpr int FORM = decltype(form)::value;
+    auto finish = [&](int m, int raw) {
+      const unsigned a = (unsigned)raw + cn + (corr_m ? (unsigned)corr_m[m] : 0u);
+      const int64_t off = (int64_t)m * e.ldo + n;
+      if (EPI == DQ8_EPI_ACC_S32)
+        ((int32_t*)e.out)[off] = (int)a;
+      else if (EPI == DQ8_EPI_DEQUANT_F32)
+        ((float*)e.out)[off] = dequant_one<FORM>(e, c, (int)a, so_val);
+      else
+        ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, (int)a);
+    };
+    int m = m_begin;
+    for (; m + 3 < m_end; m += 4) {
+      int raw[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) raw[u] = acc[(int64_t)(m + u) * e.N + n];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) finish(m + u, raw[u]);
+    }
+    for (; m < m_end; ++m) finish(m, acc[(int64_t)m * e.N + n]);
   };
-  int m = m_begin;
-  for (; m + 3 < m_end; m += 4) {
-    int raw[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) raw[u] = acc[(int64_t)(m + u) * e.N + n];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) finish(m + u, raw[u]);
-  }
-  for (; m < m_end; ++m) finish(m, acc[(int64_t)m * e.N + n]);
+  if (EPI == DQ8_EPI_DEQUANT_F32)
+    dispatch_f32_form(e, walk);
+  else
+    walk(IntC<kF32Plain>());
 }
 
 // one MFMA of each shape, operands straight from global memory

@@ -173,12 +173,22 @@ __device__ __forceinline__ float dequant_so(const EpiParams& p) {
   return p.requant ? p.so[0] : 0.0f;
 }
 
+// The four forms of the f32 epilogue.  Which one a launch runs is uniform over the kernel:
+// the loops over the accumulators are instantiated per form (dispatch_f32_form) so that no
+// per-element code tests it.
+enum F32Form { kF32Plain = 0, kF32PlainBias = 1, kF32RequantCpu = 2, kF32RequantGpu = 3 };
+
+__device__ __forceinline__ int f32_form(const EpiParams& p) {
+  return p.requant ? 1 + p.requant : (p.bias_kind != DQ8_BIAS_NONE ? 1 : 0);
+}
+
+template <int FORM>
 __device__ __forceinline__ float dequant_one(const EpiParams& p, const ColParams& c,
                                              int acc, float so_val) {
-  if (p.requant) {
+  if (FORM == kF32RequantCpu || FORM == kF32RequantGpu) {
     // requant_one's arithmetic, then dequantize's: (float)((int)q - zo) * so
     float d = (float)acc;
-    if (p.requant == 1) {
+    if (FORM == kF32RequantCpu) {
       d = d + c.b;
       d = d * c.os;
       d = d + (float)p.zo;
@@ -193,8 +203,32 @@ __device__ __forceinline__ float dequant_one(const EpiParams& p, const ColParams
     return d * so_val;
   }
   float d = (float)acc * c.os;
-  if (p.bias_kind != DQ8_BIAS_NONE) d = d + c.b;
+  if (FORM == kF32PlainBias) d = d + c.b;
   return d;
+}
+
+template <int V>
+struct IntC {
+  static constexpr int value = V;
+};
+
+// body(IntC<form>) for the launch's form
+template <typename Body>
+__device__ __forceinline__ void dispatch_f32_form(const EpiParams& p, Body&& body) {
+  switch (f32_form(p)) {
+    case kF32Plain: body(IntC<kF32Plain>()); break;
+    case kF32PlainBias: body(IntC<kF32PlainBias>()); break;
+    case kF32RequantCpu: body(IntC<kF32RequantCpu>()); break;
+    default: body(IntC<kF32RequantGpu>()); break;
+  }
+}
+
+// one result, form looked up per call (the slow paths)
+__device__ __forceinline__ float dequant_one_any(const EpiParams& p, const ColParams& c,
+                                                 int acc, float so_val) {
+  float r = 0.0f;
+  dispatch_f32_form(p, [&](auto form) { r = dequant_one<decltype(form)::value>(p, c, acc, so_val); });
+  return r;
 }
 
 // Stores the results for row m, columns n .. n+3 (n % 4 == 0).
@@ -230,7 +264,7 @@ __device__ __forceinline__ void store_group4(const EpiParams& p, int m, int n,
     float f[4];
     const float so_val = dequant_so(p);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) f[e] = dequant_one(p, c[e], acc[e], so_val);
+    for (int e = 0; e < 4; ++e) f[e] = dequant_one_any(p, c[e], acc[e], so_val);
     if (full && p.vec_store) {
       v4f w = {f[0], f[1], f[2], f[3]};
       *(v4f*)(out + off) = w;
@@ -552,6 +586,8 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     // 128-byte row segments (8 lanes per row) instead of 32-byte pieces of 32 rows.
     int8_t* stage = smem + CP_BYTES + wave * 4096;
     const float so_val = EPI == DQ8_EPI_DEQUANT_F32 ? dequant_so(e) : 0.0f;
+    auto store_all = [&](auto form) {
+    constexpr int FORM = decltype(form)::value;
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
 #pragma unroll
@@ -571,7 +607,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
             const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-              w[q] = __float_as_int(dequant_one(e, c[q], acc[i][j][4 * g + q], so_val));
+              w[q] = __float_as_int(dequant_one<FORM>(e, c[q], acc[i][j][4 * g + q], so_val));
           }
           *reinterpret_cast<v4i*>(stage + r * 128 + ((chunk ^ (r & 7)) << 4)) = w;
         }
@@ -593,6 +629,11 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
         }
       }
     }
+    };
+    if (EPI == DQ8_EPI_DEQUANT_F32)
+      dispatch_f32_form(e, store_all);
+    else
+      store_all(IntC<kF32Plain>());
     return;
   }
 
