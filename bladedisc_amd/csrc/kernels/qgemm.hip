@@ -725,16 +725,23 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   DQ8_REQUIRE(Ho == out_len(H, padding[0], padding[1], Kh, dh, sh) &&
                   Wo == out_len(Wd, padding[2], padding[3], Kw, dw, sw_),
               "dq8_qconv2d: output spatial size inconsistent with padding/stride/dilation");
+  // requant -> dequantize in one epilogue, as in dq8_qgemm
+  int requant = 0;
+  if (epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || epilogue == DQ8_EPI_REQUANT_GPU_DEQUANT_F32) {
+    requant = epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 ? 1 : 2;
+    epilogue = requant == 1 ? DQ8_EPI_REQUANT_CPU : DQ8_EPI_REQUANT_GPU;
+  }
   if (int s = check_epilogue("dq8_qconv2d", epilogue, bias, bias_kind, sx, sw, so, 1, n_sw, 1, Co))
     return s;
+  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
+              "dq8_qconv2d: an output zero point needs the REQUANT_CPU epilogue");
+  if (requant) epilogue = DQ8_EPI_DEQUANT_F32;
   const int64_t Mg = NB * Ho * Wo, Kg = Kh * Kw * Ci;
   DQ8_REQUIRE(Mg < (1LL << 31) && Kg < (1LL << 31) && Co < (1LL << 31) &&
                   NB * H * Wd * Ci < (1LL << 40),
               "dq8_qconv2d: problem too large");
   if (Mg == 0 || Co == 0) return 0;
   DQ8_REQUIRE(in && w && out, "dq8_qconv2d: null tensor");
-  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
-              "dq8_qconv2d: an output zero point needs the REQUANT_CPU epilogue");
   hipStream_t st = (hipStream_t)stream;
 
   EpiParams e = {};
@@ -751,6 +758,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   e.sw_stride = n_sw > 1;
   e.so_stride = 0;
   e.zo = zo;
+  e.requant = requant;
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (Co % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (Co % 16 == 0);

@@ -10,7 +10,7 @@ import torch
 from . import _lib
 
 EPI_ACC_S32, EPI_REQUANT_CPU, EPI_REQUANT_GPU, EPI_DEQUANT_F32 = 0, 1, 2, 3
-# qgemm only: requant, then dequantize with the per-tensor output scale, in one epilogue
+# requant, then dequantize with the per-tensor output scale, in one epilogue
 EPI_REQUANT_CPU_DEQUANT_F32, EPI_REQUANT_GPU_DEQUANT_F32 = 4, 5
 BIAS_NONE, BIAS_S32, BIAS_F32, BIAS_S8 = 0, 1, 2, 3
 ROUND_HALF_AWAY_FROM_ZERO, ROUND_HALF_TO_EVEN = 0, 1

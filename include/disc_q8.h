@@ -44,7 +44,7 @@ extern "C" {
 #define DQ8_EPI_REQUANT_CPU 1 /* out: int8   sat(rne((f32(acc)+b32[n])*os[n] + zo))        */
 #define DQ8_EPI_REQUANT_GPU 2 /* out: int8   sat(rne(os[n]*f32(acc) + bias[n]))            */
 #define DQ8_EPI_DEQUANT_F32 3 /* out: float  f32(acc)*(sx*sw[n]) + bias[n]                 */
-/* dq8_qgemm only: the int8 result q of REQUANT_CPU / REQUANT_GPU dequantized in the same
+/* dq8_qgemm and dq8_qconv2d: the int8 result q of REQUANT_CPU / REQUANT_GPU dequantized in the same
  * epilogue, out: float (float)(q - zo) * so -- bit for bit what dq8_dequantize makes of the
  * requantized output, without the int8 round trip through memory.  Per-tensor `so` only;
  * bias kinds and zero points as for the requant form. */

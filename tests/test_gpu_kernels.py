@@ -455,6 +455,13 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
         got = host(K.qconv2d(dev(x), dev(wt), padding, md, out_shape, K.EPI_REQUANT_CPU,
                              sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])), variant=v))
         np.testing.assert_array_equal(got, want, err_msg="variant %d" % v)
+    # requant -> dequantize in the convolution's epilogue: the bits of dequantize(requant)
+    want_f = O.dequantize(want, np.array([so], np.float32), np.array([0], np.int32))
+    for v in variants:
+        got = host(K.qconv2d(dev(x), dev(wt), padding, md, out_shape, K.EPI_REQUANT_CPU_DEQUANT_F32,
+                             sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])), variant=v))
+        assert got.dtype == np.float32
+        assert np.array_equal(got.view(np.uint32), want_f.view(np.uint32)), "variant %d" % v
 
 
 def test_qconv_direct_random_shapes(K):
