@@ -29,6 +29,16 @@
 //     reference reads element 0 only).
 //   * errors are reported through Context::signalError and the entry returns; no
 //     kernel is launched after an error.
+//   * DISC_GPU_ENABLE_PROFILE=1 (or "true") makes the GEMM and convolution entries time
+//     their kernels with a pair of events, wait for them, and log the fields the reference
+//     prints under DISC_CPU_ENABLE_PROFILE (R context/common_context_impl.cc:66-73, 116-119;
+//     R context/common_context_impl_quantization.cc:722-743): operand pointers, m / n / k,
+//     "Math Ops", "Bytes", bandwidth and rate.  Off by default; on, every call blocks.
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cctype>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -60,6 +70,56 @@ bool kernelFailed(ExecutionContext* ctx, int status, const char* who) {
   fail(ctx, std::string(who) + ": " + dq8_last_error());
   return true;
 }
+
+bool initProfileMode() {
+  const char* env = std::getenv("DISC_GPU_ENABLE_PROFILE");
+  if (!env) return false;
+  std::string v = env;
+  std::transform(v.begin(), v.end(), v.begin(),
+                 [](unsigned char c) { return (char)std::tolower(c); });
+  return v == "true" || v == "1";
+}
+
+bool isProfilingEnabled() {
+  static bool enabled = initProfileMode();
+  return enabled;
+}
+
+// Times what is put on `stream` between construction and stop() (profile mode only;
+// stop() waits for the stream).  Event failures switch the timer off rather than
+// failing the call.
+class StreamTimer {
+ public:
+  explicit StreamTimer(void* stream) : stream_(static_cast<hipStream_t>(stream)) {
+    if (!isProfilingEnabled()) return;
+    if (hipEventCreate(&begin_) != hipSuccess) return;
+    if (hipEventCreate(&end_) != hipSuccess) {
+      (void)hipEventDestroy(begin_);
+      return;
+    }
+    on_ = hipEventRecord(begin_, stream_) == hipSuccess;
+  }
+  ~StreamTimer() {
+    if (begin_) (void)hipEventDestroy(begin_);
+    if (end_) (void)hipEventDestroy(end_);
+    (void)hipGetLastError();
+  }
+  bool on() const { return on_; }
+  // nanoseconds since construction, or a negative value
+  double stop() {
+    float ms = -1.0f;
+    if (!on_ || hipEventRecord(end_, stream_) != hipSuccess ||
+        hipEventSynchronize(end_) != hipSuccess ||
+        hipEventElapsedTime(&ms, begin_, end_) != hipSuccess)
+      return -1.0;
+    return (double)ms * 1e6;
+  }
+
+ private:
+  hipStream_t stream_;
+  hipEvent_t begin_ = nullptr, end_ = nullptr;
+  bool on_ = false;
+};
 
 GPUDriver* driverOf(ExecutionContext* ctx) {
   auto* d = ctx->getDriver<GPUDriver>(GPUDriver::name());
@@ -144,13 +204,58 @@ void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const 
     ws = drv->alloc(ctx, ws_bytes);
     if (!ws) return;
   }
+  StreamTimer timer(stream);
   int st = dq8_qgemm(op.a, lda, op.w, ldw, out, op.n, op.m, op.n, op.k, op.tp_a, op.tp_b,
                      e.mode, e.bias, e.bias_kind, e.sx, e.n_sx, e.sw, e.n_sw, e.so, e.n_so,
                      op.zx, op.zw, e.zo, ws, ws_bytes, stream);
+  if (timer.on() && st == 0) {
+    const double ns = timer.stop();
+    const int64_t bytes = op.m * op.k + op.k * op.n + op.m * op.n;
+    TAO_LOG(INFO) << who << " (gpu):\n"
+                << "\tpa = " << (const void*)op.a << "\n"
+                << "\tpb = " << (const void*)op.w << "\n"
+                << "\tpc = " << (const void*)out << "\n"
+                << "\tm = " << op.m << "\n"
+                << "\tn = " << op.n << "\n"
+                << "\tk = " << op.k << "\n"
+                << "\ttp_a = " << op.tp_a << "\n"
+                << "\ttp_b = " << op.tp_b << "\n"
+                << "\tweight_is_const = " << op.weight_is_const << "\n"
+                << "\tMath Ops = " << 2 * op.m * op.n * op.k << "\n"
+                << "\tBytes = " << bytes << "\n"
+                << "\tElapsed = " << ns / 1e3 << " us\n"
+                << "\tBandwidth = " << double(bytes) / ns << " GB\n"
+                << "\tGOPS = " << double(2 * op.m * op.n * op.k) / ns << "\n";
+  }
   // the pool hands `ws` out again only to later work on the same stream, which is
   // ordered after this launch
   if (ws) drv->dealloc(ctx, ws);
   kernelFailed(ctx, st, who);
+}
+
+// The profile record of a convolution (the reference's dumpConvLikeKernelProflingInfo,
+// R context/common_context_impl_mkldnn.h:605): sizes, work and rates.
+void logConvProfile(const char* who, const int64_t in[4], const int64_t w[4], const int64_t out[4],
+                    double ns) {
+  int64_t out_elems = 1, in_elems = 1, w_elems = 1;
+  for (int i = 0; i < 4; ++i) {
+    out_elems *= out[i];
+    in_elems *= in[i];
+    w_elems *= w[i];
+  }
+  // every output element takes (filter elements per output channel) multiply-adds
+  const int64_t per_out = w[0] > 0 ? w_elems / w[0] : 0;
+  const int64_t ops = 2 * out_elems * per_out;
+  const int64_t bytes = in_elems + w_elems + out_elems;
+  TAO_LOG(INFO) << who << " (gpu):\n"
+              << "\tinput = " << in[0] << "x" << in[1] << "x" << in[2] << "x" << in[3] << "\n"
+              << "\tkernel = " << w[0] << "x" << w[1] << "x" << w[2] << "x" << w[3] << "\n"
+              << "\toutput = " << out[0] << "x" << out[1] << "x" << out[2] << "x" << out[3] << "\n"
+              << "\tMath Ops = " << ops << "\n"
+              << "\tBytes = " << bytes << "\n"
+              << "\tElapsed = " << ns / 1e3 << " us\n"
+              << "\tBandwidth = " << double(bytes) / ns << " GB\n"
+              << "\tGOPS = " << double(ops) / ns << "\n";
 }
 
 template <typename T, int N>
@@ -538,10 +643,19 @@ void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4>
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return;
   void* stream = drv->asCUStream(ctx, stream_handle);
+  StreamTimer timer(stream);
   int st = dq8_qconv2d(input.data, input.sizes, kernel.data, kernel.sizes, padding.data,
                        metadata.data, output.data, output.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
                        DQ8_BIAS_NONE, inputScales.data, weightScales.data,
                        weightScales.sizes[0], resultScales.data, 0, stream);
+  if (timer.on() && st == 0) {
+    // the output-channel extent first, as logConvProfile expects
+    const int ko = metadata.data[5];
+    int64_t w[4] = {kernel.sizes[ko], 1, 1, 1};
+    for (int i = 0, j = 1; i < 4; ++i)
+      if (i != ko) w[j++] = kernel.sizes[i];
+    logConvProfile(who, input.sizes, w, output.sizes, timer.stop());
+  }
   kernelFailed(ctx, st, who);
 }
 
@@ -620,10 +734,13 @@ MemRefType<int8_t, 4> ral_pdll_qconv2d(ExecutionContext* ctx, void* stream_handl
   result = assignMemRef<int8_t, 4>(data, plan.result_sizes);
   void* stream = drv->asCUStream(ctx, stream_handle);
   const int32_t zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
+  StreamTimer timer(stream);
   int st = dq8_qconv2d(input.data, input.sizes, weight.data, weight.sizes, plan.padding,
                        plan.metadata, result.data, result.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
                        DQ8_BIAS_NONE, inputScales.data, weightScales.data,
                        weightScales.sizes[0], resultScales.data, zo, stream);
+  if (timer.on() && st == 0)   // weights are [out_channels, h, w, in_channels] here
+    logConvProfile(who, input.sizes, weight.sizes, result.sizes, timer.stop());
   kernelFailed(ctx, st, who);
   return result;
 }

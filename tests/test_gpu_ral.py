@@ -350,3 +350,56 @@ def test_concurrent_executions_on_one_context(rt):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+_PROFILE_CHILD = r"""
+import numpy as np, torch
+from bladedisc_amd import ral, ral_ops as ops
+ctx = ral.RalContext(stream=torch.cuda.current_stream().cuda_stream)
+d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+f1 = lambda v: d(np.array([v], np.float32))
+rng = np.random.default_rng(0)
+a = rng.integers(-128, 128, (96, 256), dtype=np.int8)
+w = rng.integers(-128, 128, (128, 256), dtype=np.int8)
+out = torch.empty((96, 128), dtype=torch.int8, device="cuda")
+x = rng.integers(-128, 128, (2, 8, 8, 32), dtype=np.int8)
+k = rng.integers(-128, 128, (16, 3, 3, 32), dtype=np.int8)
+co = torch.empty((2, 8, 8, 16), dtype=torch.int8, device="cuda")
+with ctx.execution() as ex:
+    ops.qgemm(ex, d(a), d(w), f1(0.02), f1(0.01), f1(3.0), out, tp_b=True)
+    ops.qconv(ex, d(x), d(k), [1, 1, 1, 1], [0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2, 1, 1, 1, 1, 1],
+              f1(0.02), d(np.full(16, 0.01, np.float32)), f1(3.0), co)
+torch.cuda.synchronize()
+print("checksum", int(out.to(torch.int32).sum()), int(co.to(torch.int32).sum()))
+ctx.close()
+"""
+
+
+def test_profile_mode_logs_the_reference_fields():
+    """DISC_GPU_ENABLE_PROFILE=1: each GEMM / convolution entry logs sizes, "Math Ops", "Bytes",
+    bandwidth and rate (the fields of the reference's DISC_CPU_ENABLE_PROFILE dump), and the
+    results are the same as without it.  The switch is read once per process, hence the
+    child processes."""
+    import os
+    import re
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    runs = {}
+    for flag in ("1", "0"):
+        env = dict(os.environ, DISC_GPU_ENABLE_PROFILE=flag, PYTHONPATH=root)
+        r = subprocess.run([sys.executable, "-c", _PROFILE_CHILD], env=env, capture_output=True,
+                           text=True, timeout=110)
+        assert r.returncode == 0, r.stderr[-2000:]
+        runs[flag] = r
+    log = runs["1"].stderr + runs["1"].stdout
+    assert "ral_qgemm (gpu):" in log and "ral_qconv (gpu):" in log
+    assert re.search(r"m = 96\s+n = 128\s+k = 256", log)
+    assert "Math Ops = %d" % (2 * 96 * 128 * 256) in log
+    assert "Bytes = %d" % (96 * 256 + 256 * 128 + 96 * 128) in log
+    assert "Math Ops = %d" % (2 * 2 * 8 * 8 * 16 * 3 * 3 * 32) in log       # the convolution
+    assert re.search(r"Elapsed = [0-9.e+-]+ us", log) and "Bandwidth = " in log and "GOPS = " in log
+    quiet = runs["0"].stderr + runs["0"].stdout
+    assert "Math Ops" not in quiet
+    line = [l for l in runs["1"].stdout.splitlines() if l.startswith("checksum")]
+    assert line and line == [l for l in runs["0"].stdout.splitlines() if l.startswith("checksum")]
