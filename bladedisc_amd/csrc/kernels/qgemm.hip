@@ -140,53 +140,6 @@ rowsum_s8_kernel(const int8_t* __restrict__ X, int64_t ld, int rows, int K, int 
   if (lane == 0) out[row] = mul * s + add;
 }
 
-// Second pass of a GEMM with zero points: the symmetric MFMA kernels have left
-// sum_k A W in `acc` ([M, N] int32, dense); with SA[m] and SW[n] the row sums,
-//   sum_k (A - zx)(W - zw) = acc - zx SW[n] - zw SA[m] + K zx zw
-// (corr_n[n] = -zx SW[n] + K zx zw, corr_m[m] = -zw SA[m]; int32 arithmetic wraps exactly
-// like the direct sum), then the epilogue.
-// A thread owns one output channel (its scale, bias and column correction are computed
-// once) and walks `rows` rows, four loads in flight; consecutive threads read and write
-// consecutive addresses.
-template <int EPI>
-__global__ void __launch_bounds__(256)
-zero_point_epilogue_kernel(const int32_t* __restrict__ acc, const int32_t* __restrict__ corr_n,
-                           const int32_t* __restrict__ corr_m, int rows, const EpiParams e) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= e.N) return;
-  const ColParams c = col_params<EPI>(e, n);
-  const float so_val = EPI == DQ8_EPI_DEQUANT_F32 ? dequant_so(e) : 0.0f;
-  const unsigned cn = (unsigned)corr_n[n];
-  const int m_begin = blockIdx.y * rows;
-  const int m_end = m_begin + rows < e.M ? m_begin + rows : e.M;
-  auto walk = [&](auto form) {
-    constexpr int FORM = decltype(form)::value;
-    auto finish = [&](int m, int raw) {
-      const unsigned a = (unsigned)raw + cn + (corr_m ? (unsigned)corr_m[m] : 0u);
-      const int64_t off = (int64_t)m * e.ldo + n;
-      if (EPI == DQ8_EPI_ACC_S32)
-        ((int32_t*)e.out)[off] = (int)a;
-      else if (EPI == DQ8_EPI_DEQUANT_F32)
-        ((float*)e.out)[off] = dequant_one<FORM>(e, c, (int)a, so_val);
-      else
-        ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, (int)a);
-    };
-    int m = m_begin;
-    for (; m + 3 < m_end; m += 4) {
-      int raw[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) raw[u] = acc[(int64_t)(m + u) * e.N + n];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) finish(m + u, raw[u]);
-    }
-    for (; m < m_end; ++m) finish(m, acc[(int64_t)m * e.N + n]);
-  };
-  if (EPI == DQ8_EPI_DEQUANT_F32)
-    dispatch_f32_form(e, walk);
-  else
-    walk(IntC<kF32Plain>());
-}
-
 // one MFMA of each shape, operands straight from global memory
 __global__ void __launch_bounds__(64)
 mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* a16,
@@ -252,6 +205,11 @@ constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct 
 constexpr int kPipe256w8 = 12, kPipe128w8 = 13;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
+
+bool is_pipe_variant(int v) {
+  return v == kPipe256 || v == kPipe128 || v == kPipe64 || v == kPipe256x64 || v == kPipe64k2 ||
+         v == kPipe256w8 || v == kPipe128w8;
+}
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
@@ -460,9 +418,9 @@ extern "C" size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int
 extern "C" size_t dq8_qgemm_workspace_bytes_zp(int64_t M, int64_t N, int64_t K, int tp_a,
                                                int tp_b, int32_t zx, int32_t zw) {
   size_t bytes = dq8_qgemm_workspace_bytes(M, N, K, tp_a, tp_b);
-  if (zx != 0 || zw != 0) {
+  if (zx != 0 || zw != 0) {   // the per-column and per-row corrections
     auto pad = [](int64_t v) { return (size_t)((v + 255) / 256 * 256); };
-    bytes += pad(M * N * 4) + pad(N * 4) + pad(M * 4);
+    bytes += pad(N * 4) + pad(M * 4);
   }
   return bytes;
 }
@@ -534,16 +492,18 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
 
-  // Zero points: the MFMA kernels are symmetric.  With scratch for an int32 [M, N]
-  // intermediate the heuristic runs them and corrects the sums in a second pass; without it
-  // (or for operands they cannot take) the generic kernel subtracts the zero points itself.
+  // Zero points: sum (a - zx)(w - zw) = sum a w - zx SW[n] - zw SA[m] + K zx zw with the row
+  // sums SW, SA.  Given scratch for the two correction vectors the heuristic keeps the
+  // problem on the pipelined MFMA kernels, whose accumulators start at the corrections;
+  // otherwise (or for operands those kernels cannot take) the generic kernel subtracts the
+  // zero points itself.
   const bool has_zp = zx != 0 || zw != 0;
   const bool auto_pick = variant == -1;
-  const bool zp_two_pass =
-      has_zp && auto_pick && K > 0 && K % 16 == 0 && workspace != nullptr && aligned(workspace, 256) &&
+  const bool zp_mfma =
+      has_zp && auto_pick && K >= 16 && K % 16 == 0 && workspace != nullptr && aligned(workspace, 256) &&
       workspace_bytes >= dq8_qgemm_workspace_bytes_zp(M, N, K, tp_a, tp_b, zx, zw) &&
       (tp_a || (aligned(A, 16) && lda % 16 == 0)) && (!tp_b || (aligned(W, 16) && ldw % 16 == 0));
-  if (auto_pick && has_zp && !zp_two_pass) variant = 0;
+  if (auto_pick && has_zp && !zp_mfma) variant = 0;
   if (variant == 0) {
     GenericParams g;
     g.A = A;
@@ -561,7 +521,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
         qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
         epilogue, g, M * N, st);
   }
-  DQ8_REQUIRE(!has_zp || zp_two_pass,
+  DQ8_REQUIRE(!has_zp || zp_mfma,
               "dq8_qgemm: input/weight zero points need the heuristic (variant -1) or the "
               "generic variant");
 
@@ -625,23 +585,30 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.K = (int)K;
   p.epi = e;
   if (auto_pick)
-    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false), zp_two_pass ? 4 : es);
-  if (!zp_two_pass) return launch_epi<false>(variant, p, epilogue, st);
+    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false), es);
+  if (!zp_mfma) return launch_epi<false>(variant, p, epilogue, st);
 
-  // ---- zero points: raw sums into scratch, row-sum corrections, then the epilogue
-  int32_t* acc = reinterpret_cast<int32_t*>((int8_t*)workspace + ws_off);
-  int32_t* corr_n = reinterpret_cast<int32_t*>((int8_t*)acc + pad(M * N * 4));
+  // ---- zero points: row sums -> corrections -> a pipelined kernel that starts from them
+  if (!is_pipe_variant(variant)) variant = kPipe64;   // (small M, or tiles the others cannot address)
+  if (!pipe_ok(kVariants[variant].bm, kVariants[variant].bn, p, false)) {
+    GenericParams g;
+    g.A = a_use;
+    g.W = w_use;
+    g.a_sm = lda_use;
+    g.a_sk = 1;
+    g.w_sn = ldw_use;
+    g.w_sk = 1;
+    g.K = (int)K;
+    g.zx = zx;
+    g.zw = zw;
+    g.epi = e;
+    return launch_generic_epi<GenericParams>(
+        qgemm_generic_kernel<DQ8_EPI_ACC_S32>, qgemm_generic_kernel<DQ8_EPI_REQUANT_CPU>,
+        qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
+        epilogue, g, M * N, st);
+  }
+  int32_t* corr_n = reinterpret_cast<int32_t*>((int8_t*)workspace + ws_off);
   int32_t* corr_m = reinterpret_cast<int32_t*>((int8_t*)corr_n + pad(N * 4));
-  EpiParams raw = {};
-  raw.out = acc;
-  raw.ldo = N;
-  raw.M = (int)M;
-  raw.N = (int)N;
-  raw.bias_kind = DQ8_BIAS_NONE;
-  raw.vec_store = N % 4 == 0;
-  raw.vec_store16 = N % 4 == 0;
-  p.epi = raw;
-  if (int s = launch_epi<false>(variant, p, DQ8_EPI_ACC_S32, st)) return s;
   // (wrapping int32 arithmetic on purpose, as in the kernels)
   const int kzz = (int)((uint32_t)K * (uint32_t)zx * (uint32_t)zw);
   hipLaunchKernelGGL(rowsum_s8_kernel, dim3((unsigned)ceil_div(N, 4)), dim3(256), 0, st, w_use,
@@ -650,30 +617,9 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
     hipLaunchKernelGGL(rowsum_s8_kernel, dim3((unsigned)ceil_div(M, 4)), dim3(256), 0, st, a_use,
                        lda_use, (int)M, (int)K, -zw, 0, corr_m);
   DQ8_HIP(hipGetLastError());
-  const int32_t* cm = zw != 0 ? corr_m : nullptr;
-  // rows per workgroup: 64 for large outputs, fewer while that leaves under ~2048 workgroups
-  const int64_t col_blocks = ceil_div(N, 256);
-  const int zp_rows = (int)std::min<int64_t>(64, std::max<int64_t>(4, M * col_blocks / 2048));
-  const dim3 blocks((unsigned)col_blocks, (unsigned)ceil_div(M, zp_rows));
-  DQ8_REQUIRE(blocks.y <= 65535u, "dq8_qgemm: too many rows for the zero-point pass");
-  switch (epilogue) {
-    case DQ8_EPI_ACC_S32:
-      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_ACC_S32>, blocks, dim3(256), 0,
-                         st, acc, corr_n, cm, zp_rows, e);
-      break;
-    case DQ8_EPI_REQUANT_CPU:
-      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_REQUANT_CPU>, blocks, dim3(256),
-                         0, st, acc, corr_n, cm, zp_rows, e);
-      break;
-    case DQ8_EPI_REQUANT_GPU:
-      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_REQUANT_GPU>, blocks, dim3(256),
-                         0, st, acc, corr_n, cm, zp_rows, e);
-      break;
-    default:
-      hipLaunchKernelGGL(zero_point_epilogue_kernel<DQ8_EPI_DEQUANT_F32>, blocks, dim3(256),
-                         0, st, acc, corr_n, cm, zp_rows, e);
-  }
-  return check_hip(hipGetLastError(), "zero_point_epilogue launch");
+  p.corr_n = corr_n;
+  p.corr_m = zw != 0 ? corr_m : nullptr;
+  return launch_epi<false>(variant, p, epilogue, st);
 }
 
 extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,

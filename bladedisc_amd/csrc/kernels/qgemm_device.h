@@ -58,6 +58,10 @@ struct MainParams {
   int pad_t, pad_l, sh, sw_, dh, dw;
   int64_t conv_bytes;   // size of the NHWC image tensor in bytes
   int tiles_m, tiles_n;
+  // Zero-point corrections (pipelined GEMM kernels; null = none): the accumulator of
+  // output (m, n) starts at corr_n[n] + corr_m[m] instead of 0.
+  const int32_t* corr_n;
+  const int32_t* corr_m;
   EpiParams epi;
 };
 

@@ -251,6 +251,29 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+  if (!CONV && (p.corr_n || p.corr_m) && kg == 0) {
+    // Zero points: sum (a - zx)(w - zw) = sum a w + corr_n[n] + corr_m[m]; starting the sums at
+    // the corrections costs a few loads here and nothing in the epilogue, and int32
+    // wraps the same way whichever end the terms are added at.  Element 4g+q of fragment
+    // (i, j) is row i*32 + lane%32, column j*32 + 8g + 4(lane/32) + q of the wave tile.
+    int cm[FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      const int m = m0 + wm * TM + i * 32 + (lane & 31);
+      cm[i] = p.corr_m ? p.corr_m[m < p.M ? m : p.M - 1] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * TN + j * 32 + 8 * g + 4 * (lane >> 5) + q;
+          const int cn = p.corr_n ? p.corr_n[n < p.N ? n : p.N - 1] : 0;
+#pragma unroll
+          for (int i = 0; i < FM; ++i) acc[i][j][4 * g + q] = cn + cm[i];
+        }
+  }
 
   // Load schedule: the LD loads of tile t+2 are issued during k-steps 2 and 3 of tile
   // t, LPR per row of MFMAs, into the stage tile t has just released.

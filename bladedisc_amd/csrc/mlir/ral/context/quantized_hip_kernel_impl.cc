@@ -195,7 +195,7 @@ void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const 
 
   const int64_t lda = op.tp_a ? op.m : op.k;
   const int64_t ldw = op.tp_b ? op.k : op.n;
-  // (with a zero point: room for the int32 intermediate that keeps the problem on the MFMA
+  // (with a zero point: room for the correction vectors that keep the problem on the MFMA
   // kernels)
   const size_t ws_bytes =
       dq8_qgemm_workspace_bytes_zp(op.m, op.n, op.k, op.tp_a, op.tp_b, op.zx, op.zw);

@@ -164,8 +164,8 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
     sw = _scale(sw, dev) if sw is not None else None
     so = _scale(so, dev) if so is not None else None
     bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
-    # with zero points and the heuristic this includes the int32 intermediate of the
-    # two-pass path; a forced generic variant (0) needs none of it
+    # with zero points and the heuristic this includes the two correction vectors of the
+    # MFMA path; a forced generic variant (0) needs none of it
     ws_bytes = (L.dq8_qgemm_workspace_bytes_zp(m, n, k, int(tp_a), int(tp_b), zx, zw)
                 if variant == -1 else L.dq8_qgemm_workspace_bytes(m, n, k, int(tp_a), int(tp_b)))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None

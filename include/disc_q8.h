@@ -163,10 +163,10 @@ int dq8_tf_dequantize(const void* q, int in_kind, float* out, int64_t outer, int
  * needs none: tp_a == 0 and tp_b == 1). */
 size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
                                  int tp_b);
-/* The same for given input / weight zero points: with a non-zero one it adds an int32
- * [M, N] intermediate and two correction vectors, which lets dq8_qgemm keep such a problem
- * on the MFMA kernels.  A caller that passes less (but at least
- * dq8_qgemm_workspace_bytes()) still gets the right result, from the generic kernel. */
+/* The same for given input / weight zero points: with a non-zero one it adds two correction
+ * vectors (4 (M + N) bytes), which lets dq8_qgemm keep such a problem on the MFMA kernels.
+ * A caller that passes less (but at least dq8_qgemm_workspace_bytes()) still gets the
+ * right result, from the generic kernel. */
 size_t dq8_qgemm_workspace_bytes_zp(int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
                                     int32_t zx, int32_t zw);
 
@@ -180,10 +180,10 @@ size_t dq8_qgemm_workspace_bytes_zp(int64_t M, int64_t N, int64_t K, int tp_a, i
  *   zx / zw: input and weight zero points, acc = sum (A - zx) * (W - zw) (what oneDNN
  *      computes for the reference's CPU entries, R ral/context/mkldnn/ideep/ideep/
  *      operators/matmul.hpp:516-549: one source zero point, the first weight zero point).
- *      With scratch of dq8_qgemm_workspace_bytes_zp() the symmetric MFMA kernels compute
- *      sum A W into an int32 intermediate and a second pass applies
- *      - zx sum_k W - zw sum_k A + K zx zw and the epilogue; with less scratch, or
- *      operands the MFMA kernels cannot take, the generic scalar kernel is used.
+ *      With scratch of dq8_qgemm_workspace_bytes_zp() the MFMA kernels start their sums at
+ *      - zx sum_k W[n,k] - zw sum_k A[m,k] + K zx zw (row sums from a small kernel); with
+ *      less scratch, or operands the MFMA kernels cannot take, the generic scalar kernel
+ *      is used.
  *   zo: output zero point (REQUANT_CPU only).
  *   workspace: device scratch of at least dq8_qgemm_workspace_bytes(), may be
  *      NULL when that is 0.

@@ -219,10 +219,13 @@ def test_qgemm_zero_points_generic(K):
     (64, 768, 768, 0, 1, 7, 0), (300, 130, 400, 0, 1, -128, 0), (33, 48, 64, 0, 1, 5, -3),
     (256, 512, 1040, 0, 0, 100, 0), (100, 96, 128, 1, 1, 127, 2), (1, 768, 3072, 0, 1, 11, 0),
     (1000, 768, 768, 0, 1, -77, 9),
+    # one shape per pipelined tile: 256x256 and 128x128 on eight waves, 256x64, 64x64 with K split
+    (4096, 2560, 128, 0, 1, 9, -4), (2048, 2048, 256, 0, 1, -128, 127), (16384, 64, 128, 0, 1, 3, 1),
+    (256, 256, 2048, 0, 1, 100, -100), (4100, 2570, 4096, 0, 1, 1, 0),
 ])
 def test_qgemm_zero_points_on_the_mfma_path(K, m, n, k, tp_a, tp_b, zx, zw):
     """Asymmetric operands stay on the MFMA kernels when the caller provides the scratch for
-    the two-pass scheme: every epilogue equals the oracle's direct sum of (a - zx)(w - zw);
+    the correction vectors (the accumulators start at them): every epilogue equals the oracle's direct sum of (a - zx)(w - zw);
     without the scratch the generic kernel gives the same result."""
     rng = np.random.default_rng(m + n + k + zx)
     a = rng.integers(-128, 128, (m, k), dtype=np.int8)
@@ -254,7 +257,7 @@ def test_qgemm_zero_points_on_the_mfma_path(K, m, n, k, tp_a, tp_b, zx, zw):
 
 
 def test_qgemm_zero_points_full_size_property(K):
-    """4096^3 with an input zero point: the two-pass result equals the symmetric result of
+    """4096^3 with an input zero point: the result equals the symmetric result of
     the shifted problem computed another way -- acc(a - zx, w) = acc(a, w) - zx * colsum(w)
     -- with both sides from the GPU in int32 and the column sums from numpy."""
     n = 4096
