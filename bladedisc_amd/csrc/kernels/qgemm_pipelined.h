@@ -251,7 +251,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-  if (!CONV && (p.corr_n || p.corr_m) && kg == 0) {
+  if (!CONV && __builtin_expect((p.corr_n != nullptr || p.corr_m != nullptr) && kg == 0, 0)) {
     // Zero points: sum (a - zx)(w - zw) = sum a w + corr_n[n] + corr_m[m]; starting the sums at
     // the corrections costs a few loads here and nothing in the epilogue, and int32
     // wraps the same way whichever end the terms are added at.  Element 4g+q of fragment
