@@ -99,10 +99,11 @@ __global__ void __launch_bounds__(256) qconv_generic_kernel(const GenericConvPar
   }
 }
 
-// int8 [R, C] (row stride ld) -> [C, R] contiguous, 64x64 tiles through LDS
+// int8 [R, C] (row stride ld) -> [C, R] with row stride ldd >= R, columns R .. ldd-1 zero;
+// 64x64 tiles through LDS, blockIdx.y over ceil(ldd / 64)
 __global__ void __launch_bounds__(256)
 transpose_s8_kernel(const int8_t* __restrict__ src, int64_t ld, int8_t* __restrict__ dst,
-                    int R, int C) {
+                    int R, int C, int ldd) {
   __shared__ int8_t tile[64][65];
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -113,7 +114,27 @@ transpose_s8_kernel(const int8_t* __restrict__ src, int64_t ld, int8_t* __restri
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
     const int c = c0 + i, r = r0 + tx;
-    if (c < C && r < R) dst[(int64_t)c * R + r] = tile[tx][i];
+    if (c < C && r < ldd) dst[(int64_t)c * ldd + r] = tile[tx][i];   // (zero for r >= R)
+  }
+}
+
+// int8 [R, C] (row stride ld, any alignment) -> [R, ldd], ldd % 16 == 0 and dst 16-byte
+// aligned, columns C .. ldd-1 zero.  One 16-byte store per thread and step.
+__global__ void __launch_bounds__(256)
+pad_rows_s8_kernel(const int8_t* __restrict__ src, int64_t ld, int8_t* __restrict__ dst,
+                   int64_t R, int C, int ldd) {
+  const int chunks = ldd / 16;
+  const int64_t total = R * chunks;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * 256) {
+    const int64_t r = idx / chunks;
+    const int c0 = (int)(idx - r * chunks) * 16;
+    const int8_t* s = src + r * ld + c0;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int b = 0; b < 16; ++b)
+      if (c0 + b < C) w[b >> 2] |= (uint32_t)(uint8_t)s[b] << (8 * (b & 3));
+    *reinterpret_cast<v4i*>(dst + r * ldd + c0) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
   }
 }
 
@@ -408,10 +429,13 @@ extern "C" const char* dq8_qgemm_variant_name(int variant) {
 
 extern "C" size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
                                             int tp_b) {
+  // an operand that is not k-contiguous, or whose K is not a multiple of 16, is rewritten
+  // as [rows, K rounded up to 16] (zero filled) for the MFMA kernels
   size_t bytes = 0;
   auto pad = [](int64_t v) { return (size_t)((v + 255) / 256 * 256); };
-  if (tp_a) bytes += pad(M * K);
-  if (!tp_b) bytes += pad(N * K);
+  const int64_t kp = (K + 15) / 16 * 16;
+  if (tp_a || K % 16 != 0) bytes += pad(M * kp);
+  if (!tp_b || K % 16 != 0) bytes += pad(N * kp);
   return bytes;
 }
 
@@ -434,7 +458,7 @@ extern "C" int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int6
   DQ8_REQUIRE(src && dst, "dq8_transpose_s8: null pointer");
   hipLaunchKernelGGL(transpose_s8_kernel,
                      dim3((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(rows, 64)), dim3(256),
-                     0, (hipStream_t)stream, src, ld, dst, (int)rows, (int)cols);
+                     0, (hipStream_t)stream, src, ld, dst, (int)rows, (int)cols, (int)rows);
   return check_hip(hipGetLastError(), "dq8_transpose_s8 launch");
 }
 
@@ -499,11 +523,24 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   // zero points itself.
   const bool has_zp = zx != 0 || zw != 0;
   const bool auto_pick = variant == -1;
+  // The MFMA kernels want A [M, K'] and W [N, K'], k-contiguous, rows 16-byte aligned, K' a
+  // multiple of 16: operands in another layout, or with a ragged K, are rewritten into the
+  // workspace (zero-filled up to K'; zeros add nothing to the sums).
+  const int64_t Kp = (K + 15) / 16 * 16;
+  const bool repack_a = K > 0 && (tp_a || K % 16 != 0);
+  const bool repack_w = K > 0 && (!tp_b || K % 16 != 0);
+  const bool have_ws = workspace != nullptr && aligned(workspace, 256) &&
+                       workspace_bytes >= dq8_qgemm_workspace_bytes(M, N, K, tp_a, tp_b);
+  const bool mfma_operands = (repack_a ? have_ws : (aligned(A, 16) && lda % 16 == 0)) &&
+                             (repack_w ? have_ws : (aligned(W, 16) && ldw % 16 == 0));
   const bool zp_mfma =
-      has_zp && auto_pick && K >= 16 && K % 16 == 0 && workspace != nullptr && aligned(workspace, 256) &&
-      workspace_bytes >= dq8_qgemm_workspace_bytes_zp(M, N, K, tp_a, tp_b, zx, zw) &&
-      (tp_a || (aligned(A, 16) && lda % 16 == 0)) && (!tp_b || (aligned(W, 16) && ldw % 16 == 0));
+      has_zp && auto_pick && K > 0 && mfma_operands && workspace != nullptr &&
+      aligned(workspace, 256) &&
+      workspace_bytes >= dq8_qgemm_workspace_bytes_zp(M, N, K, tp_a, tp_b, zx, zw);
   if (auto_pick && has_zp && !zp_mfma) variant = 0;
+  // (a ragged K without the scratch to pad it, or unaligned operands: the generic kernel
+  // takes any strides; a transposed operand without scratch stays an error below)
+  if (variant != 0 && !mfma_operands && !((tp_a || !tp_b) && !have_ws)) variant = 0;
   if (variant == 0) {
     GenericParams g;
     g.A = A;
@@ -524,56 +561,37 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   DQ8_REQUIRE(!has_zp || zp_mfma,
               "dq8_qgemm: input/weight zero points need the heuristic (variant -1) or the "
               "generic variant");
+  DQ8_REQUIRE(mfma_operands, "dq8_qgemm: workspace too small for the requested transposes");
 
-  // MFMA path wants A [M,K] and W [N,K], both k-contiguous: transpose the others
-  // into the workspace.
   const int8_t* a_use = A;
   const int8_t* w_use = W;
   int64_t lda_use = lda, ldw_use = ldw;
   size_t ws_off = 0;
   auto pad = [](int64_t v) { return (size_t)((v + 255) / 256 * 256); };
-  if (K > 0 && (tp_a || !tp_b)) {
-    DQ8_REQUIRE(workspace != nullptr &&
-                    workspace_bytes >= dq8_qgemm_workspace_bytes(M, N, K, tp_a, tp_b),
-                "dq8_qgemm: workspace too small for the requested transposes");
-    if (tp_a) {  // A is [K, M] -> [M, K]
-      int8_t* dst = (int8_t*)workspace + ws_off;
-      hipLaunchKernelGGL(transpose_s8_kernel, dim3((unsigned)ceil_div(M, 64), (unsigned)ceil_div(K, 64)),
-                         dim3(256), 0, st, A, lda, dst, (int)K, (int)M);
-      a_use = dst;
-      lda_use = K;
-      ws_off += pad(M * K);
-    }
-    if (!tp_b) {  // W is [K, N] -> [N, K]
-      int8_t* dst = (int8_t*)workspace + ws_off;
-      hipLaunchKernelGGL(transpose_s8_kernel, dim3((unsigned)ceil_div(N, 64), (unsigned)ceil_div(K, 64)),
-                         dim3(256), 0, st, W, ldw, dst, (int)K, (int)N);
-      w_use = dst;
-      ldw_use = K;
-      ws_off += pad(N * K);
-    }
-    DQ8_HIP(hipGetLastError());
+  auto repack = [&](const int8_t* src, int64_t ld, bool transposed, int64_t rows) {
+    int8_t* dst = (int8_t*)workspace + ws_off;
+    if (transposed)   // src is [K, rows]
+      hipLaunchKernelGGL(transpose_s8_kernel,
+                         dim3((unsigned)ceil_div(rows, 64), (unsigned)ceil_div(Kp, 64)), dim3(256),
+                         0, st, src, ld, dst, (int)K, (int)rows, (int)Kp);
+    else
+      hipLaunchKernelGGL(pad_rows_s8_kernel,
+                         dim3((unsigned)std::min<int64_t>(ceil_div(rows * (Kp / 16), 256), 1 << 20)),
+                         dim3(256), 0, st, src, ld, dst, rows, (int)K, (int)Kp);
+    ws_off += pad(rows * Kp);
+    return dst;
+  };
+  if (repack_a) {
+    a_use = repack(A, lda, tp_a != 0, M);
+    lda_use = Kp;
   }
-  // 16-byte loads: rows must start 16-byte aligned and K must be a multiple of 16
-  const bool fast_ok = K % 16 == 0 && (K == 0 || (aligned(a_use, 16) && aligned(w_use, 16) &&
-                                                  lda_use % 16 == 0 && ldw_use % 16 == 0));
-  if (!fast_ok) {
-    GenericParams g;
-    g.A = a_use;
-    g.W = w_use;
-    g.a_sm = lda_use;
-    g.a_sk = 1;
-    g.w_sn = ldw_use;
-    g.w_sk = 1;
-    g.K = (int)K;
-    g.zx = zx;
-    g.zw = zw;
-    g.epi = e;
-    return launch_generic_epi<GenericParams>(
-        qgemm_generic_kernel<DQ8_EPI_ACC_S32>, qgemm_generic_kernel<DQ8_EPI_REQUANT_CPU>,
-        qgemm_generic_kernel<DQ8_EPI_REQUANT_GPU>, qgemm_generic_kernel<DQ8_EPI_DEQUANT_F32>,
-        epilogue, g, M * N, st);
+  if (repack_w) {
+    w_use = repack(W, ldw, tp_b == 0, N);
+    ldw_use = Kp;
   }
+  if (repack_a || repack_w) DQ8_HIP(hipGetLastError());
+  const int64_t K_true = K;
+  K = Kp;   // what the kernels below see; the padding is zero
 
   MainParams p = {};
   p.A = a_use;
@@ -598,7 +616,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
     g.a_sk = 1;
     g.w_sn = ldw_use;
     g.w_sk = 1;
-    g.K = (int)K;
+    g.K = (int)K_true;   // (the padding is not part of the sums)
     g.zx = zx;
     g.zw = zw;
     g.epi = e;
@@ -610,7 +628,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   int32_t* corr_n = reinterpret_cast<int32_t*>((int8_t*)workspace + ws_off);
   int32_t* corr_m = reinterpret_cast<int32_t*>((int8_t*)corr_n + pad(N * 4));
   // (wrapping int32 arithmetic on purpose, as in the kernels)
-  const int kzz = (int)((uint32_t)K * (uint32_t)zx * (uint32_t)zw);
+  const int kzz = (int)((uint32_t)K_true * (uint32_t)zx * (uint32_t)zw);
   hipLaunchKernelGGL(rowsum_s8_kernel, dim3((unsigned)ceil_div(N, 4)), dim3(256), 0, st, w_use,
                      ldw_use, (int)N, (int)K, -zx, kzz, corr_n);
   if (zw != 0)

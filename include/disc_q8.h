@@ -160,7 +160,10 @@ int dq8_tf_dequantize(const void* q, int in_kind, float* out, int64_t outer, int
 /* ---- int8 GEMM -------------------------------------------------------- */
 
 /* Bytes of device scratch dq8_qgemm needs for this problem with zx == zw == 0 (0 when it
- * needs none: tp_a == 0 and tp_b == 1). */
+ * needs none: tp_a == 0, tp_b == 1 and K % 16 == 0).  Operands in the other layout, or with
+ * a K that is not a multiple of 16, are rewritten there as [rows, K rounded up to 16].  A
+ * ragged K without the scratch still gives the right result, from the generic kernel; a
+ * transposed operand without it is an error. */
 size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
                                  int tp_b);
 /* The same for given input / weight zero points: with a non-zero one it adds two correction
@@ -198,8 +201,8 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
 /* Same, forcing one kernel variant (for tests and tuning):
  *  -1 heuristic, 0 generic scalar kernel, 1.. MFMA tile configurations
  *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()).  A problem
- *  an MFMA variant cannot take (K % 16 != 0, unaligned rows) runs on the generic
- *  kernel whatever the variant; non-zero zx / zw with a forced MFMA variant is an error
+ *  an MFMA variant cannot take (unaligned rows; K % 16 != 0 without scratch) runs on the
+ *  generic kernel whatever the variant; non-zero zx / zw with a forced MFMA variant is an error
  *  (they need the heuristic or the generic variant). */
 int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                       const int8_t* W, int64_t ldw, void* out, int64_t ldo,

@@ -25,8 +25,7 @@ def host(t):
 
 
 def gemm_variants(K, k):
-    """All variant ids.  (With a contraction length that is not a multiple of 16 the MFMA
-    variants hand the problem to the generic kernel.)"""
+    """All variant ids of the GEMM."""
     return [i for i, nm in enumerate(K.variant_names()) if not nm.startswith("direct3x3_")]
 
 
@@ -56,7 +55,9 @@ def test_mfma_operand_and_result_layouts(K):
 
 # ------------------------------------------------------------------------ qgemm
 SHAPES = [(1, 768, 768), (16, 768, 768), (64, 768, 768), (128, 3072, 768), (1000, 768, 3072),
-          (257, 130, 64), (33, 36, 16), (300, 260, 1040), (512, 512, 512), (5, 7, 48)]
+          (257, 130, 64), (33, 36, 16), (300, 260, 1040), (512, 512, 512), (5, 7, 48),
+          # contraction lengths that are not a multiple of 16: padded into the scratch
+          (4, 71, 25), (300, 260, 1041), (1000, 768, 777), (64, 64, 1), (2048, 1024, 15)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -201,6 +202,43 @@ def test_qgemm_transposed_operands(K, tp_a, tp_b):
         got = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_ACC_S32, tp_a=bool(tp_a), tp_b=bool(tp_b),
                            variant=v))
         np.testing.assert_array_equal(got, want)
+
+
+def test_qgemm_ragged_k_stays_on_the_mfma_kernels(K):
+    """K % 16 != 0: with the scratch dq8_qgemm_workspace_bytes asks for, the operands are
+    padded and the MFMA kernels run (every layout, zero points, every epilogue); the result
+    is the oracle's, and it is not the generic kernel's speed."""
+    import time
+    rng = np.random.default_rng(77)
+    m, n, k = 1000, 520, 777
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    for tp_a, tp_b, zx, zw in [(0, 1, 0, 0), (1, 0, 0, 0), (0, 0, 5, 0), (1, 1, -9, 4)]:
+        acc = O.gemm_s32(a, w, tp_b=True, zx=zx, zw=zw)
+        a_in = np.ascontiguousarray(a.T) if tp_a else a
+        w_in = w if tp_b else np.ascontiguousarray(w.T)
+        kw = dict(tp_a=bool(tp_a), tp_b=bool(tp_b), zx=zx, zw=zw)
+        np.testing.assert_array_equal(host(K.qgemm(dev(a_in), dev(w_in), K.EPI_ACC_S32, **kw)), acc)
+        sx, sw = make_scales(rng, n)
+        so = pick_so(acc, sx, sw)
+        bias = (rng.standard_normal(n) * 3).astype(np.float32)
+        want = O.requant_cpu(acc, sx, sw, so, b32=O.bias_f32_to_s32(bias, sx, sw))
+        got = host(K.qgemm(dev(a_in), dev(w_in), K.EPI_REQUANT_CPU, sx=dev(np.array([sx])),
+                           sw=dev(sw), so=dev(np.array([so])), bias=dev(bias), **kw))
+        np.testing.assert_array_equal(got, want)
+    # speed: 4096 x 4096 x 4095 would take the generic kernel seconds
+    big = 4096
+    ab = torch.randint(-128, 128, (big, big - 1), dtype=torch.int8, device="cuda")
+    wb = torch.randint(-128, 128, (big, big - 1), dtype=torch.int8, device="cuda")
+    out = K.qgemm(ab, wb, K.EPI_ACC_S32)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = K.qgemm(ab, wb, K.EPI_ACC_S32)
+    torch.cuda.synchronize()
+    assert time.perf_counter() - t0 < 0.01
+    rows = [0, 1234, big - 1]
+    want = O.gemm_s32(ab[rows].cpu().numpy(), wb.cpu().numpy(), tp_b=True)
+    np.testing.assert_array_equal(out[rows].cpu().numpy(), want)
 
 
 def test_qgemm_zero_points_generic(K):
