@@ -37,7 +37,11 @@ _PROTOS = {
     "dq8_qconv2d_variant": (_INT, [_INT, _VP, C.POINTER(_I64), _VP, C.POINTER(_I64),
                                    C.POINTER(_I32), C.POINTER(_I32), _VP,
                                    C.POINTER(_I64), _INT, _VP, _INT, _VP, _VP, _I64,
-                                   _VP, _I32, _VP]),
+                                   _VP, _I32, _VP, _SZ, _VP]),
+    "dq8_qconv2d_ws": (_INT, [_VP, C.POINTER(_I64), _VP, C.POINTER(_I64), C.POINTER(_I32),
+                              C.POINTER(_I32), _VP, C.POINTER(_I64), _INT, _VP, _INT, _VP,
+                              _VP, _I64, _VP, _I32, _VP, _SZ, _VP]),
+    "dq8_qconv2d_workspace_bytes": (_SZ, [C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I32)]),
     "dq8_mfma_probe": (_INT, [_VP] * 7),
     "dq8_lut8": (_INT, [_VP, _VP, _I64, _VP, _VP]),
     "dq8_tf_params_bytes": (_SZ, [_I64]),

@@ -652,13 +652,22 @@ extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t 
                            workspace, workspace_bytes, stream);
 }
 
-extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t in_sizes[4],
-                                   const int8_t* w, const int64_t w_sizes[4],
-                                   const int32_t padding[4], const int32_t md[17],
-                                   void* out, const int64_t out_sizes[4], int epilogue,
-                                   const void* bias, int bias_kind, const float* sx,
-                                   const float* sw, int64_t n_sw, const float* so,
-                                   int32_t zo, void* stream) {
+namespace {
+
+bool is_nhwc_ohwi(const int32_t md[17]) {
+  static const int32_t want[12] = {0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2};
+  for (int i = 0; i < 12; ++i)
+    if (md[i] != want[i]) return false;
+  return true;
+}
+
+size_t pad256(int64_t v) { return (size_t)((v + 255) / 256 * 256); }
+
+int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                 const int64_t w_sizes[4], const int32_t padding[4], const int32_t md[17],
+                 void* out, const int64_t out_sizes[4], int epilogue, const void* bias,
+                 int bias_kind, const float* sx, const float* sw, int64_t n_sw, const float* so,
+                 int32_t zo, void* workspace, size_t workspace_bytes, void* stream) {
   clear_error();
   DQ8_REQUIRE(in_sizes && w_sizes && padding && md && out_sizes, "dq8_qconv2d: null descriptor");
   DQ8_REQUIRE(variant >= -1 && variant < kNumVariants, "dq8_qconv2d: unknown variant");
@@ -672,7 +681,8 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   const int ib = md[0], ic = md[1], ih = md[2], iw = md[3];
   const int ki = md[4], ko = md[5], kh = md[6], kw = md[7];
   const int ob = md[8], oc = md[9], oh = md[10], ow = md[11];
-  const int64_t NB = in_sizes[ib], Ci = in_sizes[ic], H = in_sizes[ih], Wd = in_sizes[iw];
+  const int64_t NB = in_sizes[ib], H = in_sizes[ih], Wd = in_sizes[iw];
+  int64_t Ci = in_sizes[ic];
   const int64_t Co = w_sizes[ko], Kh = w_sizes[kh], Kw = w_sizes[kw];
   const int64_t Ho = out_sizes[oh], Wo = out_sizes[ow];
   DQ8_REQUIRE(w_sizes[ki] == Ci, "dq8_qconv2d: kernel input features differ from the input's");
@@ -700,7 +710,8 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
               "dq8_qconv2d: an output zero point needs the REQUANT_CPU epilogue");
   if (requant) epilogue = DQ8_EPI_DEQUANT_F32;
-  const int64_t Mg = NB * Ho * Wo, Kg = Kh * Kw * Ci;
+  const int64_t Mg = NB * Ho * Wo;
+  int64_t Kg = Kh * Kw * Ci;
   DQ8_REQUIRE(Mg < (1LL << 31) && Kg < (1LL << 31) && Co < (1LL << 31) &&
                   NB * H * Wd * Ci < (1LL << 40),
               "dq8_qconv2d: problem too large");
@@ -727,10 +738,32 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   e.vec_store = aligned(out, 4 * es) && (Co % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (Co % 16 == 0);
 
-  const bool nhwc_ohwi = ib == 0 && ic == 3 && ih == 1 && iw == 2 && ki == 3 && ko == 0 &&
-                         kh == 1 && kw == 2 && ob == 0 && oc == 3 && oh == 1 && ow == 2;
-  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16);
+  const bool nhwc_ohwi = is_nhwc_ohwi(md);
   const bool auto_pick = variant == -1;
+  // Channel counts that are not a multiple of 16 (an RGB first layer): with scratch, input
+  // and weights are rewritten with the channels zero-filled up to the next multiple; the
+  // added channels contribute nothing and the MFMA kernels run on the padded tensors.
+  const int64_t Cip = (Ci + 15) / 16 * 16;
+  if (nhwc_ohwi && Ci % 16 != 0 && variant != 0 && workspace != nullptr &&
+      aligned(workspace, 256) &&
+      workspace_bytes >= pad256(NB * H * Wd * Cip) + pad256(Co * Kh * Kw * Cip) &&
+      NB * H * Wd * Cip < (1LL << 40) && Kh * Kw * Cip < (1LL << 31)) {
+    int8_t* in_p = (int8_t*)workspace;
+    int8_t* w_p = in_p + pad256(NB * H * Wd * Cip);
+    auto blocks = [](int64_t rows, int64_t ldd) {
+      return dim3((unsigned)std::min<int64_t>(ceil_div(rows * (ldd / 16), 256), 1 << 20));
+    };
+    hipLaunchKernelGGL(pad_rows_s8_kernel, blocks(NB * H * Wd, Cip), dim3(256), 0, st, in, Ci,
+                       in_p, NB * H * Wd, (int)Ci, (int)Cip);
+    hipLaunchKernelGGL(pad_rows_s8_kernel, blocks(Co * Kh * Kw, Cip), dim3(256), 0, st, w, Ci,
+                       w_p, Co * Kh * Kw, (int)Ci, (int)Cip);
+    DQ8_HIP(hipGetLastError());
+    in = in_p;
+    w = w_p;
+    Ci = Cip;
+    Kg = Kh * Kw * Ci;
+  }
+  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16);
   if (auto_pick && !fast_ok) variant = 0;
   if (variant != 0)
     DQ8_REQUIRE(fast_ok, "dq8_qconv2d: the MFMA variants need NHWC x OHWI, Ci % 16 == 0 and "
@@ -818,14 +851,48 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   return launch_epi<true>(variant, p, epilogue, st);
 }
 
+}  // namespace
+
+extern "C" size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const int64_t w_sizes[4],
+                                              const int32_t metadata[17]) {
+  if (!in_sizes || !w_sizes || !metadata || !is_nhwc_ohwi(metadata)) return 0;
+  const int64_t ci = in_sizes[3];
+  if (ci % 16 == 0) return 0;
+  const int64_t cip = (ci + 15) / 16 * 16;
+  return pad256(in_sizes[0] * in_sizes[1] * in_sizes[2] * cip) +
+         pad256(w_sizes[0] * w_sizes[1] * w_sizes[2] * cip);
+}
+
+extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t in_sizes[4],
+                                   const int8_t* w, const int64_t w_sizes[4],
+                                   const int32_t padding[4], const int32_t md[17],
+                                   void* out, const int64_t out_sizes[4], int epilogue,
+                                   const void* bias, int bias_kind, const float* sx,
+                                   const float* sw, int64_t n_sw, const float* so,
+                                   int32_t zo, void* workspace, size_t workspace_bytes,
+                                   void* stream) {
+  return qconv2d_impl(variant, in, in_sizes, w, w_sizes, padding, md, out, out_sizes, epilogue,
+                      bias, bias_kind, sx, sw, n_sw, so, zo, workspace, workspace_bytes, stream);
+}
+
+extern "C" int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                              const int64_t w_sizes[4], const int32_t padding[4],
+                              const int32_t metadata[17], void* out, const int64_t out_sizes[4],
+                              int epilogue, const void* bias, int bias_kind, const float* sx,
+                              const float* sw, int64_t n_sw, const float* so, int32_t zo,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  return qconv2d_impl(-1, in, in_sizes, w, w_sizes, padding, metadata, out, out_sizes, epilogue,
+                      bias, bias_kind, sx, sw, n_sw, so, zo, workspace, workspace_bytes, stream);
+}
+
 extern "C" int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                            const int64_t w_sizes[4], const int32_t padding[4],
                            const int32_t metadata[17], void* out, const int64_t out_sizes[4],
                            int epilogue, const void* bias, int bias_kind, const float* sx,
                            const float* sw, int64_t n_sw, const float* so, int32_t zo,
                            void* stream) {
-  return dq8_qconv2d_variant(-1, in, in_sizes, w, w_sizes, padding, metadata, out, out_sizes,
-                             epilogue, bias, bias_kind, sx, sw, n_sw, so, zo, stream);
+  return qconv2d_impl(-1, in, in_sizes, w, w_sizes, padding, metadata, out, out_sizes, epilogue,
+                      bias, bias_kind, sx, sw, n_sw, so, zo, nullptr, 0, stream);
 }
 
 extern "C" int dq8_mfma_probe(const int8_t* a, const int8_t* b, int32_t* d32,

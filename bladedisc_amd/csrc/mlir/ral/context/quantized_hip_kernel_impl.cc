@@ -643,11 +643,17 @@ void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4>
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return;
   void* stream = drv->asCUStream(ctx, stream_handle);
+  // (scratch for channel counts that are not a multiple of 16; handed back to the pool
+  // right after the launch, which later work on the same stream is ordered behind)
+  const size_t ws_bytes = dq8_qconv2d_workspace_bytes(input.sizes, kernel.sizes, metadata.data);
+  void* ws = ws_bytes ? drv->alloc(ctx, ws_bytes) : nullptr;
+  if (ws_bytes && !ws) return;
   StreamTimer timer(stream);
-  int st = dq8_qconv2d(input.data, input.sizes, kernel.data, kernel.sizes, padding.data,
-                       metadata.data, output.data, output.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
-                       DQ8_BIAS_NONE, inputScales.data, weightScales.data,
-                       weightScales.sizes[0], resultScales.data, 0, stream);
+  int st = dq8_qconv2d_ws(input.data, input.sizes, kernel.data, kernel.sizes, padding.data,
+                          metadata.data, output.data, output.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
+                          DQ8_BIAS_NONE, inputScales.data, weightScales.data,
+                          weightScales.sizes[0], resultScales.data, 0, ws, ws_bytes, stream);
+  if (ws) drv->dealloc(ctx, ws);
   if (timer.on() && st == 0) {
     // the output-channel extent first, as logConvProfile expects
     const int ko = metadata.data[5];
@@ -734,11 +740,15 @@ MemRefType<int8_t, 4> ral_pdll_qconv2d(ExecutionContext* ctx, void* stream_handl
   result = assignMemRef<int8_t, 4>(data, plan.result_sizes);
   void* stream = drv->asCUStream(ctx, stream_handle);
   const int32_t zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
+  const size_t ws_bytes = dq8_qconv2d_workspace_bytes(input.sizes, weight.sizes, plan.metadata);
+  void* ws = ws_bytes ? drv->alloc(ctx, ws_bytes) : nullptr;
+  if (ws_bytes && !ws) return result;
   StreamTimer timer(stream);
-  int st = dq8_qconv2d(input.data, input.sizes, weight.data, weight.sizes, plan.padding,
-                       plan.metadata, result.data, result.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
-                       DQ8_BIAS_NONE, inputScales.data, weightScales.data,
-                       weightScales.sizes[0], resultScales.data, zo, stream);
+  int st = dq8_qconv2d_ws(input.data, input.sizes, weight.data, weight.sizes, plan.padding,
+                          plan.metadata, result.data, result.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
+                          DQ8_BIAS_NONE, inputScales.data, weightScales.data,
+                          weightScales.sizes[0], resultScales.data, zo, ws, ws_bytes, stream);
+  if (ws) drv->dealloc(ctx, ws);
   if (timer.on() && st == 0)   // weights are [out_channels, h, w, in_channels] here
     logConvProfile(who, input.sizes, weight.sizes, result.sizes, timer.stop());
   kernelFailed(ctx, st, who);

@@ -185,9 +185,10 @@ NHWC_OHWI = (0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2)
 
 
 def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=None,
-            bias=None, zo=0, variant=-1, out=None):
+            bias=None, zo=0, variant=-1, out=None, workspace=True):
     """int8 convolution; layouts/strides/dilations from the 17-entry ral_qconv
-    metadata, padding = (top, bottom, left, right)."""
+    metadata, padding = (top, bottom, left, right).  workspace=False withholds the scratch
+    that keeps channel counts off a multiple of 16 on the MFMA kernels."""
     _need_cuda(x, w, bias)
     L = _lib.lib()
     x = x.contiguous()
@@ -200,11 +201,14 @@ def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=N
     so = _scale(so, dev) if so is not None else None
     bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
     i64x4 = C.c_int64 * 4
+    md = (C.c_int32 * 17)(*metadata)
+    ws_bytes = L.dq8_qconv2d_workspace_bytes(i64x4(*x.shape), i64x4(*w.shape), md) if workspace else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     st = L.dq8_qconv2d_variant(
         variant, _ptr(x), i64x4(*x.shape), _ptr(w), i64x4(*w.shape),
-        (C.c_int32 * 4)(*padding), (C.c_int32 * 17)(*metadata), _ptr(out),
+        (C.c_int32 * 4)(*padding), md, _ptr(out),
         i64x4(*out_shape), epilogue, _ptr(bias), bias_kind, _ptr(sx), _ptr(sw),
-        sw.numel() if sw is not None else 0, _ptr(so), zo, _stream())
+        sw.numel() if sw is not None else 0, _ptr(so), zo, _ptr(ws), ws_bytes, _stream())
     _lib.check(st, "dq8_qconv2d")
     return out
 

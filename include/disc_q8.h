@@ -236,6 +236,19 @@ int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                 const int64_t out_sizes[4], int epilogue, const void* bias,
                 int bias_kind, const float* sx, const float* sw, int64_t n_sw,
                 const float* so, int32_t zo, void* stream);
+/* The same with device scratch: NHWC x OHWI with Ci % 16 != 0 (an RGB first layer) then
+ * stays on the MFMA path -- input and weights are rewritten into `workspace`
+ * (256-byte aligned, dq8_qconv2d_workspace_bytes() bytes) with the channels zero-filled
+ * to the next multiple of 16.  With less scratch the result is the same, from the
+ * generic kernel.  dq8_qconv2d_workspace_bytes() is 0 when nothing would be rewritten. */
+size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const int64_t w_sizes[4],
+                                   const int32_t metadata[17]);
+int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                   const int64_t w_sizes[4], const int32_t padding[4],
+                   const int32_t metadata[17], void* out, const int64_t out_sizes[4],
+                   int epilogue, const void* bias, int bias_kind, const float* sx,
+                   const float* sw, int64_t n_sw, const float* so, int32_t zo,
+                   void* workspace, size_t workspace_bytes, void* stream);
 int dq8_qconv2d_variant(int variant, const int8_t* in,
                         const int64_t in_sizes[4], const int8_t* w,
                         const int64_t w_sizes[4], const int32_t padding[4],
@@ -243,7 +256,8 @@ int dq8_qconv2d_variant(int variant, const int8_t* in,
                         const int64_t out_sizes[4], int epilogue,
                         const void* bias, int bias_kind, const float* sx,
                         const float* sw, int64_t n_sw, const float* so,
-                        int32_t zo, void* stream);
+                        int32_t zo, void* workspace, size_t workspace_bytes,
+                        void* stream);
 
 /* ---- self-test hook ---------------------------------------------------- */
 

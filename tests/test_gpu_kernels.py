@@ -452,6 +452,8 @@ def test_activation_table_equals_the_operator_chain(K):
 
 # ------------------------------------------------------------------------- conv
 CONVS = [  # nb, h, w, ci, co, k, stride, pad, dil
+    (2, 30, 30, 3, 64, 7, 2, 3, 1),      # an RGB first layer: channels padded into scratch
+    (1, 9, 9, 20, 24, 3, 1, 1, 1),
     (2, 14, 14, 64, 64, 3, 1, 1, 1),
     (2, 9, 11, 32, 48, 3, 2, 1, 1),
     (1, 8, 8, 16, 16, 3, 1, 2, 2),

@@ -202,7 +202,7 @@ def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
 
 
 @pytest.mark.parametrize("nb,h,ci,co,k,stride,pad", [(2, 14, 64, 64, 3, 1, 1), (2, 7, 256, 128, 1, 1, 0),
-                                                      (1, 9, 32, 16, 3, 2, 1)])
+                                                      (1, 9, 32, 16, 3, 2, 1), (2, 30, 3, 64, 7, 2, 3)])
 def test_ral_qconv(rt, nb, h, ci, co, k, stride, pad):
     ctx, ral, ops = rt
     rng = np.random.default_rng(h + ci)
