@@ -468,7 +468,16 @@ def extras(torch, steps, warmup, which="all"):
         gbps = nbytes * reps / ev / 1e9
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 5}
-    del x, q, f
+    # 256-entry table over an int8 tensor: 1 byte read + 1 written per element
+    table = torch.arange(256, dtype=torch.int16, device="cuda").to(torch.uint8).view(torch.int8)
+    q2 = torch.empty_like(q)
+    for _ in range(3):
+        K.lut8(q, table, out=q2)
+    _, ev = time_steps(torch, lambda: K.lut8(q, table, out=q2), reps, 3)
+    gbps = 2.0 * rows * cols * reps / ev / 1e9
+    out["lut8"] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
+                   "shape": [rows, cols], "bytes_per_elem": 2}
+    del x, q, f, q2
     # smaller activations (they fit the 256 MB last-level cache; launches captured in a graph)
     small = {}
     for shape in ((16, 768), (1000, 768), (4096, 768), (16384, 768), (32, 56, 56, 64),
