@@ -134,3 +134,39 @@ def test_gpu_signature_entry_against_eager_fake_quant(rt, shape, bias_kind):
         torch.cuda.synchronize()
         exact = pre_round(x_q, w_q, sw, bias_model)
         check(got.reshape(-1, 64), want.reshape(-1, 64), exact)
+
+
+@pytest.mark.parametrize("shape,s_o", [((512, 512), 0.05), ((8, 512, 512), 0.1)])
+def test_reference_gpu_cases_512(rt, shape, s_o):
+    """The two GPU cases of the reference's end-to-end test (test_quantization.py:356-460):
+    512 x 512 weights, inputs [512, 512] and [8, 512, 512], f32 bias, output scale 0.05 /
+    0.1, checked the way it checks them -- within one output step (atol = output scale) --
+    and, more strictly, equal wherever the exact pre-rounding value is neither saturated nor
+    within 0.02 of a rounding tie (the eager model sums 512 products in float32)."""
+    ctx, ral, ops = rt
+    from bladedisc_amd import kernels as K
+    g = torch.Generator(device="cuda").manual_seed(len(shape))
+    x = torch.randn(shape, device="cuda", generator=g)
+    w = torch.randn((512, 512), device="cuda", generator=g)
+    bias = torch.randn(512, device="cuda", generator=g)
+    z1 = torch.zeros(1, dtype=torch.int32, device="cuda")
+    xf = torch.fake_quantize_per_tensor_affine(x, S_X, 0, -128, 127)
+    wf = torch.fake_quantize_per_tensor_affine(w, S_W, 0, -128, 127)
+    want = torch.fake_quantize_per_tensor_affine(torch.nn.functional.linear(xf, wf, bias=bias),
+                                                 s_o, 0, -128, 127)
+    w_q = K.quantize(w, t1(S_W), z1)
+    with ctx.execution() as ex:
+        x_q = ops.quantize(ex, x, t1(S_X), z1)
+        y_q = ops.pdll_qgemm_gpu(ex, x_q, w_q, bias / s_o, t1(S_X), t1(S_W), t1(s_o))
+        got = ops.dequantize(ex, y_q, t1(s_o), z1)
+        torch.cuda.synchronize()
+    assert tuple(got.shape) == tuple(shape)
+    diff = (got - want).abs().double().reshape(-1, 512)
+    assert float(diff.max()) <= s_o * 1.0001
+    acc = (x_q.reshape(-1, 512).to(torch.float64) @ w_q.to(torch.float64).T)      # exact: < 2^53
+    exact = acc * (S_X * S_W / s_o) + bias.double()[None, :] / s_o
+    frac = (exact - torch.floor(exact) - 0.5).abs()
+    clear = (frac > 0.02) & (exact.abs() < 127)
+    assert bool((diff[clear] == 0).all())
+    assert float(clear.double().mean()) > 0.05        # (most outputs saturate with these scales)
+    assert float((diff == 0).double().mean()) > 0.99
