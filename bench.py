@@ -468,6 +468,15 @@ def extras(torch, steps, warmup, which="all"):
         gbps = nbytes * reps / ev / 1e9
         out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
                      "shape": [rows, cols], "bytes_per_elem": 5}
+    # quantize -> dequantize in one pass: 4 bytes read + 4 written per element
+    for _ in range(3):
+        K.fake_quant(x, s1, z1, out=f)
+    for name, fn in (("fake_quant_per_tensor", lambda: K.fake_quant(x, s1, z1, out=f)),
+                     ("fake_quant_per_channel_last_axis", lambda: K.fake_quant(x, sc, zc, axis=1, out=f))):
+        _, ev = time_steps(torch, fn, reps, 3)
+        gbps = 8.0 * rows * cols * reps / ev / 1e9
+        out[name] = {"GB/s": round(gbps, 1), "frac_of_hbm_peak": round(gbps / PEAK_HBM_GBPS, 4),
+                     "shape": [rows, cols], "bytes_per_elem": 8}
     # 256-entry table over an int8 tensor: 1 byte read + 1 written per element
     table = torch.arange(256, dtype=torch.int16, device="cuda").to(torch.uint8).view(torch.int8)
     q2 = torch.empty_like(q)

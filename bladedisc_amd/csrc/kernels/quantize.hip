@@ -198,6 +198,91 @@ dequantize_rows(const uint32_t* __restrict__ q, float4* __restrict__ out,
   }
 }
 
+// ------------------------------------------------------------------ fake quant
+// quantize followed by dequantize without the 8-bit tensor in between: f32 in, f32 out,
+// the two functions' arithmetic unchanged (the integer result is subtracted from the zero
+// point as an integer, as dequantize does).
+template <int ROUND>
+__device__ __forceinline__ float fake_one(float x, float s, int zi, float lo, float hi) {
+  const int q = quant_one<ROUND>(x, s, (float)zi, lo, hi);
+  return (float)(q - zi) * s;
+}
+
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+fake_quant_tensor_v4(const float4* __restrict__ x, float4* __restrict__ out, int64_t n4,
+                     const float* __restrict__ scale, const int32_t* __restrict__ zp, float lo,
+                     float hi) {
+  const float s = scale[0];
+  const int z = zp[0];
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n4; i += stride) {
+    const float4 v = x[i];
+    out[i] = make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
+                         fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi));
+  }
+}
+
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+fake_quant_lastaxis_v4(const float4* __restrict__ x, float4* __restrict__ out, int64_t rows,
+                       int nch4, int rows_per_block, const float4* __restrict__ scale,
+                       const int4* __restrict__ zp, float lo, float hi) {
+  const int c4 = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c4 >= nch4) return;
+  const float4 s = scale[c4];
+  const int4 z = zp[c4];
+  const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
+  const int64_t r_end = r_begin + rows_per_block < rows ? r_begin + rows_per_block : rows;
+  const int64_t step = blockDim.y;
+  const int64_t hop = step * nch4;
+  int64_t r = r_begin + threadIdx.y;
+  const float4* px = x + r * nch4 + c4;
+  float4* po = out + r * nch4 + c4;
+  auto one = [&](const float4& v) {
+    return make_float4(fake_one<ROUND>(v.x, s.x, z.x, lo, hi), fake_one<ROUND>(v.y, s.y, z.y, lo, hi),
+                       fake_one<ROUND>(v.z, s.z, z.z, lo, hi), fake_one<ROUND>(v.w, s.w, z.w, lo, hi));
+  };
+  for (; r + 3 * step < r_end; r += 4 * step, px += 4 * hop, po += 4 * hop) {
+    const float4 v0 = px[0], v1 = px[hop], v2 = px[2 * hop], v3 = px[3 * hop];
+    po[0] = one(v0);
+    po[hop] = one(v1);
+    po[2 * hop] = one(v2);
+    po[3 * hop] = one(v3);
+  }
+  for (; r < r_end; r += step, px += hop, po += hop) po[0] = one(px[0]);
+}
+
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+fake_quant_rows_v4(const float4* __restrict__ x, float4* __restrict__ out, unsigned rows,
+                   int64_t inner4, unsigned nch, const float* __restrict__ scale,
+                   const int32_t* __restrict__ zp, float lo, float hi) {
+  const unsigned row = blockIdx.y + blockIdx.z * gridDim.y;
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (row >= rows || i >= inner4) return;
+  const float4 v = x[(int64_t)row * inner4 + i];
+  __builtin_amdgcn_sched_barrier(0);   // parameters after the data load, as in quantize_rows_v4
+  const unsigned c = row % nch;
+  const float s = scale[c];
+  const int z = zp[c];
+  out[(int64_t)row * inner4 + i] =
+      make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
+                  fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi));
+}
+
+template <int ROUND>
+__global__ void __launch_bounds__(kThreads)
+fake_quant_scalar(const float* __restrict__ x, float* __restrict__ out, int64_t begin, int64_t n,
+                  int64_t nch, int64_t inner, int per_channel, const float* __restrict__ scale,
+                  const int32_t* __restrict__ zp, float lo, float hi) {
+  for (int64_t i = begin + (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kThreads) {
+    const int64_t c = per_channel ? (i / inner) % nch : 0;
+    out[i] = fake_one<ROUND>(x[i], scale[c], zp[c], lo, hi);
+  }
+}
+
 // ------------------------------------------------------------ scalar fallback
 template <int ROUND>
 __global__ void __launch_bounds__(kThreads)
@@ -355,4 +440,66 @@ extern "C" int dq8_dequantize(const void* q, int in_kind, float* out,
                        scale, zp, is_signed);
   }
   return dq8::check_hip(hipGetLastError(), "dq8_dequantize launch");
+}
+
+extern "C" int dq8_fake_quant(const float* x, float* out, int64_t outer, int64_t nch,
+                              int64_t inner, const float* scale, const int32_t* zp, int64_t n_q,
+                              int32_t qmin, int32_t qmax, int round_mode, void* stream) {
+  dq8::clear_error();
+  DQ8_REQUIRE(outer >= 0 && nch >= 0 && inner >= 0, "dq8_fake_quant: negative size");
+  DQ8_REQUIRE(round_mode == DQ8_ROUND_HALF_TO_EVEN ||
+                  round_mode == DQ8_ROUND_HALF_AWAY_FROM_ZERO,
+              "dq8_fake_quant: unknown round_mode");
+  DQ8_REQUIRE(n_q == 1 || n_q == nch, "dq8_fake_quant: n_q must be 1 or nch");
+  DQ8_REQUIRE(qmin <= qmax && qmin >= -32768 && qmax <= 65535,
+              "dq8_fake_quant: quant_min/quant_max outside the 8- and 16-bit ranges");
+  const int64_t n = outer * nch * inner;
+  if (n == 0) return 0;
+  DQ8_REQUIRE(x && out && scale && zp, "dq8_fake_quant: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const float lo = (float)qmin, hi = (float)qmax;
+  const bool per_channel = n_q > 1;
+  const bool vec_ok = dq8::aligned(x, 16) && dq8::aligned(out, 16);
+  const bool rne = round_mode == DQ8_ROUND_HALF_TO_EVEN;
+
+#define LAUNCH_RND(kernel, grid, block, ...)                                        \
+  do {                                                                              \
+    if (rne)                                                                        \
+      hipLaunchKernelGGL((kernel<DQ8_ROUND_HALF_TO_EVEN>), grid, block, 0, st,      \
+                         __VA_ARGS__);                                              \
+    else                                                                            \
+      hipLaunchKernelGGL((kernel<DQ8_ROUND_HALF_AWAY_FROM_ZERO>), grid, block, 0,   \
+                         st, __VA_ARGS__);                                          \
+  } while (0)
+
+  if (!per_channel) {
+    const int64_t n4 = vec_ok ? n / 4 : 0;
+    if (n4 > 0)
+      LAUNCH_RND(fake_quant_tensor_v4, dim3(sweep_grid(n4)), dim3(kThreads), (const float4*)x,
+                 (float4*)out, n4, scale, zp, lo, hi);
+    if (n4 * 4 < n)
+      LAUNCH_RND(fake_quant_scalar, dim3(grid_for(n - n4 * 4, 1)), dim3(kThreads), x, out,
+                 n4 * 4, n, (int64_t)1, (int64_t)1, 0, scale, zp, lo, hi);
+  } else if (vec_ok && inner == 1 && nch % 4 == 0 && nch / 4 < (1 << 30) &&
+             dq8::aligned(scale, 16) && dq8::aligned(zp, 16)) {
+    const int nch4 = (int)(nch / 4);
+    const LastAxisPlan lp = plan_last_axis(outer, nch4);
+    LAUNCH_RND(fake_quant_lastaxis_v4, dim3(lp.gx, lp.gy), dim3(lp.bx, lp.by), (const float4*)x,
+               (float4*)out, outer, nch4, lp.rows_per_block, (const float4*)scale,
+               (const int4*)zp, lo, hi);
+  } else if (vec_ok && inner % 4 == 0 && outer * nch < (1LL << 31) &&
+             inner / 4 < (1LL << 38) && dq8::ceil_div(outer * nch, 32768) <= 65535) {
+    const int64_t rows = outer * nch;
+    const int64_t inner4 = inner / 4;
+    const unsigned gx = (unsigned)dq8::ceil_div(inner4, kThreads);
+    const int gy = (int)std::min<int64_t>(rows, 32768);
+    const int64_t gz = dq8::ceil_div(rows, gy);
+    LAUNCH_RND(fake_quant_rows_v4, dim3(gx, gy, (unsigned)gz), dim3(kThreads), (const float4*)x,
+               (float4*)out, (unsigned)rows, inner4, (unsigned)nch, scale, zp, lo, hi);
+  } else {
+    LAUNCH_RND(fake_quant_scalar, dim3(grid_for(n, 1)), dim3(kThreads), x, out, (int64_t)0, n,
+               nch, inner, 1, scale, zp, lo, hi);
+  }
+#undef LAUNCH_RND
+  return dq8::check_hip(hipGetLastError(), "dq8_fake_quant launch");
 }

@@ -78,6 +78,23 @@ def quantize(x, scale, zero_point, axis=None, qmin=-128, qmax=127,
     return out
 
 
+def fake_quant(x, scale, zero_point, axis=None, qmin=-128, qmax=127,
+               round_mode=ROUND_HALF_TO_EVEN, out=None):
+    """dequantize(quantize(x)) in one pass: f32 -> f32, the same bits as the two calls."""
+    _need_cuda(x, scale, zero_point)
+    if x.dtype != torch.float32:
+        raise TypeError("fake_quant takes float32 tensors")
+    x = x.contiguous()
+    outer, nch, inner = _view3(tuple(x.shape), axis)
+    if out is None:
+        out = torch.empty_like(x)
+    n_q = scale.numel() if axis is not None else 1
+    st = _lib.lib().dq8_fake_quant(_ptr(x), _ptr(out), outer, nch, inner, _ptr(scale),
+                                   _ptr(zero_point), n_q, qmin, qmax, round_mode, _stream())
+    _lib.check(st, "dq8_fake_quant")
+    return out
+
+
 def minmax(x, min_io, max_io, axis=None, workspace=None):
     """Folds the minimum and maximum of `x` (device f32), per tensor (axis None) or per
     slice along `axis`, into the running values min_io / max_io (device f32, one entry or

@@ -7,8 +7,8 @@ modes (``observe`` / ``fake_quant``), state (``min_val``, ``max_val``, ``scale``
 
 * the statistic -- running min / max per tensor or per channel -- is ``dq8_minmax`` (the
   reference calls ``torch.aminmax``, observer.py:238, 270-275);
-* fake quantization is ``dq8_quantize`` followed by ``dq8_dequantize``: the arithmetic a
-  compiled program executes for the observer's qparams (``x / scale`` as a true division;
+* fake quantization is ``dq8_fake_quant``, ``dq8_quantize`` followed by ``dq8_dequantize`` in
+  one pass: the arithmetic a compiled program executes for the observer's qparams (``x / scale`` as a true division;
   ``torch.fake_quantize_per_tensor_affine``, which the reference calls at observer.py:203-206,
   multiplies by ``1 / scale`` and can differ from it in the last bit at ties).
 
@@ -122,16 +122,13 @@ class Observer:
         return scale, zero_point
 
     def _fake_quant(self, x, scale, zero_point):
-        """quantize -> dequantize with the observer's qparams on the GPU kernels (8-bit
+        """quantize -> dequantize with the observer's qparams in one GPU kernel (8-bit
         types); the int32 bias grid is evaluated with the same formula in torch."""
         scale = scale.reshape(-1).float()
         zero_point = zero_point.reshape(-1).to(torch.int32)
         axis = self.ch_axis if self.per_channel else None
         if self.bit == 8:
-            dt = torch.int8 if self.signed else torch.uint8
-            q = K.quantize(x, scale, zero_point, axis=axis, qmin=self.q_min, qmax=self.q_max,
-                           dtype=dt)
-            return K.dequantize(q, scale, zero_point, axis=axis)
+            return K.fake_quant(x, scale, zero_point, axis=axis, qmin=self.q_min, qmax=self.q_max)
         shape = [1] * x.dim()
         if axis is not None:
             shape[axis] = -1

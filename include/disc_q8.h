@@ -112,6 +112,15 @@ int dq8_dequantize(const void* q, int in_kind, float* out, int64_t outer,
                    int64_t nch, int64_t inner, const float* scale,
                    const int32_t* zp, int64_t n_q, void* stream);
 
+/* Fake quantization: dq8_dequantize(dq8_quantize(x)) in one pass, f32 -> f32, without
+ * the integer tensor in between; bit for bit the result of the two calls (what the
+ * reference's observers apply while calibrating, R tools/torch_quant/torch_quant/
+ * observer.py:181-208; the compiler rewrites mhlo_disc.fake_quant into exactly this pair,
+ * R disc/transforms/disc_convert_fake_quant_op.cc).  Arguments as for dq8_quantize; qmin / qmax within [-32768, 65535].  out may be x. */
+int dq8_fake_quant(const float* x, float* out, int64_t outer, int64_t nch, int64_t inner,
+                   const float* scale, const int32_t* zp, int64_t n_q, int32_t qmin,
+                   int32_t qmax, int round_mode, void* stream);
+
 /* ---- elementwise function between two quantized tensors ----------------- */
 
 /* out[i] = table[in[i]] over n bytes (device; in == out allowed), `table` = 256 device bytes

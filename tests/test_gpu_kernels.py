@@ -376,6 +376,38 @@ def test_quantize_dequantize_parity(K, shape, axis, round_mode):
     np.testing.assert_array_equal(got_f, want_f)
 
 
+@pytest.mark.parametrize("shape,axis", [((1000, 768), None), ((1003,), None), ((64, 768), 1), ((768, 768), 0),
+                                        ((2, 3, 4, 5), 1), ((32, 8, 8, 64), 3), ((33, 52), 1), ((5, 7), 1)])
+@pytest.mark.parametrize("round_mode", [0, 1])
+@pytest.mark.parametrize("unsigned", [False, True])
+def test_fake_quant_equals_quantize_then_dequantize(K, shape, axis, round_mode, unsigned):
+    """dq8_fake_quant against the oracle's quantize -> dequantize and against the two GPU
+    kernels, bit for bit (ties, saturation, non-zero zero points, in place)."""
+    rng = np.random.default_rng(len(shape) * 31 + shape[0] + round_mode + 2 * unsigned)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    flat = x.reshape(-1)
+    flat[::7] = np.round(flat[::7] * 4) / 8          # plenty of exact halves after scaling by 1/0.125
+    flat[::11] = 1e9
+    nq = shape[axis] if axis is not None else 1
+    scale = np.full(nq, 0.125, np.float32) if nq == 1 else rng.choice([0.125, 0.25, 0.1], nq).astype(np.float32)
+    zp = rng.integers(-10, 11, nq).astype(np.int32) + (128 if unsigned else 0)
+    qmin, qmax = (0, 255) if unsigned else (-128, 127)
+    dt = np.uint8 if unsigned else np.int8
+    want = O.dequantize(O.quantize(x, scale, zp, axis=axis, qmin=qmin, qmax=qmax,
+                                   round_mode=round_mode, dtype=dt), scale, zp, axis=axis)
+    dx, ds, dz = dev(x), dev(scale), dev(zp)
+    got = K.fake_quant(dx, ds, dz, axis=axis, qmin=qmin, qmax=qmax, round_mode=round_mode)
+    assert np.array_equal(host(got).view(np.uint32), want.view(np.uint32))
+    two = K.dequantize(K.quantize(dx, ds, dz, axis=axis, qmin=qmin, qmax=qmax, round_mode=round_mode,
+                                  dtype=torch.uint8 if unsigned else torch.int8), ds, dz, axis=axis)
+    assert torch.equal(got.view(torch.int32), two.view(torch.int32))
+    K.fake_quant(dx, ds, dz, axis=axis, qmin=qmin, qmax=qmax, round_mode=round_mode, out=dx)   # in place
+    assert torch.equal(dx.view(torch.int32), got.view(torch.int32))
+    # idempotent on its own output
+    again = K.fake_quant(got, ds, dz, axis=axis, qmin=qmin, qmax=qmax, round_mode=round_mode)
+    assert torch.equal(again, got)
+
+
 def test_quantize_golden_vectors(K, golden):
     for case in golden["quantize_fold"]:
         if case["dtype"] not in ("int8", "uint8"):
