@@ -221,11 +221,14 @@ def test_config5_bert_layer_dequantize_in_the_gemm_epilogue_is_bit_identical(C, 
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
 
 
-def test_config5_bert_layer_graph_replays_match_eager(C):
+@pytest.mark.parametrize("fused", [False, True])
+def test_config5_bert_layer_graph_replays_match_eager(C, fused):
     """The captured layer against eager execution: several replays, with eager work and
-    synchronisations in between, each compared bit for bit."""
+    synchronisations in between, each compared bit for bit; also with the GELU table and the
+    dequantize-in-epilogue forms switched on."""
     from bladedisc_amd import bert_layer as B
-    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend())
+    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend(), fuse_gelu=fused,
+                             fuse_dequant=fused)
     h0 = layer.embed(C.config5_tokens(8, 32))
     layer.calibrate(h0)
     replay, static_in, static_out = layer.capture(h0)
