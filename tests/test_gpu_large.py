@@ -108,3 +108,37 @@ def test_quantize_dequantize_more_than_2_31_elements(axis):
         lim_hi = (127 - zp).float() * scale
         err = (ys - torch.maximum(torch.minimum(xs, lim_hi), lim_lo)).abs()
         assert bool((err <= scale * 0.5001).all()), lo
+
+
+def test_qconv_input_larger_than_2_gib():
+    """NHWC input of 2.2 GB (33 x 256 x 256 x 1024), 1x1 filter with stride 2: beyond the 32-bit
+    buffer offsets of the pipelined kernels, so the implicit GEMM must take the path with
+    64-bit image bases.  The oracle convolves the first and the last image, and the image
+    that straddles the 2^31-byte mark."""
+    from bladedisc_amd import kernels as K
+    nb, h, ci, co = 33, 256, 1024, 16
+    g = torch.Generator(device="cuda").manual_seed(8)
+    x = torch.randint(-128, 128, (nb, h, h, ci), dtype=torch.int8, device="cuda", generator=g)
+    w = torch.randint(-128, 128, (co, 1, 1, ci), dtype=torch.int8, device="cuda", generator=g)
+    md = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
+    out_shape = [nb, h // 2, h // 2, co]
+    sx = torch.full((1,), 0.02, device="cuda")
+    sw = torch.rand(co, device="cuda", generator=g) * 0.05 + 0.001
+    so = torch.full((1,), 8.0, device="cuda")
+    acc = K.qconv2d(x, w, [0, 0, 0, 0], md, out_shape, K.EPI_ACC_S32)
+    y = K.qconv2d(x, w, [0, 0, 0, 0], md, out_shape, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so)
+    torch.cuda.synchronize()
+    w_h = w.cpu().numpy()
+    straddling = (1 << 31) // (h * h * ci)
+    for b in (0, straddling, nb - 1):
+        want = O.conv_s32(x[b:b + 1].cpu().numpy(), w_h, [0, 0, 0, 0], md, [1] + out_shape[1:])
+        assert np.array_equal(acc[b:b + 1].cpu().numpy(), want), b
+        want_q = O.requant_cpu(want.reshape(-1, co), np.float32(0.02), sw.cpu().numpy(),
+                               np.float32(8.0)).reshape(want.shape)
+        assert np.array_equal(y[b:b + 1].cpu().numpy(), want_q), b
+    # every image equals the convolution of that image alone
+    for b in range(nb):
+        one = K.qconv2d(x[b:b + 1], w, [0, 0, 0, 0], md, [1] + out_shape[1:], K.EPI_REQUANT_CPU,
+                        sx=sx, sw=sw, so=so)
+        assert torch.equal(one, y[b:b + 1]), b
+    assert float(((y == 127) | (y == -128)).float().mean()) < 0.5
