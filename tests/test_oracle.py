@@ -347,3 +347,52 @@ def test_requant_cpu_tie_margin_audit():
         assert np.abs(q - base).max() <= 1
         assert np.all(dist_to_tie[differs] < margin)
         assert differs.mean() < 0.01
+
+
+def test_requant_cpu_agrees_with_library_quantized_linear_away_from_ties():
+    """Cross-check of E1 against library routines of this image (PyTorch's CPU quantized
+    linear on its qnnpack, fbgemm and oneDNN-3 engines) -- not the reference, whose oneDNN 2.x
+    is absent, but independent implementations of the same contract: int32 accumulate, bias
+    quantized to int32 with scale s_x s_w[n], one multiplication by s_x s_w[n] / s_o, round to
+    nearest even, saturate.  They must agree with the oracle wherever the exact pre-rounding
+    value is further than 2^-10 from a rounding tie (the margin of the audit above), and never
+    differ by more than one step."""
+    torch = pytest.importorskip("torch")
+    engines = [e for e in torch.backends.quantized.supported_engines if e in ("qnnpack", "fbgemm", "onednn")]
+    if not engines:
+        pytest.skip("no CPU quantized engine in this torch build")
+    rng = np.random.default_rng(0)
+    saved = torch.backends.quantized.engine
+    checked = 0
+    try:
+        for m, k, n in [(64, 256, 128), (128, 768, 768), (33, 100, 77)]:
+            x_q = rng.integers(-128, 128, (m, k), dtype=np.int8)
+            w_q = rng.integers(-128, 128, (n, k), dtype=np.int8)
+            sx = np.float32(rng.uniform(0.01, 0.03))
+            sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+            acc = O.gemm_s32(x_q, w_q, tp_b=True)
+            so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40)
+            bias = (rng.standard_normal(n) * 3 * so).astype(np.float32)
+            b32 = O.bias_f32_to_s32(bias, sx, sw)
+            want = O.requant_cpu(acc, sx, sw, so, b32=b32)
+            exact = (acc.astype(np.float64) + b32.astype(np.float64)[None, :]) * \
+                (np.float64(sx) * sw.astype(np.float64) / np.float64(so))[None, :]
+            near_tie = np.abs(exact - np.floor(exact) - 0.5) < 2.0 ** -10
+            for eng in engines:
+                torch.backends.quantized.engine = eng
+                # these engines take unsigned activations: the same values with zero point 128
+                xq = torch._make_per_tensor_quantized_tensor(
+                    torch.from_numpy((x_q.astype(np.int16) + 128).astype(np.uint8)), float(sx), 128)
+                wq = torch._make_per_channel_quantized_tensor(
+                    torch.from_numpy(w_q), torch.from_numpy(sw.astype(np.float64)),
+                    torch.zeros(n, dtype=torch.int64), 0)
+                packed = torch.ops.quantized.linear_prepack(wq, torch.from_numpy(bias))
+                y = torch.ops.quantized.linear(xq, packed, float(so), 128)
+                got = y.int_repr().numpy().astype(np.int16) - 128
+                differs = got != want
+                assert np.abs(got - want).max() <= 1, eng
+                assert not (differs & ~near_tie).any(), eng
+                checked += int((~near_tie).sum())
+    finally:
+        torch.backends.quantized.engine = saved
+    assert checked > 100000
