@@ -396,3 +396,48 @@ def test_requant_cpu_agrees_with_library_quantized_linear_away_from_ties():
     finally:
         torch.backends.quantized.engine = saved
     assert checked > 100000
+
+
+def test_conv_oracle_agrees_with_library_quantized_conv2d():
+    """The convolution geometry (padding, stride, dilation, NHWC x OHWI) and its requant against
+    PyTorch's CPU quantized conv2d on the fbgemm and qnnpack engines (libraries of this image,
+    not the reference): equal wherever the pre-rounding value is further than 2^-10 from a tie,
+    within one step elsewhere."""
+    torch = pytest.importorskip("torch")
+    engines = [e for e in torch.backends.quantized.supported_engines if e in ("qnnpack", "fbgemm")]
+    if not engines:
+        pytest.skip("no CPU quantized engine in this torch build")
+    rng = np.random.default_rng(1)
+    saved = torch.backends.quantized.engine
+    try:
+        for nb, h, w_, ci, co, k, stride, pad, dil in [(2, 14, 14, 32, 48, 3, 1, 1, 1), (1, 9, 11, 16, 24, 3, 2, 1, 1),
+                                                       (1, 12, 12, 8, 16, 3, 1, 2, 2), (2, 7, 7, 64, 32, 1, 1, 0, 1)]:
+            x_q = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+            wt = rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8)
+            ho = (h + 2 * pad - dil * (k - 1) - 1) // stride + 1
+            wo = (w_ + 2 * pad - dil * (k - 1) - 1) // stride + 1
+            md = list(O.NHWC_OHWI_METADATA) + [stride, stride, dil, dil, 1]
+            acc = O.conv_s32(x_q, wt, [pad] * 4, md, [nb, ho, wo, co])
+            sx = np.float32(0.02)
+            sw = rng.uniform(0.001, 0.05, co).astype(np.float32)
+            so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40)
+            want = O.requant_cpu(acc.reshape(-1, co), sx, sw, so).reshape(nb, ho, wo, co)
+            exact = acc.astype(np.float64) * (np.float64(sx) * sw.astype(np.float64) / np.float64(so))
+            near_tie = np.abs(exact - np.floor(exact) - 0.5) < 2.0 ** -10
+            for eng in engines:
+                torch.backends.quantized.engine = eng
+                xu = torch.from_numpy((x_q.astype(np.int16) + 128).astype(np.uint8))
+                xq = torch._make_per_tensor_quantized_tensor(
+                    xu.permute(0, 3, 1, 2).contiguous(memory_format=torch.channels_last), float(sx), 128)
+                wq = torch._make_per_channel_quantized_tensor(
+                    torch.from_numpy(wt).permute(0, 3, 1, 2).contiguous(),
+                    torch.from_numpy(sw.astype(np.float64)), torch.zeros(co, dtype=torch.int64), 0)
+                packed = torch.ops.quantized.conv2d_prepack(wq, None, [stride, stride], [pad, pad],
+                                                            [dil, dil], 1)
+                y = torch.ops.quantized.conv2d(xq, packed, float(so), 128)
+                got = y.int_repr().permute(0, 2, 3, 1).numpy().astype(np.int16) - 128
+                assert got.shape == want.shape
+                assert np.abs(got - want).max() <= 1, eng
+                assert not ((got != want) & ~near_tie).any(), eng
+    finally:
+        torch.backends.quantized.engine = saved
