@@ -120,7 +120,10 @@ class GemmCall:
         self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def __call__(self):
-        st = self.L.dq8_qgemm_variant(self.variant, *self.args, self.stream)
+        if self.variant < 0:
+            st = self.L.dq8_qgemm(*self.args, self.stream)
+        else:
+            st = self.L.dq8_qgemm_variant(self.variant, *self.args, self.stream)
         if st != 0:
             raise RuntimeError(self.L.dq8_last_error().decode())
 
