@@ -46,52 +46,7 @@ def parse():
                         "launches would blur per-kernel durations and counters)")
     p.add_argument("--extras", choices=("all", "qdq"), default="all",
                    help="'qdq': only the quantize / dequantize bandwidth cases (for profiling)")
-    p.add_argument("--pattern", choices=("uniform", "ones"), default="uniform",
-                   help="operand values: 'uniform' is the benchmark's definition (integers uniform "
-                        "in [-127,127]); 'ones' is a diagnosis aid that shows how much of the time "
-                        "is the power drawn by toggling operands (same instructions, same traffic)")
-    p.add_argument("--copy-probe", action="store_true",
-                   help="also launch one plain streaming kernel of known size before the timed "
-                        "loop (dst = src + 1 over 1 GiB of int8: reads 1 GiB, writes 1 GiB), the "
-                        "yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
-    p.add_argument("--occupancy-sweep", action="store_true",
-                   help="diagnosis aid instead of the benchmark: the headline kernel on the first "
-                        "512 ... 4096 rows of the problem -- one 256x256x4096 tile per CU on 32 ... 256 "
-                        "CUs, the same work per CU every time -- with the benchmark's operands and "
-                        "with all-ones operands; prints one JSON line")
     return p.parse_args()
-
-
-def occupancy_sweep(torch, size, steps, warmup):
-    """How long one CU takes for its 256 x 256 x K tile as more CUs run the same thing beside
-    it.  Every launch gives each busy CU exactly one tile (M = 256 * tiles / (N / 256)), so a
-    launch time that grows with the number of busy CUs is the chip, not the kernel."""
-    import numpy as np
-    from bladedisc_amd import kernels as K
-    a, w, sx, sw, so, bias_q = make_problem(torch, size)
-    d = lambda v: torch.from_numpy(np.ascontiguousarray(v)).cuda()  # noqa: E731
-    dsx, dsw, dso, dbias = d(np.array([sx])), d(sw), d(np.array([so])), d(bias_q)
-    tile = K.variant_names().index("pipe_256x256x128_w8")    # what the heuristic runs at full size
-    rows = []
-    for pattern in ("uniform", "ones"):
-        if pattern == "ones":
-            a = np.ones_like(a)
-            w = np.ones_like(w)
-        dw = d(w)
-        for m in (size // 8, size // 4, size // 2, 3 * size // 4, size):
-            da = d(a[:m])
-            out = torch.empty((m, size), dtype=torch.int8, device="cuda")
-            call = GemmCall(torch, da, dw, dsx, dsw, dso, dbias, 2, 2, out, variant=tile)
-            _, ev = time_steps(torch, call, steps, warmup)
-            us = ev / steps * 1e6
-            tiles = (m // 256) * (size // 256)
-            rows.append({"operands": pattern, "M": m, "busy_cus": min(tiles, 256),
-                         "us_per_launch": round(us, 1),
-                         "TOPS": round(2.0 * m * size * size / us / 1e6, 1),
-                         "TOPS_per_busy_cu": round(2.0 * m * size * size / us / 1e6 / min(tiles, 256), 2)})
-    print(json.dumps({"kernel": "dq8_qgemm_variant pipe_256x256x128_w8, epilogue REQUANT_GPU, "
-                                "N = K = %d" % size,
-                      "steps": steps, "warmup": warmup, "rows": rows}))
 
 
 def make_problem(torch, size):
@@ -105,10 +60,9 @@ class GemmCall:
     """dq8_qgemm bound once with all arguments, so the timed loop is one ctypes call
     per step."""
 
-    def __init__(self, torch, a, w, sx, sw, so, bias, epilogue, bias_kind, out, variant=-1):
+    def __init__(self, torch, a, w, sx, sw, so, bias, epilogue, bias_kind, out):
         from bladedisc_amd import _lib
         self.L = _lib.lib()
-        self.variant = variant      # -1: the library's own choice of tile
         self._keep = (a, w, sx, sw, so, bias, out)
         m, k = a.shape
         n = w.shape[0]
@@ -120,10 +74,7 @@ class GemmCall:
         self.stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def __call__(self):
-        if self.variant < 0:
-            st = self.L.dq8_qgemm(*self.args, self.stream)
-        else:
-            st = self.L.dq8_qgemm_variant(self.variant, *self.args, self.stream)
+        st = self.L.dq8_qgemm(*self.args, self.stream)
         if st != 0:
             raise RuntimeError(self.L.dq8_last_error().decode())
 
@@ -610,15 +561,8 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
 
-    if args.occupancy_sweep:
-        occupancy_sweep(torch, args.size, min(args.steps, 200), min(args.warmup, 200))
-        return
-
     size = args.size
     a, w, sx, sw, so, bias_q = make_problem(torch, size)
-    if args.pattern == "ones":
-        a[:] = 1
-        w[:] = 1
     d = lambda v: torch.from_numpy(v).cuda()  # noqa: E731
     import numpy as np
     da, dw = d(a), d(w)
@@ -627,13 +571,6 @@ def main():
     out = torch.empty((size, size), dtype=torch.int8, device="cuda")
     # REQUANT_GPU epilogue (2) with an f32 bias (kind 2): out = sat8(rne(os[n]*acc + b[n]))
     call = GemmCall(torch, da, dw, dsx, dsw, dso, dbias, 2, 2, out)
-
-    if args.copy_probe:
-        src = torch.ones(1 << 30, dtype=torch.int8, device="cuda")
-        dst = torch.empty_like(src)
-        torch.add(src, 1, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
 
     wall, ev = time_steps(torch, call, args.steps, args.warmup)
     ops = 2.0 * size * size * size
@@ -665,8 +602,7 @@ def main():
                         "f32 bias + requant to s8 (round-half-even, saturate)" % size,
             "entry": "dq8_qgemm (C ABI), epilogue REQUANT_GPU",
             "saturated_fraction": round(sat_frac, 4),
-            "operand_values": "uniform integers in [-127,127]" if args.pattern == "uniform"
-                              else "all ones (diagnosis run, not the benchmark's data)",
+            "operand_values": "uniform integers in [-127,127]",
         },
         "roofline": {
             "bound": "mfma",
@@ -674,7 +610,7 @@ def main():
             "peak": PEAK_INT8_TOPS,
             "unit": "TOP/s",
             "frac": round(achieved / PEAK_INT8_TOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(size) if args.pattern == "uniform" else None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(size),
             "algorithmic_bytes": 3 * size * size + 8 * size,
             "kernel_us": round(kernel_s * 1e6, 2),
             "ops_per_launch": ops,

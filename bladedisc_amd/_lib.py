@@ -52,6 +52,7 @@ _PROTOS = {
                                  _VP]),
     "dq8_minmax_workspace_bytes": (_SZ, [_I64, _I64, _I64]),
     "dq8_minmax": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP, _SZ, _VP]),
+    "dq8_fill": (_INT, [_VP, _INT, _SZ, _VP]),
 }
 
 

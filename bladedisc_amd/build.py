@@ -30,12 +30,9 @@ DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
 
 
 def sources():
-    """Sources of the library (everything under csrc except the standalone profiling
-    programs)."""
+    """Sources of the library: everything under csrc."""
     out = []
     for d, _, files in os.walk(CSRC):
-        if os.path.basename(d) == "profiling":
-            continue
         for f in sorted(files):
             if f.endswith((".hip", ".cc")):
                 out.append(os.path.join(d, f))
@@ -65,23 +62,6 @@ def _compile(src, force, hdr_m):
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
     return obj, log
-
-
-def build_profiling_tools():
-    """Standalone profiling programs (csrc/profiling/*.hip) -> bladedisc_amd/build/<name>."""
-    os.makedirs(OBJ, exist_ok=True)
-    built = []
-    prof = os.path.join(CSRC, "profiling")
-    for f in sorted(os.listdir(prof)):
-        if not f.endswith(".hip"):
-            continue
-        exe = os.path.join(OBJ, f[:-4])
-        cmd = [HIPCC] + [c for c in COMMON if c != "-fPIC"] + DEVICE + ["-o", exe, os.path.join(prof, f)]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("hipcc failed for %s:\n%s" % (f, r.stdout + r.stderr))
-        built.append(exe)
-    return built
 
 
 def build_test_code_objects():

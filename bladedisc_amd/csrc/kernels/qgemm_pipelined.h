@@ -86,7 +86,7 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, unsigned lds_addr
       "buffer_load_dwordx4 %1, %2, 0 offen lds"
       :
       : "s"(lds_addr), "v"(voffset), "s"(rsrc)
-      : "memory");
+      : "memory", "m0");
 }
 
 // s_waitcnt immediate for gfx9: vmcnt = n (6 bits, split), lgkmcnt = 0, expcnt = any

@@ -4,6 +4,7 @@
 #include <sstream>
 #include <unordered_set>
 
+#include "disc_q8.h"
 #include "mlir/ral/ral_helper.h"
 #include "mlir/ral/ral_logging.h"
 
@@ -177,7 +178,8 @@ void ral_base_hip_dealloc(ExecutionContext* ctx, buffer_t buffer) {
     return;
   }
   if (--it->second == 0) {
-    state->gpu_allocator->dealloc(buffer);
+    // an alias of a program input was pinned by inc_ref; the buffer is the caller's
+    if (!exec->input_ptr_set.count(buffer)) state->gpu_allocator->dealloc(buffer);
     exec->device_ptr_map.erase(it);
   }
 }
@@ -281,7 +283,9 @@ void ral_base_hip_memset(ExecutionContext* ctx, stream_t sidx, buffer_t buffer, 
                          size_t bytes) {
   auto* state = stateOf(ctx);
   if (!state || !validStream(ctx, sidx) || !buffer || !bytes) return;
-  hipOk(hipMemsetAsync(buffer, value, bytes, state->stream), ctx, "memset");
+  // a fill kernel, not hipMemsetAsync: the launch may be recorded into a captured graph
+  if (dq8_fill(buffer, value, bytes, state->stream) != 0)
+    ctx->signalError(Context::FAILURE, std::string("GPU failed in memset: ") + dq8_last_error());
 }
 
 void ral_base_hip_sync_on_stream(ExecutionContext* ctx, stream_t sidx) {
@@ -344,12 +348,18 @@ void BaseHipExecutionContext::bindOutput(int output_idx,
 }
 
 BaseHipExecutionContext::~BaseHipExecutionContext() {
-  // buffers the program never handed back return to the pool with the execution
+  // Buffers the program allocated and never handed back return to the pool with the
+  // execution.  The map also holds entries inc_ref pinned for aliases of program inputs and
+  // of persistent buffers (constants, packed weights): those belong to the caller and to
+  // the context and are left alone.
   auto* state = getResource<BaseHipContextState>(kRalBaseHipContextState);
   if (state) {
     std::lock_guard<std::mutex> guard(state->mu);
-    for (auto& kv : device_ptr_map)
+    for (auto& kv : device_ptr_map) {
+      if (input_ptr_set.count(kv.first) || state->device_persistent_buffers.count(kv.first))
+        continue;
       state->gpu_allocator->dealloc(const_cast<buffer_t>(kv.first));
+    }
   }
   device_ptr_map.clear();
   onExecutionFinish();

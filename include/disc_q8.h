@@ -80,6 +80,12 @@ int dq8_version(void);
  * device; fills what it can, returns 0 on success. */
 int dq8_device_info(int* compute_units, int* lds_bytes_per_cu, int* clock_khz);
 
+/* dst[0 .. bytes) = (uint8_t)value, as a kernel launch (any alignment).  What the runtime's
+ * ral_gpu_memset issues in place of the reference's cudaMemsetAsync
+ * (R ral/context/base/cuda/cuda_context_impl.cc:272-281): a compiled program whose execution
+ * is captured into a HIP graph then records a kernel node, not a memset node. */
+int dq8_fill(void* dst, int value, size_t bytes, void* stream);
+
 /* ---- calibration statistics -------------------------------------------- */
 
 /* Running minimum and maximum of a float tensor, per tensor or per channel: what the
@@ -207,23 +213,6 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
               const float* so, int64_t n_so, int32_t zx, int32_t zw, int32_t zo,
               void* workspace, size_t workspace_bytes, void* stream);
 
-/* Same, forcing one kernel variant (for tests and tuning):
- *  -1 heuristic, 0 generic scalar kernel, 1.. MFMA tile configurations
- *  (dq8_qgemm_num_variants() of them, names from dq8_qgemm_variant_name()).  A problem
- *  an MFMA variant cannot take (unaligned rows; K % 16 != 0 without scratch) runs on the
- *  generic kernel whatever the variant; non-zero zx / zw with a forced MFMA variant is an error
- *  (they need the heuristic or the generic variant). */
-int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
-                      const int8_t* W, int64_t ldw, void* out, int64_t ldo,
-                      int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
-                      int epilogue, const void* bias, int bias_kind,
-                      const float* sx, int64_t n_sx, const float* sw,
-                      int64_t n_sw, const float* so, int64_t n_so, int32_t zx,
-                      int32_t zw, int32_t zo, void* workspace,
-                      size_t workspace_bytes, void* stream);
-int dq8_qgemm_num_variants(void);
-const char* dq8_qgemm_variant_name(int variant);
-
 /* dst[c, r] = src[r, c] for an int8 matrix src [rows, cols] with row stride ld;
  * dst is dense [cols, rows].  Used to put [K,N] weights into the kernels' [N,K]
  * layout once (the reference's counterpart is oneDNN's weight pre-packing,
@@ -258,26 +247,6 @@ int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                    int epilogue, const void* bias, int bias_kind, const float* sx,
                    const float* sw, int64_t n_sw, const float* so, int32_t zo,
                    void* workspace, size_t workspace_bytes, void* stream);
-int dq8_qconv2d_variant(int variant, const int8_t* in,
-                        const int64_t in_sizes[4], const int8_t* w,
-                        const int64_t w_sizes[4], const int32_t padding[4],
-                        const int32_t metadata[17], void* out,
-                        const int64_t out_sizes[4], int epilogue,
-                        const void* bias, int bias_kind, const float* sx,
-                        const float* sw, int64_t n_sw, const float* so,
-                        int32_t zo, void* workspace, size_t workspace_bytes,
-                        void* stream);
-
-/* ---- self-test hook ---------------------------------------------------- */
-
-/* Runs one v_mfma_i32_32x32x32_i8 and one v_mfma_i32_16x16x64_i8 on device
- * buffers: a[32*32] (row i, k contiguous), b[32*32] (column j, k contiguous) ->
- * d32[32*32] row-major; a16[16*64], b16[16*64] -> d16[16*16].  Lets a test pin
- * the operand and result register layouts against brute force. */
-int dq8_mfma_probe(const int8_t* a, const int8_t* b, int32_t* d32,
-                   const int8_t* a16, const int8_t* b16, int32_t* d16,
-                   void* stream);
-
 #ifdef __cplusplus
 }
 #endif

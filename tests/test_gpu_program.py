@@ -238,3 +238,124 @@ def test_dispatch_path_cost_per_call(program, capsys):
         L.disc_ral_execution_context_destroy(C.c_void_p(ex))
         torch.cuda.synchronize()
         L.disc_ral_context_destroy(C.c_void_p(ctx))
+
+
+class _CountingAllocator:
+    """Device memory for a context through the C callbacks of disc_ral_context_create, with
+    every request and every return recorded (backed by torch tensors)."""
+
+    def __init__(self):
+        self.live, self.allocated, self.freed = {}, [], []
+        self._alloc = C.CFUNCTYPE(C.c_void_p, C.c_size_t, C.c_void_p)(self._on_alloc)
+        self._dealloc = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)(self._on_dealloc)
+
+    def _on_alloc(self, nbytes, _user):
+        t = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device="cuda")
+        self.live[t.data_ptr()] = t
+        self.allocated.append(t.data_ptr())
+        return t.data_ptr()
+
+    def _on_dealloc(self, ptr, _user):
+        self.freed.append(ptr)
+        self.live.pop(ptr, None)
+
+
+def test_inc_ref_aliases_of_inputs_and_constants_outlive_the_execution(program):
+    """A compiled graph usually starts by reshaping an input and a constant (inc_ref), and
+    later drops the aliases (dealloc).  Neither the caller's input nor the context's
+    constant may ever reach the allocator's dealloc -- not from the program's dealloc and
+    not when the execution ends -- and the constant serves the next execution intact."""
+    _, d = program
+    from bladedisc_amd import ral
+    L = ral.lib()
+    w = (np.arange(24 * 16, dtype=np.int32) % 251 - 125).astype(np.int8).reshape(24, 16)
+    meta = str(d / "alias.metadata").encode()
+    assert L.disc_ral_metadata_emit(meta, 1, (C.c_uint8 * 1)(0), (C.c_char_p * 1)(b"w0_i8_24x16"),
+                                    (C.c_char_p * 1)(hexstr(w).encode())) == 0
+    L.disc_ral_context_create_for_program.restype = C.c_void_p
+    alloc = _CountingAllocator()
+    stream = torch.cuda.current_stream().cuda_stream
+    ctx_h = L.disc_ral_context_create_for_program(C.c_void_p(stream), 0, alloc._alloc, alloc._dealloc,
+                                                  None, 1, meta)
+    assert ctx_h
+    name = C.create_string_buffer(b"w0_i8_24x16")
+    x = torch.arange(6 * 8, dtype=torch.float32, device="cuda").reshape(6, 8)
+    const_ptrs = []
+
+    class _Ctx:                      # the little of ral.RalContext that RalExecution uses
+        handle, _L, _names = ctx_h, L, {}
+        _name = ral.RalContext._name
+        last_error = ral.RalContext.last_error
+        clear_error = ral.RalContext.clear_error
+
+    try:
+        for run in range(2):
+            ex = ral.RalExecution(_Ctx())
+            assert L.disc_ral_execution_bind_input(C.c_void_p(ex.handle), 0, C.c_void_p(x.data_ptr()),
+                                                   (C.c_int64 * 2)(6, 8), 2) == 0
+            # the constant, as a [24, 16] memref
+            a = ex.new_args().scalar("pvoid", C.addressof(name)).scalar("i32", 0)
+            cst = a.result_memref("i8", 2)
+            ex.call("ral_const", "gpu", a)
+            const_ptrs.append(cst.data)
+            # reshape it to [384] and the input to [48] (inc_ref with a host shape operand)
+            a = ex.new_args().memref("i8", cst.data, [24, 16]).host_array(np.array([384], np.int64))
+            flat_w = a.result_memref("i8", 1)
+            ex.call("inc_ref", "gpu", a)
+            a = ex.new_args().memref("f32", x.data_ptr(), [6, 8]).host_array(np.array([48], np.int64))
+            flat_x = a.result_memref("f32", 1)
+            ex.call("inc_ref", "gpu", a)
+            assert flat_w.data == cst.data and flat_x.data == x.data_ptr()
+            assert flat_w.sizes[0] == 384 and flat_x.sizes[0] == 48
+            # a buffer of the program's own, never handed back: returns with the execution
+            own = ex.alloc(1000)
+            if run == 0:
+                ex.dealloc(flat_w.data)      # the program drops its aliases ...
+                ex.dealloc(flat_x.data)
+            ex.sync()                        # ... or (second run) leaves them to the end
+            got = ral.device_view(cst.data, (24, 16), torch.int8).cpu().numpy()
+            np.testing.assert_array_equal(got, w)
+            ex.close()
+            assert own in alloc.freed
+            assert x.data_ptr() not in alloc.freed
+            assert not set(const_ptrs) & set(alloc.freed)
+        assert const_ptrs[0] == const_ptrs[1]      # served from the context's store
+    finally:
+        torch.cuda.synchronize()
+        L.disc_ral_context_destroy(C.c_void_p(ctx_h))
+    # the context returns its constants when it goes, and only then
+    assert const_ptrs[0] in alloc.freed
+    assert x.data_ptr() not in alloc.freed
+
+
+def test_memset_service_inside_a_captured_graph():
+    """ral_gpu_memset is a kernel launch, so an execution captured into a HIP graph can
+    contain it: every replay clears the buffer again (odd sizes and alignments included),
+    with the program's own eager work between replays."""
+    from bladedisc_amd import ral
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        ctx = ral.RalContext(stream=side.cuda_stream)
+        buf = torch.full((4099,), 7, dtype=torch.uint8, device="cuda")
+        graph = torch.cuda.CUDAGraph()
+        with ctx.execution() as ex:
+            def memset(ptr, value, nbytes):
+                a = ex.new_args().scalar("pvoid", ptr).scalar("i32", value).scalar("i64", nbytes)
+                ex.call("ral_gpu_memset", "gpu", a)
+            memset(buf.data_ptr() + 3, 0x5a, 4090)          # eager, unaligned head and tail
+            side.synchronize()
+            want = np.full(4099, 7, np.uint8)
+            want[3:4093] = 0x5a
+            np.testing.assert_array_equal(buf.cpu().numpy(), want)
+            with torch.cuda.graph(graph, stream=side):
+                memset(buf.data_ptr() + 1, 0, 4097)
+                memset(buf.data_ptr() + 64, 0xff, 16)
+            want[1:4098] = 0
+            want[64:80] = 0xff
+            for rep in range(4):
+                buf.fill_(9 + rep)                           # eager work between the replays
+                want[0] = want[4098] = 9 + rep
+                graph.replay()
+                side.synchronize()
+                np.testing.assert_array_equal(buf.cpu().numpy(), want, err_msg="replay %d" % rep)
+        ctx.close()
