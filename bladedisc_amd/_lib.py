@@ -52,6 +52,8 @@ _PROTOS = {
                                  _VP]),
     "dq8_minmax_workspace_bytes": (_SZ, [_I64, _I64, _I64]),
     "dq8_minmax": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP, _SZ, _VP]),
+    "dq8_minmax_static_max_bytes": (_SZ, []),
+    "dq8_minmax_static": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP]),
     "dq8_fill": (_INT, [_VP, _INT, _SZ, _VP]),
 }
 

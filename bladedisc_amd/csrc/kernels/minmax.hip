@@ -17,6 +17,7 @@
 //    four channels each, a workgroup walks a block of rows.
 #include <algorithm>
 #include <limits>
+#include <mutex>
 
 #include "dq8_common.h"
 #include "disc_q8.h"
@@ -308,22 +309,13 @@ extern "C" size_t dq8_minmax_workspace_bytes(int64_t outer, int64_t channels, in
   return (size_t)p.pairs * sizeof(float2);
 }
 
-extern "C" int dq8_minmax(const float* x, int64_t outer, int64_t channels, int64_t inner,
-                          float* min_io, float* max_io, void* workspace,
-                          size_t workspace_bytes, void* stream) {
-  clear_error();
-  DQ8_REQUIRE(outer >= 0 && channels >= 0 && inner >= 0, "dq8_minmax: negative extent");
-  if (outer == 0 || channels == 0 || inner == 0) return 0;   // nothing observed: state kept
-  DQ8_REQUIRE(x && min_io && max_io, "dq8_minmax: null pointer");
-  DQ8_REQUIRE(channels < (1LL << 31), "dq8_minmax: too many channels");
-  const bool last_axis = inner == 1 && channels > 1;
-  const bool vec = aligned(x, 16) && (last_axis ? channels % 4 == 0 : inner % 4 == 0);
-  Plan p;
-  DQ8_REQUIRE(make_plan(outer, channels, inner, vec, &p), "dq8_minmax: tensor too large");
-  DQ8_REQUIRE(workspace && workspace_bytes >= (size_t)p.pairs * sizeof(float2),
-              "dq8_minmax: workspace too small (see dq8_minmax_workspace_bytes)");
-  hipStream_t st = (hipStream_t)stream;
-  float2* partial = static_cast<float2*>(workspace);
+namespace {
+
+// Shared by the two entry points: both passes with the (min, max) pairs in `partial`.  Pass 1
+// writes every pair pass 2 reads, so the scratch needs no particular contents beforehand.
+int run_minmax(const float* x, int64_t outer, int64_t channels, int64_t inner,
+               float* min_io, float* max_io, float2* partial, const Plan& p, bool vec,
+               hipStream_t st) {
   if (p.last_axis) {
     const dim3 grid((unsigned)p.gx, (unsigned)p.gy), block((unsigned)p.bx, (unsigned)p.by);
     if (vec)
@@ -351,4 +343,83 @@ extern "C" int dq8_minmax(const float* x, int64_t outer, int64_t channels, int64
     hipLaunchKernelGGL(minmax_fold_rows, dim3((unsigned)channels), dim3(kThreads), 0, st, partial,
                        outer, (int)channels, p.segs, min_io, max_io);
   return check_hip(hipGetLastError(), "minmax_fold_rows launch");
+}
+
+}  // namespace
+
+extern "C" int dq8_minmax(const float* x, int64_t outer, int64_t channels, int64_t inner,
+                          float* min_io, float* max_io, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(outer >= 0 && channels >= 0 && inner >= 0, "dq8_minmax: negative extent");
+  if (outer == 0 || channels == 0 || inner == 0) return 0;   // nothing observed: state kept
+  DQ8_REQUIRE(x && min_io && max_io, "dq8_minmax: null pointer");
+  DQ8_REQUIRE(channels < (1LL << 31), "dq8_minmax: too many channels");
+  const bool last_axis = inner == 1 && channels > 1;
+  const bool vec = aligned(x, 16) && (last_axis ? channels % 4 == 0 : inner % 4 == 0);
+  Plan p;
+  DQ8_REQUIRE(make_plan(outer, channels, inner, vec, &p), "dq8_minmax: tensor too large");
+  DQ8_REQUIRE(workspace && workspace_bytes >= (size_t)p.pairs * sizeof(float2),
+              "dq8_minmax: workspace too small (see dq8_minmax_workspace_bytes)");
+  return run_minmax(x, outer, channels, inner, min_io, max_io,
+                    static_cast<float2*>(workspace), p, vec, (hipStream_t)stream);
+}
+
+// ---- the same with the pairs in memory the library brings along -------------------------
+// For callers that cannot allocate (code under graph capture, serving loops that forbid
+// hipMalloc): the (min, max) pairs of pass 1 live in a fixed array in device memory.  Every
+// device the library runs on holds its own copy of the array at its own address, looked up
+// once per device, with that device current, and kept; host code never uses the array's
+// name for anything else.
+namespace {
+
+constexpr size_t kStaticScratchBytes = 4u << 20;   // 524288 (min, max) pairs
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device (nullptr + error status on failure)
+int static_scratch(void** out) {
+  int dev = 0;
+  if (int s = check_hip(hipGetDevice(&dev), "hipGetDevice")) return s;
+  DQ8_REQUIRE(dev >= 0 && dev < kMaxDevices, "dq8_minmax_static: device ordinal out of range");
+  std::lock_guard<std::mutex> guard(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (int s = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)),
+                          "hipGetSymbolAddress(scratch)"))
+      return s;
+    DQ8_REQUIRE(ptr != nullptr, "dq8_minmax_static: no device address for the scratch array");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+}  // namespace
+
+extern "C" size_t dq8_minmax_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int dq8_minmax_static(const float* x, int64_t outer, int64_t channels, int64_t inner,
+                                 float* min_io, float* max_io, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(outer >= 0 && channels >= 0 && inner >= 0, "dq8_minmax_static: negative extent");
+  if (outer == 0 || channels == 0 || inner == 0) return 0;
+  DQ8_REQUIRE(x && min_io && max_io, "dq8_minmax_static: null pointer");
+  DQ8_REQUIRE(channels < (1LL << 31), "dq8_minmax_static: too many channels");
+  const bool last_axis = inner == 1 && channels > 1;
+  const bool vec = aligned(x, 16) && (last_axis ? channels % 4 == 0 : inner % 4 == 0);
+  Plan p;
+  DQ8_REQUIRE(make_plan(outer, channels, inner, vec, &p), "dq8_minmax_static: tensor too large");
+  DQ8_REQUIRE((size_t)p.pairs * sizeof(float2) <= kStaticScratchBytes,
+              "dq8_minmax_static: this tensor needs " +
+                  std::to_string((size_t)p.pairs * sizeof(float2)) +
+                  " bytes of scratch, more than the built-in " +
+                  std::to_string(kStaticScratchBytes) + "; use dq8_minmax with a workspace");
+  void* ptr = nullptr;
+  if (int s = static_scratch(&ptr)) return s;
+  return run_minmax(x, outer, channels, inner, min_io, max_io,
+                    static_cast<float2*>(ptr), p, vec, (hipStream_t)stream);
 }

@@ -103,6 +103,21 @@ size_t dq8_minmax_workspace_bytes(int64_t outer, int64_t channels, int64_t inner
 int dq8_minmax(const float* x, int64_t outer, int64_t channels, int64_t inner, float* min_io,
                float* max_io, void* workspace, size_t workspace_bytes, void* stream);
 
+/* dq8_minmax without a workspace argument and without any allocation: no hipMalloc, hipFree
+ * or allocating library routine is called.  No counterpart in the reference; it is for
+ * callers that cannot allocate -- code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  The (min, max) pairs of the first pass go to an array
+ * of dq8_minmax_static_max_bytes() bytes (4 MiB) that the library holds in the memory of
+ * every device it runs on until the process ends; a tensor that needs more
+ * (dq8_minmax_workspace_bytes() tells) is refused with an error and must use dq8_minmax.
+ * Same results as dq8_minmax, bit for bit.  All calls on one device share that array:
+ * calls that overlap on one device (different streams, different threads) race; calls on
+ * one stream are ordered and safe.  Nothing in the array needs clearing between calls
+ * (the first pass writes every pair the second reads). */
+size_t dq8_minmax_static_max_bytes(void);
+int dq8_minmax_static(const float* x, int64_t outer, int64_t channels, int64_t inner,
+                      float* min_io, float* max_io, void* stream);
+
 /* ---- quantize / dequantize -------------------------------------------- */
 
 /* x (device, f32) is viewed as [outer, nch, inner]; scale (device f32) and zp
