@@ -2,11 +2,13 @@
 // (any layout, any alignment, zero points) scalar kernels, and the MFMA layout
 // probe.  The tile shape is chosen at run time from the dynamic M.
 #include <algorithm>
+#include <cmath>
 
 #include "dq8_common.h"
 #include "disc_q8.h"
 #include "qgemm_device.h"
 #include "qgemm_pipelined.h"
+#include "qgemm_persistent.h"
 #include "qgemm_skinny.h"
 #include "qconv_direct.h"
 
@@ -218,20 +220,46 @@ const Variant kVariants[] = {
     // with wave tile 64x32 (two workgroups per CU: four waves per SIMD)
     {"pipe_256x256x128_w8", 256, 256, 128, 512},
     {"pipe_128x128x128_w8", 128, 128, 128, 512},
+    // persistent forms: one workgroup per slot walks several tiles, the next tile's first
+    // loads fly during the epilogue
+    {"persist_256x256x128_w8", 256, 256, 128, 512},
+    {"persist_128x128x128_w8", 128, 128, 128, 512},
+    // 256x192 on eight waves (wave tile 64x96): for problems whose 256x256 tiles would leave
+    // a quarter of the compute units idle
+    {"pipe_256x192x128_w8", 256, 192, 128, 512},
+    {"persist_256x192x128_w8", 256, 192, 128, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
 constexpr int kSkinnyVariant = 9;
 constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct variants
 constexpr int kPipe256w8 = 12, kPipe128w8 = 13;
+constexpr int kPersist256 = 14, kPersist128 = 15;
+constexpr int kPipe256x192 = 16, kPersist256x192 = 17;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 
 bool is_pipe_variant(int v) {
   return v == kPipe256 || v == kPipe128 || v == kPipe64 || v == kPipe256x64 || v == kPipe64k2 ||
-         v == kPipe256w8 || v == kPipe128w8;
+         v == kPipe256w8 || v == kPipe128w8 || v == kPersist256 ||
+         v == kPersist128 || v == kPipe256x192 || v == kPersist256x192;
 }
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+int compute_units() {
+  static std::atomic<int> cached{0};
+  int v = cached.load(std::memory_order_relaxed);
+  if (v > 0) return v;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  v = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  cached.store(v, std::memory_order_relaxed);
+  return v;
+}
 
 template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
 int launch_mfma(const MainParams& p, hipStream_t st) {
@@ -267,6 +295,22 @@ int launch_pipe(const MainParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_pipe launch");
 }
 
+// `per_cu`: workgroups of this shape a compute unit holds at a time
+template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
+int launch_persist(const MainParams& p, int per_cu, hipStream_t st) {
+  constexpr int stage = (BM + BN) * 128;
+  constexpr int lds = 2 * stage + (WM * WN * 4096 + BN * 8 <= stage ? 0 : BN * 8);
+  DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
+              "persistent qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
+  auto kern = qgemm_persist_kernel<BM, BN, WM, WN, CONV, EPI>;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int slots = compute_units() * per_cu;
+  hipLaunchKernelGGL(kern, dim3(tiles < slots ? tiles : slots), dim3(WM * WN * 64), lds, st, p);
+  return check_hip(hipGetLastError(), "qgemm_persist launch");
+}
+
 template <int NW, int MT, int EPI>
 int launch_skinny_t(const MainParams& p, hipStream_t st) {
   const dim3 grid((unsigned)ceil_div(p.N, 16), (unsigned)ceil_div(p.M, 16 * MT));
@@ -300,6 +344,10 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, CONV, EPI>(p, st);
     case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, CONV, EPI>(p, st);
     case kPipe128w8: return launch_pipe<128, 128, 2, 4, 1, CONV, EPI>(p, st);
+    case kPipe256x192: return launch_pipe<256, 192, 4, 2, 1, CONV, EPI>(p, st);
+    case kPersist256: return launch_persist<256, 256, 2, 4, CONV, EPI>(p, 1, st);
+    case kPersist128: return launch_persist<128, 128, 2, 4, CONV, EPI>(p, 2, st);
+    case kPersist256x192: return launch_persist<256, 192, 4, 2, CONV, EPI>(p, 1, st);
   }
   if constexpr (!CONV) {
     if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
@@ -336,15 +384,45 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 //    256x256 tile per CU, all of it at the very end; while the main loop is short (K < 2048)
 //    128x128 tiles, several per CU, write under each other's main loops instead
 //    (3072 x 3072 x 768 to f32: 21.8 us against 26.1).
+//  * int8 output, big tiles: 256x256 against 256x192 (wave tile 64x96), one-shot against
+//    persistent.  Measured per workgroup with all compute units busy and K = 768: 1.8 us until
+//    the first k tile has landed, 1.6 us (256x256) or 1.27 us (256x192) per k tile, 2.8 / 2.1 us
+//    of requantisation (4 VALU instructions per result at 4 cycles each per SIMD: bound by the
+//    vector ALU), 0.75 us before the next workgroup starts on the compute unit.  The matrix
+//    pipe is power-limited: a k tile takes 1.0 us with a few compute units busy and 1.65 us
+//    with all 256, which is why a shape that fills 192 compute units with 256x256 tiles gains
+//    only 6-10 % from 256 tiles of 256x192 and not the 25 % its idle quarter suggests.  The
+//    persistent form saves the first-tile latency and the hand-over (1.5 us per tile) from
+//    the second tile of a workgroup on and costs about 1 us per launch.
 int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) {
   auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
   if (pipe) {
     if (N <= 64 && M >= 256 * 64) return kPipe256x64;
+    const int64_t cus = compute_units();
     const int64_t t256 = tiles(kPipe256w8);
-    const int64_t rounds = ceil_div(t256, 256);
-    if (t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * 256 * rounds) &&
-        (out_bytes == 1 || K >= 2048))
+    const int64_t rounds = ceil_div(t256, cus);
+    const bool big256 = t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * cus * rounds) &&
+                        (out_bytes == 1 || K >= 2048);
+    if (out_bytes == 1) {
+      // estimated time in us of a launch of `t` tiles whose k tile costs `per_k` us with all
+      // compute units busy and whose fixed parts cost `fixed` us
+      const double kt = (double)ceil_div(K, 128);
+      auto estimate = [&](int64_t t, double per_k, double fixed, bool* persistent) {
+        const int64_t r = ceil_div(t, cus);
+        const double busy = (double)(t < cus ? t : cus) / (double)cus;
+        const double throttle = (1.0 + 0.65 * busy * std::sqrt(busy)) / 1.65;
+        *persistent = r >= 2;
+        return (double)r * (kt * per_k * throttle + fixed) - (*persistent ? (double)(r - 1) * 1.5 - 1.0 : 0.0);
+      };
+      const int64_t t192 = tiles(kPipe256x192);
+      bool p256 = false, p192 = false;
+      const double e256 = big256 ? estimate(t256, 1.6, 5.4, &p256) : 1e30;
+      const double e192 = t192 >= 200 ? estimate(t192, 1.27, 4.7, &p192) : 1e30;
+      if (e192 < e256) return p192 ? kPersist256x192 : kPipe256x192;
+      if (big256) return p256 ? kPersist256 : kPipe256w8;
+    } else if (big256) {
       return kPipe256w8;
+    }
     if (tiles(kPipe128) >= 120) return K < 4096 ? kPipe128w8 : kPipe128;
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
@@ -847,6 +925,10 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
       if (c >= 0 && direct_conv_plan(c, &d)) return launch_direct_conv(c, epilogue, d, st);
     }
     variant = pick_variant(Mg, Co, Kg, pipe_ok(256, 256, p, true), es);
+    // (the persistent forms are tuned for the plain GEMM: with the convolution's row geometry
+    // on top they run out of registers)
+    if (variant == kPersist256) variant = kPipe256w8;
+    if (variant == kPersist256x192) variant = kPipe256x192;
   }
   return launch_epi<true>(variant, p, epilogue, st);
 }

@@ -22,6 +22,11 @@
 
 #pragma clang fp contract(off)
 
+// Timeline hook for profiling builds (see qgemm_pipelined.h): expands to nothing in the library.
+#ifndef DQ8_TRACE_POINT
+#define DQ8_TRACE_POINT(i)
+#endif
+
 namespace dq8 {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -144,31 +149,48 @@ __device__ __forceinline__ int requant_one(const EpiParams& p, const ColParams& 
 // Same arithmetic as requant_one; rounding and conversion are done by adding
 // 1.5 * 2^23: for |d| <= 128 the sum is rounded to an integer by the addition itself
 // (round-to-nearest-even) and its low mantissa byte is the two's-complement int8.
-template <int EPI>
+//
+// PLAIN: the launch has no bias and no output zero point, so the additive terms are +0.0f and
+// are left out.  Adding +0.0f changes nothing but the sign of a zero, and a zero of either
+// sign gives the byte 0 below, so the result is the same bit for bit.
+template <int EPI, bool PLAIN = false>
 __device__ __forceinline__ uint32_t requant_pack4(const EpiParams& p, const ColParams (&c)[4],
                                                   int a0, int a1, int a2, int a3) {
   const int acc[4] = {a0, a1, a2, a3};
-  uint32_t bits[4];
+  float clamped[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     float d = (float)acc[e];
     if (EPI == DQ8_EPI_REQUANT_CPU) {
-      d = d + c[e].b;
+      if (!PLAIN) d = d + c[e].b;
       d = d * c[e].os;
-      d = d + (float)p.zo;
+      if (!PLAIN) d = d + (float)p.zo;
     } else {
       d = c[e].os * d;
-      d = d + c[e].b;
+      if (!PLAIN) d = d + c[e].b;
     }
     // v_med3_f32: one instruction for the clamp; with a NaN operand it returns the
     // minimum of the other two, so NaN -> -128 like the CPU path
-    d = __builtin_amdgcn_fmed3f(d, -128.0f, 127.0f);
-    d = d + 12582912.0f;
-    bits[e] = __float_as_uint(d);
+    clamped[e] = __builtin_amdgcn_fmed3f(d, -128.0f, 127.0f);
   }
-  const uint32_t lo = __builtin_amdgcn_perm(bits[1], bits[0], 0x0c0c0400u);
-  const uint32_t hi = __builtin_amdgcn_perm(bits[3], bits[2], 0x04000c0cu);
-  return lo | hi;
+  // Rounding, conversion and packing in one instruction per result: adding 1.5 * 2^23 rounds
+  // the clamped value to an integer (nearest even) and leaves its two's-complement int8 in
+  // the low byte of the sum; the sub-dword form of the add (SDWA) writes exactly that byte
+  // into byte e of the packed word and keeps the other bytes.
+  const float magic = 12582912.0f;
+  uint32_t word = __float_as_uint(clamped[0] + magic);   // byte 0; bytes 1 .. 3 are replaced below
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(word) : "v"(clamped[1]), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(word) : "v"(clamped[2]), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(word) : "v"(clamped[3]), "v"(magic));
+#else
+  word &= 0xffu;
+  for (int e = 1; e < 4; ++e) word |= (__float_as_uint(clamped[e] + magic) & 0xffu) << (8 * e);
+#endif
+  return word;
 }
 
 // The output scale the fused requant -> dequantize forms multiply by (one load per kernel;
@@ -307,12 +329,19 @@ __device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, i
   tn = in_panel / rows;
 }
 
-template <int EPI, int FM, int FN, int NT, int BN>
+// Hook of mfma_epilogue: called once, after the int8 results have been computed into
+// registers and before the first of them is stored (the default does nothing).
+struct NoHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores = NoHook>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
                                               int n_blk0, const ColParams* early = nullptr,
                                               int wave_slot = -1, bool active = true,
-                                              int m_limit = -1);
+                                              int m_limit = -1, int8_t* stage_base = nullptr,
+                                              BeforeStores before_stores = BeforeStores());
 
 // The per-channel factors of the channels thread t is responsible for in the epilogue
 // (t, t + NT, ...), fetched at the start of a kernel so that the cold loads of scales
@@ -497,17 +526,22 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
 // instruction would touch 32 different rows with 8 bytes each.  The staging tile
 // swizzles its 16-byte chunks with the row number to keep both the dword writes
 // and the 16-byte reads spread over the banks.
-template <int EPI, int FM, int FN, int NT, int BN>
+template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
                                               int n_blk0, const ColParams* early,
-                                              int wave_slot, bool active, int m_limit) {
+                                              int wave_slot, bool active, int m_limit,
+                                              int8_t* stage_base, BeforeStores before_stores) {
   // `wave_slot`: which per-wave staging tile this wave uses (default: its index in the
   // workgroup); waves with `active` false only take part in the barriers; rows at or
-  // past `m_limit` (default: M) are not stored.
+  // past `m_limit` (default: M) are not stored; `stage_base`: where the per-wave staging
+  // tiles start (default: right behind the per-channel factors at `smem`).
   const int m_end = m_limit >= 0 ? m_limit : e.M;
   constexpr int TM = FM * 32, TN = FN * 32;
-  constexpr int CH = TN / 16;                 // 16-byte chunks per staged row
+  // staged rows are TNP bytes apart, TN rounded up to a power of two, so that the chunk
+  // swizzle below stays inside the row for wave tiles such as 64 x 96
+  constexpr int TNP = TN <= 32 ? 32 : TN <= 64 ? 64 : TN <= 128 ? 128 : 256;
+  constexpr int CH = TNP / 16;                // 16-byte chunk slots per staged row
   constexpr int CP_BYTES = BN * 8;            // per-channel (scale, addend) pairs
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = wave_slot >= 0 ? wave_slot : tid >> 6;
@@ -529,41 +563,131 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     }
   }
   __syncthreads();
+  DQ8_TRACE_POINT(5);
   if (!active) return;
 
   constexpr bool kInt8Out = EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU;
+#ifndef DQ8_EPILOGUE_STAGED_INT8
   if (kInt8Out && e.vec_store16) {
-    int8_t* stage = smem + CP_BYTES + wave * (TM * TN);
+    // int8 results straight from the registers.  Of a 32 x 32 fragment a lane holds row
+    // lane % 32 and the four channel quads 8 g + 4 (lane / 32) .. + 3, g = 0 .. 3, one packed
+    // word each.  Two half-wave swaps (v_permlane32_swap) trade quads between lane l and
+    // lane l + 32 so that the lower lane ends up with channels 0 .. 15 of its row and the
+    // upper one with channels 16 .. 31: one 16-byte store per lane, 32 contiguous bytes per
+    // row and instruction.  No LDS traffic (the first version staged the tile through LDS
+    // with four-byte writes, eight to a bank).
+    const bool plain = e.bias_kind == DQ8_BIAS_NONE && e.zo == 0;
+    int8_t* out = static_cast<int8_t*>(e.out);
+    // With a hook the results of the whole wave tile are formed first (32 registers per
+    // 128 x 64), the hook runs, and the stores follow in one go; without one each fragment is
+    // stored as soon as it is packed.
+    constexpr bool kHook = !__is_same(BeforeStores, NoHook);
+    v4i held[kHook ? FM : 1][kHook ? FN : 1];
+    auto store_frag = [&](const v4i v, int i, int j) {
+      const int n = n_wave0 + j * 32 + 16 * (lane >> 5);
+      const int m = m_wave0 + i * 32 + (lane & 31);
+      if (m < m_end && n < e.N) {
+        int8_t* dst = out + (int64_t)m * e.ldo + n;
+        if (n + 15 < e.N) {
+          *reinterpret_cast<v4i*>(dst) = v;
+        } else {
 #pragma unroll
-    for (int j = 0; j < FN; ++j) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
-        const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
-        const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
-        const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
-        const int chunk = j * 2 + (g >> 1);
-        const int dw = (2 * g + (lane >> 5)) & 3;
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-          const int r = i * 32 + (lane & 31);
-          const uint32_t w = requant_pack4<EPI>(e, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
-                                                acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-          *reinterpret_cast<uint32_t*>(stage + r * TN + ((chunk ^ (r & (CH - 1))) << 4) + dw * 4) = w;
+          for (int b = 0; b < 16; ++b)
+            if (n + b < e.N) dst[b] = (int8_t)((uint32_t)v[b >> 2] >> (8 * (b & 3)));
         }
       }
+    };
+    auto store_all = [&](auto plain_c) {
+      constexpr bool PLAIN = decltype(plain_c)::value != 0;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int cl0 = wn_off + j * 32 + 4 * (lane >> 5);
+        ColParams c[4][4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g]);
+          const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g + 2]);
+          c[g][0] = {p01[0], p01[1]};
+          c[g][1] = {p01[2], p01[3]};
+          c[g][2] = {p23[0], p23[1]};
+          c[g][3] = {p23[2], p23[3]};
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          uint32_t w[4];
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            w[g] = requant_pack4<EPI, PLAIN>(e, c[g], acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
+                                             acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+          // swap(a, b): the upper half of a trades places with the lower half of b
+          const auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+          const auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+          const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+          if (kHook)
+            held[kHook ? i : 0][kHook ? j : 0] = v;
+          else
+            store_frag(v, i, j);
+        }
+      }
+    };
+    if (plain)
+      store_all(IntC<1>());
+    else
+      store_all(IntC<0>());
+    if (kHook) {
+      before_stores();
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int i = 0; i < FM; ++i) store_frag(held[kHook ? i : 0][kHook ? j : 0], i, j);
     }
+    DQ8_TRACE_POINT(6);
+    return;
+  }
+#endif
+  before_stores();
+  if (kInt8Out && e.vec_store16) {
+    int8_t* stage = (stage_base ? stage_base : smem + CP_BYTES) + wave * (TM * TNP);
+    // (kernel-uniform: which of the two instantiations of the loop runs)
+    const bool plain = e.bias_kind == DQ8_BIAS_NONE && e.zo == 0;
+    auto requant_all = [&](auto plain_c) {
+      constexpr bool PLAIN = decltype(plain_c)::value != 0;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
+          const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
+          const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
+          const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
+          const int chunk = j * 2 + (g >> 1);
+          const int dw = (2 * g + (lane >> 5)) & 3;
+#pragma unroll
+          for (int i = 0; i < FM; ++i) {
+            const int r = i * 32 + (lane & 31);
+            const uint32_t w = requant_pack4<EPI, PLAIN>(e, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
+                                                         acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+            *reinterpret_cast<uint32_t*>(stage + r * TNP + ((chunk ^ (r & (CH - 1))) << 4) + dw * 4) = w;
+          }
+        }
+      }
+    };
+    if (plain)
+      requant_all(IntC<1>());
+    else
+      requant_all(IntC<0>());
+    DQ8_TRACE_POINT(6);
     // the staging tile is private to the wave and LDS operations of one wave
     // execute in order: no barrier needed before reading it back
-    constexpr int ROWS_PER_IT = 1024 / TN;
+    constexpr int ROWS_PER_IT = 1024 / TNP;
     int8_t* out = static_cast<int8_t*>(e.out);
 #pragma unroll
     for (int it = 0; it < TM / ROWS_PER_IT; ++it) {
       const int row = it * ROWS_PER_IT + lane / CH;
       const int chunk = lane % CH;
-      const v4i v = *reinterpret_cast<const v4i*>(stage + row * TN + ((chunk ^ (row & (CH - 1))) << 4));
+      const v4i v = *reinterpret_cast<const v4i*>(stage + row * TNP + ((chunk ^ (row & (CH - 1))) << 4));
       const int m = m_wave0 + row, n = n_wave0 + chunk * 16;
-      if (m < m_end && n < e.N) {
+      if (chunk * 16 < TN && m < m_end && n < e.N) {
         int8_t* dst = out + (int64_t)m * e.ldo + n;
         if (n + 15 < e.N) {
           // A wave tile at least 128 channels wide writes whole 128-byte lines: streamed past
@@ -588,7 +712,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     // int32 / f32 results: one 32 x 32 fragment (4 KiB) at a time through a per-wave LDS
     // tile, 128-byte rows with the 16-byte chunks swizzled by the row, then out as full
     // 128-byte row segments (8 lanes per row) instead of 32-byte pieces of 32 rows.
-    int8_t* stage = smem + CP_BYTES + wave * 4096;
+    int8_t* stage = (stage_base ? stage_base : smem + CP_BYTES) + wave * 4096;
     const float so_val = EPI == DQ8_EPI_DEQUANT_F32 ? dequant_so(e) : 0.0f;
     auto store_all = [&](auto form) {
     constexpr int FORM = decltype(form)::value;

@@ -66,11 +66,14 @@ constexpr int kBufferRsrcWord3 = 0x00020000;
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
-// 128-bit raw buffer descriptor (stride 0): base address, byte count, format word
+// 128-bit raw buffer descriptor (stride 0): base address, byte count, format word.  The
+// descriptor is a scalar operand of the load: base and size are the same in every lane, and
+// the readfirstlane says so where the compiler cannot see it (it folds away where it can).
 __device__ __forceinline__ v4i make_rsrc(const void* base, int64_t num_records) {
   const uint64_t b = (uint64_t)base;
-  v4i r = {(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xffff), (int)num_records,
-           kBufferRsrcWord3};
+  v4i r = {__builtin_amdgcn_readfirstlane((int)(uint32_t)b),
+           __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xffff)),
+           __builtin_amdgcn_readfirstlane((int)num_records), kBufferRsrcWord3};
   return r;
 }
 
@@ -80,6 +83,10 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, int64_t num_records) 
 // s_waitcnt vmcnt, when it needs the data; through the compiler builtin every LDS
 // read would first wait for all loads in flight.
 __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, unsigned lds_addr, int voffset) {
+  // (wave-uniform by construction; said explicitly for where the compiler cannot prove it)
+  lds_addr = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_addr);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) rsrc[c] = __builtin_amdgcn_readfirstlane(rsrc[c]);
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
       "s_nop 0\n\t"
@@ -110,7 +117,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   constexpr int B_LD = (BN / 8) / NW;
   constexpr int LD = A_LD + B_LD;           // load instructions per tile per wave
   static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile does not split over the waves");
-  static_assert(FM >= 1 && FN >= 1 && FN <= FM, "fragment mismatch");
+  static_assert(FM >= 1 && FN >= 1, "fragment mismatch");
   static_assert(LD <= 63, "vmcnt is a 6-bit counter");
   static_assert(NW % 2 == 0, "the chunk a lane loads must not depend on the load slot");
 
@@ -322,20 +329,25 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
       }
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
+        // (row i of the MFMA grid also fetches the W fragments j = i, i + FM, ...)
         if (ks == 0) {
           load_frag_a(1, cur, 1, i);
-          if (i < FN) load_frag_b(1, cur, 1, i);
+#pragma unroll
+          for (int j = i; j < FN; j += FM) load_frag_b(1, cur, 1, j);
         } else if (ks == 1) {
           load_frag_a(2, cur, 2, i);
-          if (i < FN) load_frag_b(2, cur, 2, i);
+#pragma unroll
+          for (int j = i; j < FN; j += FM) load_frag_b(2, cur, 2, j);
           load_frag_a(3, cur, 3, i);
-          if (i < FN) load_frag_b(3, cur, 3, i);
+#pragma unroll
+          for (int j = i; j < FN; j += FM) load_frag_b(3, cur, 3, j);
         } else if (ks == 2) {
 #pragma unroll
           for (int l = 0; l < LPR; ++l) issue_load(i * LPR + l, cur);
         } else {
           load_frag_a(0, nxt, 0, i);
-          if (i < FN) load_frag_b(0, nxt, 0, i);
+#pragma unroll
+          for (int j = i; j < FN; j += FM) load_frag_b(0, nxt, 0, j);
 #pragma unroll
           for (int l = 0; l < LPR; ++l) issue_load((FM + i) * LPR + l, cur);
         }

@@ -99,6 +99,45 @@ def test_qgemm_requant_cpu(K, m, n, k, bias):
     assert sat < 0.5, "degenerate test: %.2f saturated" % sat
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (4133, 4109, 272),     # 17 x 17 tiles of 256 x 256: more tiles than compute units, not a multiple of 8
+    (4096, 4300, 144),     # 16 x 17 = 272 tiles: dealt per XCD; two k tiles, the second ragged
+    (5000, 3840, 128),     # 20 x 20 tiles of 256 x 192 / 20 x 15 of 256 x 256; one k tile
+    (16384, 1536, 400),    # three and four rounds of the two big tile shapes
+])
+def test_qgemm_persistent_variants_walk_many_tiles(K, m, n, k):
+    """The persistent kernels with several output tiles per workgroup: ragged last tiles in
+    M, N and K, tile counts that do and do not divide over the XCDs, all epilogue families
+    (int8 with and without additive terms, int32, f32), and the heuristic's own pick at these
+    sizes -- bit-exact against the oracle."""
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    bf = (rng.standard_normal(n) * 10 * so).astype(np.float32)
+    b32 = O.bias_f32_to_s32(bf, sx, sw)
+    want_plain = O.requant_cpu(acc, sx, sw, so)
+    want_bias = O.requant_cpu(acc, sx, sw, so, b32=b32, zo=3)
+    want_f32 = O.dequant_acc(acc, sx, sw, bias=bf)
+    da, dw = dev(a), dev(w)
+    dsx, dsw, dso = dev(np.array([sx])), dev(sw), dev(np.array([so]))
+    names = K.variant_names()
+    persistent = [i for i, nm in enumerate(names) if nm.startswith("persist_")]
+    assert len(persistent) >= 2
+    for v in [-1] + persistent:
+        tag = names[v] if v >= 0 else "heuristic"
+        got = host(K.qgemm(da, dw, K.EPI_REQUANT_CPU, sx=dsx, sw=dsw, so=dso, variant=v))
+        np.testing.assert_array_equal(got, want_plain, err_msg=tag)
+        got = host(K.qgemm(da, dw, K.EPI_REQUANT_CPU, sx=dsx, sw=dsw, so=dso, bias=dev(bf), zo=3,
+                           variant=v))
+        np.testing.assert_array_equal(got, want_bias, err_msg=tag)
+        np.testing.assert_array_equal(host(K.qgemm(da, dw, K.EPI_ACC_S32, variant=v)), acc, err_msg=tag)
+        got = host(K.qgemm(da, dw, K.EPI_DEQUANT_F32, sx=dsx, sw=dsw, bias=dev(bf), variant=v))
+        assert np.array_equal(got.view(np.uint32), want_f32.view(np.uint32)), tag
+
+
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("bias", ["none", "f32", "s8"])
 def test_qgemm_requant_gpu(K, per_channel, bias):
@@ -516,7 +555,7 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
     out_shape = [nb, ho, wo, co]
     acc = O.conv_s32(x, wt, padding, md, out_shape)
     names = K.variant_names()
-    variants = [-1, 0] + ([i for i, nm in enumerate(names) if nm.startswith(("mfma_", "pipe_"))]
+    variants = [-1, 0] + ([i for i, nm in enumerate(names) if nm.startswith(("mfma_", "pipe_", "dual_"))]
                           if ci % 16 == 0 else [])
     if k == 3 and stride == 1 and dil == 1 and ci in (32, 64, 128, 256):
         variants += [i for i, nm in enumerate(names) if nm.startswith("direct3x3_")]
