@@ -299,7 +299,8 @@ int launch_pipe(const MainParams& p, hipStream_t st) {
 template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
 int launch_persist(const MainParams& p, int per_cu, hipStream_t st) {
   constexpr int stage = (BM + BN) * 128;
-  constexpr int lds = 2 * stage + (WM * WN * 4096 + BN * 8 <= stage ? 0 : BN * 8);
+  // (per-channel factors: 8 bytes, plus 4 for the shifts of the fixed-point output stage)
+  constexpr int lds = 2 * stage + (WM * WN * 4096 + BN * 8 <= stage ? 0 : BN * 12);
   DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
               "persistent qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
   auto kern = qgemm_persist_kernel<BM, BN, WM, WN, CONV, EPI>;
@@ -562,6 +563,15 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                            "output scale");
     epilogue = requant == 1 ? DQ8_EPI_REQUANT_CPU : DQ8_EPI_REQUANT_GPU;
   }
+  int fixedpoint = 0;
+  if (epilogue == DQ8_EPI_REQUANT_FIXEDPOINT) {
+    fixedpoint = 1;
+    DQ8_REQUIRE(n_sx == 1 && n_so == 1, "dq8_qgemm: the fixed-point stage takes per-tensor input "
+                                        "and output scales");
+    DQ8_REQUIRE(bias_kind == DQ8_BIAS_NONE || bias_kind == DQ8_BIAS_S32,
+                "dq8_qgemm: the fixed-point stage takes an s32 bias or none");
+    epilogue = DQ8_EPI_REQUANT_CPU;
+  }
   if (int s = check_epilogue("dq8_qgemm", epilogue, bias, bias_kind, sx, sw, so, n_sx,
                              n_sw, n_so, N))
     return s;
@@ -590,6 +600,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   e.so_stride = n_so > 1;
   e.zo = zo;
   e.requant = requant;
+  e.fixedpoint = fixedpoint;
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
@@ -783,6 +794,13 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     requant = epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 ? 1 : 2;
     epilogue = requant == 1 ? DQ8_EPI_REQUANT_CPU : DQ8_EPI_REQUANT_GPU;
   }
+  int fixedpoint = 0;
+  if (epilogue == DQ8_EPI_REQUANT_FIXEDPOINT) {
+    fixedpoint = 1;
+    DQ8_REQUIRE(bias_kind == DQ8_BIAS_NONE || bias_kind == DQ8_BIAS_S32,
+                "dq8_qconv2d: the fixed-point stage takes an s32 bias or none");
+    epilogue = DQ8_EPI_REQUANT_CPU;
+  }
   if (int s = check_epilogue("dq8_qconv2d", epilogue, bias, bias_kind, sx, sw, so, 1, n_sw, 1, Co))
     return s;
   DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
@@ -812,6 +830,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   e.so_stride = 0;
   e.zo = zo;
   e.requant = requant;
+  e.fixedpoint = fixedpoint;
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (Co % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (Co % 16 == 0);

@@ -47,6 +47,10 @@ struct EpiParams {
   // DEQUANT_F32 only.  0: out = f32(acc) * (sx sw) + bias.  1 / 2: the REQUANT_CPU /
   // REQUANT_GPU result q, dequantized in place: out = (float)(q - zo) * so[0].
   int requant;
+  // REQUANT_CPU only.  1: the output stage is the integer one of the reference's AArch64
+  // path -- (acc + bias) times a fixed-point multiplier and shift derived from
+  // (sx sw[n]) / so, plus zo, clamped (see fixedpoint_one).
+  int fixedpoint;
   int vec_store;    // 1: a group of 4 consecutive n may be stored as one 4/16-byte word
   int vec_store16;  // 1: int8 rows may be written with aligned 16-byte stores
 };
@@ -74,7 +78,44 @@ struct MainParams {
 struct ColParams {  // per output channel
   float os;   // output scale (requant) or dequant scale
   float b;    // additive term, already in the units the mode needs
+  int sh;     // fixed-point output stage only: the shift; os and b then hold the bit
+              // patterns of the int32 multiplier and of the int32 bias
 };
+
+// ---- the integer output stage of the reference's AArch64 path
+// (R ral/context/common_context_impl_quantization.cc:671-679, 865-872: Arm Compute Library's
+// GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT; the library's published algorithm)
+// saturating rounding doubling multiply, high half: (2 a b + 2^31) >> 32
+__device__ __forceinline__ int sqrdmulh(int a, int b) {
+  const long long t = (long long)a * (long long)b + (1ll << 30);
+  const int r = (int)(t >> 31);
+  return (a == (int)0x80000000 && b == (int)0x80000000) ? 0x7fffffff : r;
+}
+// x / 2^e, ties away from zero, e in [0, 31]
+__device__ __forceinline__ int rounding_divide_by_pow2(int x, int e) {
+  const int mask = (int)((1u << e) - 1u);
+  const int threshold = (mask >> 1) + (x < 0 ? 1 : 0);
+  return (x >> e) + ((x & mask) > threshold ? 1 : 0);
+}
+__device__ __forceinline__ int fixedpoint_one(int acc, int bias, int m0, int sh, int zo) {
+  int v = (int)((unsigned)acc + (unsigned)bias);
+  if (sh < 0) {
+    const int left = -sh < 31 ? -sh : 31;
+    v = sqrdmulh((int)((unsigned)v << left), m0);   // (the pre-multiplication wraps)
+  } else {
+    v = rounding_divide_by_pow2(sqrdmulh(v, m0), sh < 31 ? sh : 31);
+  }
+  v = (int)((unsigned)v + (unsigned)zo);
+  return v < -128 ? -128 : (v > 127 ? 127 : v);
+}
+// multiplier = M0 2^-31 2^-shift with M0 in [2^30, 2^31): a binary32 has 24 significant bits,
+// so q 2^31 below is an integer and the library's round() of it is the identity
+__device__ __forceinline__ void fixedpoint_multiplier(float multiplier, int& m0, int& sh) {
+  int e = 0;
+  const float q = frexpf(multiplier, &e);
+  m0 = (int)(q * 2147483648.0f);
+  sh = -e;
+}
 
 __device__ __forceinline__ float sat_rne_s32_as_float(float v) {
   // saturate to int32 in float (the largest float below 2^31 is 2147483520), then
@@ -89,6 +130,7 @@ __device__ __forceinline__ ColParams col_params(const EpiParams& p, int n) {
   ColParams c;
   c.os = 1.0f;
   c.b = 0.0f;
+  c.sh = 0;
   if (EPI == DQ8_EPI_ACC_S32) return c;
   const float sx = p.sx[(int64_t)n * p.sx_stride];
   const float sw = p.sw[(int64_t)n * p.sw_stride];
@@ -104,6 +146,14 @@ __device__ __forceinline__ ColParams col_params(const EpiParams& p, int n) {
     return c;
   }
   const float so = p.so[(int64_t)n * p.so_stride];
+  if (mode == DQ8_EPI_REQUANT_CPU && p.fixedpoint) {
+    int m0, sh;
+    fixedpoint_multiplier(prod / so, m0, sh);
+    c.os = __int_as_float(m0);
+    c.sh = sh;
+    c.b = __int_as_float(p.bias_kind == DQ8_BIAS_S32 ? ((const int32_t*)p.bias)[n] : 0);
+    return c;
+  }
   if (mode == DQ8_EPI_REQUANT_CPU) {
     c.os = prod / (1.0f * so);
     if (p.bias_kind == DQ8_BIAS_S32) {
@@ -133,6 +183,8 @@ __device__ __forceinline__ int sat_rne_s8(float d) {
 template <int EPI>
 __device__ __forceinline__ int requant_one(const EpiParams& p, const ColParams& c,
                                            int acc) {
+  if (EPI == DQ8_EPI_REQUANT_CPU && p.fixedpoint)
+    return fixedpoint_one(acc, __float_as_int(c.b), __float_as_int(c.os), c.sh, p.zo);
   float d = (float)acc;
   if (EPI == DQ8_EPI_REQUANT_CPU) {
     d = d + c.b;
@@ -267,7 +319,15 @@ __device__ __forceinline__ void store_group4(const EpiParams& p, int m, int n,
   const bool full = n + 3 < p.N;
   if (EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU) {
     int8_t* out = (int8_t*)p.out;
-    const uint32_t w = requant_pack4<EPI>(p, c, a0, a1, a2, a3);
+    uint32_t w;
+    if (EPI == DQ8_EPI_REQUANT_CPU && p.fixedpoint) {
+      w = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        w |= ((uint32_t)requant_one<EPI>(p, c[e], acc[e]) & 0xffu) << (8 * e);
+    } else {
+      w = requant_pack4<EPI>(p, c, a0, a1, a2, a3);
+    }
     if (full && p.vec_store) {
       *(uint32_t*)(out + off) = w;
     } else {
@@ -354,7 +414,7 @@ struct EarlyColParams {
 #pragma unroll
     for (int i = 0; i < kPerThread; ++i) {
       // (a wave whose channels all lie past the block's BN has nothing to fetch)
-      c[i] = ColParams{0.f, 0.f};
+      c[i] = ColParams{0.f, 0.f, 0};
       if ((int)(threadIdx.x & ~63u) + i * NT >= BN) continue;
       const int n = n_blk0 + (int)threadIdx.x + i * NT;
       c[i] = col_params<EPI>(e, n < e.N ? n : e.N - 1);
@@ -519,13 +579,11 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
 // output row m_wave0 + i*32 + lane%32 and channel n_wave0 + j*32 + 8*(v/4) +
 // 4*(lane/32) + v%4.
 //
-// The per-channel factors are computed once per block (thread t -> channel t) and
-// parked in LDS.  int8 results are then staged through LDS so that they leave the
-// CU as 16-byte stores with eight consecutive lanes covering one 128-byte line of
-// an output row: written straight from the accumulator layout, every store
-// instruction would touch 32 different rows with 8 bytes each.  The staging tile
-// swizzles its 16-byte chunks with the row number to keep both the dword writes
-// and the 16-byte reads spread over the banks.
+// The per-channel factors are computed once per block (thread t -> channel t) and parked in
+// LDS.  int8 results are packed four to a word, traded between the two halves of the wave so
+// that a lane holds 16 consecutive channels of its row, and stored from the registers;
+// int32 / f32 results are staged through LDS one fragment at a time so that they leave as
+// full 128-byte row segments.
 template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
@@ -537,11 +595,6 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
   // past `m_limit` (default: M) are not stored; `stage_base`: where the per-wave staging
   // tiles start (default: right behind the per-channel factors at `smem`).
   const int m_end = m_limit >= 0 ? m_limit : e.M;
-  constexpr int TM = FM * 32, TN = FN * 32;
-  // staged rows are TNP bytes apart, TN rounded up to a power of two, so that the chunk
-  // swizzle below stays inside the row for wave tiles such as 64 x 96
-  constexpr int TNP = TN <= 32 ? 32 : TN <= 64 ? 64 : TN <= 128 ? 128 : 256;
-  constexpr int CH = TNP / 16;                // 16-byte chunk slots per staged row
   constexpr int CP_BYTES = BN * 8;            // per-channel (scale, addend) pairs
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = wave_slot >= 0 ? wave_slot : tid >> 6;
@@ -549,17 +602,25 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
 
   __syncthreads();  // every wave is done with the operand tiles
   float2* cp = reinterpret_cast<float2*>(smem);
+  // (fixed-point output stage: the shifts, behind the pairs; that space is otherwise the
+  // result staging of the 4-byte epilogues, which the stage does not use)
+  int* cps = reinterpret_cast<int*>(smem + CP_BYTES);
+  const bool fixedpoint = EPI == DQ8_EPI_REQUANT_CPU && e.fixedpoint;
   if (early) {
 #pragma unroll
     for (int i = 0; i < (BN + NT - 1) / NT; ++i) {
       const int t = tid + i * NT;
-      if (t < BN) cp[t] = make_float2(early[i].os, early[i].b);
+      if (t < BN) {
+        cp[t] = make_float2(early[i].os, early[i].b);
+        if (fixedpoint) cps[t] = early[i].sh;
+      }
     }
   } else {
     for (int t = tid; t < BN; t += NT) {
       const int n = n_blk0 + t;
       const ColParams c = col_params<EPI>(e, n < e.N ? n : e.N - 1);
       cp[t] = make_float2(c.os, c.b);
+      if (fixedpoint) cps[t] = c.sh;
     }
   }
   __syncthreads();
@@ -567,7 +628,6 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
   if (!active) return;
 
   constexpr bool kInt8Out = EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU;
-#ifndef DQ8_EPILOGUE_STAGED_INT8
   if (kInt8Out && e.vec_store16) {
     // int8 results straight from the registers.  Of a 32 x 32 fragment a lane holds row
     // lane % 32 and the four channel quads 8 g + 4 (lane / 32) .. + 3, g = 0 .. 3, one packed
@@ -589,6 +649,8 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
       if (m < m_end && n < e.N) {
         int8_t* dst = out + (int64_t)m * e.ldo + n;
         if (n + 15 < e.N) {
+          // (an ordinary store: the L2 merges the 32-byte pieces of a line; streamed past it,
+          // non-temporal, the same stores take half as long again for the whole launch)
           *reinterpret_cast<v4i*>(dst) = v;
         } else {
 #pragma unroll
@@ -597,8 +659,9 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
         }
       }
     };
-    auto store_all = [&](auto plain_c) {
-      constexpr bool PLAIN = decltype(plain_c)::value != 0;
+    // MODE 0: float stage with its additive terms, 1: without them, 2: fixed-point stage
+    auto store_all = [&](auto mode_c) {
+      constexpr int MODE = decltype(mode_c)::value;
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
         const int cl0 = wn_off + j * 32 + 4 * (lane >> 5);
@@ -607,18 +670,31 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
         for (int g = 0; g < 4; ++g) {
           const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g]);
           const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g + 2]);
-          c[g][0] = {p01[0], p01[1]};
-          c[g][1] = {p01[2], p01[3]};
-          c[g][2] = {p23[0], p23[1]};
-          c[g][3] = {p23[2], p23[3]};
+          v4i sh = {0, 0, 0, 0};
+          if (MODE == 2) sh = *reinterpret_cast<const v4i*>(&cps[cl0 + 8 * g]);
+          c[g][0] = {p01[0], p01[1], sh[0]};
+          c[g][1] = {p01[2], p01[3], sh[1]};
+          c[g][2] = {p23[0], p23[1], sh[2]};
+          c[g][3] = {p23[2], p23[3], sh[3]};
         }
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           uint32_t w[4];
 #pragma unroll
-          for (int g = 0; g < 4; ++g)
-            w[g] = requant_pack4<EPI, PLAIN>(e, c[g], acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
-                                             acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+          for (int g = 0; g < 4; ++g) {
+            if (MODE == 2) {
+              w[g] = 0;
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                w[g] |= ((uint32_t)fixedpoint_one(acc[i][j][4 * g + q], __float_as_int(c[g][q].b),
+                                                  __float_as_int(c[g][q].os), c[g][q].sh, e.zo) &
+                         0xffu)
+                        << (8 * q);
+            } else {
+              w[g] = requant_pack4<EPI, MODE == 1>(e, c[g], acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
+                                                   acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+            }
+          }
           // swap(a, b): the upper half of a trades places with the lower half of b
           const auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
           const auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
@@ -630,7 +706,9 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
         }
       }
     };
-    if (plain)
+    if (fixedpoint)
+      store_all(IntC<2>());
+    else if (plain)
       store_all(IntC<1>());
     else
       store_all(IntC<0>());
@@ -644,69 +722,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     DQ8_TRACE_POINT(6);
     return;
   }
-#endif
   before_stores();
-  if (kInt8Out && e.vec_store16) {
-    int8_t* stage = (stage_base ? stage_base : smem + CP_BYTES) + wave * (TM * TNP);
-    // (kernel-uniform: which of the two instantiations of the loop runs)
-    const bool plain = e.bias_kind == DQ8_BIAS_NONE && e.zo == 0;
-    auto requant_all = [&](auto plain_c) {
-      constexpr bool PLAIN = decltype(plain_c)::value != 0;
-#pragma unroll
-      for (int j = 0; j < FN; ++j) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
-          const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
-          const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
-          const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
-          const int chunk = j * 2 + (g >> 1);
-          const int dw = (2 * g + (lane >> 5)) & 3;
-#pragma unroll
-          for (int i = 0; i < FM; ++i) {
-            const int r = i * 32 + (lane & 31);
-            const uint32_t w = requant_pack4<EPI, PLAIN>(e, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
-                                                         acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-            *reinterpret_cast<uint32_t*>(stage + r * TNP + ((chunk ^ (r & (CH - 1))) << 4) + dw * 4) = w;
-          }
-        }
-      }
-    };
-    if (plain)
-      requant_all(IntC<1>());
-    else
-      requant_all(IntC<0>());
-    DQ8_TRACE_POINT(6);
-    // the staging tile is private to the wave and LDS operations of one wave
-    // execute in order: no barrier needed before reading it back
-    constexpr int ROWS_PER_IT = 1024 / TNP;
-    int8_t* out = static_cast<int8_t*>(e.out);
-#pragma unroll
-    for (int it = 0; it < TM / ROWS_PER_IT; ++it) {
-      const int row = it * ROWS_PER_IT + lane / CH;
-      const int chunk = lane % CH;
-      const v4i v = *reinterpret_cast<const v4i*>(stage + row * TNP + ((chunk ^ (row & (CH - 1))) << 4));
-      const int m = m_wave0 + row, n = n_wave0 + chunk * 16;
-      if (chunk * 16 < TN && m < m_end && n < e.N) {
-        int8_t* dst = out + (int64_t)m * e.ldo + n;
-        if (n + 15 < e.N) {
-          // A wave tile at least 128 channels wide writes whole 128-byte lines: streamed past
-          // the L2 (non-temporal), which shortens the write-back at the end of the kernel.  A
-          // 64-wide tile writes half lines; ordinary stores let the L2 merge them with the
-          // neighbouring wave's half (same speed, a third less write traffic).
-          if (TN >= 128)
-            __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
-          else
-            *reinterpret_cast<v4i*>(dst) = v;
-        } else {
-#pragma unroll
-          for (int b = 0; b < 16; ++b)
-            if (n + b < e.N) dst[b] = (int8_t)((uint32_t)v[b >> 2] >> (8 * (b & 3)));
-        }
-      }
-    }
-    return;
-  }
 
   if (!kInt8Out && e.vec_store) {
     // int32 / f32 results: one 32 x 32 fragment (4 KiB) at a time through a per-wave LDS
@@ -732,7 +748,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
           } else {
             const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
             const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
-            const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
+            const ColParams c[4] = {{p01[0], p01[1], 0}, {p01[2], p01[3], 0}, {p23[0], p23[1], 0}, {p23[2], p23[3], 0}};
 #pragma unroll
             for (int q = 0; q < 4; ++q)
               w[q] = __float_as_int(dequant_one<FORM>(e, c[q], acc[i][j][4 * g + q], so_val));
@@ -775,7 +791,10 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
       if (n >= e.N) continue;
       const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
       const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
-      const ColParams c[4] = {{p01[0], p01[1]}, {p01[2], p01[3]}, {p23[0], p23[1]}, {p23[2], p23[3]}};
+      v4i sh = {0, 0, 0, 0};
+      if (fixedpoint) sh = *reinterpret_cast<const v4i*>(&cps[cl]);
+      const ColParams c[4] = {{p01[0], p01[1], sh[0]}, {p01[2], p01[3], sh[1]},
+                              {p23[0], p23[1], sh[2]}, {p23[2], p23[3], sh[3]}};
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
         const int m = m_wave0 + i * 32 + (lane & 31);

@@ -121,6 +121,21 @@ class StreamTimer {
   bool on_ = false;
 };
 
+// Which output stage the entries use whose signature the reference implements twice on the
+// CPU -- with oneDNN's float post-ops on x86 and with Arm Compute Library's fixed-point
+// multiplier and shift on AArch64 (ral_qgemm with per-channel weight scales, ral_qconv,
+// ral_pdll_qconv2d: R context/common_context_impl_quantization.cc:1680-1696 against
+// :1699-1719).  Default: the float stage; DISC_GPU_REQUANT_FIXEDPOINT=1 selects the integer
+// one, for results identical to the reference's AArch64 build.
+// (Read at every call, like the reference reads its DISC_* switches at the point of use: a
+// host may run graphs of both kinds in one process.)
+int sharedSignatureStage() {
+  const char* v = std::getenv("DISC_GPU_REQUANT_FIXEDPOINT");
+  return v && *v && std::strcmp(v, "0") != 0 && std::strcmp(v, "false") != 0
+             ? DQ8_EPI_REQUANT_FIXEDPOINT
+             : DQ8_EPI_REQUANT_CPU;
+}
+
 GPUDriver* driverOf(ExecutionContext* ctx) {
   auto* d = ctx->getDriver<GPUDriver>(GPUDriver::name());
   if (!d) fail(ctx, "GPUDriver not found");
@@ -303,7 +318,7 @@ void ral_qgemm_impl(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_
   op.tp_b = tp_b;
   op.weight_is_const = weight_is_const;
   Epilogue e;
-  e.mode = DQ8_EPI_REQUANT_CPU;
+  e.mode = WS_RANK == 1 ? sharedSignatureStage() : DQ8_EPI_REQUANT_CPU;
   e.sx = inputScales.data;
   e.sw = weightScales.data;
   e.so = resultScales.data;
@@ -509,7 +524,7 @@ MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_hand
                                         MemRefType<int32_t, 1> weightZeroPoints,
                                         MemRefType<float, 0> resultScales,
                                         MemRefType<int32_t, 0> resultZeroPoints,
-                                        void* customAttrs) {
+                                        void* customAttrs, int stage = DQ8_EPI_REQUANT_CPU) {
   static const char* who = "ral_pdll_qgemm";
   int64_t zeros[N] = {0};
   MemRefType<int8_t, N> result = assignMemRef<int8_t, N>(nullptr, zeros);
@@ -567,7 +582,7 @@ MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_hand
   op.tp_b = tp_b;
   op.weight_is_const = weight_is_const;
   Epilogue e;
-  e.mode = DQ8_EPI_REQUANT_CPU;
+  e.mode = stage;
   e.bias = bias;
   e.bias_kind = bias_kind;
   e.sx = inputScales.data;
@@ -618,6 +633,61 @@ MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_per_channel(
                               resultScales, resultZeroPoints, customAttrs);
 }
 
+// The per-tensor signatures of ral_pdll_qgemm: in the reference they exist only in the
+// AArch64 build, on Arm Compute Library's fixed-point output stage
+// (ral_pdll_qgemm_acl_s8_s8_s8_per_tensor<2,3,4> and ..._s32_per_tensor<2,3>,
+// R context/common_context_impl_quantization.cc:747-1187, registered :1689-1695):
+//   out = clamp8(stage(acc + bias[n]; multiplier = (s_x s_w) / s_o) + z_o)
+// Mirrored here for device "gpu" with the same stage, so that a graph rewritten with the
+// AArch64 pattern set gives the AArch64 results.
+namespace {
+MemRefType<float, 1> asVector(const MemRefType<float, 0>& m) {
+  MemRefType<float, 1> v;
+  v.basePtr = m.basePtr;
+  v.data = m.data;
+  v.offset = m.offset;
+  v.sizes[0] = 1;
+  v.strides[0] = 1;
+  return v;
+}
+MemRefType<int32_t, 1> asVector(const MemRefType<int32_t, 0>& m) {
+  MemRefType<int32_t, 1> v;
+  v.basePtr = m.basePtr;
+  v.data = m.data;
+  v.offset = m.offset;
+  v.sizes[0] = 1;
+  v.strides[0] = 1;
+  return v;
+}
+}  // namespace
+
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_per_tensor(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 0> weightScales,
+    MemRefType<int32_t, 0> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, void* customAttrs) {
+  return pdllQgemmCpuStyle<N>(ctx, stream_handle, input, weight, nullptr, 0, DQ8_BIAS_NONE,
+                              inputScales, inputZeroPoints, asVector(weightScales),
+                              asVector(weightZeroPoints), resultScales, resultZeroPoints,
+                              customAttrs, DQ8_EPI_REQUANT_FIXEDPOINT);
+}
+
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_s32_per_tensor(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<int32_t, 1> bias,
+    MemRefType<float, 0> inputScales, MemRefType<int32_t, 0> inputZeroPoints,
+    MemRefType<float, 0> weightScales, MemRefType<int32_t, 0> weightZeroPoints,
+    MemRefType<float, 0> resultScales, MemRefType<int32_t, 0> resultZeroPoints,
+    void* customAttrs) {
+  return pdllQgemmCpuStyle<N>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0],
+                              DQ8_BIAS_S32, inputScales, inputZeroPoints, asVector(weightScales),
+                              asVector(weightZeroPoints), resultScales, resultZeroPoints,
+                              customAttrs, DQ8_EPI_REQUANT_FIXEDPOINT);
+}
+
 // ------------------------------------------------------------------ ral_qconv
 // out = sat8(rne(((s_x*s_w[co])/s_o) * conv_s32(in, w))); padding and metadata are
 // host memrefs; zero points are not read.
@@ -650,8 +720,8 @@ void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4>
   if (ws_bytes && !ws) return;
   StreamTimer timer(stream);
   int st = dq8_qconv2d_ws(input.data, input.sizes, kernel.data, kernel.sizes, padding.data,
-                          metadata.data, output.data, output.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
-                          DQ8_BIAS_NONE, inputScales.data, weightScales.data,
+                          metadata.data, output.data, output.sizes, sharedSignatureStage(),
+                          nullptr, DQ8_BIAS_NONE, inputScales.data, weightScales.data,
                           weightScales.sizes[0], resultScales.data, 0, ws, ws_bytes, stream);
   if (ws) drv->dealloc(ctx, ws);
   if (timer.on() && st == 0) {
@@ -745,8 +815,8 @@ MemRefType<int8_t, 4> ral_pdll_qconv2d(ExecutionContext* ctx, void* stream_handl
   if (ws_bytes && !ws) return result;
   StreamTimer timer(stream);
   int st = dq8_qconv2d_ws(input.data, input.sizes, weight.data, weight.sizes, plan.padding,
-                          plan.metadata, result.data, result.sizes, DQ8_EPI_REQUANT_CPU, nullptr,
-                          DQ8_BIAS_NONE, inputScales.data, weightScales.data,
+                          plan.metadata, result.data, result.sizes, sharedSignatureStage(),
+                          nullptr, DQ8_BIAS_NONE, inputScales.data, weightScales.data,
                           weightScales.sizes[0], resultScales.data, zo, ws, ws_bytes, stream);
   if (ws) drv->dealloc(ctx, ws);
   if (timer.on() && st == 0)   // weights are [out_channels, h, w, in_channels] here
@@ -875,6 +945,13 @@ TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_ch
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<2>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<3>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<4>);
+
+// the AArch64 build's per-tensor signatures (fixed-point output stage)
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<2>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<3>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<4>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_tensor<2>);
+TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_tensor<3>);
 
 TAO_RAL_API("ral_qconv", "gpu", gpu::q8::ral_qconv);
 TAO_RAL_API("ral_pdll_qconv2d", "gpu", gpu::q8::ral_pdll_qconv2d);

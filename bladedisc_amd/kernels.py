@@ -12,6 +12,7 @@ from . import _lib
 EPI_ACC_S32, EPI_REQUANT_CPU, EPI_REQUANT_GPU, EPI_DEQUANT_F32 = 0, 1, 2, 3
 # requant, then dequantize with the per-tensor output scale, in one epilogue
 EPI_REQUANT_CPU_DEQUANT_F32, EPI_REQUANT_GPU_DEQUANT_F32 = 4, 5
+EPI_REQUANT_FIXEDPOINT = 6
 BIAS_NONE, BIAS_S32, BIAS_F32, BIAS_S8 = 0, 1, 2, 3
 ROUND_HALF_AWAY_FROM_ZERO, ROUND_HALF_TO_EVEN = 0, 1
 
@@ -19,7 +20,8 @@ _BIAS_KIND = {torch.int32: BIAS_S32, torch.float32: BIAS_F32, torch.int8: BIAS_S
 _OUT_DTYPE = {EPI_ACC_S32: torch.int32, EPI_REQUANT_CPU: torch.int8,
               EPI_REQUANT_GPU: torch.int8, EPI_DEQUANT_F32: torch.float32,
               EPI_REQUANT_CPU_DEQUANT_F32: torch.float32,
-              EPI_REQUANT_GPU_DEQUANT_F32: torch.float32}
+              EPI_REQUANT_GPU_DEQUANT_F32: torch.float32,
+              EPI_REQUANT_FIXEDPOINT: torch.int8}
 
 
 def _ptr(t):

@@ -100,6 +100,30 @@ def pdll_qgemm_cpu_style(ex, x, w, bias, sx, sw_n, so, zo=0, transpose_b=False,
     return ral.memref_to_tensor(res, torch.int8)
 
 
+def pdll_qgemm_per_tensor(ex, x, w, bias_s32, sx, sw, so, zo=0, transpose_b=False,
+                          weight_is_const=True):
+    """ral_pdll_qgemm with the AArch64 patterns' per-tensor signature on the gpu device
+    (fixed-point output stage): weight [K,N] unless transpose_b, bias s32 or None, rank-0
+    device scales, rank-0 host zero points."""
+    n = w.shape[0] if transpose_b else w.shape[1]
+    a = ex.new_args().tensor(x).tensor(w)
+    if bias_s32 is not None:
+        a.tensor(bias_s32)
+    a.tensor(sx, rank0=True)
+    _zp0(a, host=True)
+    a.tensor(sw, rank0=True)
+    _zp0(a, host=True)
+    a.tensor(so, rank0=True)
+    a.host_array(np.array([zo], np.int32), rank0=True)
+    a.blob(ral.encode_attr({"transpose_a": False, "transpose_b": bool(transpose_b),
+                            "weight_is_const": bool(weight_is_const),
+                            "bias_is_const": True}))
+    res = a.result_memref("i8", x.dim())
+    ex.call("ral_pdll_qgemm", "gpu", a)
+    assert n == res.sizes[x.dim() - 1]
+    return ral.memref_to_tensor(res, torch.int8)
+
+
 def qconv(ex, x, w, padding, metadata, sx, sw_c, so, out):
     """ral_qconv: padding [4] and metadata [17] are host int32 memrefs."""
     a = ex.new_args().tensor(x).tensor(w)

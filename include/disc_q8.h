@@ -51,6 +51,17 @@ extern "C" {
 #define DQ8_EPI_REQUANT_CPU_DEQUANT_F32 4
 #define DQ8_EPI_REQUANT_GPU_DEQUANT_F32 5
 /* os[n] = (sx*sw[n])/so evaluated in binary32, left to right.                            */
+/* dq8_qgemm and dq8_qconv2d: the integer output stage of the reference's AArch64 path
+ * (R ral/context/common_context_impl_quantization.cc:671-679, 865-872, 1083-1090:
+ * GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT of Arm Compute Library), out: int8
+ *   multiplier[n] = (sx*sw[n])/so in binary32 = M0[n] 2^-31 2^-shift[n], M0 in [2^30, 2^31)
+ *   v = acc + bias[n];  shift >= 0: v = rdivpot(sqrdmulh(v, M0), shift)
+ *                       shift <  0: v = sqrdmulh(v 2^-shift, M0)
+ *   out = clamp(v + zo, -128, 127)
+ * with sqrdmulh(a, b) = (2ab + 2^31) >> 32 and rdivpot rounding ties away from zero.  Bias:
+ * none or DQ8_BIAS_S32; sx and so per tensor, sw per tensor or per channel.  Not bit-identical
+ * to the float stages (different rounding), by design of the reference's two CPU paths. */
+#define DQ8_EPI_REQUANT_FIXEDPOINT 6
 
 /* bias operand kinds */
 #define DQ8_BIAS_NONE 0

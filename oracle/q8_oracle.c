@@ -9,6 +9,7 @@
 
 #include <fenv.h>
 #include <math.h>
+#include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -240,6 +241,96 @@ void q8o_requant_cpu(const int32_t* acc, int64_t M, int64_t N,
     }
   }
   free(os);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Fixed-point requantisation of the AArch64 path.                           */
+/* R: ral/context/common_context_impl_quantization.cc:671-679 (per channel), */
+/*    :865-872 and :1083-1090 (per tensor) select                            */
+/*    GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT and call             */
+/*    arm_compute::quantization::calculate_quantized_multipliers.  The       */
+/*    arithmetic itself lives in Arm Compute Library v23.02.1 (an            */
+/*    http_archive of R/tao/third_party/..., blade_disc_dnn_workspace.bzl    */
+/*    :27-38; its sources are not in the reference tree).  What follows      */
+/*    restates the library's published algorithm:                            */
+/*      multiplier[n] = s_x * s_w[n] / s_o              (binary32)           */
+/*      frexp(multiplier) = q * 2^e, q in [0.5, 1);  M0 = round(q * 2^31),   */
+/*      shift = -e  (M0 == 2^31 -> M0 /= 2, shift -= 1)                      */
+/*      (AsymmHelpers.cpp: calculate_quantized_multiplier[_less_than_one |   */
+/*       _greater_than_one])                                                 */
+/*      v = acc + bias;                                                      */
+/*      shift >= 0: v = rounding_divide_by_pow2(sqrdmulh(v, M0), shift)      */
+/*      shift <  0: v = sqrdmulh(v * 2^-shift, M0)         (NEAsymm.h:       */
+/*      finalize_quantization), v += z_o, clamp to [-128, 127].              */
+/*    sqrdmulh is the AArch64 instruction the library's vqrdmulhq_n_s32      */
+/*    compiles to: (2 a b + 2^31) >> 32, saturated; rounding_divide_by_pow2  */
+/*    rounds half away from zero.  Parity beyond this published algorithm    */
+/*    is unpinned: the reference holds no vectors for it but the 12.0 /      */
+/*    108.0 closed forms of its AArch64 tests.                               */
+/* ------------------------------------------------------------------------ */
+int32_t q8o_sqrdmulh(int32_t a, int32_t b) {
+  if (a == INT32_MIN && b == INT32_MIN) return INT32_MAX;
+  const int64_t prod = (int64_t)a * (int64_t)b;
+  /* (2 prod + 2^31) >> 32 with an arithmetic shift, written without overflow */
+  const int64_t t = prod + ((int64_t)1 << 30);
+  return (int32_t)(t >> 31);
+}
+
+int32_t q8o_rounding_divide_by_pow2(int32_t x, int exponent) {
+  if (exponent <= 0) return x;
+  if (exponent > 31) exponent = 31;
+  const int32_t mask = (int32_t)(((uint32_t)1 << exponent) - 1u);
+  const int32_t threshold = (mask >> 1) + (x < 0 ? 1 : 0);
+  return (x >> exponent) + ((x & mask) > threshold ? 1 : 0);
+}
+
+void q8o_fixedpoint_multiplier(float multiplier, int32_t* quant_multiplier, int32_t* shift) {
+  int e = 0;
+  const double q = frexp((double)multiplier, &e);
+  int64_t q_fixed = (int64_t)round(q * (double)((int64_t)1 << 31));
+  int sh = -e;
+  if (q_fixed == ((int64_t)1 << 31)) {
+    q_fixed /= 2;
+    --sh;
+  }
+  *quant_multiplier = (int32_t)q_fixed;
+  *shift = sh;
+}
+
+int8_t q8o_finalize_fixedpoint(int32_t v, int32_t quant_multiplier, int32_t shift, int32_t zo) {
+  if (shift < 0) {
+    /* vmulq_n_s32: the product wraps */
+    const int32_t scaled = (int32_t)((uint32_t)v * ((uint32_t)1 << (-shift > 31 ? 31 : -shift)));
+    v = q8o_sqrdmulh(scaled, quant_multiplier);
+  } else {
+    v = q8o_rounding_divide_by_pow2(q8o_sqrdmulh(v, quant_multiplier), shift);
+  }
+  v = (int32_t)((uint32_t)v + (uint32_t)zo);
+  if (v < -128) v = -128;
+  if (v > 127) v = 127;
+  return (int8_t)v;
+}
+
+void q8o_requant_fixedpoint(const int32_t* acc, int64_t M, int64_t N, const int32_t* b32,
+                            float sx, const float* sw, int64_t n_sw, float so, int32_t zo,
+                            int8_t* out) {
+  int32_t* mult = (int32_t*)malloc(sizeof(int32_t) * (size_t)(N > 0 ? N : 1));
+  int32_t* shift = (int32_t*)malloc(sizeof(int32_t) * (size_t)(N > 0 ? N : 1));
+  for (int64_t n = 0; n < N; ++n) {
+    const float num = sx * sw[n_sw > 1 ? n : 0];
+    const float multiplier = num / so;
+    q8o_fixedpoint_multiplier(multiplier, &mult[n], &shift[n]);
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      int32_t v = acc[m * N + n];
+      if (b32) v = (int32_t)((uint32_t)v + (uint32_t)b32[n]);
+      out[m * N + n] = q8o_finalize_fixedpoint(v, mult[n], shift[n], zo);
+    }
+  }
+  free(mult);
+  free(shift);
 }
 
 /* R: quantized_gpu_kernel_impl.cc:262-265 (per channel) / :385 (per tensor):

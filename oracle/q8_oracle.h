@@ -26,6 +26,12 @@
  *                           ral/context/quantized_gpu_kernel_impl.cc:262-265,385,416-420
  *                           (cublasLt alpha + EPILOGUE_BIAS) and
  *                           ral/context/stream_executor_based_impl.cc:458.
+ *   q8o_requant_fixedpoint  the AArch64 path's requantisation by a fixed-point multiplier
+ *                           and shift (GEMMLowpOutputStageType::QUANTIZE_DOWN_FIXEDPOINT,
+ *                           ral/context/common_context_impl_quantization.cc:671-679,
+ *                           865-872, 1083-1090); the arithmetic is Arm Compute Library's
+ *                           (v23.02.1, not in the reference tree): published algorithm
+ *                           restated, PARITY UNPINNED beyond it.
  *   q8o_dequant_acc  (E3)   f32(acc)*(s_x*s_w[n]) + bias[n]: qgemm followed by
  *                           mhlo_disc.dequantize with a per-channel scale.
  *   q8o_quantize_f32        disc/transforms/disc_lower_quantize_and_dequantize.cc:77-94
@@ -93,6 +99,22 @@ void q8o_requant_gpu(const int32_t* acc, int64_t M, int64_t N,
                      const float* bias_f32, const int8_t* bias_i8,
                      const float* sx, int64_t n_sx, const float* sw,
                      int64_t n_sw, const float* so, int64_t n_so, int8_t* out);
+
+/* Fixed-point requantisation (see q8_oracle.c for the algorithm and its source).
+ *   q8o_sqrdmulh               saturating rounding doubling multiply, high half
+ *   q8o_rounding_divide_by_pow2  x / 2^exponent, ties away from zero
+ *   q8o_fixedpoint_multiplier  multiplier -> (M0 in [2^30, 2^31), shift), multiplier =
+ *                              M0 * 2^-31 * 2^-shift exactly (a binary32 has 24 bits)
+ *   q8o_finalize_fixedpoint    one value through the output stage
+ *   q8o_requant_fixedpoint     out = clamp8(stage(acc + b32[n], M0[n], shift[n]) + zo),
+ *                              multiplier[n] = (sx * sw[n]) / so in binary32; b32 may be NULL */
+int32_t q8o_sqrdmulh(int32_t a, int32_t b);
+int32_t q8o_rounding_divide_by_pow2(int32_t x, int exponent);
+void q8o_fixedpoint_multiplier(float multiplier, int32_t* quant_multiplier, int32_t* shift);
+int8_t q8o_finalize_fixedpoint(int32_t v, int32_t quant_multiplier, int32_t shift, int32_t zo);
+void q8o_requant_fixedpoint(const int32_t* acc, int64_t M, int64_t N, const int32_t* b32,
+                            float sx, const float* sw, int64_t n_sw, float so, int32_t zo,
+                            int8_t* out);
 
 /* E3.  bias may be NULL. */
 void q8o_dequant_acc(const int32_t* acc, int64_t M, int64_t N, float sx,

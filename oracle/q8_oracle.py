@@ -142,6 +142,46 @@ def requant_gpu(acc, sx, sw, so, bias_f32=None, bias_i8=None):
     return out
 
 
+def requant_fixedpoint(acc, sx, sw, so, b32=None, zo=0):
+    """The AArch64 path's output stage: (acc + b32[n]) times a fixed-point multiplier and
+    shift derived from (sx * sw[n]) / so, plus zo, clamped to int8."""
+    acc = _c(acc, np.int32)
+    m, n = acc.shape
+    sw = _c(np.atleast_1d(sw), np.float32)
+    if sw.size not in (1, n):
+        raise ValueError("weight scales must have 1 or N entries")
+    b = _c(b32, np.int32) if b32 is not None else None
+    out = np.empty((m, n), np.int8)
+    lib().q8o_requant_fixedpoint(_p(acc), _i64(m), _i64(n), _p(b), C.c_float(sx), _p(sw),
+                                 _i64(sw.size), C.c_float(so), C.c_int32(int(zo)), _p(out))
+    return out
+
+
+def fixedpoint_multiplier(multiplier):
+    """(M0, shift) of a binary32 multiplier."""
+    m0, sh = C.c_int32(), C.c_int32()
+    lib().q8o_fixedpoint_multiplier(C.c_float(multiplier), C.byref(m0), C.byref(sh))
+    return m0.value, sh.value
+
+
+def sqrdmulh(a, b):
+    f = lib().q8o_sqrdmulh
+    f.restype = C.c_int32
+    return f(C.c_int32(int(a)), C.c_int32(int(b)))
+
+
+def rounding_divide_by_pow2(x, exponent):
+    f = lib().q8o_rounding_divide_by_pow2
+    f.restype = C.c_int32
+    return f(C.c_int32(int(x)), C.c_int(int(exponent)))
+
+
+def finalize_fixedpoint(v, m0, shift, zo=0):
+    f = lib().q8o_finalize_fixedpoint
+    f.restype = C.c_int8
+    return f(C.c_int32(int(v)), C.c_int32(int(m0)), C.c_int32(int(shift)), C.c_int32(int(zo)))
+
+
 def dequant_acc(acc, sx, sw, bias=None):
     """E3: f32(acc) * (sx*sw[n]) + bias[n]."""
     acc = _c(acc, np.int32)

@@ -138,6 +138,38 @@ def test_qgemm_persistent_variants_walk_many_tiles(K, m, n, k):
         assert np.array_equal(got.view(np.uint32), want_f32.view(np.uint32)), tag
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 768, 768), (1000, 768, 3072), (257, 130, 64), (5, 7, 48),
+                                   (4096, 768, 768), (300, 260, 1041)])
+@pytest.mark.parametrize("bias", ["none", "s32"])
+def test_qgemm_requant_fixedpoint(K, m, n, k, bias):
+    """The integer output stage of the reference's AArch64 path (multiplier + shift) in every
+    kernel variant, per-channel and per-tensor weight scales, with and without an output zero
+    point, multipliers below and above one -- bit-exact against the oracle's restatement."""
+    rng = np.random.default_rng(m + 5 * n + k + len(bias))
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    b32 = rng.integers(-200000, 200000, n).astype(np.int32) if bias == "s32" else None
+    bias_t = dev(b32) if b32 is not None else None
+    cases = [(sw, so, 0), (sw, so, -5), (sw[:1], so, 0),
+             (sw, np.float32(so * 1e-5), 7)]          # multipliers above one: left shifts, saturation
+    for swv, sov, zo in cases:
+        want = O.requant_fixedpoint(acc, sx, swv, sov, b32=b32, zo=zo)
+        for v in [-1] + gemm_variants(K, k):
+            got = host(K.qgemm(dev(a), dev(w), K.EPI_REQUANT_FIXEDPOINT, sx=dev(np.array([sx])),
+                               sw=dev(swv), so=dev(np.array([sov], np.float32)), bias=bias_t, zo=zo,
+                               variant=v))
+            np.testing.assert_array_equal(got, want, err_msg="variant %d zo %d" % (v, zo))
+    want = O.requant_fixedpoint(acc, sx, sw, so, b32=b32)
+    sat = np.mean((want == 127) | (want == -128))
+    assert sat < 0.5, "degenerate test: %.2f saturated" % sat
+    # it is a different rounding from the float stage, not the same numbers by another route
+    other = O.requant_cpu(acc, sx, sw, so, b32=b32)
+    assert np.max(np.abs(other.astype(np.int32) - want.astype(np.int32))) <= 1
+
+
 @pytest.mark.parametrize("per_channel", [False, True])
 @pytest.mark.parametrize("bias", ["none", "f32", "s8"])
 def test_qgemm_requant_gpu(K, per_channel, bias):
@@ -569,6 +601,14 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
         got = host(K.qconv2d(dev(x), dev(wt), padding, md, out_shape, K.EPI_REQUANT_CPU,
                              sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])), variant=v))
         np.testing.assert_array_equal(got, want, err_msg="variant %d" % v)
+    # the integer output stage of the reference's AArch64 convolution, with an s32 bias
+    b32 = rng.integers(-100000, 100000, co).astype(np.int32)
+    want_fx = O.requant_fixedpoint(acc.reshape(-1, co), sx, sw, so, b32=b32, zo=-2).reshape(out_shape)
+    for v in variants:
+        got = host(K.qconv2d(dev(x), dev(wt), padding, md, out_shape, K.EPI_REQUANT_FIXEDPOINT,
+                             sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])),
+                             bias=dev(b32), zo=-2, variant=v))
+        np.testing.assert_array_equal(got, want_fx, err_msg="fixed-point, variant %d" % v)
     # requant -> dequantize in the convolution's epilogue: the bits of dequantize(requant)
     want_f = O.dequantize(want, np.array([so], np.float32), np.array([0], np.int32))
     for v in variants:

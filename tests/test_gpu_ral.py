@@ -252,6 +252,87 @@ def test_ral_pdll_qconv2d(rt, fmt, padding, k, stride, dil):
         np.testing.assert_array_equal(host(got), want)
 
 
+@pytest.mark.parametrize("rank", [2, 3, 4])
+@pytest.mark.parametrize("bias", [False, True])
+def test_ral_pdll_qgemm_per_tensor_signature_uses_the_fixed_point_stage(rt, rank, bias):
+    """The per-tensor ral_pdll_qgemm signatures exist in the reference only in the AArch64
+    build, on Arm Compute Library's multiplier-and-shift output stage
+    (common_context_impl_quantization.cc:747-1187, registered :1689-1695): mirrored on gpu
+    with the same stage, bit-exact against its restatement; config 1 sizes."""
+    if bias and rank == 4:
+        pytest.skip("the reference registers the s32-bias form for ranks 2 and 3 only")
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(40 + rank)
+    lead = {2: (64,), 3: (4, 16), 4: (2, 2, 16)}[rank]
+    k, n = 768, 768
+    x = rng.integers(-128, 128, lead + (k,), dtype=np.int8)
+    w_kn = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(x.reshape(-1, k), np.ascontiguousarray(w_kn.T))
+    sx, sw = np.float32(0.02), np.float32(0.011)
+    so = np.float32(np.std(acc * float(sx) * float(sw)) / 40.0)
+    b32 = rng.integers(-100000, 100000, n).astype(np.int32) if bias else None
+    want = O.requant_fixedpoint(acc, sx, np.array([sw]), so, b32=b32, zo=2).reshape(lead + (n,))
+    with ctx.execution() as ex:
+        # (weight_is_const would let the context cache the repacked weight by its address,
+        # and these test tensors come and go)
+        got = ops.pdll_qgemm_per_tensor(ex, dev(x), dev(w_kn), dev(b32) if bias else None, f1(sx),
+                                        f1(sw), f1(so), zo=2, weight_is_const=False)
+        assert list(got.shape) == list(lead + (n,))
+        np.testing.assert_array_equal(host(got), want)
+    # a different rounding from the float stage of the per-channel signatures, one step at most
+    flt = O.requant_cpu(acc, sx, np.array([sw]), so, b32=b32, zo=2).reshape(lead + (n,))
+    assert np.max(np.abs(flt.astype(np.int32) - want.astype(np.int32))) <= 1
+
+
+def test_shared_signatures_switch_to_the_fixed_point_stage(rt, monkeypatch):
+    """ral_qgemm with per-channel weight scales, ral_qconv and ral_pdll_qconv2d have one
+    signature and two CPU implementations in the reference (oneDNN's float post-ops on x86,
+    Arm Compute Library's fixed-point stage on AArch64): DISC_GPU_REQUANT_FIXEDPOINT=1 selects
+    the second here.  Known answers of the reference's AArch64 tests (12.0, 108.0) and seeded
+    tensors against the oracle."""
+    ctx, ral, ops = rt
+    monkeypatch.setenv("DISC_GPU_REQUANT_FIXEDPOINT", "1")
+    rng = np.random.default_rng(99)
+    # -- ral_qgemm, per channel
+    m, k, n = 100, 400, 136
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx = np.float32(0.02)
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40.0)
+    with ctx.execution() as ex:
+        got = ops.qgemm(ex, dev(a), dev(w), f1(sx), dev(sw), f1(so))
+        np.testing.assert_array_equal(host(got), O.requant_fixedpoint(acc, sx, sw, so))
+    # -- ral_qconv: 3x3, 25 channels of (-72)(-51) -> 108 (quantized_conv2d.cc cases 2, 3)
+    x = np.full((1, 5, 5, 25), -72, np.int8)
+    wt = np.full((4, 3, 3, 25), -51, np.int8)
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    out = torch.empty((1, 3, 3, 4), dtype=torch.int8, device="cuda")
+    with ctx.execution() as ex:
+        ops.qconv(ex, dev(x), dev(wt), [0, 0, 0, 0], md, f1(8.333333e-3),
+                  dev(np.full(4, 1.568627e-2, np.float32)), f1(1.0), out)
+        assert np.all(host(out) == 108)
+    # -- ral_pdll_qconv2d on seeded tensors, SAME padding, with an output zero point
+    nb, h, w_, ci, co = 2, 14, 12, 32, 48
+    x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+    wt = rng.integers(-128, 128, (co, 3, 3, ci), dtype=np.int8)
+    pad4, md, out_shape = O.conv_attrs(x.shape, wt.shape, "NHWC", [1, 1, 1, 1], [1, 1, 1, 1], "SAME")
+    acc = O.conv_s32(x, wt, pad4, md, out_shape)
+    sw = rng.uniform(0.001, 0.05, co).astype(np.float32)
+    so = np.float32(np.std(acc * float(sx) * float(sw.mean())) / 40.0)
+    want = O.requant_fixedpoint(acc.reshape(-1, co), sx, sw, so, zo=3).reshape(acc.shape)
+    with ctx.execution() as ex:
+        got = ops.pdll_qconv2d(ex, dev(x), dev(wt), f1(sx), dev(sw), f1(so), zo=3)
+        np.testing.assert_array_equal(host(got), want)
+    # ... and back: without the switch the float stage answers
+    monkeypatch.delenv("DISC_GPU_REQUANT_FIXEDPOINT")
+    with ctx.execution() as ex:
+        got = ops.pdll_qconv2d(ex, dev(x), dev(wt), f1(sx), dev(sw), f1(so), zo=3)
+        np.testing.assert_array_equal(
+            host(got), O.requant_cpu(acc.reshape(-1, co), sx, sw, so, zo=3).reshape(acc.shape))
+
+
 def test_ral_pdll_qconv2d_rejects_bad_attrs(rt):
     ctx, ral, ops = rt
     x = torch.zeros((1, 4, 4, 16), dtype=torch.int8, device="cuda")

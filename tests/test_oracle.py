@@ -441,3 +441,131 @@ def test_conv_oracle_agrees_with_library_quantized_conv2d():
                 assert not ((got != want) & ~near_tie).any(), eng
     finally:
         torch.backends.quantized.engine = saved
+
+
+# ---------------------------------------------------------------- fixed-point requantisation
+# Pins for the restatement of Arm Compute Library's QUANTIZE_DOWN_FIXEDPOINT output stage (the
+# reference's AArch64 entries, common_context_impl_quantization.cc:671-679, 865-872, 1083-1090).
+# The library is not in the reference tree, so the pins are what the arithmetic fixes: the two
+# rounding primitives against exact rationals, the multiplier decomposition against exact
+# equality, the whole stage against an independent evaluation in exact arithmetic, the
+# reference's 12.0 / 108.0 closed forms, saturation and left shifts.
+def _floor_div(a, b):
+    return a // b
+
+
+def test_sqrdmulh_is_round_half_up_of_the_doubled_high_half():
+    from fractions import Fraction
+    import math
+    rng = np.random.default_rng(5)
+    cases = [(0, 0), (1, 1 << 30), (-1, 1 << 30), (3, 1 << 30), (-3, 1 << 30), (5, 1 << 29),
+             (-5, 1 << 29), (2**31 - 1, 2**31 - 1), (-2**31, 2**31 - 1), (-2**31, -2**31),
+             (-2**31, 1 << 30), (12345, -(1 << 30))]
+    cases += [(int(a), int(b)) for a, b in zip(rng.integers(-2**31, 2**31, 2000),
+                                               rng.integers(-2**31, 2**31, 2000))]
+    for a, b in cases:
+        exact = Fraction(a * b, 1 << 31)                 # the doubled product's high half
+        want = math.floor(exact + Fraction(1, 2))        # ties toward +infinity
+        want = min(want, 2**31 - 1)                      # only -2^31 * -2^31 saturates
+        assert O.sqrdmulh(a, b) == want, (a, b)
+    assert O.sqrdmulh(-3, 1 << 30) == -1                 # -1.5 -> -1: not half away from zero
+
+
+def test_rounding_divide_by_pow2_rounds_half_away_from_zero():
+    from fractions import Fraction
+    import math
+    rng = np.random.default_rng(6)
+    xs = [0, 1, -1, 2, -2, 3, -3, 5, -5, 6, -6, 2**31 - 1, -2**31] + \
+        [int(v) for v in rng.integers(-2**31, 2**31, 500)]
+    for x in xs:
+        for e in (0, 1, 2, 3, 7, 16, 30, 31):
+            q = Fraction(x, 1 << e)
+            fl = math.floor(q)
+            frac = q - fl
+            if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and x > 0):
+                want = fl + 1
+            else:
+                want = fl
+            assert O.rounding_divide_by_pow2(x, e) == want, (x, e)
+
+
+def test_fixedpoint_multiplier_represents_the_binary32_value_exactly():
+    from fractions import Fraction
+    rng = np.random.default_rng(7)
+    vals = [1.3071891e-4, 0.5, 0.25, 0.75, 1.0, 1.5, 2.0, 3.999, 1e-5, 0.99999994, 123.456]
+    vals += list(np.exp(rng.uniform(np.log(1e-6), np.log(64.0), 500)))
+    for v in vals:
+        f = np.float32(v)
+        m0, sh = O.fixedpoint_multiplier(float(f))
+        assert (1 << 30) <= m0 < (1 << 31), (v, m0)
+        assert Fraction(m0, 1 << 31) / (Fraction(2) ** sh) == Fraction(float(f)), (v, m0, sh)
+    assert O.fixedpoint_multiplier(0.0) == (0, 0)
+    assert O.fixedpoint_multiplier(0.5) == (1 << 30, 0)
+    assert O.fixedpoint_multiplier(1.0) == (1 << 30, -1)     # a left shift
+
+
+def _stage_exact(v, mult_f32, zo):
+    """The output stage evaluated independently in exact arithmetic: the high-half product
+    rounded half up, then the power-of-two division rounded half away from zero."""
+    from fractions import Fraction
+    import math
+    m = Fraction(float(np.float32(mult_f32)))
+    e = 0
+    q = m
+    while q >= 1:
+        q /= 2
+        e += 1
+    while 0 < q < Fraction(1, 2):
+        q *= 2
+        e -= 1
+    m0 = int(q * (1 << 31))                       # exact: q has 24 significant bits
+    shift = -e
+    if shift < 0:
+        v = ((v << -shift) + 2**31) % 2**32 - 2**31      # vmulq_n_s32 wraps
+        v = math.floor(Fraction(v * m0, 1 << 31) + Fraction(1, 2))
+    else:
+        h = math.floor(Fraction(v * m0, 1 << 31) + Fraction(1, 2))
+        qq = Fraction(h, 1 << shift)
+        fl = math.floor(qq)
+        v = fl + 1 if (qq - fl > Fraction(1, 2) or (qq - fl == Fraction(1, 2) and h > 0)) else fl
+    return int(min(127, max(-128, v + zo)))
+
+
+def test_requant_fixedpoint_known_answers_and_exact_stage():
+    # the reference's AArch64 closed forms: 25 x (-72)(-51) -> 12, nine taps of it -> 108
+    # (disc/tests/tensorflow_ops/quantized_matmul.cc:26-55, disc/tests/pdll/quantized_conv2d.cc)
+    sx, sw, so = np.float32(8.333333e-3), np.float32(1.568627e-2), np.float32(1.0)
+    acc = np.array([[91800, 826200, 0, -91800, -826200]], np.int32)
+    got = O.requant_fixedpoint(acc, sx, np.array([sw] * 5, np.float32), so)
+    np.testing.assert_array_equal(got, [[12, 108, 0, -12, -108]])
+    # random accumulators, per-channel scales (right shifts), bias and zero point
+    rng = np.random.default_rng(8)
+    m, n = 37, 29
+    acc = rng.integers(-3_000_000, 3_000_000, (m, n)).astype(np.int32)
+    acc[0, :5] = [2**31 - 1, -2**31, 0, 1, -1]
+    b32 = rng.integers(-100000, 100000, n).astype(np.int32)
+    sx = np.float32(0.02)
+    swv = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    so = np.float32(0.7)
+    got = O.requant_fixedpoint(acc, sx, swv, so, b32=b32, zo=-3)
+    for i in range(m):
+        for j in range(n):
+            mult = np.float32(np.float32(sx * swv[j]) / so)
+            v = int(acc[i, j]) + int(b32[j])
+            v = (v + 2**31) % 2**32 - 2**31
+            assert got[i, j] == _stage_exact(v, mult, -3), (i, j)
+    # within one step of the real-valued product wherever nothing saturates
+    real = (acc.astype(np.float64) + b32) * (np.float64(sx) * swv.astype(np.float64) / np.float64(so)) - 3
+    inside = np.abs(real) < 126
+    assert np.all(np.abs(got.astype(np.float64) - real)[inside] <= 0.5 + 1e-3)
+    # multipliers of one and more: left shifts, saturation on both sides
+    # (the pre-multiplication by 2^-shift wraps like the library's vmulq_n_s32: 2^30 * 2 is
+    # -2^31, which the last two columns show)
+    acc = np.array([[1, -1, 50, -50, 100, -100, 2**28, -2**28, 2**30, -2**30]], np.int32)
+    for mult in (1.0, 1.5, 2.0, 3.25):
+        got = O.requant_fixedpoint(acc, np.float32(mult), np.ones(10, np.float32), np.float32(1.0))
+        want = [_stage_exact(int(v), mult, 0) for v in acc[0]]
+        np.testing.assert_array_equal(got[0], want, err_msg=str(mult))
+        assert got[0, 6] == 127 and got[0, 7] == -128
+    got = O.requant_fixedpoint(acc, np.float32(1.0), np.ones(10, np.float32), np.float32(1.0))
+    assert got[0, 8] == -128 and got[0, 9] == -128

@@ -33,6 +33,11 @@ GOLDEN_NAMES = [
     "ral_kernel_launch___gpu___pvoid_ppvoid_i64_pvoid_i64_i64_i64_i64_i64_i64_i32_pvoid_i32_ppvoid___void",
     "d2h____gpu___pvoid_pvoid_pvoid_pvoid_i64___void",
     "ral_gpu_get_stream___gpu___pvoid_i32___pvoid",
+    # the AArch64 build's per-tensor ral_pdll_qgemm signatures (weight scale and zero point
+    # of rank 0; common_context_impl_quantization.cc:1689-1695), mirrored for device gpu
+    "ral_pdll_qgemm___gpu___pvoid_pvoid_m2di8_m2di8_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m2di8",
+    "ral_pdll_qgemm___gpu___pvoid_pvoid_m4di8_m2di8_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m4di8",
+    "ral_pdll_qgemm___gpu___pvoid_pvoid_m3di8_m2di8_m1di32_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m3di8",
 ]
 
 
