@@ -50,12 +50,25 @@ _PROTOS = {
                                   _VP, _VP, _VP, _SZ, _VP]),
     "dq8_tf_dequantize": (_INT, [_VP, _INT, _VP, _I64, _I64, _I64, _VP, _VP, _INT, _VP, _SZ,
                                  _VP]),
+    "dq8_qgemm_fused": (_INT, [_VP, _I64, _VP, _I64, _VP, _I64, _I64, _I64, _I64, _INT, _INT,
+                               _INT, _VP, _INT, _VP, _I64, _VP, _I64, _VP, _I64, _I32, _I32,
+                               _I32, _VP, _SZ, _VP, _VP]),
+    "dq8_qconv2d_fused": (_INT, [_VP, C.POINTER(_I64), _VP, C.POINTER(_I64), C.POINTER(_I32),
+                                 C.POINTER(_I32), _VP, C.POINTER(_I64), _INT, _VP, _INT, _VP,
+                                 _VP, _I64, _VP, _I32, _VP, _SZ, _VP, _VP]),
     "dq8_minmax_workspace_bytes": (_SZ, [_I64, _I64, _I64]),
     "dq8_minmax": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP, _SZ, _VP]),
     "dq8_minmax_static_max_bytes": (_SZ, []),
     "dq8_minmax_static": (_INT, [_VP, _I64, _I64, _I64, _VP, _VP, _VP]),
     "dq8_fill": (_INT, [_VP, _INT, _SZ, _VP]),
 }
+
+
+class PostOps(C.Structure):
+    """dq8_postops_t (include/disc_q8.h)."""
+    _fields_ = [("residual", _VP), ("residual_kind", _INT), ("ldr", _I64),
+                ("residual_scale", _VP), ("residual_zp", _I32), ("relu", _INT),
+                ("out_scale", _VP), ("out_zp", _I32), ("table", _VP)]
 
 
 def lib():

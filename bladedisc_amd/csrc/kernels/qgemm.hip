@@ -35,9 +35,9 @@ __device__ __forceinline__ void store_one(const EpiParams& e, int m, int n, int 
   if (EPI == DQ8_EPI_ACC_S32)
     ((int32_t*)e.out)[off] = acc;
   else if (EPI == DQ8_EPI_DEQUANT_F32)
-    ((float*)e.out)[off] = dequant_one_any(e, c, acc, dequant_so(e));
+    ((float*)e.out)[off] = finish_f32(e, dequant_one_any(e, c, acc, dequant_so(e)), m, n);
   else
-    ((int8_t*)e.out)[off] = (int8_t)requant_one<EPI>(e, c, acc);
+    ((int8_t*)e.out)[off] = (int8_t)finish_s8(e, requant_one<EPI>(e, c, acc), m, n);
 }
 
 template <int EPI>
@@ -94,10 +94,10 @@ __global__ void __launch_bounds__(256) qconv_generic_kernel(const GenericConvPar
     const int64_t off = b * p.o_sb + co * p.o_sc + y * p.o_sh + x * p.o_sw;
     if (EPI == DQ8_EPI_ACC_S32)
       ((int32_t*)p.epi.out)[off] = acc;
-    else if (EPI == DQ8_EPI_DEQUANT_F32)
-      ((float*)p.epi.out)[off] = dequant_one_any(p.epi, c, acc, dequant_so(p.epi));
+    else if (EPI == DQ8_EPI_DEQUANT_F32)   // (a fused residual has the output's layout)
+      ((float*)p.epi.out)[off] = finish_f32_at(p.epi, dequant_one_any(p.epi, c, acc, dequant_so(p.epi)), off);
     else
-      ((int8_t*)p.epi.out)[off] = (int8_t)requant_one<EPI>(p.epi, c, acc);
+      ((int8_t*)p.epi.out)[off] = (int8_t)finish_s8_at(p.epi, requant_one<EPI>(p.epi, c, acc), off);
   }
 }
 
@@ -299,8 +299,9 @@ int launch_pipe(const MainParams& p, hipStream_t st) {
 template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
 int launch_persist(const MainParams& p, int per_cu, hipStream_t st) {
   constexpr int stage = (BM + BN) * 128;
-  // (per-channel factors: 8 bytes, plus 4 for the shifts of the fixed-point output stage)
-  constexpr int lds = 2 * stage + (WM * WN * 4096 + BN * 8 <= stage ? 0 : BN * 12);
+  // (per-channel factors: 8 bytes, plus 4 for the shifts of the fixed-point output stage, and
+  // the 256-byte table of a fused lookup)
+  constexpr int lds = 2 * stage + (WM * WN * 4096 + BN * 12 + 256 <= stage ? 0 : BN * 12 + 256);
   DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
               "persistent qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
   auto kern = qgemm_persist_kernel<BM, BN, WM, WN, CONV, EPI>;
@@ -346,12 +347,12 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, CONV, EPI>(p, st);
     case kPipe128w8: return launch_pipe<128, 128, 2, 4, 1, CONV, EPI>(p, st);
     case kPipe256x192: return launch_pipe<256, 192, 4, 2, 1, CONV, EPI>(p, st);
-    case kPersist256: return launch_persist<256, 256, 2, 4, CONV, EPI>(p, 1, st);
-    case kPersist128: return launch_persist<128, 128, 2, 4, CONV, EPI>(p, 2, st);
-    case kPersist256x192: return launch_persist<256, 192, 4, 2, CONV, EPI>(p, 1, st);
   }
-  if constexpr (!CONV) {
+  if constexpr (!CONV) {   // GEMM only: the small-M kernel and the persistent forms
     if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
+    if (variant == kPersist256) return launch_persist<256, 256, 2, 4, false, EPI>(p, 1, st);
+    if (variant == kPersist128) return launch_persist<128, 128, 2, 4, false, EPI>(p, 2, st);
+    if (variant == kPersist256x192) return launch_persist<256, 192, 4, 2, false, EPI>(p, 1, st);
   }
   return fail("unknown or unsupported qgemm variant for this operation");
 }
@@ -481,6 +482,41 @@ int check_epilogue(const char* who, int epilogue, const void* bias, int bias_kin
   return 0;
 }
 
+// Validates the fused operators against the epilogue and puts them into the kernel
+// parameters.  `int8_out`: the epilogue proper writes int8; `n_so`: entries of the output scale.
+int apply_postops(const char* who, const dq8_postops_t* post, bool int8_out, bool f32_requant,
+                  int64_t n_so, int64_t N, EpiParams* e) {
+  if (!post || (post->residual_kind == DQ8_RESIDUAL_NONE && !post->table)) return 0;
+  const std::string w(who);
+  DQ8_REQUIRE(int8_out || f32_requant,
+              w + ": fused operators need a requantising epilogue");
+  if (post->table) {
+    DQ8_REQUIRE(int8_out && post->residual_kind == DQ8_RESIDUAL_NONE,
+                w + ": a fused table takes an int8 result and no residual");
+    e->table = static_cast<const uint8_t*>(post->table);
+    return 0;
+  }
+  DQ8_REQUIRE(post->residual_kind == DQ8_RESIDUAL_F32 || post->residual_kind == DQ8_RESIDUAL_S8,
+              w + ": unknown residual kind");
+  DQ8_REQUIRE(post->residual != nullptr && post->ldr >= N, w + ": residual missing or too narrow");
+  DQ8_REQUIRE(n_so == 1, w + ": a fused residual takes a per-tensor output scale");
+  DQ8_REQUIRE(post->residual_kind != DQ8_RESIDUAL_S8 || post->residual_scale != nullptr,
+              w + ": an int8 residual needs its scale");
+  DQ8_REQUIRE(int8_out == (post->out_scale != nullptr),
+              w + ": int8 results with a residual need out_scale, f32 results take none");
+  e->resid = post->residual;
+  e->resid_kind = post->residual_kind;
+  e->ldr = post->ldr;
+  e->resid_scale = post->residual_scale;
+  e->resid_zp = post->residual_zp;
+  e->relu = post->relu != 0;
+  e->out_scale = post->out_scale;
+  e->out_zp = post->out_zp;
+  const int esz = post->residual_kind == DQ8_RESIDUAL_F32 ? 4 : 1;
+  e->resid_vec = aligned(post->residual, 16) && (post->ldr * esz) % 16 == 0;
+  return 0;
+}
+
 template <typename P>
 int launch_generic_epi(void (*k0)(const P), void (*k1)(const P), void (*k2)(const P),
                        void (*k3)(const P), int epilogue, const P& p, int64_t total,
@@ -541,14 +577,12 @@ extern "C" int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int6
   return check_hip(hipGetLastError(), "dq8_transpose_s8 launch");
 }
 
-extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
-                                 const int8_t* W, int64_t ldw, void* out, int64_t ldo,
-                                 int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
-                                 int epilogue, const void* bias, int bias_kind,
-                                 const float* sx, int64_t n_sx, const float* sw,
-                                 int64_t n_sw, const float* so, int64_t n_so,
-                                 int32_t zx, int32_t zw, int32_t zo, void* workspace,
-                                 size_t workspace_bytes, void* stream) {
+namespace {
+int qgemm_impl(int variant, const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, void* out,
+               int64_t ldo, int64_t M, int64_t N, int64_t K, int tp_a, int tp_b, int epilogue,
+               const void* bias, int bias_kind, const float* sx, int64_t n_sx, const float* sw,
+               int64_t n_sw, const float* so, int64_t n_so, int32_t zx, int32_t zw, int32_t zo,
+               void* workspace, size_t workspace_bytes, const dq8_postops_t* post, void* stream) {
   clear_error();
   DQ8_REQUIRE(M >= 0 && N >= 0 && K >= 0, "dq8_qgemm: negative size");
   DQ8_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
@@ -604,6 +638,9 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
+  if (int s = apply_postops("dq8_qgemm", post, es == 1 && epilogue != DQ8_EPI_ACC_S32, requant != 0,
+                            n_so, N, &e))
+    return s;
 
   // Zero points: sum (a - zx)(w - zw) = sum a w - zx SW[n] - zw SA[m] + K zx zw with the row
   // sums SW, SA.  Given scratch for the two correction vectors the heuristic keeps the
@@ -627,6 +664,10 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
       aligned(workspace, 256) &&
       workspace_bytes >= dq8_qgemm_workspace_bytes_zp(M, N, K, tp_a, tp_b, zx, zw);
   if (auto_pick && has_zp && !zp_mfma) variant = 0;
+  // fused operators are implemented on the vector store paths of the MFMA kernels (and in
+  // the generic kernel): output rows that are not 16-byte aligned take the generic kernel
+  const bool fused = e.table != nullptr || e.resid_kind != 0;
+  if (fused && !(es == 1 ? e.vec_store16 : e.vec_store)) variant = 0;
   // (a ragged K without the scratch to pad it, or unaligned operands: the generic kernel
   // takes any strides; a transposed operand without scratch stays an error below)
   if (variant != 0 && !mfma_operands && !((tp_a || !tp_b) && !have_ws)) variant = 0;
@@ -693,6 +734,13 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.epi = e;
   if (auto_pick)
     variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false), es);
+  if (fused || e.fixedpoint) {   // the persistent forms carry neither
+    DQ8_REQUIRE(auto_pick || (variant != kPersist256 && variant != kPersist256x192 && variant != kPersist128),
+                "dq8_qgemm: the persistent variants take neither fused operators nor the fixed-point stage");
+    if (variant == kPersist256) variant = kPipe256w8;
+    if (variant == kPersist256x192) variant = kPipe256x192;
+    if (variant == kPersist128) variant = kPipe128w8;
+  }
   if (!zp_mfma) return launch_epi<false>(variant, p, epilogue, st);
 
   // ---- zero points: row sums -> corrections -> a pipelined kernel that starts from them
@@ -728,6 +776,32 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
   p.corr_m = zw != 0 ? corr_m : nullptr;
   return launch_epi<false>(variant, p, epilogue, st);
 }
+}  // namespace
+
+extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
+                                 const int8_t* W, int64_t ldw, void* out, int64_t ldo,
+                                 int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
+                                 int epilogue, const void* bias, int bias_kind,
+                                 const float* sx, int64_t n_sx, const float* sw,
+                                 int64_t n_sw, const float* so, int64_t n_so,
+                                 int32_t zx, int32_t zw, int32_t zo, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  return qgemm_impl(variant, A, lda, W, ldw, out, ldo, M, N, K, tp_a, tp_b, epilogue, bias,
+                    bias_kind, sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo, workspace,
+                    workspace_bytes, nullptr, stream);
+}
+
+extern "C" int dq8_qgemm_fused(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
+                               void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int tp_a,
+                               int tp_b, int epilogue, const void* bias, int bias_kind,
+                               const float* sx, int64_t n_sx, const float* sw, int64_t n_sw,
+                               const float* so, int64_t n_so, int32_t zx, int32_t zw, int32_t zo,
+                               void* workspace, size_t workspace_bytes,
+                               const dq8_postops_t* post, void* stream) {
+  return qgemm_impl(-1, A, lda, W, ldw, out, ldo, M, N, K, tp_a, tp_b, epilogue, bias, bias_kind,
+                    sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo, workspace, workspace_bytes, post,
+                    stream);
+}
 
 extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
                          void* out, int64_t ldo, int64_t M, int64_t N, int64_t K,
@@ -756,7 +830,8 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
                  const int64_t w_sizes[4], const int32_t padding[4], const int32_t md[17],
                  void* out, const int64_t out_sizes[4], int epilogue, const void* bias,
                  int bias_kind, const float* sx, const float* sw, int64_t n_sw, const float* so,
-                 int32_t zo, void* workspace, size_t workspace_bytes, void* stream) {
+                 int32_t zo, void* workspace, size_t workspace_bytes, void* stream,
+                 const dq8_postops_t* post = nullptr) {
   clear_error();
   DQ8_REQUIRE(in_sizes && w_sizes && padding && md && out_sizes, "dq8_qconv2d: null descriptor");
   DQ8_REQUIRE(variant >= -1 && variant < kNumVariants, "dq8_qconv2d: unknown variant");
@@ -834,6 +909,11 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   const int es = elem_size(epilogue);
   e.vec_store = aligned(out, 4 * es) && (Co % 4 == 0);
   e.vec_store16 = aligned(out, 16) && (Co % 16 == 0);
+  if (int s = apply_postops("dq8_qconv2d", post, es == 1 && epilogue != DQ8_EPI_ACC_S32,
+                            requant != 0, 1, Co, &e))
+    return s;
+  DQ8_REQUIRE(!e.resid_kind || is_nhwc_ohwi(md) || e.ldr == Co,
+              "dq8_qconv2d: a fused residual has the layout of the output");
 
   const bool nhwc_ohwi = is_nhwc_ohwi(md);
   const bool auto_pick = variant == -1;
@@ -860,7 +940,9 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     Ci = Cip;
     Kg = Kh * Kw * Ci;
   }
-  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16);
+  const bool fused = e.table != nullptr || e.resid_kind != 0;
+  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16) &&
+                       (!fused || (es == 1 ? e.vec_store16 : e.vec_store));
   if (auto_pick && !fast_ok) variant = 0;
   if (variant != 0)
     DQ8_REQUIRE(fast_ok, "dq8_qconv2d: the MFMA variants need NHWC x OHWI, Ci % 16 == 0 and "
@@ -984,6 +1066,18 @@ extern "C" int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const
                               void* workspace, size_t workspace_bytes, void* stream) {
   return qconv2d_impl(-1, in, in_sizes, w, w_sizes, padding, metadata, out, out_sizes, epilogue,
                       bias, bias_kind, sx, sw, n_sw, so, zo, workspace, workspace_bytes, stream);
+}
+
+extern "C" int dq8_qconv2d_fused(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                                 const int64_t w_sizes[4], const int32_t padding[4],
+                                 const int32_t metadata[17], void* out,
+                                 const int64_t out_sizes[4], int epilogue, const void* bias,
+                                 int bias_kind, const float* sx, const float* sw, int64_t n_sw,
+                                 const float* so, int32_t zo, void* workspace,
+                                 size_t workspace_bytes, const dq8_postops_t* post, void* stream) {
+  return qconv2d_impl(-1, in, in_sizes, w, w_sizes, padding, metadata, out, out_sizes, epilogue,
+                      bias, bias_kind, sx, sw, n_sw, so, zo, workspace, workspace_bytes, stream,
+                      post);
 }
 
 extern "C" int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,

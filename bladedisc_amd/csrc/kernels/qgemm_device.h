@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <utility>
 
 #include "disc_q8.h"
 
@@ -51,6 +52,20 @@ struct EpiParams {
   // path -- (acc + bias) times a fixed-point multiplier and shift derived from
   // (sx sw[n]) / so, plus zo, clamped (see fixedpoint_one).
   int fixedpoint;
+  // ---- operators fused behind the quantized result q (all optional; see disc_q8.h,
+  // dq8_postops_t).  Residual: t = (float)(q - zo) * so[0] + r(m, n), then ReLU, then either
+  // the f32 value is the output or it is quantized again: sat8(rne(t / out_scale + out_zp)).
+  // Table: the int8 result indexes a 256-byte table.
+  const void* resid;         // [M, N], row stride ldr elements; f32 or int8
+  int64_t ldr;
+  int resid_kind;            // 0 none, 1 f32, 2 int8 with (resid_scale[0], resid_zp)
+  int resid_zp;
+  const float* resid_scale;
+  int relu;
+  int out_zp;
+  const float* out_scale;    // null: the residual form writes f32
+  const uint8_t* table;
+  int resid_vec;    // 1: residual rows may be read with aligned 16-byte loads
   int vec_store;    // 1: a group of 4 consecutive n may be stored as one 4/16-byte word
   int vec_store16;  // 1: int8 rows may be written with aligned 16-byte stores
 };
@@ -251,6 +266,48 @@ __device__ __forceinline__ float dequant_so(const EpiParams& p) {
   return p.requant ? p.so[0] : 0.0f;
 }
 
+// ---- fused operators behind the quantized result (scalar forms; the hot paths below do the
+// same arithmetic on vectors)
+__device__ __forceinline__ float resid_at(const EpiParams& p, int64_t off) {
+  if (p.resid_kind == 1) return ((const float*)p.resid)[off];
+  return (float)((int)((const int8_t*)p.resid)[off] - p.resid_zp) * p.resid_scale[0];
+}
+// t = y + r, ReLU (a NaN stays a NaN)
+__device__ __forceinline__ float resid_add(const EpiParams& p, float y, float r) {
+  float t = y + r;
+  if (p.relu) t = t < 0.0f ? 0.0f : t;
+  return t;
+}
+// mhlo_disc.quantize to int8, round half to even: the arithmetic of dq8_quantize
+__device__ __forceinline__ int quantize_s8(float t, float s, float z) {
+  float v = t / s;
+  v = v + z;
+  v = rintf(v);
+  v = fminf(fmaxf(v, -128.0f), 127.0f);
+  return (int)v;
+}
+// the int8 that leaves the kernel for the stage's int8 result q; `roff` is the element's
+// offset in the residual tensor
+__device__ __forceinline__ int finish_s8_at(const EpiParams& p, int q, int64_t roff) {
+  if (p.table) return (int)(int8_t)p.table[(uint8_t)q];
+  if (p.resid_kind) {
+    const float y = (float)(q - p.zo) * p.so[0];
+    return quantize_s8(resid_add(p, y, resid_at(p, roff)), p.out_scale[0], (float)p.out_zp);
+  }
+  return q;
+}
+__device__ __forceinline__ int finish_s8(const EpiParams& p, int q, int64_t m, int n) {
+  return finish_s8_at(p, q, m * p.ldr + n);
+}
+// the f32 that leaves the kernel for the dequantized stage result y
+__device__ __forceinline__ float finish_f32_at(const EpiParams& p, float y, int64_t roff) {
+  if (!p.resid_kind) return y;
+  return resid_add(p, y, resid_at(p, roff));
+}
+__device__ __forceinline__ float finish_f32(const EpiParams& p, float y, int64_t m, int n) {
+  return finish_f32_at(p, y, m * p.ldr + n);
+}
+
 // The four forms of the f32 epilogue.  Which one a launch runs is uniform over the kernel:
 // the loops over the accumulators are instantiated per form (dispatch_f32_form) so that no
 // per-element code tests it.
@@ -290,6 +347,18 @@ struct IntC {
   static constexpr int value = V;
 };
 
+// body(IntC<0>()), ..., body(IntC<N-1>()): a loop that is unrolled by construction, for code
+// that indexes registers (an index the compiler does not see as a constant sends the whole
+// array to scratch memory)
+template <typename Body, int... I>
+__device__ __forceinline__ void static_for_impl(Body&& body, std::integer_sequence<int, I...>) {
+  (body(IntC<I>()), ...);
+}
+template <int N, typename Body>
+__device__ __forceinline__ void static_for(Body&& body) {
+  static_for_impl(body, std::make_integer_sequence<int, N>());
+}
+
 // body(IntC<form>) for the launch's form
 template <typename Body>
 __device__ __forceinline__ void dispatch_f32_form(const EpiParams& p, Body&& body) {
@@ -320,6 +389,8 @@ __device__ __forceinline__ void store_group4(const EpiParams& p, int m, int n,
   if (EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU) {
     int8_t* out = (int8_t*)p.out;
     uint32_t w;
+    // (launches with fused operators never come here: without 16-byte aligned output rows
+    // they run on the generic kernel)
     if (EPI == DQ8_EPI_REQUANT_CPU && p.fixedpoint) {
       w = 0;
 #pragma unroll
@@ -391,7 +462,11 @@ __device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, i
 
 // Hook of mfma_epilogue: called once, after the int8 results have been computed into
 // registers and before the first of them is stored (the default does nothing).
+// kPostOps: whether the epilogue carries the code of the fused operators (residual, table) and
+// of the fixed-point output stage; a kernel that is short of registers leaves them out and is
+// not chosen for such launches.
 struct NoHook {
+  static constexpr bool kPostOps = true;
   __device__ __forceinline__ void operator()() const {}
 };
 
@@ -605,7 +680,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
   // (fixed-point output stage: the shifts, behind the pairs; that space is otherwise the
   // result staging of the 4-byte epilogues, which the stage does not use)
   int* cps = reinterpret_cast<int*>(smem + CP_BYTES);
-  const bool fixedpoint = EPI == DQ8_EPI_REQUANT_CPU && e.fixedpoint;
+  const bool fixedpoint = BeforeStores::kPostOps && EPI == DQ8_EPI_REQUANT_CPU && e.fixedpoint;
   if (early) {
 #pragma unroll
     for (int i = 0; i < (BN + NT - 1) / NT; ++i) {
@@ -623,6 +698,10 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
       if (fixedpoint) cps[t] = c.sh;
     }
   }
+  // (fused table lookup: the 256 bytes behind the shifts)
+  uint8_t* tab = reinterpret_cast<uint8_t*>(smem + CP_BYTES + BN * 4);
+  if (BeforeStores::kPostOps && e.table && tid < 64)
+    reinterpret_cast<uint32_t*>(tab)[tid] = reinterpret_cast<const uint32_t*>(e.table)[tid];
   __syncthreads();
   DQ8_TRACE_POINT(5);
   if (!active) return;
@@ -698,7 +777,60 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
           // swap(a, b): the upper half of a trades places with the lower half of b
           const auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
           const auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
-          const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+          v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+          if (BeforeStores::kPostOps && (e.table || e.resid_kind)) {
+            // operators fused behind the quantized result: the lane holds 16 consecutive
+            // channels of one row, which is also how it reads the residual
+            const int n = n_wave0 + j * 32 + 16 * (lane >> 5);
+            const int64_t m = m_wave0 + i * 32 + (lane & 31);
+            if (e.table) {
+              static_for<4>([&](auto dc) {
+                constexpr int d = decltype(dc)::value;
+                const uint32_t x = (uint32_t)v[d];
+                v[d] = (int)((uint32_t)tab[x & 0xff] | ((uint32_t)tab[(x >> 8) & 0xff] << 8) |
+                             ((uint32_t)tab[(x >> 16) & 0xff] << 16) | ((uint32_t)tab[x >> 24] << 24));
+              });
+            } else if (m < m_end && n < e.N) {
+              const float so_v = e.so[0], s2 = e.out_scale[0], z2 = (float)e.out_zp;
+              const bool whole = e.resid_vec && n + 15 < e.N;
+              const int64_t roff = m * e.ldr + n;
+              // the residual of the 16 channels, as f32 (channels past N: unused zeros)
+              v4f r[4];
+              if (whole && e.resid_kind == 1) {
+                const v4f* rp = reinterpret_cast<const v4f*>((const float*)e.resid + roff);
+                static_for<4>([&](auto dc) { r[decltype(dc)::value] = rp[decltype(dc)::value]; });
+              } else if (whole) {
+                const float rs = e.resid_scale[0];
+                const v4i rv = *reinterpret_cast<const v4i*>((const int8_t*)e.resid + roff);
+                static_for<4>([&](auto dc) {
+                  constexpr int d = decltype(dc)::value;
+                  static_for<4>([&](auto bc) {
+                    constexpr int b = decltype(bc)::value;
+                    r[d][b] = (float)((int)(int8_t)((uint32_t)rv[d] >> (8 * b)) - e.resid_zp) * rs;
+                  });
+                });
+              } else {
+                static_for<4>([&](auto dc) {
+                  constexpr int d = decltype(dc)::value;
+                  static_for<4>([&](auto bc) {
+                    constexpr int b = decltype(bc)::value;
+                    r[d][b] = n + 4 * d + b < e.N ? resid_at(e, roff + 4 * d + b) : 0.0f;
+                  });
+                });
+              }
+              static_for<4>([&](auto dc) {
+                constexpr int d = decltype(dc)::value;
+                uint32_t w2 = 0;
+                static_for<4>([&](auto bc) {
+                  constexpr int b = decltype(bc)::value;
+                  const int q = (int)(int8_t)((uint32_t)v[d] >> (8 * b));
+                  const float t = resid_add(e, (float)(q - e.zo) * so_v, r[d][b]);
+                  w2 |= ((uint32_t)quantize_s8(t, s2, z2) & 0xffu) << (8 * b);
+                });
+                v[d] = (int)w2;
+              });
+            }
+          }
           if (kHook)
             held[kHook ? i : 0][kHook ? j : 0] = v;
           else
@@ -758,10 +890,32 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
           const int row = it * 8 + (lane >> 3), chunk = lane & 7;
-          const v4i v = *reinterpret_cast<const v4i*>(stage + row * 128 + ((chunk ^ (row & 7)) << 4));
+          v4i v = *reinterpret_cast<const v4i*>(stage + row * 128 + ((chunk ^ (row & 7)) << 4));
           const int m = m_wave0 + i * 32 + row, n = n_wave0 + j * 32 + chunk * 4;
           if (m < m_end && n < e.N) {
             int32_t* dst = static_cast<int32_t*>(e.out) + (int64_t)m * e.ldo + n;
+            if (BeforeStores::kPostOps && EPI == DQ8_EPI_DEQUANT_F32 && e.resid_kind) {
+              // + residual (and ReLU) behind the dequantized result, read the way it is stored
+              if (e.resid_vec && n + 3 < e.N) {
+                float r[4];
+                if (e.resid_kind == 1) {
+                  const v4f rv = *reinterpret_cast<const v4f*>((const float*)e.resid + (int64_t)m * e.ldr + n);
+#pragma unroll
+                  for (int q = 0; q < 4; ++q) r[q] = rv[q];
+                } else {
+                  const float rs = e.resid_scale[0];
+                  const uint32_t rw = *reinterpret_cast<const uint32_t*>((const int8_t*)e.resid + (int64_t)m * e.ldr + n);
+#pragma unroll
+                  for (int q = 0; q < 4; ++q) r[q] = (float)((int)(int8_t)(rw >> (8 * q)) - e.resid_zp) * rs;
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] = __float_as_int(resid_add(e, __int_as_float(v[q]), r[q]));
+              } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                  if (n + q < e.N) v[q] = __float_as_int(finish_f32(e, __int_as_float(v[q]), m, n + q));
+              }
+            }
             if (n + 3 < e.N) {
               __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
             } else {

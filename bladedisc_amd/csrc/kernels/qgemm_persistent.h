@@ -39,6 +39,14 @@ __device__ __forceinline__ void panel_coords(int t, int tiles_m, int tiles_n, in
   tn = in_panel / rows;
 }
 
+// Hook of the persistent kernel's epilogue: wait until this wave's loads have landed.
+struct LoadsLanded {
+  static constexpr bool kPostOps = false;   // (no registers to spare for the fused operators)
+  __device__ __forceinline__ void operator()() const {
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  }
+};
+
 template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
 __global__ void __launch_bounds__(WM* WN * 64) qgemm_persist_kernel(const MainParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -63,7 +71,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_persist_kernel(const MainPa
   // Per-channel factors: in stage 0 behind the result staging of the 4-byte epilogues when
   // there is room (stage 0 holds no operands between the end of a main loop and the barrier
   // at the top of the next tile), else behind the two stages.
-  constexpr int kCpInStage0 = NW * 4096 + BN * 8 <= STAGE;
+  constexpr int kCpInStage0 = NW * 4096 + BN * 12 + 256 <= STAGE;
   extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
   int8_t* const cp_smem = smem + (kCpInStage0 ? NW * 4096 : 2 * STAGE);
 
@@ -328,11 +336,6 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_persist_kernel(const MainPa
     // (they have had the whole requantisation to do so), then stores: the wait at the top of
     // the next tile therefore finds only stores in flight and does not wait for them (loads
     // and stores share the one counter).
-    struct LoadsLanded {
-      __device__ __forceinline__ void operator()() const {
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-      }
-    };
     mfma_epilogue<EPI, FM, FN, NT, BN, LoadsLanded>(acc, p.epi, cp_smem, m0e + wm * TM,
                                                     n0e + wn * TN, n0e, early.c, wave, true, -1,
                                                     smem, LoadsLanded());

@@ -82,9 +82,9 @@ __global__ void __launch_bounds__(NW * 64) qgemm_skinny_kernel(const MainParams 
     if (EPI == DQ8_EPI_ACC_S32)
       ((int32_t*)ep.out)[off] = sum;
     else if (EPI == DQ8_EPI_DEQUANT_F32)
-      ((float*)ep.out)[off] = dequant_one_any(ep, c, sum, dequant_so(ep));
+      ((float*)ep.out)[off] = finish_f32(ep, dequant_one_any(ep, c, sum, dequant_so(ep)), m, n);
     else
-      ((int8_t*)ep.out)[off] = (int8_t)requant_one<EPI>(ep, c, sum);
+      ((int8_t*)ep.out)[off] = (int8_t)finish_s8(ep, requant_one<EPI>(ep, c, sum), m, n);
   }
 }
 

@@ -160,8 +160,40 @@ def dequantize(q, scale, zero_point, axis=None, out=None):
     return out
 
 
+def make_postops(residual=None, residual_scale=None, residual_zp=0, relu=False, out_scale=None,
+                 out_zp=0, table=None):
+    """dq8_postops_t for the operators fused behind a quantized GEMM / convolution; returns
+    (struct, objects to keep alive).  residual: f32 or int8 device tensor of the output's
+    shape (int8: with residual_scale, a one-element device tensor, and residual_zp);
+    out_scale: one-element device tensor of the quantize that follows (int8 results);
+    table: 256-entry int8 / uint8 device tensor."""
+    po = _lib.PostOps()
+    keep = []
+    if residual is not None:
+        if residual.stride(-1) != 1:
+            residual = residual.contiguous()
+        r2 = residual.reshape(-1, residual.shape[-1]) if residual.is_contiguous() else residual
+        po.residual = r2.data_ptr()
+        po.residual_kind = 1 if residual.dtype == torch.float32 else 2
+        po.ldr = r2.stride(0)
+        keep.append(r2)
+        if residual_scale is not None:
+            po.residual_scale = residual_scale.data_ptr()
+            keep.append(residual_scale)
+        po.residual_zp = int(residual_zp)
+    po.relu = int(bool(relu))
+    if out_scale is not None:
+        po.out_scale = out_scale.data_ptr()
+        keep.append(out_scale)
+    po.out_zp = int(out_zp)
+    if table is not None:
+        po.table = table.data_ptr()
+        keep.append(table)
+    return po, keep
+
+
 def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b=True,
-          zx=0, zw=0, zo=0, variant=-1, out=None):
+          zx=0, zw=0, zo=0, variant=-1, out=None, post=None):
     """int8 GEMM with a fused epilogue.  a: [M,K] ([K,M] if tp_a); w: [N,K] if tp_b
     else [K,N]; scales are device f32 tensors with 1 or N entries."""
     _need_cuda(a, w, bias)
@@ -188,14 +220,20 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
     ws_bytes = (L.dq8_qgemm_workspace_bytes_zp(m, n, k, int(tp_a), int(tp_b), zx, zw)
                 if variant == -1 else L.dq8_qgemm_workspace_bytes(m, n, k, int(tp_a), int(tp_b)))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-    st = L.dq8_qgemm_variant(
-        variant, _ptr(a), max(a.stride(0), a.shape[1]), _ptr(w), max(w.stride(0), w.shape[1]),
-        _ptr(out), out.stride(0) if m else n,
-        m, n, k, int(tp_a), int(tp_b), epilogue, _ptr(bias), bias_kind,
-        _ptr(sx), sx.numel() if sx is not None else 0,
-        _ptr(sw), sw.numel() if sw is not None else 0,
-        _ptr(so), so.numel() if so is not None else 0,
-        zx, zw, zo, _ptr(ws), ws_bytes, _stream())
+    args = (_ptr(a), max(a.stride(0), a.shape[1]), _ptr(w), max(w.stride(0), w.shape[1]),
+            _ptr(out), out.stride(0) if m else n,
+            m, n, k, int(tp_a), int(tp_b), epilogue, _ptr(bias), bias_kind,
+            _ptr(sx), sx.numel() if sx is not None else 0,
+            _ptr(sw), sw.numel() if sw is not None else 0,
+            _ptr(so), so.numel() if so is not None else 0,
+            zx, zw, zo, _ptr(ws), ws_bytes)
+    if post is not None:
+        if variant != -1:
+            raise ValueError("fused operators go with the library's own choice of kernel")
+        po, keep = post if isinstance(post, tuple) else (post, None)
+        st = L.dq8_qgemm_fused(*args, C.byref(po), _stream())
+    else:
+        st = L.dq8_qgemm_variant(variant, *args, _stream())
     _lib.check(st, "dq8_qgemm")
     return out
 
@@ -204,7 +242,7 @@ NHWC_OHWI = (0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2)
 
 
 def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=None,
-            bias=None, zo=0, variant=-1, out=None, workspace=True):
+            bias=None, zo=0, variant=-1, out=None, workspace=True, post=None):
     """int8 convolution; layouts/strides/dilations from the 17-entry ral_qconv
     metadata, padding = (top, bottom, left, right).  workspace=False withholds the scratch
     that keeps channel counts off a multiple of 16 on the MFMA kernels."""
@@ -223,11 +261,17 @@ def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=N
     md = (C.c_int32 * 17)(*metadata)
     ws_bytes = L.dq8_qconv2d_workspace_bytes(i64x4(*x.shape), i64x4(*w.shape), md) if workspace else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-    st = L.dq8_qconv2d_variant(
-        variant, _ptr(x), i64x4(*x.shape), _ptr(w), i64x4(*w.shape),
-        (C.c_int32 * 4)(*padding), md, _ptr(out),
-        i64x4(*out_shape), epilogue, _ptr(bias), bias_kind, _ptr(sx), _ptr(sw),
-        sw.numel() if sw is not None else 0, _ptr(so), zo, _ptr(ws), ws_bytes, _stream())
+    args = (_ptr(x), i64x4(*x.shape), _ptr(w), i64x4(*w.shape),
+            (C.c_int32 * 4)(*padding), md, _ptr(out),
+            i64x4(*out_shape), epilogue, _ptr(bias), bias_kind, _ptr(sx), _ptr(sw),
+            sw.numel() if sw is not None else 0, _ptr(so), zo, _ptr(ws), ws_bytes)
+    if post is not None:
+        if variant != -1:
+            raise ValueError("fused operators go with the library's own choice of kernel")
+        po, keep = post if isinstance(post, tuple) else (post, None)
+        st = L.dq8_qconv2d_fused(*args, C.byref(po), _stream())
+    else:
+        st = L.dq8_qconv2d_variant(variant, *args, _stream())
     _lib.check(st, "dq8_qconv2d")
     return out
 

@@ -239,6 +239,45 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
               const float* so, int64_t n_so, int32_t zx, int32_t zw, int32_t zo,
               void* workspace, size_t workspace_bytes, void* stream);
 
+/* Operators the compiler fuses behind a quantized GEMM or convolution (its elementwise
+ * fusion around quantized_dot_general / quantized_conv, next to the graph rewrites of
+ * R disc/transforms/disc_quantized_dot_merge.cc:155-456): done in the producing kernel's
+ * epilogue, bit for bit what the separate operators give.  With q the int8 result of the
+ * requantisation stage (output scale so[0], zero point zo):
+ *   table     out = table[(uint8_t) q]: any dequantize -> activation -> quantize chain
+ *             (256 device bytes, as for dq8_lut8); int8 out, no residual
+ *   residual  t = (float)(q - zo) * so[0] + r(m, n)        [dq8_dequantize, then an f32 add]
+ *             r = residual[m, n] (DQ8_RESIDUAL_F32) or
+ *                 (float)(residual[m, n] - residual_zp) * residual_scale[0] (DQ8_RESIDUAL_S8)
+ *             relu: t = t < 0 ? 0 : t
+ *             out_scale given: out = sat8(rne(t / out_scale[0] + out_zp))   [dq8_quantize]
+ *             (epilogues REQUANT_CPU / REQUANT_GPU / REQUANT_FIXEDPOINT, int8 out);
+ *             out_scale NULL: out = t (epilogues REQUANT_*_DEQUANT_F32, f32 out)
+ * The residual is [M, N] with row stride ldr elements (a convolution's: the layout of its
+ * output).  Scales are device pointers. */
+#define DQ8_RESIDUAL_NONE 0
+#define DQ8_RESIDUAL_F32 1
+#define DQ8_RESIDUAL_S8 2
+typedef struct dq8_postops {
+  const void* residual;
+  int residual_kind;
+  int64_t ldr;
+  const float* residual_scale;
+  int32_t residual_zp;
+  int relu;
+  const float* out_scale;
+  int32_t out_zp;
+  const void* table;
+} dq8_postops_t;
+
+/* dq8_qgemm with operators fused behind it (post may be NULL: then it is dq8_qgemm). */
+int dq8_qgemm_fused(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, void* out,
+                    int64_t ldo, int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
+                    int epilogue, const void* bias, int bias_kind, const float* sx,
+                    int64_t n_sx, const float* sw, int64_t n_sw, const float* so, int64_t n_so,
+                    int32_t zx, int32_t zw, int32_t zo, void* workspace, size_t workspace_bytes,
+                    const dq8_postops_t* post, void* stream);
+
 /* dst[c, r] = src[r, c] for an int8 matrix src [rows, cols] with row stride ld;
  * dst is dense [cols, rows].  Used to put [K,N] weights into the kernels' [N,K]
  * layout once (the reference's counterpart is oneDNN's weight pre-packing,
@@ -273,6 +312,15 @@ int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                    int epilogue, const void* bias, int bias_kind, const float* sx,
                    const float* sw, int64_t n_sw, const float* so, int32_t zo,
                    void* workspace, size_t workspace_bytes, void* stream);
+/* dq8_qconv2d_ws with operators fused behind it (post may be NULL). */
+int dq8_qconv2d_fused(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
+                      const int64_t w_sizes[4], const int32_t padding[4],
+                      const int32_t metadata[17], void* out, const int64_t out_sizes[4],
+                      int epilogue, const void* bias, int bias_kind, const float* sx,
+                      const float* sw, int64_t n_sw, const float* so, int32_t zo,
+                      void* workspace, size_t workspace_bytes, const dq8_postops_t* post,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -158,6 +158,13 @@ def test_qgemm_requant_fixedpoint(K, m, n, k, bias):
     for swv, sov, zo in cases:
         want = O.requant_fixedpoint(acc, sx, swv, sov, b32=b32, zo=zo)
         for v in [-1] + gemm_variants(K, k):
+            if K.variant_names()[v].startswith("persist_") and v >= 0:
+                # (the persistent kernels leave this stage out and say so when forced)
+                with pytest.raises(RuntimeError, match="persistent"):
+                    K.qgemm(dev(a), dev(w), K.EPI_REQUANT_FIXEDPOINT, sx=dev(np.array([sx])),
+                            sw=dev(swv), so=dev(np.array([sov], np.float32)), bias=bias_t, zo=zo,
+                            variant=v)
+                continue
             got = host(K.qgemm(dev(a), dev(w), K.EPI_REQUANT_FIXEDPOINT, sx=dev(np.array([sx])),
                                sw=dev(swv), so=dev(np.array([sov], np.float32)), bias=bias_t, zo=zo,
                                variant=v))
@@ -168,6 +175,73 @@ def test_qgemm_requant_fixedpoint(K, m, n, k, bias):
     # it is a different rounding from the float stage, not the same numbers by another route
     other = O.requant_cpu(acc, sx, sw, so, b32=b32)
     assert np.max(np.abs(other.astype(np.int32) - want.astype(np.int32))) <= 1
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 768, 768), (1000, 768, 3072), (257, 132, 64), (5, 16, 48),
+                                   (4096, 768, 768), (3072, 3072, 768), (300, 260, 96)])
+def test_qgemm_fused_operators_equal_the_separate_ones(K, m, n, k):
+    """Operators fused behind a quantized GEMM -- dequantize -> +residual (f32 or int8) ->
+    ReLU -> quantize, dequantize -> +residual -> f32, and a 256-entry table on the int8
+    result -- give the bits of the chain of separate library calls (qgemm, dq8_dequantize, an
+    f32 add, a clamp at zero, dq8_quantize, dq8_lut8), for every epilogue family."""
+    rng = np.random.default_rng(11 * m + n + k)
+    a = dev(rng.integers(-128, 128, (m, k), dtype=np.int8))
+    w = dev(rng.integers(-128, 128, (n, k), dtype=np.int8))
+    acc, _ = O.gemm_s32_fast(host(a), host(w))
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    dsx, dsw, dso = dev(np.array([sx])), dev(sw), dev(np.array([so], np.float32))
+    bias = dev((rng.standard_normal(n) * 10 * so).astype(np.float32))
+    b32 = dev(rng.integers(-100000, 100000, n).astype(np.int32))
+    rf = dev((rng.standard_normal((m, n)) * 40 * so).astype(np.float32))
+    rq = dev(rng.integers(-128, 128, (m, n), dtype=np.int8))
+    rs, rz = dev(np.array([so * 1.7], np.float32)), 4
+    s2, z2 = dev(np.array([so * 1.3], np.float32)), -7
+    zero = torch.zeros(1, dtype=torch.int32, device="cuda")
+    table = dev(rng.integers(-128, 128, 256, dtype=np.int8))
+
+    def unfused(q, zo, resid, relu, requant):
+        y = K.dequantize(q, dso, torch.full((1,), zo, dtype=torch.int32, device="cuda"))
+        r = resid if resid.dtype == torch.float32 else \
+            K.dequantize(resid, rs, torch.full((1,), rz, dtype=torch.int32, device="cuda"))
+        t = y + r
+        if relu:
+            t = torch.where(t < 0, torch.zeros_like(t), t)
+        if not requant:
+            return t
+        return K.quantize(t, s2, torch.full((1,), z2, dtype=torch.int32, device="cuda"))
+
+    stages = [(K.EPI_REQUANT_CPU, K.EPI_REQUANT_CPU_DEQUANT_F32, bias, 3),
+              (K.EPI_REQUANT_GPU, K.EPI_REQUANT_GPU_DEQUANT_F32, bias, 0),
+              (K.EPI_REQUANT_FIXEDPOINT, None, b32, -2)]
+    for epi, epi_f32, b, zo in stages:
+        q = K.qgemm(a, w, epi, sx=dsx, sw=dsw, so=dso, bias=b, zo=zo)
+        for resid in (rf, rq):
+            for relu in (False, True):
+                kw = dict(residual=resid, relu=relu)
+                if resid.dtype == torch.int8:
+                    kw.update(residual_scale=rs, residual_zp=rz)
+                got = K.qgemm(a, w, epi, sx=dsx, sw=dsw, so=dso, bias=b, zo=zo,
+                              post=K.make_postops(out_scale=s2, out_zp=z2, **kw))
+                assert torch.equal(got, unfused(q, zo, resid, relu, True)), (epi, resid.dtype, relu)
+                if epi_f32 is not None:
+                    got = K.qgemm(a, w, epi_f32, sx=dsx, sw=dsw, so=dso, bias=b, zo=zo,
+                                  post=K.make_postops(**kw))
+                    want = unfused(q, zo, resid, relu, False)
+                    assert torch.equal(got.view(torch.int32), want.view(torch.int32)), \
+                        (epi_f32, resid.dtype, relu)
+        got = K.qgemm(a, w, epi, sx=dsx, sw=dsw, so=dso, bias=b, zo=zo,
+                      post=K.make_postops(table=table))
+        assert torch.equal(got, K.lut8(q, table)), epi
+    # what the API refuses
+    with pytest.raises(RuntimeError, match="out_scale"):
+        K.qgemm(a, w, K.EPI_REQUANT_CPU, sx=dsx, sw=dsw, so=dso, post=K.make_postops(residual=rf))
+    with pytest.raises(RuntimeError, match="requantising"):
+        K.qgemm(a, w, K.EPI_ACC_S32, post=K.make_postops(table=table))
+    with pytest.raises(RuntimeError, match="no residual"):
+        K.qgemm(a, w, K.EPI_REQUANT_CPU, sx=dsx, sw=dsw, so=dso,
+                post=K.make_postops(table=table, residual=rf, out_scale=s2))
+    assert zero.item() == 0
 
 
 @pytest.mark.parametrize("per_channel", [False, True])
