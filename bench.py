@@ -341,61 +341,41 @@ def config_reports(torch, K):
             layer.forward(h)
         torch.cuda.synchronize()
         eager_us = (time.perf_counter() - t0) / 10 * 1e6
-        # the same layer replayed from a HIP graph
-        graph_us = None
-        try:
-            replay, _, _ = layer.capture(h)
-            for _ in range(3):
-                replay()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(20):
-                replay()
-            torch.cuda.synchronize()
-            graph_us = round((time.perf_counter() - t0) / 20 * 1e6, 1)
-        except Exception as exc:  # capture is an optimisation, not the path under test
-            graph_us = "capture failed: %s" % str(exc)[:100]
-        # the same with dequantize -> GELU -> quantize between the FFN linears run as one
-        # 256-entry table lookup on the int8 tensor (bit-identical output)
-        fused_us = None
-        try:
-            layer.fuse_gelu = True
-            replay, _, _ = layer.capture(h)
-            for _ in range(3):
-                replay()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(20):
-                replay()
-            torch.cuda.synchronize()
-            fused_us = round((time.perf_counter() - t0) / 20 * 1e6, 1)
-        except Exception as exc:
-            fused_us = "capture failed: %s" % str(exc)[:100]
-        finally:
-            layer.fuse_gelu = False
-        # ... and with each trailing dequantize done in its GEMM's epilogue as well
-        try:
-            layer.fuse_gelu = layer.fuse_dequant = True
-            replay, _, _ = layer.capture(h)
-            for _ in range(3):
-                replay()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(20):
-                replay()
-            torch.cuda.synchronize()
-            fused2_us = round((time.perf_counter() - t0) / 20 * 1e6, 1)
-        except Exception as exc:
-            fused2_us = "capture failed: %s" % str(exc)[:100]
-        finally:
-            layer.fuse_gelu = layer.fuse_dequant = False
+        # the same layer replayed from a HIP graph: as separate operators; with dequantize ->
+        # GELU -> quantize between the FFN linears as one 256-entry table lookup on the int8
+        # tensor; with each trailing dequantize done in its GEMM's epilogue as well; and with
+        # the table and both residual additions in the epilogues too (all bit-identical)
+        def replay_us(**flags):
+            saved = {k: getattr(layer, k) for k in flags}
+            try:
+                for k, v in flags.items():
+                    setattr(layer, k, v)
+                replay, _, _ = layer.capture(h)
+                for _ in range(3):
+                    replay()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    replay()
+                torch.cuda.synchronize()
+                return round((time.perf_counter() - t0) / 20 * 1e6, 1)
+            except Exception as exc:  # capture is an optimisation, not the path under test
+                return "capture failed: %s" % str(exc)[:100]
+            finally:
+                for k, v in saved.items():
+                    setattr(layer, k, v)
+        graph_us = replay_us()
+        fused_us = replay_us(fuse_gelu=True)
+        fused2_us = replay_us(fuse_gelu=True, fuse_dequant=True)
+        fused3_us = replay_us(fuse_gelu=True, fuse_dequant=True, fuse_epilogue=True)
         bert["seq%d" % seq] = {"linears_q_gemm_dq": per,
                                "quantized_ops_gpu_us": round(gpu_sum * 1e6, 2),
                                "quantized_ops_cpu_us": round(cpu_sum * 1e6, 1),
                                "layer_eager_wall_us": round(eager_us, 1),
                                "layer_graph_replay_us": graph_us,
                                "layer_graph_replay_fused_gelu_table_us": fused_us,
-                               "layer_graph_replay_fused_gelu_table_and_dequantize_us": fused2_us}
+                               "layer_graph_replay_fused_gelu_table_and_dequantize_us": fused2_us,
+                               "layer_graph_replay_fused_epilogues_us": fused3_us}
     rep["5_bert_base_layer_batch8"] = bert
     return rep
 

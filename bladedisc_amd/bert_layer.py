@@ -45,6 +45,18 @@ class RawBackend:
         """qlinear followed by dequantize(., so), in the GEMM's epilogue: f32 out."""
         return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU_DEQUANT_F32, sx=sx, sw=sw, so=so, bias=bias)
 
+    def qlinear_table(self, x_q, w_q, bias, sx, sw, so, table):
+        """qlinear followed by a 256-entry table lookup on its int8 result, in the epilogue."""
+        post = K.make_postops(table=table)
+        return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so, bias=bias, post=post)
+
+    def qlinear_dequantized_residual(self, x_q, w_q, bias, sx, sw, so, residual):
+        """qlinear, dequantize(., so) and the addition of an f32 tensor of the result's
+        shape, in the epilogue: f32 out."""
+        post = K.make_postops(residual=residual)
+        return K.qgemm(x_q, w_q, K.EPI_REQUANT_CPU_DEQUANT_F32, sx=sx, sw=sw, so=so, bias=bias,
+                       post=post)
+
     def lut8(self, q, table):
         return K.lut8(q, table)
 
@@ -80,15 +92,19 @@ class QuantBertLayer:
     """One encoder layer; hidden 768, 12 heads, FFN 3072 by default."""
 
     def __init__(self, weights, backend, heads=12, device="cuda", fuse_gelu=False,
-                 fuse_dequant=False):
+                 fuse_dequant=False, fuse_epilogue=False):
         """fuse_dequant (raw backend): a linear whose int8 result is only dequantized writes
         the dequantized f32 from the GEMM's epilogue (same bits, no int8 round trip).
         fuse_gelu: run dequantize -> GELU -> quantize between the two FFN linears as one
         256-entry table lookup on the int8 tensor (what the compiler's fusion of those three
         elementwise operators amounts to); the result is bit-identical to the three separate
-        operators because the table is built by running exactly them on all 256 inputs."""
-        self.fuse_gelu = fuse_gelu
-        self.fuse_dequant = fuse_dequant
+        operators because the table is built by running exactly them on all 256 inputs.
+        fuse_epilogue (raw backend): the operators behind three of the linears run in the
+        GEMM's epilogue -- the residual additions behind the attention output and FFN2
+        (dequantize + add, f32 out) and the GELU table behind FFN1 -- again the same bits."""
+        self.fuse_gelu = fuse_gelu or fuse_epilogue
+        self.fuse_dequant = fuse_dequant or fuse_epilogue
+        self.fuse_epilogue = fuse_epilogue
         self.gelu_table = None
         self.be = backend
         self.heads = heads
@@ -178,11 +194,37 @@ class QuantBertLayer:
             rec[name] = dict(x=x2, x_q=x_q, y_q=y_q, y=y)
         return y.reshape(*shape[:-1], y.shape[-1])
 
+    def _qlinear_residual(self, name, x, residual, rec):
+        """residual + dequantize(linear(quantize(x))) with everything behind the GEMM fused."""
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        x_q = self.be.quantize(x2, self.s_in[name])
+        r2 = residual.reshape(-1, residual.shape[-1])
+        y = self.be.qlinear_dequantized_residual(x_q, self.w_q[name], self.bias[name],
+                                                 self.s_in[name], self.sw[name],
+                                                 self.s_out[name], r2)
+        if rec is not None:
+            rec[name] = dict(x=x2, x_q=x_q, y_plus_residual=y)
+        return y.reshape(*shape[:-1], y.shape[-1])
+
     def _ffn_fused(self, h1, rec):
         """quantize -> ffn1 -> [table: dequantize, GELU, quantize] -> ffn2 -> dequantize."""
         shape = h1.shape
         x2 = h1.reshape(-1, shape[-1])
         x_q = self.be.quantize(x2, self.s_in["ffn1"])
+        if self.fuse_epilogue:
+            y1_q = None
+            x2_q = self.be.qlinear_table(x_q, self.w_q["ffn1"], self.bias["ffn1"],
+                                         self.s_in["ffn1"], self.sw["ffn1"],
+                                         self.s_out["ffn1"], self.gelu_table)
+            r2 = x2
+            y2 = self.be.qlinear_dequantized_residual(
+                x2_q, self.w_q["ffn2"], self.bias["ffn2"], self.s_in["ffn2"], self.sw["ffn2"],
+                self.s_out["ffn2"], r2)
+            if rec is not None:
+                rec["ffn1"] = dict(x=x2, x_q=x_q)
+                rec["ffn2"] = dict(x_q=x2_q, y_plus_residual=y2)
+            return y2.reshape(*shape[:-1], y2.shape[-1])
         y1_q = self._gemm("ffn1", x_q)
         x2_q = self.be.lut8(y1_q, self.gelu_table)
         y2_q, y2 = self._gemm_dequantized("ffn2", x2_q)
@@ -217,6 +259,13 @@ class QuantBertLayer:
             raise RuntimeError("calibrate() first")
         qkv = self._qlinear("qkv", h, record)
         ctx = self.attention(qkv)
+        if self.fuse_epilogue:
+            if not isinstance(self.be, RawBackend):
+                raise RuntimeError("fused epilogues need the raw backend")
+            pre1 = self._qlinear_residual("out", ctx, h, record)
+            h1 = _layer_norm(pre1, self.f["ln1_g"], self.f["ln1_b"])
+            pre2 = self._ffn_fused(h1, record)       # h1 + ffn2(gelu(ffn1(h1)))
+            return _layer_norm(pre2, self.f["ln2_g"], self.f["ln2_b"])
         attn = self._qlinear("out", ctx, record)
         h1 = _layer_norm(h + attn, self.f["ln1_g"], self.f["ln1_b"])
         if self.fuse_gelu:

@@ -920,8 +920,12 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   // Channel counts that are not a multiple of 16 (an RGB first layer): with scratch, input
   // and weights are rewritten with the channels zero-filled up to the next multiple; the
   // added channels contribute nothing and the MFMA kernels run on the padded tensors.
+  // (fused operators with an output the 16-byte stores cannot take run on the generic kernel,
+  // which reads the tensors as they were passed)
+  const bool fused = e.table != nullptr || e.resid_kind != 0;
+  const bool fused_ok = !fused || (es == 1 ? e.vec_store16 : e.vec_store);
   const int64_t Cip = (Ci + 15) / 16 * 16;
-  if (nhwc_ohwi && Ci % 16 != 0 && variant != 0 && workspace != nullptr &&
+  if (nhwc_ohwi && Ci % 16 != 0 && variant != 0 && fused_ok && workspace != nullptr &&
       aligned(workspace, 256) &&
       workspace_bytes >= pad256(NB * H * Wd * Cip) + pad256(Co * Kh * Kw * Cip) &&
       NB * H * Wd * Cip < (1LL << 40) && Kh * Kw * Cip < (1LL << 31)) {
@@ -940,9 +944,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     Ci = Cip;
     Kg = Kh * Kw * Ci;
   }
-  const bool fused = e.table != nullptr || e.resid_kind != 0;
-  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16) &&
-                       (!fused || (es == 1 ? e.vec_store16 : e.vec_store));
+  const bool fast_ok = nhwc_ohwi && Ci % 16 == 0 && aligned(in, 16) && aligned(w, 16) && fused_ok;
   if (auto_pick && !fast_ok) variant = 0;
   if (variant != 0)
     DQ8_REQUIRE(fast_ok, "dq8_qconv2d: the MFMA variants need NHWC x OHWI, Ci % 16 == 0 and "

@@ -221,14 +221,36 @@ def test_config5_bert_layer_dequantize_in_the_gemm_epilogue_is_bit_identical(C, 
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
 
 
-@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("seq", [32, 384])
+def test_config5_bert_layer_operators_in_the_gemm_epilogues_are_bit_identical(C, seq):
+    """The residual additions behind the attention output and FFN2 and the GELU table behind
+    FFN1 run in the producing GEMM's epilogue: the int8 input of FFN2, the two pre-LayerNorm
+    sums and the layer output keep their bits."""
+    from bladedisc_amd import bert_layer as B
+    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend())
+    h = layer.embed(C.config5_tokens(8, seq))
+    layer.calibrate(h)
+    rec_a, rec_b = {}, {}
+    want = layer.forward(h, rec_a)
+    layer.fuse_epilogue = layer.fuse_gelu = layer.fuse_dequant = True
+    got = layer.forward(h, rec_b)
+    torch.cuda.synchronize()
+    assert torch.equal(rec_b["ffn2"]["x_q"], rec_a["ffn2"]["x_q"])
+    pre1 = h.reshape(-1, h.shape[-1]) + rec_a["out"]["y"]
+    assert torch.equal(rec_b["out"]["y_plus_residual"].view(torch.int32), pre1.view(torch.int32))
+    pre2 = rec_a["ffn1"]["x"] + rec_a["ffn2"]["y"]
+    assert torch.equal(rec_b["ffn2"]["y_plus_residual"].view(torch.int32), pre2.view(torch.int32))
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+
+
+@pytest.mark.parametrize("fused", [False, True, "epilogue"])
 def test_config5_bert_layer_graph_replays_match_eager(C, fused):
     """The captured layer against eager execution: several replays, with eager work and
     synchronisations in between, each compared bit for bit; also with the GELU table and the
     dequantize-in-epilogue forms switched on."""
     from bladedisc_amd import bert_layer as B
-    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend(), fuse_gelu=fused,
-                             fuse_dequant=fused)
+    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend(), fuse_gelu=bool(fused),
+                             fuse_dequant=bool(fused), fuse_epilogue=fused == "epilogue")
     h0 = layer.embed(C.config5_tokens(8, 32))
     layer.calibrate(h0)
     replay, static_in, static_out = layer.capture(h0)

@@ -692,6 +692,46 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
         assert np.array_equal(got.view(np.uint32), want_f.view(np.uint32)), "variant %d" % v
 
 
+@pytest.mark.parametrize("nb,h,w_,ci,co,k,pad", [(2, 14, 14, 64, 256, 1, 0), (1, 28, 28, 128, 128, 3, 1),
+                                                 (2, 9, 11, 48, 72, 3, 1), (1, 7, 7, 24, 40, 1, 0)])
+def test_qconv_fused_residual_relu_quantize(K, nb, h, w_, ci, co, k, pad):
+    """The tail of a ResNet block in the convolution's epilogue: dequantize -> + the block's
+    int8 input (its own scale and zero point) -> ReLU -> quantize gives the bits of the
+    separate library calls; so does an f32 residual with an f32 result, and a table."""
+    rng = np.random.default_rng(h * 31 + ci + co)
+    x = dev(rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8))
+    wt = dev(rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8))
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    padding = [pad] * 4
+    out_shape = [nb, h, w_, co]
+    acc = O.conv_s32(host(x), host(wt), padding, md, out_shape)
+    sx, sw = make_scales(rng, co)
+    so = pick_so(acc, sx, sw)
+    sc = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so], np.float32)))
+    bias = dev((rng.standard_normal(co) * 10 * so).astype(np.float32))
+    q = K.qconv2d(x, wt, padding, md, out_shape, K.EPI_REQUANT_CPU, bias=bias, zo=2, **sc)
+    zi = lambda v: torch.full((1,), v, dtype=torch.int32, device="cuda")  # noqa: E731
+    y = K.dequantize(q, sc["so"], zi(2))
+    rq = dev(rng.integers(-128, 128, out_shape, dtype=np.int8))
+    rs, rz = dev(np.array([so * 0.8], np.float32)), -5
+    s2, z2 = dev(np.array([so * 1.1], np.float32)), -128
+    t = y + K.dequantize(rq, rs, zi(rz))
+    t = torch.where(t < 0, torch.zeros_like(t), t)
+    want = K.quantize(t, s2, zi(z2))
+    got = K.qconv2d(x, wt, padding, md, out_shape, K.EPI_REQUANT_CPU, bias=bias, zo=2, **sc,
+                    post=K.make_postops(residual=rq, residual_scale=rs, residual_zp=rz,
+                                        relu=True, out_scale=s2, out_zp=z2))
+    assert torch.equal(got, want)
+    rf = dev((rng.standard_normal(out_shape) * 40 * so).astype(np.float32))
+    got = K.qconv2d(x, wt, padding, md, out_shape, K.EPI_REQUANT_CPU_DEQUANT_F32, bias=bias, zo=2,
+                    **sc, post=K.make_postops(residual=rf))
+    assert torch.equal(got.view(torch.int32), (y + rf).view(torch.int32))
+    table = dev(rng.integers(-128, 128, 256, dtype=np.int8))
+    got = K.qconv2d(x, wt, padding, md, out_shape, K.EPI_REQUANT_CPU, bias=bias, zo=2, **sc,
+                    post=K.make_postops(table=table))
+    assert torch.equal(got, K.lut8(q, table))
+
+
 def test_qconv_direct_random_shapes(K):
     """Seeded sweep for the kernels that keep the input patch in LDS: image sizes that make
     tiles start and end anywhere in a row, every channel count, ragged output channels,
