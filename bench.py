@@ -34,11 +34,19 @@ MEASURED_TRAFFIC_BYTES = {4096: (98660 + 16384) * 1024}
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    # After idling the GPU needs about 20 ms of load before its clocks settle (the first
-    # 300 launches of this 60 us kernel run 5-15 % slow), hence the long default warm-up.
+    # After idling the GPU needs some tens of milliseconds of load before its clocks settle
+    # (the first 300 launches of this 60 us kernel run 5-15 % slow): --prewarm-ms of the
+    # same kernel run before the warm-up steps, untimed and reported separately.
     p.add_argument("--steps", type=int, default=400)
-    p.add_argument("--warmup", type=int, default=400)
+    p.add_argument("--warmup", type=int, default=50)
+    p.add_argument("--prewarm-ms", type=float, default=50.0,
+                   help="milliseconds of GPU time of the headline kernel before the warm-up "
+                        "steps (0: none)")
     p.add_argument("--size", type=int, default=4096, help="M = N = K of the headline GEMM")
+    p.add_argument("--workload", default="headline",
+                   help="'headline' (default), or one parity-test configuration on its own, "
+                        "e.g. for a profiler: 'gemm:MxKxN' (dynamic-M sweep shape, requant to "
+                        "int8) or 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS)")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extra", action="store_true", help="skip the extras")
     p.add_argument("--no-two-stream", action="store_true",
@@ -79,10 +87,25 @@ class GemmCall:
             raise RuntimeError(self.L.dq8_last_error().decode())
 
 
-def time_graph(torch, calls, launches=20, replays=10):
+class Timing(float):
+    """Seconds per pass: the median over the timed graph replays (the float itself), with
+    the fastest replay kept beside it."""
+
+    def __new__(cls, median, fastest):
+        t = super().__new__(cls, median)
+        t.fastest = fastest
+        return t
+
+
+def time_graph(torch, calls, launches=20, replays=7, warm_replays=3, warm_seconds=0.03):
     """GPU time per pass over `calls` (objects with a .stream attribute and __call__)
     with the launches captured into a HIP graph, so that short kernels are timed back to
-    back instead of at the rate Python can launch them.  Returns seconds per pass."""
+    back instead of at the rate Python can launch them.  The graph is first replayed untimed,
+    at least warm_replays times and for at least warm_seconds (the first replays after capture
+    upload the graph and, after idle, run at a lower clock: a single timed batch that includes
+    them has read up to ten times too long for the shortest kernels, and 10-15 % too long for
+    the long ones), then `replays` times with an event pair around each;
+    returns the median as a Timing, the fastest replay in .fastest."""
     side = torch.cuda.Stream()
     saved = [c.stream for c in calls]
     graph = torch.cuda.CUDAGraph()
@@ -97,15 +120,45 @@ def time_graph(torch, calls, launches=20, replays=10):
     finally:
         for c, st in zip(calls, saved):
             c.stream = st
-    graph.replay()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(replays):
+    # warm: at least warm_replays replays and at least warm_seconds of GPU time (the CPU legs
+    # between two measurements leave the GPU idle long enough for its clocks to drop)
+    warm_t, warm_n = 0.0, 0
+    while warm_n < max(3, warm_replays) or warm_t < warm_seconds:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        warm_t += e0.elapsed_time(e1) * 1e-3
+        warm_n += 3
+    times = []
+    for _ in range(max(5, replays)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / (launches * replays)
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e-3 / launches)
+    times.sort()
+    return Timing(times[len(times) // 2], times[0])
+
+
+def prewarm(torch, fn, min_seconds=0.05):
+    """Runs fn back to back until at least min_seconds of GPU time have gone by: after
+    idling, the clocks need some tens of milliseconds of load to settle.  Untimed work,
+    reported separately from the warm-up steps.  Returns (launches, seconds)."""
+    launches, total = 0, 0.0
+    while total < min_seconds:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(100):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        launches += 100
+        total += e0.elapsed_time(e1) * 1e-3
+    return launches, total
 
 
 def time_steps(torch, fn, steps, warmup):
@@ -187,8 +240,11 @@ def cpu_time(fn, min_time=0.3, max_reps=10, min_reps=5):
 def roof(ops, byts, seconds):
     """TOP/s, GB/s and the larger of the two roofline fractions."""
     tops, gbps = ops / seconds / 1e12, byts / seconds / 1e9
-    return {"us": round(seconds * 1e6, 2), "TOPS": round(tops, 2), "GB/s": round(gbps, 1),
-            "roofline_frac": round(max(tops / PEAK_INT8_TOPS, gbps / PEAK_HBM_GBPS), 4)}
+    r = {"us": round(seconds * 1e6, 2), "TOPS": round(tops, 2), "GB/s": round(gbps, 1),
+         "roofline_frac": round(max(tops / PEAK_INT8_TOPS, gbps / PEAK_HBM_GBPS), 4)}
+    if isinstance(seconds, Timing):
+        r["us_fastest_replay"] = round(seconds.fastest * 1e6, 2)
+    return r
 
 
 def config_reports(torch, K):
@@ -354,11 +410,17 @@ def config_reports(torch, K):
                 for _ in range(3):
                     replay()
                 torch.cuda.synchronize()
-                t0 = time.perf_counter()
-                for _ in range(20):
-                    replay()
-                torch.cuda.synchronize()
-                return round((time.perf_counter() - t0) / 20 * 1e6, 1)
+                ts = []
+                for _ in range(9):                   # median of batches of 4 replays
+                    e0 = torch.cuda.Event(enable_timing=True)
+                    e1 = torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(4):
+                        replay()
+                    e1.record()
+                    torch.cuda.synchronize()
+                    ts.append(e0.elapsed_time(e1) / 4)
+                return round(sorted(ts)[len(ts) // 2] * 1e3, 1)
             except Exception as exc:  # capture is an optimisation, not the path under test
                 return "capture failed: %s" % str(exc)[:100]
             finally:
@@ -529,6 +591,61 @@ def two_stream(torch, args, ops, da, dw, dsx, dsw, dso, dbias, out):
             "note": "same GEMM, launches alternating over two HIP streams"}
 
 
+def single_workload(torch, args):
+    """One configuration of the dynamic-M sweep or one convolution, launched back to back on
+    the current stream (pre-warm, warm-up steps, then exactly --steps timed launches): the
+    command a profiler is attached to for these shapes.  Prints its own JSON line."""
+    import numpy as np
+    import oracle as O
+    from bladedisc_amd import baseline_configs as cfg
+    from bladedisc_amd import kernels as K
+    dev = lambda v: torch.from_numpy(np.ascontiguousarray(v)).cuda()  # noqa: E731
+    f1 = lambda v: dev(np.array([v], np.float32))                     # noqa: E731
+    kind, _, what = args.workload.partition(":")
+    if kind == "gemm":
+        m, k, n = (int(v) for v in what.split("x"))
+        c = cfg.config2(m, k, n)
+        o = torch.empty((m, n), dtype=torch.int8, device="cuda")
+        call = GemmCall(torch, dev(c["a_q"]), dev(c["w_q"]), f1(c["sx"]), dev(c["sw"]), f1(c["so"]),
+                        None, 1, 0, o)
+        ops, byts = 2.0 * m * n * k, m * k + n * k + m * n + 4 * n
+        name = "int8 qgemm M=%d K=%d N=%d, requant to int8 (E1)" % (m, k, n)
+    elif kind == "conv":
+        conv = {c["name"]: c for c in cfg.RESNET_CONVS}[what]
+        c = cfg.config4(conv)
+        nb, h, w_, ci, co, kk = (conv[t] for t in ("nb", "h", "w", "ci", "co", "k"))
+        pad4, md, osh = O.conv_attrs((nb, h, w_, ci), (co, kk, kk, ci), "NHWC", [1, 1, 1, 1],
+                                     [1, 1, 1, 1], "EXPLICIT",
+                                     explicit_paddings=[0, 0, conv["pad"], conv["pad"],
+                                                        conv["pad"], conv["pad"], 0, 0])
+        md[:12] = O.NHWC_OHWI_METADATA
+        xq, wq = dev(c["x_q"]), dev(c["w_q"])
+        sx, sw, so = f1(c["sx"]), dev(c["sw"]), f1(c["so"])
+        o = torch.empty(tuple(osh), dtype=torch.int8, device="cuda")
+        call = lambda: K.qconv2d(xq, wq, pad4, md, osh, K.EPI_REQUANT_CPU, sx=sx, sw=sw,  # noqa: E731
+                                 so=so, out=o)
+        mg, kg = nb * osh[1] * osh[2], kk * kk * ci
+        ops, byts = 2.0 * mg * co * kg, nb * h * w_ * ci + co * kg + mg * co + 4 * co
+        name = "int8 NHWC conv %s, batch %d, requant to int8 (E1)" % (what, nb)
+    else:
+        raise SystemExit("bench.py: unknown --workload %r" % args.workload)
+    pre_launches, pre_s = prewarm(torch, call, args.prewarm_ms * 1e-3) if args.prewarm_ms > 0 \
+        else (0, 0.0)
+    wall, ev = time_steps(torch, call, args.steps, args.warmup)
+    r = roof(ops, byts, ev / args.steps)
+    print(json.dumps({
+        "metric": "int8 TOPS", "value": round(ops * args.steps / wall / 1e12, 2), "unit": "TOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 5),
+        "prewarm": {"ms": round(pre_s * 1e3, 1), "launches": pre_launches},
+        "higher_is_better": True, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": name},
+        "roofline": {"bound": "mfma" if r["TOPS"] / PEAK_INT8_TOPS >= r["GB/s"] / PEAK_HBM_GBPS
+                     else "hbm", "kernel_us": r["us"], "TOPS": r["TOPS"], "GB/s": r["GB/s"],
+                     "frac": r["roofline_frac"], "ops_per_launch": ops,
+                     "algorithmic_bytes": byts}}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -540,6 +657,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.workload != "headline":
+        single_workload(torch, args)
+        return
 
     size = args.size
     a, w, sx, sw, so, bias_q = make_problem(torch, size)
@@ -552,6 +672,8 @@ def main():
     # REQUANT_GPU epilogue (2) with an f32 bias (kind 2): out = sat8(rne(os[n]*acc + b[n]))
     call = GemmCall(torch, da, dw, dsx, dsw, dso, dbias, 2, 2, out)
 
+    pre_launches, pre_s = prewarm(torch, call, args.prewarm_ms * 1e-3) if args.prewarm_ms > 0 \
+        else (0, 0.0)
     wall, ev = time_steps(torch, call, args.steps, args.warmup)
     ops = 2.0 * size * size * size
     ms_per_step = wall / args.steps * 1e3
@@ -572,6 +694,9 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
+        "prewarm": {"ms": round(pre_s * 1e3, 1), "launches": pre_launches,
+                    "note": "untimed launches of the same kernel before the warm-up steps, "
+                            "until the clocks have settled"},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -591,6 +716,9 @@ def main():
             "unit": "TOP/s",
             "frac": round(achieved / PEAK_INT8_TOPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(size),
+            "traffic_source": "recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over "
+                              "this command (profiles/qgemm_4096_requant_hbm_traffic.md); "
+                              "counters cannot be read from inside the run",
             "algorithmic_bytes": 3 * size * size + 8 * size,
             "kernel_us": round(kernel_s * 1e6, 2),
             "ops_per_launch": ops,

@@ -7,9 +7,7 @@
 #include "dq8_common.h"
 #include "disc_q8.h"
 #include "qgemm_device.h"
-#include "qgemm_pipelined.h"
-#include "qgemm_persistent.h"
-#include "qgemm_skinny.h"
+#include "qgemm_launch.h"
 #include "qconv_direct.h"
 
 #pragma clang fp contract(off)
@@ -194,57 +192,19 @@ mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* 
 }
 
 // ------------------------------------------------------------- tile variants
-struct Variant {
-  const char* name;
-  int bm, bn, bk, threads;
-};
-// index 0 is the generic scalar kernel
-const Variant kVariants[] = {
-    {"generic", 1, 1, 1, 256},
-    {"mfma_256x256x64_w2x2", 256, 256, 64, 256},
-    {"mfma_128x128x64_w2x2", 128, 128, 64, 256},
-    {"mfma_64x64x64_w2x2", 64, 64, 64, 256},
-    // software-pipelined kernels, operands loaded straight into LDS
-    {"pipe_256x256x128", 256, 256, 128, 256},
-    {"pipe_128x128x128", 128, 128, 128, 256},
-    {"pipe_64x64x128", 64, 64, 128, 256},
-    {"pipe_256x64x128", 256, 64, 128, 256},
-    // the same with the k tiles split over 2 groups of waves inside the workgroup
-    {"pipe_64x64x128_k2", 64, 64, 128, 512},
-    // small-M kernel: 16 output channels per workgroup, K split over the waves (GEMM only)
-    {"skinny_16", 16, 16, 64, 512},
-    // 3x3 stride-1 convolution with the input patch resident in LDS (convolution only)
-    {"direct3x3_256x64", 256, 64, 128, 256},
-    {"direct3x3_128x64", 128, 64, 128, 256},
-    // eight waves per workgroup: 256x256 with wave tile 128x64 (two waves per SIMD), 128x128
-    // with wave tile 64x32 (two workgroups per CU: four waves per SIMD)
-    {"pipe_256x256x128_w8", 256, 256, 128, 512},
-    {"pipe_128x128x128_w8", 128, 128, 128, 512},
-    // persistent forms: one workgroup per slot walks several tiles, the next tile's first
-    // loads fly during the epilogue
-    {"persist_256x256x128_w8", 256, 256, 128, 512},
-    {"persist_128x128x128_w8", 128, 128, 128, 512},
-    // 256x192 on eight waves (wave tile 64x96): for problems whose 256x256 tiles would leave
-    // a quarter of the compute units idle
-    {"pipe_256x192x128_w8", 256, 192, 128, 512},
-    {"persist_256x192x128_w8", 256, 192, 128, 512},
-};
-constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
-constexpr int kPipe64k2 = 8;
-constexpr int kSkinnyVariant = 9;
-constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct variants
-constexpr int kPipe256w8 = 12, kPipe128w8 = 13;
-constexpr int kPersist256 = 14, kPersist128 = 15;
-constexpr int kPipe256x192 = 16, kPersist256x192 = 17;
-// largest M the heuristic hands to the small-M kernel
-constexpr int64_t kSkinnyMaxM = 32;
-
-bool is_pipe_variant(int v) {
-  return v == kPipe256 || v == kPipe128 || v == kPipe64 || v == kPipe256x64 || v == kPipe64k2 ||
-         v == kPipe256w8 || v == kPipe128w8 || v == kPersist256 ||
-         v == kPersist128 || v == kPipe256x192 || v == kPersist256x192;
-}
-constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+// (qgemm_launch.h; every launch_variant<CONV, EPI> is instantiated in a qgemm_launch_*.hip)
+}  // namespace
+#define DQ8_DECLARE_LAUNCH(CONV, EPI) \
+  extern template int launch_variant<CONV, EPI>(int, MainParams&, hipStream_t);
+DQ8_DECLARE_LAUNCH(false, DQ8_EPI_ACC_S32)
+DQ8_DECLARE_LAUNCH(false, DQ8_EPI_REQUANT_CPU)
+DQ8_DECLARE_LAUNCH(false, DQ8_EPI_REQUANT_GPU)
+DQ8_DECLARE_LAUNCH(false, DQ8_EPI_DEQUANT_F32)
+DQ8_DECLARE_LAUNCH(true, DQ8_EPI_ACC_S32)
+DQ8_DECLARE_LAUNCH(true, DQ8_EPI_REQUANT_CPU)
+DQ8_DECLARE_LAUNCH(true, DQ8_EPI_REQUANT_GPU)
+DQ8_DECLARE_LAUNCH(true, DQ8_EPI_DEQUANT_F32)
+#undef DQ8_DECLARE_LAUNCH
 
 int compute_units() {
   static std::atomic<int> cached{0};
@@ -261,101 +221,7 @@ int compute_units() {
   return v;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
-int launch_mfma(const MainParams& p, hipStream_t st) {
-  constexpr int lds = 2 * (BM + BN) * (BK + 16);
-  auto kern = qgemm_mfma_kernel<BM, BN, BK, WM, WN, CONV, EPI>;
-  static std::atomic<uint64_t> lds_allowed{0};
-  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
-  const int grid = p.tiles_m * p.tiles_n;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, st, p);
-  return check_hip(hipGetLastError(), "qgemm_mfma launch");
-}
-
-// The pipelined kernels address each block's rows (GEMM) or the whole image
-// (convolution) with 32-bit buffer offsets.
-bool pipe_ok(int bm, int bn, const MainParams& p, bool conv) {
-  constexpr int BK = 128;
-  if (p.K < 16 || p.K % 16 != 0) return false;
-  if ((int64_t)bn * p.ldw + p.K + 2 * BK >= (1LL << 31)) return false;
-  if (conv) return p.conv_bytes < (1LL << 31) && p.Ci % 16 == 0;
-  return (int64_t)bm * p.lda + p.K + 2 * BK < (1LL << 31);
-}
-
-template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI>
-int launch_pipe(const MainParams& p, hipStream_t st) {
-  constexpr int BK = 128;
-  constexpr int lds = KSPLIT * 2 * (BM + BN) * BK;
-  DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
-              "pipelined qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
-  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, KSPLIT, CONV, EPI>;
-  static std::atomic<uint64_t> lds_allowed{0};
-  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
-  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(WM * WN * KSPLIT * 64), lds, st, p);
-  return check_hip(hipGetLastError(), "qgemm_pipe launch");
-}
-
-// `per_cu`: workgroups of this shape a compute unit holds at a time
-template <int BM, int BN, int WM, int WN, bool CONV, int EPI>
-int launch_persist(const MainParams& p, int per_cu, hipStream_t st) {
-  constexpr int stage = (BM + BN) * 128;
-  // (per-channel factors: 8 bytes, plus 4 for the shifts of the fixed-point output stage, and
-  // the 256-byte table of a fused lookup)
-  constexpr int lds = 2 * stage + (WM * WN * 4096 + BN * 12 + 256 <= stage ? 0 : BN * 12 + 256);
-  DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
-              "persistent qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
-  auto kern = qgemm_persist_kernel<BM, BN, WM, WN, CONV, EPI>;
-  static std::atomic<uint64_t> lds_allowed{0};
-  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
-  const int tiles = p.tiles_m * p.tiles_n;
-  const int slots = compute_units() * per_cu;
-  hipLaunchKernelGGL(kern, dim3(tiles < slots ? tiles : slots), dim3(WM * WN * 64), lds, st, p);
-  return check_hip(hipGetLastError(), "qgemm_persist launch");
-}
-
-template <int NW, int MT, int EPI>
-int launch_skinny_t(const MainParams& p, hipStream_t st) {
-  const dim3 grid((unsigned)ceil_div(p.N, 16), (unsigned)ceil_div(p.M, 16 * MT));
-  DQ8_REQUIRE(grid.y <= 65535, "small-M qgemm: M too large for this variant");
-  hipLaunchKernelGGL((qgemm_skinny_kernel<NW, MT, EPI>), grid, dim3(NW * 64), 0, st, p);
-  return check_hip(hipGetLastError(), "qgemm_skinny launch");
-}
-
-// rows per workgroup grow with M (fewer passes over W), waves with the depth of K
-template <int EPI>
-int launch_skinny(const MainParams& p, hipStream_t st) {
-  const bool deep = p.K >= 1024;
-  if (p.M <= 16) return deep ? launch_skinny_t<8, 1, EPI>(p, st) : launch_skinny_t<4, 1, EPI>(p, st);
-  if (p.M <= 32) return deep ? launch_skinny_t<8, 2, EPI>(p, st) : launch_skinny_t<4, 2, EPI>(p, st);
-  return deep ? launch_skinny_t<8, 4, EPI>(p, st) : launch_skinny_t<4, 4, EPI>(p, st);
-}
-
-template <bool CONV, int EPI>
-int launch_variant(int variant, MainParams& p, hipStream_t st) {
-  const Variant& v = kVariants[variant];
-  p.tiles_m = (int)ceil_div(p.M, v.bm);
-  p.tiles_n = (int)ceil_div(p.N, v.bn);
-  switch (variant) {
-    case 1: return launch_mfma<256, 256, 64, 2, 2, CONV, EPI>(p, st);
-    case 2: return launch_mfma<128, 128, 64, 2, 2, CONV, EPI>(p, st);
-    case 3: return launch_mfma<64, 64, 64, 2, 2, CONV, EPI>(p, st);
-    case kPipe256: return launch_pipe<256, 256, 2, 2, 1, CONV, EPI>(p, st);
-    case kPipe128: return launch_pipe<128, 128, 2, 2, 1, CONV, EPI>(p, st);
-    case kPipe64: return launch_pipe<64, 64, 2, 2, 1, CONV, EPI>(p, st);
-    case kPipe256x64: return launch_pipe<256, 64, 4, 1, 1, CONV, EPI>(p, st);
-    case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, CONV, EPI>(p, st);
-    case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, CONV, EPI>(p, st);
-    case kPipe128w8: return launch_pipe<128, 128, 2, 4, 1, CONV, EPI>(p, st);
-    case kPipe256x192: return launch_pipe<256, 192, 4, 2, 1, CONV, EPI>(p, st);
-  }
-  if constexpr (!CONV) {   // GEMM only: the small-M kernel and the persistent forms
-    if (variant == kSkinnyVariant) return launch_skinny<EPI>(p, st);
-    if (variant == kPersist256) return launch_persist<256, 256, 2, 4, false, EPI>(p, 1, st);
-    if (variant == kPersist128) return launch_persist<128, 128, 2, 4, false, EPI>(p, 2, st);
-    if (variant == kPersist256x192) return launch_persist<256, 192, 4, 2, false, EPI>(p, 1, st);
-  }
-  return fail("unknown or unsupported qgemm variant for this operation");
-}
+namespace {
 
 template <bool CONV>
 int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
@@ -425,7 +291,11 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
     } else if (big256) {
       return kPipe256w8;
     }
-    if (tiles(kPipe128) >= 120) return K < 4096 ? kPipe128w8 : kPipe128;
+    // 128x128: eight waves while every tile has a compute unit to itself (more waves to cover
+    // the load latency: 6.3 against 7.1 us at M = 2048, 768 -> 768); with two tiles on a
+    // compute unit, or a deep K, four waves (10.0 against 11.2 us at M = 2048, 768 -> 3072)
+    const int64_t t128 = tiles(kPipe128);
+    if (t128 >= 120) return (K < 4096 && t128 <= cus) ? kPipe128w8 : kPipe128;
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
   constexpr int64_t kCus = 256;

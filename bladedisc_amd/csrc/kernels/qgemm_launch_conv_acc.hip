@@ -1,0 +1,4 @@
+// The tiled kernels of one (operation, epilogue) pair: implicit-GEMM convolution, DQ8_EPI_ACC_S32.
+#include "qgemm_launch.h"
+
+DQ8_INSTANTIATE_LAUNCH(true, DQ8_EPI_ACC_S32)

@@ -1,0 +1,4 @@
+// The tiled kernels of one (operation, epilogue) pair: GEMM, DQ8_EPI_ACC_S32.
+#include "qgemm_launch.h"
+
+DQ8_INSTANTIATE_LAUNCH(false, DQ8_EPI_ACC_S32)
