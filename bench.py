@@ -547,6 +547,24 @@ def extras(torch, steps, warmup, which="all"):
     out["quantize_dequantize_shapes"] = small
     if which == "qdq":
         return out
+    # weight-only quantized linear (f16 activations x uint8 weights, per-channel scale and zero
+    # point): bound by the weight bytes for small M, by the f16 matrix cores (2.5 PFLOP/s) above
+    wo = {}
+    for (k, n) in ((768, 3072), (4096, 4096)):
+        wq = torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda")
+        sc = (torch.rand(n, device="cuda") * 0.02 + 0.002).half()
+        zp = torch.full((n,), 128, dtype=torch.int32, device="cuda")
+        for m in (1, 16, 128, 1024, 4096):
+            xh = torch.randn((m, k), device="cuda").half()
+            oh = torch.empty((m, n), dtype=torch.float16, device="cuda")
+            t = time_graph(torch, [FnCall(lambda: K.weight_only_qgemm(xh, wq, sc, zp, out=oh))])
+            byts, flops = 2.0 * m * k + n * k + 2.0 * m * n + 6.0 * n, 2.0 * m * n * k
+            wo["M%d_K%d_N%d" % (m, k, n)] = {
+                "us": round(t * 1e6, 2), "us_fastest_replay": round(t.fastest * 1e6, 2),
+                "GB/s": round(byts / t / 1e9, 1), "TFLOP/s": round(flops / t / 1e12, 1),
+                "roofline_frac": round(max(byts / t / 1e9 / PEAK_HBM_GBPS,
+                                           flops / t / 1e12 / 2500.0), 4)}
+    out["weight_only_qgemm_f16_u8"] = wo
     out["configs"] = config_reports(torch, K)
     # yardstick: the ROCm library int8 GEMM behind torch._int_mm (int32 output, no
     # epilogue) on the headline shape and data distribution -- a library, not the reference

@@ -691,6 +691,143 @@ MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_s32_per_tensor(
 // ------------------------------------------------------------------ ral_qconv
 // out = sat8(rne(((s_x*s_w[co])/s_o) * conv_s32(in, w))); padding and metadata are
 // host memrefs; zero points are not read.
+// ---- ral_pdll_weight_only_qgemm -------------------------------------------------------
+// Target of the reference's weight-only patterns (R pytorch_blade/tests/disc/pdl/pdll_files/
+// gpu/weight_only_qgemm.pdll:2-104; placements "d,d,d,d" and "d,d,d,d,d"): activations f32 or
+// f16 [..., K], weight ui8 [K, N] (the pattern transposes the [N, K] constant), [bias [N],]
+// per-channel scale [N] and zero point [N], all on the device; result [..., N] in the
+// activation type.  The reference tree has no implementation of this entry to compare with.
+// custom_attrs: `weight_should_be_reordered` -- true as the pattern emits it: the runtime may
+// put the weight into whatever layout its kernel wants, which here is [N, K], done once per
+// weight buffer and cached for the life of the context.  false means the compiler's CUDA
+// layout pass (R tao_compiler/mlir/disc/transforms/
+// disc_transform_weight_data_layout_for_weight_only_gemm.cc:305) has already interleaved the
+// bytes for NVIDIA tensor-core fragments; that layout has no meaning here and is refused.
+namespace {
+
+template <typename T>
+struct WoDtype;
+template <>
+struct WoDtype<float> {
+  static constexpr int value = DQ8_DTYPE_F32;
+};
+template <>
+struct WoDtype<float16> {
+  static constexpr int value = DQ8_DTYPE_F16;
+};
+
+template <typename T, int N>
+MemRefType<T, N> weightOnlyQgemm(ExecutionContext* ctx, void* stream_handle,
+                                 MemRefType<T, N> input, MemRefType<uint8_t, 2> weight,
+                                 const T* bias, int64_t n_bias, MemRefType<T, 1> scales,
+                                 MemRefType<int32_t, 1> zeroPoints, void* customAttrs) {
+  static const char* who = "ral_pdll_weight_only_qgemm";
+  int64_t sizes[N] = {0};
+  MemRefType<T, N> result = assignMemRef<T, N>(nullptr, sizes);
+  if (customAttrs) {
+    PDLAttr* attr = getOrParsePDLAttr(ctx, customAttrs, who);
+    if (!attr || attr->getType() != "dict") {
+      fail(ctx, "fail to parse custom_attrs\n");
+      return result;
+    }
+    auto& dict = attr->as<DictPDLAttr>();
+    if (dict.hasKey("weight_should_be_reordered") &&
+        dict.get("weight_should_be_reordered").getType() == "bool" &&
+        !dict.get("weight_should_be_reordered").as<BoolPDLAttr>().getValue()) {
+      fail(ctx, std::string(who) + ": a weight already reordered by the compiler's CUDA layout "
+                                   "pass cannot be used on this device");
+      return result;
+    }
+  }
+  const int64_t k = weight.sizes[0], n = weight.sizes[1];
+  if (input.sizes[N - 1] != k && !isEmptyMemref(input)) {
+    fail(ctx, std::string(who) + ": mismatch contraction dim");
+    return result;
+  }
+  if (scales.sizes[0] != n || zeroPoints.sizes[0] != n || (bias && n_bias != n)) {
+    fail(ctx, std::string(who) + ": scale, zero point and bias must have N entries");
+    return result;
+  }
+  int64_t m = 1;
+  for (int i = 0; i < N - 1; ++i) {
+    m *= input.sizes[i];
+    sizes[i] = input.sizes[i];
+  }
+  sizes[N - 1] = n;
+  result = assignMemRef<T, N>(nullptr, sizes);
+  if (m == 0 || n == 0) return result;
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight"))
+    return result;
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return result;
+  void* stream = drv->asCUStream(ctx, stream_handle);
+  // [K,N] -> [N,K], once per weight buffer
+  const uint8_t* w_nk = nullptr;
+  if (k > 0) {
+    auto* state = ctx->getOrCreateResource<PackedWeightState>(
+        kPackedWeightState, [] { return new PackedWeightState; });
+    if (!state) return result;
+    std::lock_guard<std::mutex> guard(state->mu);
+    PackedWeightState::Key key{weight.data, k, n};
+    auto it = state->packed.find(key);
+    if (it == state->packed.end()) {
+      auto* nk = static_cast<int8_t*>(drv->alloc_persistent(ctx, (size_t)(n * k)));
+      if (!nk) return result;
+      if (kernelFailed(ctx, dq8_transpose_s8(reinterpret_cast<const int8_t*>(weight.data), n, nk,
+                                             k, n, stream), who))
+        return result;
+      it = state->packed.emplace(key, nk).first;
+    }
+    w_nk = reinterpret_cast<const uint8_t*>(it->second);
+  }
+  void* data = drv->alloc(ctx, (size_t)(m * n) * sizeof(T));
+  if (!data) return result;
+  result = assignMemRef<T, N>(data, sizes);
+  StreamTimer timer(stream);
+  const int st = dq8_weight_only_qgemm(input.data, WoDtype<T>::value, k, w_nk, 0, k, 1, scales.data,
+                                       zeroPoints.data, bias, data, n, m, n, k, nullptr, 0, stream);
+  if (timer.on() && st == 0) {
+    const double ns = timer.stop();
+    const int64_t bytes = (m * k + m * n) * (int64_t)sizeof(T) + k * n;
+    TAO_LOG(INFO) << who << " (gpu):\n"
+                  << "\tm = " << m << "\n"
+                  << "\tn = " << n << "\n"
+                  << "\tk = " << k << "\n"
+                  << "\tMath Ops = " << 2 * m * n * k << "\n"
+                  << "\tBytes = " << bytes << "\n"
+                  << "\tElapsed = " << ns / 1e3 << " us\n"
+                  << "\tBandwidth = " << double(bytes) / ns << " GB\n"
+                  << "\tGFLOPS = " << double(2 * m * n * k) / ns << "\n";
+  }
+  kernelFailed(ctx, st, who);
+  return result;
+}
+
+}  // namespace
+
+template <typename T, int N>
+MemRefType<T, N> ral_pdll_weight_only_qgemm(ExecutionContext* ctx, void* stream_handle,
+                                            MemRefType<T, N> input,
+                                            MemRefType<uint8_t, 2> weight,
+                                            MemRefType<T, 1> scales,
+                                            MemRefType<int32_t, 1> zeroPoints,
+                                            void* customAttrs) {
+  return weightOnlyQgemm<T, N>(ctx, stream_handle, input, weight, nullptr, 0, scales, zeroPoints,
+                               customAttrs);
+}
+
+template <typename T, int N>
+MemRefType<T, N> ral_pdll_weight_only_qgemm_bias(ExecutionContext* ctx, void* stream_handle,
+                                                 MemRefType<T, N> input,
+                                                 MemRefType<uint8_t, 2> weight,
+                                                 MemRefType<T, 1> bias, MemRefType<T, 1> scales,
+                                                 MemRefType<int32_t, 1> zeroPoints,
+                                                 void* customAttrs) {
+  return weightOnlyQgemm<T, N>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0], scales,
+                               zeroPoints, customAttrs);
+}
+
 void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4> input,
                MemRefType<int8_t, 4> kernel, MemRefType<int32_t, 1> padding,
                MemRefType<float, 0> inputScales, MemRefType<int32_t, 0> /*inputZeroPoints*/,
@@ -952,6 +1089,15 @@ TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<4>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_tensor<2>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_s32_per_tensor<3>);
+
+#define DQ8_REGISTER_WEIGHT_ONLY(T, N)                                                        \
+  TAO_RAL_API("ral_pdll_weight_only_qgemm", "gpu", gpu::q8::ral_pdll_weight_only_qgemm<T, N>); \
+  TAO_RAL_API("ral_pdll_weight_only_qgemm", "gpu", gpu::q8::ral_pdll_weight_only_qgemm_bias<T, N>);
+DQ8_REGISTER_WEIGHT_ONLY(float, 2)
+DQ8_REGISTER_WEIGHT_ONLY(float, 3)
+DQ8_REGISTER_WEIGHT_ONLY(float16, 2)
+DQ8_REGISTER_WEIGHT_ONLY(float16, 3)
+#undef DQ8_REGISTER_WEIGHT_ONLY
 
 TAO_RAL_API("ral_qconv", "gpu", gpu::q8::ral_qconv);
 TAO_RAL_API("ral_pdll_qconv2d", "gpu", gpu::q8::ral_pdll_qconv2d);

@@ -132,6 +132,40 @@ def lut8(q, table, out=None):
     return out
 
 
+def weight_only_qgemm(x, w, scale, zero_points=None, bias=None, tp_b=True, out=None,
+                      workspace=True):
+    """out = x @ ((w - zero_points[:, None]) * scale[:, None]).T + bias for f16 / f32
+    activations x [M,K] and 8-bit weights (uint8 or int8) w [N,K] (tp_b) or [K,N]; scale and
+    bias have x's dtype, zero_points is int32.  workspace=False withholds the scratch that
+    [K,N] weights are transposed into."""
+    _need_cuda(x, w, scale, zero_points, bias)
+    if x.dtype not in (torch.float32, torch.float16):
+        raise TypeError("weight_only_qgemm takes f32 or f16 activations")
+    if w.dtype not in (torch.uint8, torch.int8) or w.dim() != 2:
+        raise TypeError("weight_only_qgemm takes a uint8 / int8 weight matrix")
+    if x.dim() != 2 or x.stride(1) != 1:
+        x = x.reshape(-1, x.shape[-1]).contiguous()
+    w = w.contiguous()
+    n, k = (w.shape if tp_b else (w.shape[1], w.shape[0]))
+    m = x.shape[0]
+    if x.shape[1] != k:
+        raise ValueError("contraction dimensions differ")
+    scale = scale.to(x.dtype).contiguous()
+    bias = bias.to(x.dtype).contiguous() if bias is not None else None
+    zero_points = zero_points.to(torch.int32).contiguous() if zero_points is not None else None
+    if out is None:
+        out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    L = _lib.lib()
+    ws_bytes = L.dq8_weight_only_qgemm_workspace_bytes(n, k, int(tp_b)) if workspace else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    st = L.dq8_weight_only_qgemm(_ptr(x), 0 if x.dtype == torch.float32 else 1, x.stride(0),
+                                 _ptr(w), int(w.dtype == torch.int8), w.stride(0), int(tp_b),
+                                 _ptr(scale), _ptr(zero_points), _ptr(bias), _ptr(out),
+                                 out.stride(0), m, n, k, _ptr(ws), ws_bytes, _stream())
+    _lib.check(st, "dq8_weight_only_qgemm")
+    return out
+
+
 def activation_table(fn, s_in, z_in, s_out, z_out, in_dtype=torch.int8, out_dtype=torch.int8,
                      device="cuda"):
     """The table of  q -> quantize(fn(dequantize(q, s_in, z_in)), s_out, z_out)  for every

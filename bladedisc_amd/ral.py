@@ -340,7 +340,8 @@ def memref_to_tensor(st, dtype, device="cuda"):
 
     h = _Holder()
     h.__cuda_array_interface__ = {
-        "shape": tuple(sizes), "typestr": {1: "|i1", 4: "<f4"}[itemsize] if dtype != torch.int32 else "<i4",
+        "shape": tuple(sizes),
+        "typestr": "<i4" if dtype == torch.int32 else {1: "|i1", 2: "<f2", 4: "<f4"}[itemsize],
         "data": (int(st.data), False), "version": 2,
     }
     return torch.as_tensor(h, device=device)

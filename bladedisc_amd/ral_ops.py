@@ -124,6 +124,22 @@ def pdll_qgemm_per_tensor(ex, x, w, bias_s32, sx, sw, so, zo=0, transpose_b=Fals
     return ral.memref_to_tensor(res, torch.int8)
 
 
+def pdll_weight_only_qgemm(ex, x, w_kn, scale, zero_points, bias=None, reorder=True):
+    """ral_pdll_weight_only_qgemm: f32 / f16 activations [..., K], uint8 weight [K,N], optional
+    bias [N], per-channel scale [N] (activation dtype) and zero point [N] (int32), all on the
+    device; `reorder` is the pattern's `weight_should_be_reordered` attribute."""
+    code = {torch.float32: "f32", torch.float16: "f16"}[x.dtype]
+    a = ex.new_args().tensor(x).tensor(w_kn)
+    if bias is not None:
+        a.tensor(bias)
+    a.tensor(scale).tensor(zero_points)
+    a.blob(ral.encode_attr({"weight_should_be_reordered": bool(reorder)}))
+    res = a.result_memref(code, x.dim())
+    ex.call("ral_pdll_weight_only_qgemm", "gpu", a)
+    assert w_kn.shape[1] == res.sizes[x.dim() - 1]
+    return ral.memref_to_tensor(res, x.dtype)
+
+
 def qconv(ex, x, w, padding, metadata, sx, sw_c, so, out):
     """ral_qconv: padding [4] and metadata [17] are host int32 memrefs."""
     a = ex.new_args().tensor(x).tensor(w)

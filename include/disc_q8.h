@@ -285,6 +285,34 @@ int dq8_qgemm_fused(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, 
 int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
                      int64_t cols, void* stream);
 
+/* ---- weight-only quantized GEMM ----------------------------------------- */
+
+#define DQ8_DTYPE_F32 0
+#define DQ8_DTYPE_F16 1
+
+/* out[m,n] = (sum_k x[m,k] * (w(n,k) - zero_points[n])) * scale[n] + bias[n]: floating-point
+ * activations times 8-bit weights with a per-output-channel scale and zero point, i.e.
+ * matmul(x, dequantize(w)^T) + bias.  Replaces the target of the reference's
+ * `ral_pdll_weight_only_qgemm` custom call
+ * (R pytorch_blade/tests/disc/pdl/pdll_files/gpu/weight_only_qgemm.pdll:2-104, operands
+ * input, weight, [bias,] weight_scale, weight_zero_point; the layout pass that marks the
+ * weight as reordered is R tao_compiler/mlir/disc/transforms/
+ * disc_transform_weight_data_layout_for_weight_only_gemm.cc:305).
+ * x, out, scale, bias: x_dtype (DQ8_DTYPE_*), rows ldx / ldo elements apart; bias and
+ * zero_points may be NULL; w: uint8 (w_signed = 0) or int8 (1), [N,K] with rows ldw bytes
+ * apart if tp_b, else [K,N] as the custom call passes it.  Zero points must lie in
+ * [-1024, 1024].  [K,N] weights are transposed into `workspace`
+ * (dq8_weight_only_qgemm_workspace_bytes) on every call; a runtime does that once per constant
+ * weight with dq8_transpose_s8 and passes tp_b = 1.  Without the scratch, or with K % 16 != 0
+ * or rows that are not 16-byte aligned, a slower kernel without alignment rules runs.
+ * Accumulation is f32; f32 activations enter the matrix cores as two halves (about 22
+ * significant bits). */
+size_t dq8_weight_only_qgemm_workspace_bytes(int64_t N, int64_t K, int tp_b);
+int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, const void* w, int w_signed,
+                          int64_t ldw, int tp_b, const void* scale, const int32_t* zero_points,
+                          const void* bias, void* out, int64_t ldo, int64_t M, int64_t N,
+                          int64_t K, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- int8 convolution (rank 4) ---------------------------------------- */
 
 /* Implicit-GEMM convolution.  Layouts are described exactly as ral_qconv's

@@ -194,6 +194,25 @@ def dequant_acc(acc, sx, sw, bias=None):
     return out
 
 
+def weight_only_qgemm(x, w_nk, scale, zero_points=None, bias=None):
+    """(out, bound) for the weight-only quantized linear the reference's pattern rewrites into
+    `ral_pdll_weight_only_qgemm` (pytorch_blade/tests/disc/pdl/pdll_files/gpu/
+    weight_only_qgemm.pdll:2-104): matmul(x, dequantize(w)^T) + bias with
+    dequantize(w)[n, k] = (w[n, k] - zero_points[n]) * scale[n]
+    (torch.fake_quantize_per_channel_affine's dequantized weight, the model of
+    pytorch_blade/tests/disc/pdl/test_torchscipt_to_mhlo/test_quantization.py:501-523).
+    PARITY UNPINNED beyond this definition: the reference tree holds no runtime implementation
+    and no expected values for it.  Computed in float64; `bound[m, n]` = sum_k |x| |w_deq|,
+    the quantity accumulation-error tolerances are stated against."""
+    x64 = np.asarray(x, np.float64)
+    zp = np.zeros(w_nk.shape[0], np.int64) if zero_points is None else np.asarray(zero_points, np.int64)
+    wd = (w_nk.astype(np.int64) - zp[:, None]).astype(np.float64) * np.asarray(scale, np.float64)[:, None]
+    out = x64 @ wd.T
+    if bias is not None:
+        out = out + np.asarray(bias, np.float64)[None, :]
+    return out, np.abs(x64) @ np.abs(wd).T
+
+
 def _view3(shape, axis):
     if axis is None:
         return 1, 1, int(np.prod(shape, dtype=np.int64))

@@ -946,3 +946,73 @@ def test_bad_arguments_fail_loudly(K):
     st = L.dq8_qgemm(None, one, None, one, None, one, C.c_int64(-1), one, one, 0, 1, 0, None, 0,
                      None, one, None, one, None, one, 0, 0, 0, None, C.c_size_t(0), None)
     assert st != 0 and b"negative" in L.dq8_last_error()
+
+
+def _weight_only_case(rng, m, k, n, dtype, signed):
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    x = rng.standard_normal((m, k)).astype(npdt)
+    if signed:
+        w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        zp = rng.integers(-8, 9, n).astype(np.int32)
+    else:
+        w = rng.integers(0, 256, (n, k), dtype=np.uint8)
+        zp = rng.integers(118, 139, n).astype(np.int32)
+    scale = rng.uniform(0.002, 0.02, n).astype(npdt)
+    bias = rng.standard_normal(n).astype(npdt)
+    return x, w, scale, zp, bias
+
+
+def _weight_only_check(got, x, w, scale, zp, bias, dtype):
+    """|error| <= accumulation bound: products are exact in f32 (half activations; f32 ones
+    enter as two halves, 2^-21 relative), the f32 accumulation of K terms adds K * 2^-24 of
+    sum |x||w|, then one rounding to the output type."""
+    want, bound = O.weight_only_qgemm(x, w, scale, zp, bias)
+    k = x.shape[1]
+    tol = bound * (k * 2.0 ** -24 + 2.0 ** -20) + 1e-30
+    tol = tol + (np.abs(want) + bound * 2.0 ** -12) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
+    err = np.abs(host(got).astype(np.float64) - want)
+    assert (err <= tol).all(), "max excess %.3g at %s" % (float((err - tol).max()),
+                                                          np.unravel_index(np.argmax(err - tol), err.shape))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("k,n", [(768, 768), (768, 3072), (3072, 768)])
+@pytest.mark.parametrize("m", [1, 16, 128, 1024])
+def test_weight_only_qgemm_bert_linears(K, m, k, n, dtype):
+    """Weight-only quantized linear on the BERT-base shapes: uint8 weights with per-channel
+    scale and zero point near 128 (the reference pattern's quantization), bias, f16 and f32
+    activations, every kernel form (small-M, both tile shapes)."""
+    rng = np.random.default_rng(m * 7 + k + n)
+    x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed=False)
+    got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+    assert got.dtype == dtype and tuple(got.shape) == (m, n)
+    _weight_only_check(got, x, w, scale, zp, bias, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
+    """[K,N] weights as the custom call passes them (with and without the scratch for the
+    transpose), int8 weights, no bias / no zero points, shapes that leave partial tiles, a k
+    depth that is not a multiple of 32, and the shapes the alignment rules send to the
+    kernel without them (the reference's own test uses K = 3, N = 5)."""
+    rng = np.random.default_rng(77)
+    for (m, k, n) in [(2, 3, 5), (33, 48, 40), (200, 80, 136), (1, 16, 1), (70, 2064, 100),
+                      (130, 40, 260), (5, 1000, 33)]:
+        for signed in (False, True):
+            x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed)
+            got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+            _weight_only_check(got, x, w, scale, zp, bias, dtype)
+            w_kn = np.ascontiguousarray(w.T)
+            for ws in (True, False):
+                got = K.weight_only_qgemm(dev(x), dev(w_kn), dev(scale), dev(zp), None, tp_b=False,
+                                          workspace=ws)
+                _weight_only_check(got, x, w, scale, zp, None, dtype)
+            got = K.weight_only_qgemm(dev(x), dev(w), dev(scale))
+            _weight_only_check(got, x, w, scale, None, None, dtype)
+    # strided activations (a column slice of a wider tensor)
+    x, w, scale, zp, bias = _weight_only_case(rng, 64, 64, 96, dtype, False)
+    wide = dev(np.concatenate([x, x], axis=1))
+    got = K.weight_only_qgemm(wide[:, :64], dev(w), dev(scale), dev(zp), dev(bias))
+    _weight_only_check(got, x, w, scale, zp, bias, dtype)
+    empty = K.weight_only_qgemm(dev(x[:0]), dev(w), dev(scale), dev(zp), dev(bias))
+    assert tuple(empty.shape) == (0, 96)

@@ -19,6 +19,9 @@ def rt():
     ctx.close()
 
 
+_CONSTANT_WEIGHTS = []
+
+
 def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
@@ -199,6 +202,41 @@ def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
         a.result_memref("i8", 2)
         with pytest.raises(ral.RalError, match="zero point"):
             ex.call("ral_pdll_qgemm", "gpu", a)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_ral_pdll_weight_only_qgemm(rt, dtype, with_bias):
+    """The weight-only entry by its mangled name, as the pattern calls it: rank-3 activations,
+    uint8 weight [K,N] with zero points 128 (quant range 0..255), per-channel scale, optional
+    bias; the packed weight is cached, so a second call with other activations must agree
+    too.  Tolerance: the f32 accumulation bound of the kernel tests."""
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(31 + int(with_bias))
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    b, s, k, n = 2, 40, 96, 72
+    w = rng.integers(0, 256, (n, k), dtype=np.uint8)
+    zp = np.full(n, 128, np.int32)
+    scale = rng.uniform(0.002, 0.02, n).astype(npdt)
+    bias = rng.standard_normal(n).astype(npdt) if with_bias else None
+    w_kn = dev(np.ascontiguousarray(w.T))
+    # (the entry caches the re-laid-out weight by buffer address for the life of the context, as
+    # for a program's constants: the buffer must not be freed and reused while `rt` lives)
+    _CONSTANT_WEIGHTS.append(w_kn)
+    with ctx.execution() as ex:
+        for rep in range(2):
+            x = rng.standard_normal((b, s, k)).astype(npdt)
+            got = ops.pdll_weight_only_qgemm(ex, dev(x), w_kn, dev(scale), dev(zp),
+                                             dev(bias) if with_bias else None)
+            assert got.dtype == dtype and tuple(got.shape) == (b, s, n)
+            want, bound = O.weight_only_qgemm(x.reshape(-1, k), w, scale, zp, bias)
+            tol = bound * (k * 2.0 ** -24 + 2.0 ** -20) + \
+                (np.abs(want) + bound * 2.0 ** -12) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
+            err = np.abs(host(got).astype(np.float64).reshape(-1, n) - want)
+            assert (err <= tol).all(), rep
+        # a weight the compiler's CUDA layout pass has already interleaved is refused
+        with pytest.raises(ral.RalError, match="reordered"):
+            ops.pdll_weight_only_qgemm(ex, dev(x), w_kn, dev(scale), dev(zp), None, reorder=False)
 
 
 @pytest.mark.parametrize("nb,h,ci,co,k,stride,pad", [(2, 14, 64, 64, 3, 1, 1), (2, 7, 256, 128, 1, 1, 0),

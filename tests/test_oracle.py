@@ -569,3 +569,28 @@ def test_requant_fixedpoint_known_answers_and_exact_stage():
         assert got[0, 6] == 127 and got[0, 7] == -128
     got = O.requant_fixedpoint(acc, np.float32(1.0), np.ones(10, np.float32), np.float32(1.0))
     assert got[0, 8] == -128 and got[0, 9] == -128
+
+
+def test_weight_only_qgemm_is_linear_on_the_fake_quantized_weight():
+    """The weight-only oracle against the model the reference's pattern matches
+    (test_quantization.py:501-523): F.linear on torch.fake_quantize_per_channel_affine(weight)
+    with quant range [0, 255], zero point 128 -- a library cross-check on the CPU that pins the
+    sign of the zero point, the channel axis and the place of the scale."""
+    import torch
+    rng = np.random.default_rng(5)
+    n, k, m = 5, 3, 7
+    w = torch.from_numpy(rng.standard_normal((n, k)).astype(np.float32))
+    scale = torch.from_numpy(rng.uniform(0.005, 0.03, n).astype(np.float32))
+    zp = torch.from_numpy(rng.integers(100, 156, n).astype(np.int32))
+    bias = torch.from_numpy(rng.standard_normal(n).astype(np.float32))
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32))
+    fq = torch.fake_quantize_per_channel_affine(w, scale, zp, 0, 0, 255)
+    want = torch.nn.functional.linear(x, fq, bias).numpy()
+    q = torch.clamp(torch.round(w / scale[:, None]) + zp[:, None], 0, 255).to(torch.uint8).numpy()
+    got, bound = O.weight_only_qgemm(x.numpy(), q, scale.numpy(), zp.numpy(), bias.numpy())
+    assert got.shape == (m, n) and (bound >= np.abs(got - bias.numpy()[None]) - 1e-9).all()
+    np.testing.assert_allclose(got, want, rtol=0, atol=2e-6 * float(bound.max()) + 1e-6)
+    # no zero points / no bias: plain matmul on the scaled integers
+    got2, _ = O.weight_only_qgemm(x.numpy(), q, scale.numpy())
+    np.testing.assert_allclose(got2, x.numpy().astype(np.float64) @ (q.astype(np.float64) * scale.numpy().astype(np.float64)[:, None]).T,
+                               rtol=1e-12)

@@ -38,6 +38,13 @@ GOLDEN_NAMES = [
     "ral_pdll_qgemm___gpu___pvoid_pvoid_m2di8_m2di8_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m2di8",
     "ral_pdll_qgemm___gpu___pvoid_pvoid_m4di8_m2di8_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m4di8",
     "ral_pdll_qgemm___gpu___pvoid_pvoid_m3di8_m2di8_m1di32_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m3di8",
+    # weight_only_qgemm.pdll:2-104 with the operand types of test_quantization.py:550,612 (f32) and of
+    # disc-convert-weight-layout-for-weight-only-gemm.mlir:5-10 (f16): input, weight ui8 [K,N], [bias,]
+    # scale, zero point i32, custom_attrs
+    "ral_pdll_weight_only_qgemm___gpu___pvoid_pvoid_m3df32_m2dui8_m1df32_m1di32_pvoid___m3df32",
+    "ral_pdll_weight_only_qgemm___gpu___pvoid_pvoid_m3df32_m2dui8_m1df32_m1df32_m1di32_pvoid___m3df32",
+    "ral_pdll_weight_only_qgemm___gpu___pvoid_pvoid_m3df16_m2dui8_m1df16_m1di32_pvoid___m3df16",
+    "ral_pdll_weight_only_qgemm___gpu___pvoid_pvoid_m2df16_m2dui8_m1df16_m1df16_m1di32_pvoid___m2df16",
 ]
 
 
