@@ -21,6 +21,9 @@ _PROTOS = {
     "dq8_quantize": (_INT, [_VP, _VP, _INT, _I64, _I64, _I64, _VP, _VP, _I64, _I32,
                             _I32, _INT, _VP]),
     "dq8_dequantize": (_INT, [_VP, _INT, _VP, _I64, _I64, _I64, _VP, _VP, _I64, _VP]),
+    "dq8_quantize_ex": (_INT, [_VP, _INT, _VP, _INT, _I64, _I64, _I64, _VP, _VP, _I64, _I64, _I64,
+                               _INT, _VP]),
+    "dq8_dequantize_ex": (_INT, [_VP, _INT, _VP, _I64, _I64, _I64, _VP, _VP, _I64, _VP]),
     "dq8_qgemm_workspace_bytes": (_SZ, [_I64, _I64, _I64, _INT, _INT]),
     "dq8_qgemm_workspace_bytes_zp": (_SZ, [_I64, _I64, _I64, _INT, _INT, _I32, _I32]),
     "dq8_qgemm": (_INT, [_VP, _I64, _VP, _I64, _VP, _I64, _I64, _I64, _I64, _INT, _INT,

@@ -310,6 +310,83 @@ dequantize_scalar(const uint8_t* __restrict__ q, float* __restrict__ out,
   }
 }
 
+// ------------------------------------------------- wide outputs, f16 inputs
+// 16- and 32-bit quantized types and half-precision inputs: one element per thread, the same
+// separately rounded f32 steps.  The conversion of the clamped f32 value saturates: the f32
+// images of 2^31 - 1 and 2^32 - 1 are 2^31 and 2^32, one past the integer range.
+template <typename QT>
+__device__ __forceinline__ QT convert_clamped(float t) {
+  return (QT)(int)t;
+}
+template <>
+__device__ __forceinline__ int32_t convert_clamped<int32_t>(float t) {
+  return t >= 2147483648.0f ? INT32_MAX : (int32_t)t;
+}
+template <>
+__device__ __forceinline__ uint32_t convert_clamped<uint32_t>(float t) {
+  return t >= 4294967296.0f ? UINT32_MAX : (t <= 0.0f ? 0u : (uint32_t)t);
+}
+template <>
+__device__ __forceinline__ uint16_t convert_clamped<uint16_t>(float t) {
+  return (uint16_t)(unsigned)t;
+}
+
+template <typename XT, typename QT, int ROUND>
+__global__ void __launch_bounds__(kThreads)
+quantize_wide(const XT* __restrict__ x, QT* __restrict__ out, int64_t n, int64_t nch,
+              int64_t inner, int per_channel, const float* __restrict__ scale,
+              const int32_t* __restrict__ zp, float lo, float hi) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kThreads) {
+    const int64_t c = per_channel ? (i / inner) % nch : 0;
+    const float t0 = (float)x[i] / scale[c];
+    const float t1 = t0 + (float)zp[c];
+    const float t2 = ROUND == DQ8_ROUND_HALF_TO_EVEN ? rintf(t1) : roundf(t1);
+    out[i] = convert_clamped<QT>(fminf(fmaxf(t2, lo), hi));
+  }
+}
+
+template <typename QT>
+__global__ void __launch_bounds__(kThreads)
+dequantize_wide(const QT* __restrict__ q, float* __restrict__ out, int64_t n, int64_t nch,
+                int64_t inner, int per_channel, const float* __restrict__ scale,
+                const int32_t* __restrict__ zp) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kThreads) {
+    const int64_t c = per_channel ? (i / inner) % nch : 0;
+    // the input is converted to the zero point's type (i32) before the subtraction
+    out[i] = (float)((int32_t)q[i] - zp[c]) * scale[c];
+  }
+}
+
+template <typename XT, typename QT>
+void launch_quantize_wide(bool rne, const void* x, void* out, int64_t n, int64_t nch,
+                          int64_t inner, int per_channel, const float* scale, const int32_t* zp,
+                          float lo, float hi, hipStream_t st) {
+  const dim3 grid(grid_for(n, 1)), block(kThreads);
+  if (rne)
+    hipLaunchKernelGGL((quantize_wide<XT, QT, DQ8_ROUND_HALF_TO_EVEN>), grid, block, 0, st,
+                       (const XT*)x, (QT*)out, n, nch, inner, per_channel, scale, zp, lo, hi);
+  else
+    hipLaunchKernelGGL((quantize_wide<XT, QT, DQ8_ROUND_HALF_AWAY_FROM_ZERO>), grid, block, 0, st,
+                       (const XT*)x, (QT*)out, n, nch, inner, per_channel, scale, zp, lo, hi);
+}
+
+template <typename XT>
+bool launch_quantize_kind(int out_kind, bool rne, const void* x, void* out, int64_t n,
+                          int64_t nch, int64_t inner, int per_channel, const float* scale,
+                          const int32_t* zp, float lo, float hi, hipStream_t st) {
+  switch (out_kind) {
+    case DQ8_I8: launch_quantize_wide<XT, int8_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+    case DQ8_U8: launch_quantize_wide<XT, uint8_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+    case DQ8_I16: launch_quantize_wide<XT, int16_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+    case DQ8_U16: launch_quantize_wide<XT, uint16_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+    case DQ8_I32: launch_quantize_wide<XT, int32_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+    case DQ8_U32: launch_quantize_wide<XT, uint32_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+  }
+  return false;
+}
+
 }  // namespace
 
 extern "C" int dq8_quantize(const float* x, void* out, int out_kind,
@@ -502,4 +579,75 @@ extern "C" int dq8_fake_quant(const float* x, float* out, int64_t outer, int64_t
   }
 #undef LAUNCH_RND
   return dq8::check_hip(hipGetLastError(), "dq8_fake_quant launch");
+}
+
+namespace {
+bool quant_limits(int kind, int64_t* lo, int64_t* hi) {
+  switch (kind) {
+    case DQ8_I8: *lo = -128; *hi = 127; return true;
+    case DQ8_U8: *lo = 0; *hi = 255; return true;
+    case DQ8_I16: *lo = -32768; *hi = 32767; return true;
+    case DQ8_U16: *lo = 0; *hi = 65535; return true;
+    case DQ8_I32: *lo = INT32_MIN; *hi = INT32_MAX; return true;
+    case DQ8_U32: *lo = 0; *hi = UINT32_MAX; return true;
+  }
+  return false;
+}
+}  // namespace
+
+extern "C" int dq8_quantize_ex(const void* x, int x_dtype, void* out, int out_kind, int64_t outer,
+                               int64_t nch, int64_t inner, const float* scale,
+                               const int32_t* zp, int64_t n_q, int64_t qmin, int64_t qmax,
+                               int round_mode, void* stream) {
+  dq8::clear_error();
+  int64_t lim_lo = 0, lim_hi = 0;
+  DQ8_REQUIRE(quant_limits(out_kind, &lim_lo, &lim_hi), "dq8_quantize_ex: unknown out_kind");
+  DQ8_REQUIRE(x_dtype == DQ8_DTYPE_F32 || x_dtype == DQ8_DTYPE_F16,
+              "dq8_quantize_ex: input must be f32 or f16");
+  DQ8_REQUIRE(qmin <= qmax && qmin >= lim_lo && qmax <= lim_hi,
+              "dq8_quantize_ex: quant_min/quant_max outside the output type");
+  // f32 -> 8 bit: the bandwidth-tuned kernels
+  if (x_dtype == DQ8_DTYPE_F32 && (out_kind == DQ8_I8 || out_kind == DQ8_U8))
+    return dq8_quantize(static_cast<const float*>(x), out, out_kind, outer, nch, inner, scale, zp,
+                        n_q, (int32_t)qmin, (int32_t)qmax, round_mode, stream);
+  DQ8_REQUIRE(outer >= 0 && nch >= 0 && inner >= 0, "dq8_quantize_ex: negative size");
+  DQ8_REQUIRE(round_mode == DQ8_ROUND_HALF_TO_EVEN ||
+                  round_mode == DQ8_ROUND_HALF_AWAY_FROM_ZERO,
+              "dq8_quantize_ex: unknown round_mode");
+  DQ8_REQUIRE(n_q == 1 || n_q == nch, "dq8_quantize_ex: n_q must be 1 or nch");
+  const int64_t n = outer * nch * inner;
+  if (n == 0) return 0;
+  DQ8_REQUIRE(x && out && scale && zp, "dq8_quantize_ex: null pointer");
+  const bool rne = round_mode == DQ8_ROUND_HALF_TO_EVEN;
+  const float lo = (float)qmin, hi = (float)qmax;
+  hipStream_t st = (hipStream_t)stream;
+  if (x_dtype == DQ8_DTYPE_F32)
+    launch_quantize_kind<float>(out_kind, rne, x, out, n, nch, inner, n_q > 1, scale, zp, lo, hi, st);
+  else
+    launch_quantize_kind<_Float16>(out_kind, rne, x, out, n, nch, inner, n_q > 1, scale, zp, lo, hi, st);
+  return dq8::check_hip(hipGetLastError(), "dq8_quantize_ex launch");
+}
+
+extern "C" int dq8_dequantize_ex(const void* q, int in_kind, float* out, int64_t outer,
+                                 int64_t nch, int64_t inner, const float* scale,
+                                 const int32_t* zp, int64_t n_q, void* stream) {
+  if (in_kind == DQ8_I8 || in_kind == DQ8_U8)
+    return dq8_dequantize(q, in_kind, out, outer, nch, inner, scale, zp, n_q, stream);
+  dq8::clear_error();
+  DQ8_REQUIRE(in_kind >= DQ8_I16 && in_kind <= DQ8_U32, "dq8_dequantize_ex: unknown in_kind");
+  DQ8_REQUIRE(outer >= 0 && nch >= 0 && inner >= 0, "dq8_dequantize_ex: negative size");
+  DQ8_REQUIRE(n_q == 1 || n_q == nch, "dq8_dequantize_ex: n_q must be 1 or nch");
+  const int64_t n = outer * nch * inner;
+  if (n == 0) return 0;
+  DQ8_REQUIRE(q && out && scale && zp, "dq8_dequantize_ex: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(grid_for(n, 1)), block(kThreads);
+  const int pc = n_q > 1;
+  switch (in_kind) {
+    case DQ8_I16: hipLaunchKernelGGL(dequantize_wide<int16_t>, grid, block, 0, st, (const int16_t*)q, out, n, nch, inner, pc, scale, zp); break;
+    case DQ8_U16: hipLaunchKernelGGL(dequantize_wide<uint16_t>, grid, block, 0, st, (const uint16_t*)q, out, n, nch, inner, pc, scale, zp); break;
+    case DQ8_I32: hipLaunchKernelGGL(dequantize_wide<int32_t>, grid, block, 0, st, (const int32_t*)q, out, n, nch, inner, pc, scale, zp); break;
+    default: hipLaunchKernelGGL(dequantize_wide<uint32_t>, grid, block, 0, st, (const uint32_t*)q, out, n, nch, inner, pc, scale, zp); break;
+  }
+  return dq8::check_hip(hipGetLastError(), "dq8_dequantize_ex launch");
 }

@@ -985,6 +985,15 @@ void view3(const int64_t (&sizes)[N], int64_t axis, int64_t* outer, int64_t* nch
 
 }  // namespace
 
+template <typename QT>
+struct QuantKind;
+template <> struct QuantKind<int8_t> { static constexpr int value = DQ8_I8; };
+template <> struct QuantKind<uint8_t> { static constexpr int value = DQ8_U8; };
+template <> struct QuantKind<int16_t> { static constexpr int value = DQ8_I16; };
+template <> struct QuantKind<uint16_t> { static constexpr int value = DQ8_U16; };
+template <> struct QuantKind<int32_t> { static constexpr int value = DQ8_I32; };
+template <> struct QuantKind<uint32_t> { static constexpr int value = DQ8_U32; };
+
 template <typename QT, int N, int SR>
 void ral_quantize(ExecutionContext* ctx, void* stream_handle, MemRefType<float, N> input,
                   MemRefType<float, SR> scale, MemRefType<int32_t, SR> zeroPoint,
@@ -1016,10 +1025,9 @@ void ral_quantize(ExecutionContext* ctx, void* stream_handle, MemRefType<float, 
   }
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return;
-  int st = dq8_quantize(input.data, result.data,
-                        std::is_same<QT, int8_t>::value ? DQ8_I8 : DQ8_U8, outer, nch, inner,
-                        scale.data, zeroPoint.data, SR == 0 ? 1 : n_q, (int32_t)quantMin,
-                        (int32_t)quantMax, (int)roundMode, drv->asCUStream(ctx, stream_handle));
+  int st = dq8_quantize_ex(input.data, DQ8_DTYPE_F32, result.data, QuantKind<QT>::value, outer, nch,
+                           inner, scale.data, zeroPoint.data, SR == 0 ? 1 : n_q, quantMin,
+                           quantMax, (int)roundMode, drv->asCUStream(ctx, stream_handle));
   kernelFailed(ctx, st, who);
 }
 
@@ -1053,9 +1061,9 @@ void ral_dequantize(ExecutionContext* ctx, void* stream_handle, MemRefType<QT, N
   }
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return;
-  int st = dq8_dequantize(input.data, std::is_same<QT, int8_t>::value ? DQ8_I8 : DQ8_U8,
-                          result.data, outer, nch, inner, scale.data, zeroPoint.data,
-                          SR == 0 ? 1 : n_q, drv->asCUStream(ctx, stream_handle));
+  int st = dq8_dequantize_ex(input.data, QuantKind<QT>::value, result.data, outer, nch, inner,
+                             scale.data, zeroPoint.data, SR == 0 ? 1 : n_q,
+                             drv->asCUStream(ctx, stream_handle));
   kernelFailed(ctx, st, who);
 }
 
@@ -1115,6 +1123,15 @@ DQ8_REGISTER_QDQ(uint8_t, 1)
 DQ8_REGISTER_QDQ(uint8_t, 2)
 DQ8_REGISTER_QDQ(uint8_t, 3)
 DQ8_REGISTER_QDQ(uint8_t, 4)
+// the wider quantized types of the operator (disc-fold-quantize.mlir:137-247), ranks 1-2
+DQ8_REGISTER_QDQ(int16_t, 1)
+DQ8_REGISTER_QDQ(int16_t, 2)
+DQ8_REGISTER_QDQ(uint16_t, 1)
+DQ8_REGISTER_QDQ(uint16_t, 2)
+DQ8_REGISTER_QDQ(int32_t, 1)
+DQ8_REGISTER_QDQ(int32_t, 2)
+DQ8_REGISTER_QDQ(uint32_t, 1)
+DQ8_REGISTER_QDQ(uint32_t, 2)
 #undef DQ8_REGISTER_QDQ
 
 }  // namespace ral

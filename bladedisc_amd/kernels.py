@@ -64,18 +64,38 @@ def _view3(shape, axis):
     return outer, shape[axis], inner
 
 
+# quantized element types: name -> (kind of the C ABI, torch dtype that stores the bits)
+QUANT_KINDS = {"int8": (0, torch.int8), "uint8": (1, torch.uint8), "int16": (2, torch.int16),
+               "uint16": (3, torch.int16), "int32": (4, torch.int32), "uint32": (5, torch.int32)}
+
+
+def _quant_kind(dtype):
+    if isinstance(dtype, str):
+        return QUANT_KINDS[dtype]
+    name = str(dtype).replace("torch.", "")
+    kind, _ = QUANT_KINDS[name]
+    return kind, dtype
+
+
 def quantize(x, scale, zero_point, axis=None, qmin=-128, qmax=127,
              round_mode=ROUND_HALF_TO_EVEN, dtype=torch.int8, out=None):
-    """mhlo_disc.quantize on the GPU.  scale/zero_point: device tensors (f32 / i32)."""
+    """mhlo_disc.quantize on the GPU.  scale/zero_point: device tensors (f32 / i32); x: f32 or
+    f16.  dtype: a torch dtype or one of the names in QUANT_KINDS -- the unsigned 16 / 32 bit
+    types are returned in the signed torch dtype of the same width (same bits)."""
     _need_cuda(x, scale, zero_point)
+    if x.dtype not in (torch.float32, torch.float16):
+        raise TypeError("quantize takes f32 or f16 input")
     x = x.contiguous()
     outer, nch, inner = _view3(tuple(x.shape), axis)
+    if out is not None and not isinstance(dtype, str):
+        dtype = out.dtype
+    kind, store = _quant_kind(dtype)
     if out is None:
-        out = torch.empty(x.shape, dtype=dtype, device=x.device)
-    kind = 0 if out.dtype == torch.int8 else 1
+        out = torch.empty(x.shape, dtype=store, device=x.device)
     n_q = scale.numel() if axis is not None else 1
-    st = _lib.lib().dq8_quantize(_ptr(x), _ptr(out), kind, outer, nch, inner, _ptr(scale),
-                                 _ptr(zero_point), n_q, qmin, qmax, round_mode, _stream())
+    st = _lib.lib().dq8_quantize_ex(_ptr(x), 0 if x.dtype == torch.float32 else 1, _ptr(out), kind,
+                                    outer, nch, inner, _ptr(scale), _ptr(zero_point), n_q,
+                                    int(qmin), int(qmax), round_mode, _stream())
     _lib.check(st, "dq8_quantize")
     return out
 
@@ -180,16 +200,18 @@ def activation_table(fn, s_in, z_in, s_out, z_out, in_dtype=torch.int8, out_dtyp
     return quantize(y, s_out, z_out, qmin=qmin, qmax=qmax, dtype=out_dtype)
 
 
-def dequantize(q, scale, zero_point, axis=None, out=None):
+def dequantize(q, scale, zero_point, axis=None, out=None, dtype=None):
+    """mhlo_disc.dequantize on the GPU; dtype names the quantized type where q's torch dtype
+    does not (the unsigned 16 / 32 bit types, see QUANT_KINDS)."""
     _need_cuda(q, scale, zero_point)
     q = q.contiguous()
     outer, nch, inner = _view3(tuple(q.shape), axis)
     if out is None:
         out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
-    kind = 0 if q.dtype == torch.int8 else 1
+    kind, _ = _quant_kind(dtype if dtype is not None else q.dtype)
     n_q = scale.numel() if axis is not None else 1
-    st = _lib.lib().dq8_dequantize(_ptr(q), kind, _ptr(out), outer, nch, inner, _ptr(scale),
-                                   _ptr(zero_point), n_q, _stream())
+    st = _lib.lib().dq8_dequantize_ex(_ptr(q), kind, _ptr(out), outer, nch, inner, _ptr(scale),
+                                      _ptr(zero_point), n_q, _stream())
     _lib.check(st, "dq8_dequantize")
     return out
 

@@ -26,7 +26,8 @@ def _torch_code(dtype):
         import torch
         _TORCH_CODES = {torch.int8: "i8", torch.uint8: "ui8", torch.int32: "i32",
                         torch.int64: "i64", torch.float32: "f32", torch.float64: "f64",
-                        torch.bool: "i1", torch.float16: "f16", torch.bfloat16: "bf16"}
+                        torch.bool: "i1", torch.float16: "f16", torch.bfloat16: "bf16",
+                        torch.int16: "i16"}
     return _TORCH_CODES[dtype]
 
 

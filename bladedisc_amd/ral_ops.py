@@ -197,22 +197,31 @@ def conv2d_plan(in_shape, w_shape, data_format, strides, dilations, padding,
 
 
 def quantize(ex, x, scale, zp, axis=None, qmin=-128, qmax=127, round_mode=1, out=None,
-             dtype=torch.int8):
+             dtype=torch.int8, code=None):
+    """ral_quantize; `code` names the result's element type in the mangled symbol where the
+    torch dtype that stores the bits does not ("ui16" / "ui32" in int16 / int32 storage)."""
     if out is None:
         out = torch.empty(x.shape, dtype=dtype, device=x.device)
     a = ex.new_args().tensor(x)
     a.tensor(scale, rank0=axis is None).tensor(zp, rank0=axis is None)
-    a.tensor(out)
+    if code is None:
+        a.tensor(out)
+    else:
+        a.memref(code, out.data_ptr(), list(out.shape), list(out.stride()))
     a.scalar("i64", -1 if axis is None else axis).scalar("i64", qmin).scalar("i64", qmax)
     a.scalar("i64", round_mode)
     ex.call("ral_quantize", "gpu", a)
     return out
 
 
-def dequantize(ex, q, scale, zp, axis=None, out=None):
+def dequantize(ex, q, scale, zp, axis=None, out=None, code=None):
     if out is None:
         out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
-    a = ex.new_args().tensor(q)
+    a = ex.new_args()
+    if code is None:
+        a.tensor(q)
+    else:
+        a.memref(code, q.data_ptr(), list(q.shape), list(q.stride()))
     a.tensor(scale, rank0=axis is None).tensor(zp, rank0=axis is None)
     a.tensor(out)
     a.scalar("i64", -1 if axis is None else axis)

@@ -71,8 +71,16 @@ extern "C" {
 #define DQ8_BIAS_S8 3  /* REQUANT_GPU: (float)bias                                          */
 
 /* element kinds of quantized tensors */
+/* floating-point element types (dq8_quantize_ex, dq8_weight_only_qgemm) */
+#define DQ8_DTYPE_F32 0
+#define DQ8_DTYPE_F16 1
 #define DQ8_I8 0
 #define DQ8_U8 1
+/* (dq8_quantize_ex / dq8_dequantize_ex only) */
+#define DQ8_I16 2
+#define DQ8_U16 3
+#define DQ8_I32 4
+#define DQ8_U32 5
 
 /* mhlo_disc round_mode (R disc/IR/hlo_disc_enums.td) */
 #define DQ8_ROUND_HALF_AWAY_FROM_ZERO 0
@@ -143,6 +151,20 @@ int dq8_quantize(const float* x, void* out, int out_kind, int64_t outer,
 int dq8_dequantize(const void* q, int in_kind, float* out, int64_t outer,
                    int64_t nch, int64_t inner, const float* scale,
                    const int32_t* zp, int64_t n_q, void* stream);
+
+/* dq8_quantize / dq8_dequantize for every quantized type the reference's operator takes
+ * (i8, ui8, i16, ui16, i32, ui32: R disc/transforms/tests/disc-fold-quantize.mlir:48-247) and,
+ * beyond the reference (whose lowering refuses anything but f32 input,
+ * R disc/transforms/disc_lower_quantize_and_dequantize.cc:46-48), f16 input, which is widened
+ * to f32 exactly before the same steps.  x_dtype: DQ8_DTYPE_*; kinds: DQ8_I8 .. DQ8_U32.  The
+ * conversion of the clamped f32 value saturates (the f32 images of 2^31 - 1 and 2^32 - 1 lie
+ * one past the integer range).  f32 -> 8-bit forwards to dq8_quantize. */
+int dq8_quantize_ex(const void* x, int x_dtype, void* out, int out_kind, int64_t outer,
+                    int64_t nch, int64_t inner, const float* scale, const int32_t* zp,
+                    int64_t n_q, int64_t qmin, int64_t qmax, int round_mode, void* stream);
+int dq8_dequantize_ex(const void* q, int in_kind, float* out, int64_t outer, int64_t nch,
+                      int64_t inner, const float* scale, const int32_t* zp, int64_t n_q,
+                      void* stream);
 
 /* Fake quantization: dq8_dequantize(dq8_quantize(x)) in one pass, f32 -> f32, without
  * the integer tensor in between; bit for bit the result of the two calls (what the
@@ -286,9 +308,6 @@ int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
                      int64_t cols, void* stream);
 
 /* ---- weight-only quantized GEMM ----------------------------------------- */
-
-#define DQ8_DTYPE_F32 0
-#define DQ8_DTYPE_F16 1
 
 /* out[m,n] = (sum_k x[m,k] * (w(n,k) - zero_points[n])) * scale[n] + bias[n]: floating-point
  * activations times 8-bit weights with a per-output-channel scale and zero point, i.e.

@@ -382,8 +382,11 @@ static void store_q(void* out, int64_t i, int kind, double v) {
     case Q8O_U8: ((uint8_t*)out)[i] = (uint8_t)v; break;
     case Q8O_I16: ((int16_t*)out)[i] = (int16_t)v; break;
     case Q8O_U16: ((uint16_t*)out)[i] = (uint16_t)v; break;
-    case Q8O_I32: ((int32_t*)out)[i] = (int32_t)v; break;
-    default: ((uint32_t*)out)[i] = (uint32_t)v; break;
+    /* the f32 images of the 32-bit limits lie one past the integer range (2^31, 2^32): the
+     * conversion of such a clamped value saturates -- this build's definition, the
+     * reference's mhlo.convert leaves it undefined */
+    case Q8O_I32: ((int32_t*)out)[i] = v >= 2147483648.0 ? INT32_MAX : (int32_t)v; break;
+    default: ((uint32_t*)out)[i] = v >= 4294967296.0 ? UINT32_MAX : (uint32_t)v; break;
   }
 }
 

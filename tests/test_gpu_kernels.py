@@ -554,16 +554,64 @@ def test_fake_quant_equals_quantize_then_dequantize(K, shape, axis, round_mode, 
 
 
 def test_quantize_golden_vectors(K, golden):
+    """Every vector of disc-fold-quantize.mlir, all six quantized types (the unsigned 16 / 32
+    bit results come back as bits in the signed torch dtype of the same width)."""
+    seen = set()
     for case in golden["quantize_fold"]:
-        if case["dtype"] not in ("int8", "uint8"):
-            continue
         x = np.array(case["x"], np.float32)
-        dt = torch.int8 if case["dtype"] == "int8" else torch.uint8
         got = host(K.quantize(dev(x), dev(np.array(case["scale"], np.float32)),
                               dev(np.array(case["zp"], np.int32)), axis=case["axis"],
                               qmin=case["qmin"], qmax=case["qmax"], round_mode=case["round_mode"],
-                              dtype=dt))
-        np.testing.assert_array_equal(got, np.array(case["expect"], case["dtype"]), err_msg=case["src"])
+                              dtype=case["dtype"]))
+        np.testing.assert_array_equal(got.view(case["dtype"]), np.array(case["expect"], case["dtype"]),
+                                      err_msg=case["src"])
+        seen.add(case["dtype"])
+    assert seen == {"int8", "uint8", "int16", "uint16", "int32", "uint32"}
+
+
+@pytest.mark.parametrize("name", ["int16", "uint16", "int32", "uint32"])
+@pytest.mark.parametrize("axis", [None, 0, 1])
+def test_quantize_dequantize_wide_types(K, name, axis):
+    """16- and 32-bit quantized types against the oracle: values that land inside the range,
+    on both limits and beyond them (the conversion of the clamped value saturates), both
+    rounding modes, per tensor and per channel; dequantize back."""
+    rng = np.random.default_rng(len(name) + (axis or 0) * 7)
+    npdt = np.dtype(name)
+    info = np.iinfo(npdt)
+    shape = (37, 24)
+    nq = 1 if axis is None else shape[axis]
+    scale = rng.uniform(0.001, 0.01, nq).astype(np.float32)
+    zp = rng.integers(-50, 50, nq).astype(np.int32) if info.min < 0 else rng.integers(0, 100, nq).astype(np.int32)
+    span = float(info.max) * float(scale.mean())
+    x = (rng.standard_normal(shape) * span * 0.6).astype(np.float32)
+    x[0, :4] = [span * 4, -span * 4, span, -span]
+    for rm in (0, 1):
+        want = O.quantize(x, scale, zp, axis=axis, qmin=int(info.min), qmax=int(info.max),
+                          round_mode=rm, dtype=npdt)
+        got = K.quantize(dev(x), dev(scale), dev(zp), axis=axis, qmin=int(info.min),
+                         qmax=int(info.max), round_mode=rm, dtype=name)
+        np.testing.assert_array_equal(host(got).view(npdt), want)
+        assert (want == info.max).any() and (want == info.min).any()
+    back = K.dequantize(got, dev(scale), dev(zp), axis=axis, dtype=name)
+    want_f = O.dequantize(want, scale, zp, axis=axis)
+    assert np.array_equal(host(back).view(np.uint32), want_f.view(np.uint32))
+
+
+@pytest.mark.parametrize("name", ["int8", "uint8", "int16"])
+def test_quantize_f16_input_is_the_f32_path_on_the_widened_values(K, name):
+    """Half-precision input (an extension: the reference's lowering takes f32 only) is widened
+    exactly and then quantized by the f32 steps."""
+    rng = np.random.default_rng(3)
+    npdt = np.dtype(name)
+    info = np.iinfo(npdt)
+    x16 = (rng.standard_normal((50, 33)) * 3).astype(np.float16)
+    scale = rng.uniform(0.01, 0.05, 33).astype(np.float32)
+    zp = np.full(33, int((int(info.min) + int(info.max) + 1) // 2), np.int32)
+    want = O.quantize(x16.astype(np.float32), scale, zp, axis=1, qmin=int(info.min),
+                      qmax=int(info.max), dtype=npdt)
+    got = K.quantize(dev(x16), dev(scale), dev(zp), axis=1, qmin=int(info.min), qmax=int(info.max),
+                     dtype=name)
+    np.testing.assert_array_equal(host(got).view(npdt), want)
 
 
 def test_quantize_unaligned_and_uint8(K):

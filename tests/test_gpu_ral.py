@@ -402,6 +402,24 @@ def test_ral_quantize_dequantize(rt, shape, axis):
         np.testing.assert_array_equal(host(f), O.dequantize(want, scale, zp, axis=axis))
 
 
+@pytest.mark.parametrize("name,code,store", [("int16", None, torch.int16), ("uint16", "ui16", torch.int16),
+                                             ("int32", None, torch.int32), ("uint32", "ui32", torch.int32)])
+def test_ral_quantize_dequantize_wide_types(rt, name, code, store):
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(11)
+    info = np.iinfo(name)
+    x = (rng.standard_normal((33, 20)) * 30).astype(np.float32)
+    scale = rng.uniform(0.002, 0.01, 20).astype(np.float32)
+    zp = rng.integers(0, 40, 20).astype(np.int32)
+    with ctx.execution() as ex:
+        q = ops.quantize(ex, dev(x), dev(scale), dev(zp), axis=1, qmin=int(info.min),
+                         qmax=int(info.max), dtype=store, code=code)
+        want = O.quantize(x, scale, zp, axis=1, qmin=int(info.min), qmax=int(info.max), dtype=np.dtype(name))
+        np.testing.assert_array_equal(host(q).view(name), want)
+        f = ops.dequantize(ex, q, dev(scale), dev(zp), axis=1, code=code)
+        np.testing.assert_array_equal(host(f), O.dequantize(want, scale, zp, axis=1))
+
+
 def test_driver_alloc_copy_roundtrip_and_pool_reuse(rt):
     ctx, ral, ops = rt
     import ctypes as C
