@@ -87,3 +87,43 @@ def test_running_min_max_and_bias_scale():
     np.testing.assert_array_equal(hi, [4.0, 3.0])
     np.testing.assert_array_equal(OB.bias_scale(np.array([0.5, 0.25], np.float32), np.float32(0.1)),
                                   np.array([0.5, 0.25], np.float32) * np.float32(0.1))
+
+
+def test_fake_quant_against_torch_fake_quantize():
+    """The observers' fake quantization here is quantize -> dequantize as a compiled program
+    executes it (x / scale, a true division); the reference's observer calls
+    torch.fake_quantize_per_{tensor,channel}_affine (observer.py:203-206), which multiplies
+    by 1 / scale.  On the CPU, against torch itself: the two agree wherever x / scale + zp is
+    not within a few ulp of a rounding tie, never differ by more than one quantization step,
+    and on random data differ on fewer than one element in a thousand."""
+    import torch
+    import oracle as O
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((64, 96)) * 2).astype(np.float32)
+    # per tensor, symmetric int8 and affine uint8
+    for (scale, zp, qmin, qmax, dt) in ((0.0173, 0, -128, 127, np.int8), (0.031, 117, 0, 255, np.uint8)):
+        q = O.quantize(x, np.float32(scale), zp, qmin=qmin, qmax=qmax, dtype=dt)
+        mine = O.dequantize(q, np.float32(scale), zp)
+        ref = torch.fake_quantize_per_tensor_affine(torch.from_numpy(x), scale, zp, qmin, qmax).numpy()
+        diff = np.abs(mine - ref)
+        assert diff.max() <= np.float32(scale) * 1.0001
+        t = x.astype(np.float64) / np.float32(scale) + zp
+        near_tie = np.abs(np.abs(t - np.floor(t)) - 0.5) < 1e-4
+        assert not (diff[~near_tie] > 0).any()
+        assert (diff > 0).mean() < 1e-3
+    # per channel (axis 0), the weight observers' form
+    scale = rng.uniform(0.005, 0.03, 64).astype(np.float32)
+    zp = np.zeros(64, np.int32)
+    q = O.quantize(x, scale, zp, axis=0)
+    mine = O.dequantize(q, scale, zp, axis=0)
+    ref = torch.fake_quantize_per_channel_affine(torch.from_numpy(x), torch.from_numpy(scale),
+                                                 torch.from_numpy(zp), 0, -128, 127).numpy()
+    diff = np.abs(mine - ref)
+    assert (diff <= scale[:, None] * 1.0001).all() and (diff > 0).mean() < 1e-3
+    # an exact tie where the two really part: x / s is a tie in exact arithmetic, x * (1 / s)
+    # need not be
+    s = np.float32(0.1)
+    xt = (np.arange(1, 200, 2, dtype=np.float32) * np.float32(0.05)).astype(np.float32)
+    q = O.quantize(xt, s, 0)
+    ref = torch.fake_quantize_per_tensor_affine(torch.from_numpy(xt), float(s), 0, -128, 127).numpy()
+    assert np.abs(O.dequantize(q, s, 0) - ref).max() <= s * 1.0001
