@@ -45,6 +45,8 @@ _PROTOS = {
                               C.POINTER(_I32), _VP, C.POINTER(_I64), _INT, _VP, _INT, _VP,
                               _VP, _I64, _VP, _I32, _VP, _SZ, _VP]),
     "dq8_qconv2d_workspace_bytes": (_SZ, [C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I32)]),
+    "dq8_qconv2d_workspace_bytes_ex": (_SZ, [C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I64),
+                                             C.POINTER(_I32)]),
     "dq8_mfma_probe": (_INT, [_VP] * 7),
     "dq8_lut8": (_INT, [_VP, _VP, _I64, _VP, _VP]),
     "dq8_weight_only_qgemm_workspace_bytes": (C.c_size_t, [_I64, _I64, _INT]),

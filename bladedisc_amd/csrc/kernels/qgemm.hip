@@ -118,6 +118,39 @@ transpose_s8_kernel(const int8_t* __restrict__ src, int64_t ld, int8_t* __restri
   }
 }
 
+// dst[b][c][r] = src[b][r][c] for B dense matrices [R, C] of 1- or 4-byte elements (layout
+// changes between NCHW and NHWC, OIHW and OHWI); 32x32 tiles through LDS
+template <typename T>
+__global__ void __launch_bounds__(256)
+transpose_batched_kernel(const T* __restrict__ src, T* __restrict__ dst, int R, int C,
+                         int tiles_c) {
+  __shared__ T tile[32][33];
+  const int64_t base = (int64_t)blockIdx.y * R * C;
+  const int r0 = (blockIdx.x / tiles_c) * 32, c0 = (blockIdx.x % tiles_c) * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int i = ty; i < 32; i += 8) {
+    const int r = r0 + i, c = c0 + tx;
+    if (r < R && c < C) tile[i][tx] = src[base + (int64_t)r * C + c];
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    const int c = c0 + i, r = r0 + tx;
+    if (c < C && r < R) dst[base + (int64_t)c * R + r] = tile[tx][i];
+  }
+}
+
+template <typename T>
+int transpose_batched(const void* src, void* dst, int64_t B, int64_t R, int64_t C,
+                      hipStream_t st) {
+  if (B == 0 || R == 0 || C == 0) return 0;
+  const int64_t tiles_c = ceil_div(C, 32), tiles = ceil_div(R, 32) * tiles_c;
+  DQ8_REQUIRE(B <= 65535 && tiles < (1LL << 31), "layout change: tensor too large");
+  hipLaunchKernelGGL(transpose_batched_kernel<T>, dim3((unsigned)tiles, (unsigned)B), dim3(256), 0,
+                     st, static_cast<const T*>(src), static_cast<T*>(dst), (int)R, (int)C,
+                     (int)tiles_c);
+  return check_hip(hipGetLastError(), "layout change launch");
+}
+
 // int8 [R, C] (row stride ld, any alignment) -> [R, ldd], ldd % 16 == 0 and dst 16-byte
 // aligned, columns C .. ldd-1 zero.  One 16-byte store per thread and step.
 __global__ void __launch_bounds__(256)
@@ -694,7 +727,20 @@ bool is_nhwc_ohwi(const int32_t md[17]) {
   return true;
 }
 
+bool is_nchw_oihw(const int32_t md[17]) {
+  static const int32_t want[12] = {0, 1, 2, 3, 1, 0, 2, 3, 0, 1, 2, 3};
+  for (int i = 0; i < 12; ++i)
+    if (md[i] != want[i]) return false;
+  return true;
+}
+
 size_t pad256(int64_t v) { return (size_t)((v + 255) / 256 * 256); }
+
+int out_elem_size(int epilogue) {
+  return (epilogue == DQ8_EPI_ACC_S32 || epilogue == DQ8_EPI_DEQUANT_F32 ||
+          epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || epilogue == DQ8_EPI_REQUANT_GPU_DEQUANT_F32)
+             ? 4 : 1;
+}
 
 int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                  const int64_t w_sizes[4], const int32_t padding[4], const int32_t md[17],
@@ -733,6 +779,44 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   DQ8_REQUIRE(Ho == out_len(H, padding[0], padding[1], Kh, dh, sh) &&
                   Wo == out_len(Wd, padding[2], padding[3], Kw, dw, sw_),
               "dq8_qconv2d: output spatial size inconsistent with padding/stride/dilation");
+  // NCHW x OIHW -> NCHW (the PyTorch layouts): with scratch, the input and the weights are
+  // re-laid out as NHWC / OHWI, the convolution runs on the MFMA kernels into an NHWC scratch
+  // result, and that is turned back into NCHW -- what the reference's GPU path does around its
+  // NHWC-only int8 kernels (R ral/context/stream_executor_based_impl.cc:1073-1112).  Without
+  // scratch (or with a fused residual, which has the output's layout) the generic kernel reads
+  // the tensors in place.
+  if (is_nchw_oihw(md) && variant != 0 && workspace != nullptr && aligned(workspace, 256) &&
+      !(post && post->residual_kind != DQ8_RESIDUAL_NONE) &&
+      epilogue >= DQ8_EPI_ACC_S32 && epilogue <= DQ8_EPI_REQUANT_FIXEDPOINT) {
+    const int64_t Mo = NB * out_sizes[2] * out_sizes[3];
+    const int es = out_elem_size(epilogue);
+    const size_t in_b = pad256(NB * H * Wd * Ci), w_b = pad256(Co * Kh * Kw * Ci);
+    const size_t out_b = pad256(Mo * Co * es);
+    if (workspace_bytes >= in_b + w_b + out_b && Mo > 0 && Co > 0 && in && w && out) {
+      hipStream_t st0 = (hipStream_t)stream;
+      int8_t* in_t = static_cast<int8_t*>(workspace);
+      int8_t* w_t = in_t + in_b;
+      uint8_t* out_t = reinterpret_cast<uint8_t*>(w_t + w_b);
+      if (int s = transpose_batched<int8_t>(in, in_t, NB, Ci, H * Wd, st0)) return s;
+      if (int s = transpose_batched<int8_t>(w, w_t, Co, Ci, Kh * Kw, st0)) return s;
+      const int64_t in2[4] = {NB, H, Wd, Ci}, w2[4] = {Co, Kh, Kw, Ci};
+      const int64_t out2[4] = {NB, out_sizes[2], out_sizes[3], Co};
+      int32_t md2[17];
+      static const int32_t nhwc[12] = {0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2};
+      for (int i = 0; i < 12; ++i) md2[i] = nhwc[i];
+      for (int i = 12; i < 17; ++i) md2[i] = md[i];
+      const size_t used = in_b + w_b + out_b;
+      if (int s = qconv2d_impl(variant, in_t, in2, w_t, w2, padding, md2, out_t, out2, epilogue, bias,
+                               bias_kind, sx, sw, n_sw, so, zo,
+                               static_cast<uint8_t*>(workspace) + used, workspace_bytes - used,
+                               stream, post))
+        return s;
+      const int64_t pix = out_sizes[2] * out_sizes[3];
+      return es == 4 ? transpose_batched<uint32_t>(out_t, out, NB, pix, Co, st0)
+                     : transpose_batched<int8_t>(out_t, out, NB, pix, Co, st0);
+    }
+  }
+
   // requant -> dequantize in one epilogue, as in dq8_qgemm
   int requant = 0;
   if (epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || epilogue == DQ8_EPI_REQUANT_GPU_DEQUANT_F32) {
@@ -908,14 +992,34 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
 
 }  // namespace
 
-extern "C" size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const int64_t w_sizes[4],
-                                              const int32_t metadata[17]) {
-  if (!in_sizes || !w_sizes || !metadata || !is_nhwc_ohwi(metadata)) return 0;
+extern "C" size_t dq8_qconv2d_workspace_bytes_ex(const int64_t in_sizes[4],
+                                                 const int64_t w_sizes[4],
+                                                 const int64_t out_sizes[4],
+                                                 const int32_t metadata[17]) {
+  if (!in_sizes || !w_sizes || !metadata) return 0;
+  if (is_nchw_oihw(metadata)) {
+    // NHWC copies of input and weights, an NHWC result of up to 4 bytes per element, and what
+    // the NHWC convolution may want for itself
+    if (!out_sizes) return 0;
+    const int64_t ci = in_sizes[1], cip = (ci + 15) / 16 * 16;
+    const int64_t in_e = in_sizes[0] * in_sizes[2] * in_sizes[3];
+    const int64_t w_e = w_sizes[0] * w_sizes[2] * w_sizes[3];
+    size_t need = pad256(in_e * ci) + pad256(w_e * ci) +
+                  pad256(out_sizes[0] * out_sizes[1] * out_sizes[2] * out_sizes[3] * 4);
+    if (ci % 16 != 0) need += pad256(in_e * cip) + pad256(w_e * cip);
+    return need;
+  }
+  if (!is_nhwc_ohwi(metadata)) return 0;
   const int64_t ci = in_sizes[3];
   if (ci % 16 == 0) return 0;
   const int64_t cip = (ci + 15) / 16 * 16;
   return pad256(in_sizes[0] * in_sizes[1] * in_sizes[2] * cip) +
          pad256(w_sizes[0] * w_sizes[1] * w_sizes[2] * cip);
+}
+
+extern "C" size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const int64_t w_sizes[4],
+                                              const int32_t metadata[17]) {
+  return dq8_qconv2d_workspace_bytes_ex(in_sizes, w_sizes, nullptr, metadata);
 }
 
 extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t in_sizes[4],

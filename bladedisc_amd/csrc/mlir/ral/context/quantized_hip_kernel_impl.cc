@@ -850,9 +850,11 @@ void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4>
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return;
   void* stream = drv->asCUStream(ctx, stream_handle);
-  // (scratch for channel counts that are not a multiple of 16; handed back to the pool
+  // (scratch for channel counts that are not a multiple of 16 and for the NHWC copies of
+  // NCHW tensors; handed back to the pool
   // right after the launch, which later work on the same stream is ordered behind)
-  const size_t ws_bytes = dq8_qconv2d_workspace_bytes(input.sizes, kernel.sizes, metadata.data);
+  const size_t ws_bytes =
+      dq8_qconv2d_workspace_bytes_ex(input.sizes, kernel.sizes, output.sizes, metadata.data);
   void* ws = ws_bytes ? drv->alloc(ctx, ws_bytes) : nullptr;
   if (ws_bytes && !ws) return;
   StreamTimer timer(stream);
@@ -947,7 +949,8 @@ MemRefType<int8_t, 4> ral_pdll_qconv2d(ExecutionContext* ctx, void* stream_handl
   result = assignMemRef<int8_t, 4>(data, plan.result_sizes);
   void* stream = drv->asCUStream(ctx, stream_handle);
   const int32_t zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
-  const size_t ws_bytes = dq8_qconv2d_workspace_bytes(input.sizes, weight.sizes, plan.metadata);
+  const size_t ws_bytes = dq8_qconv2d_workspace_bytes_ex(input.sizes, weight.sizes,
+                                                         plan.result_sizes, plan.metadata);
   void* ws = ws_bytes ? drv->alloc(ctx, ws_bytes) : nullptr;
   if (ws_bytes && !ws) return result;
   StreamTimer timer(stream);

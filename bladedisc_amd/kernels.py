@@ -315,7 +315,7 @@ def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=N
     bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
     i64x4 = C.c_int64 * 4
     md = (C.c_int32 * 17)(*metadata)
-    ws_bytes = L.dq8_qconv2d_workspace_bytes(i64x4(*x.shape), i64x4(*w.shape), md) if workspace else 0
+    ws_bytes = L.dq8_qconv2d_workspace_bytes_ex(i64x4(*x.shape), i64x4(*w.shape), i64x4(*out_shape), md) if workspace else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     args = (_ptr(x), i64x4(*x.shape), _ptr(w), i64x4(*w.shape),
             (C.c_int32 * 4)(*padding), md, _ptr(out),

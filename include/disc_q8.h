@@ -353,6 +353,13 @@ int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
  * generic kernel.  dq8_qconv2d_workspace_bytes() is 0 when nothing would be rewritten. */
 size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const int64_t w_sizes[4],
                                    const int32_t metadata[17]);
+/* The same with the result's sizes: additionally covers NCHW x OIHW -> NCHW convolutions, whose
+ * tensors are re-laid out as NHWC / OHWI in the scratch so that they run on the MFMA kernels
+ * (what the reference's GPU path does around its NHWC int8 kernels,
+ * R ral/context/stream_executor_based_impl.cc:1073-1112); without the scratch they take the
+ * generic kernel. */
+size_t dq8_qconv2d_workspace_bytes_ex(const int64_t in_sizes[4], const int64_t w_sizes[4],
+                                      const int64_t out_sizes[4], const int32_t metadata[17]);
 int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                    const int64_t w_sizes[4], const int32_t padding[4],
                    const int32_t metadata[17], void* out, const int64_t out_sizes[4],

@@ -854,6 +854,42 @@ def test_qconv_nchw_oihw_generic(K):
     np.testing.assert_array_equal(got, acc)
 
 
+@pytest.mark.parametrize("nb,ci,h,w_,co,k,stride,pad,dil", [(2, 32, 14, 14, 48, 3, 1, 1, 1), (3, 24, 9, 11, 40, 3, 2, 1, 1),
+                                                         (1, 64, 28, 28, 64, 1, 1, 0, 1), (2, 16, 12, 12, 20, 3, 1, 2, 2)])
+def test_qconv_nchw_oihw_on_the_mfma_path(K, nb, ci, h, w_, co, k, stride, pad, dil):
+    """NCHW x OIHW -> NCHW with scratch: tensors re-laid out as NHWC / OHWI, MFMA kernels, result
+    turned back -- the same bits as the oracle and as the generic kernel without scratch, for
+    every epilogue family (int8, int32 and f32 results)."""
+    rng = np.random.default_rng(ci + co + h)
+    x = rng.integers(-128, 128, (nb, ci, h, w_), dtype=np.int8)
+    wt = rng.integers(-128, 128, (co, ci, k, k), dtype=np.int8)
+    ho = (h + 2 * pad - dil * (k - 1) - 1) // stride + 1
+    wo = (w_ + 2 * pad - dil * (k - 1) - 1) // stride + 1
+    md = [0, 1, 2, 3, 1, 0, 2, 3, 0, 1, 2, 3, stride, stride, dil, dil, 1]
+    padding, osh = [pad] * 4, [nb, co, ho, wo]
+    acc = O.conv_s32(x, wt, padding, md, osh)
+    for ws in (True, False):
+        got = host(K.qconv2d(dev(x), dev(wt), padding, md, osh, K.EPI_ACC_S32, workspace=ws))
+        np.testing.assert_array_equal(got, acc)
+    sx, sw = make_scales(rng, co)
+    so = pick_so(acc, sx, sw)
+    sc = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so], np.float32)))
+    per_c = lambda a: np.moveaxis(a, 1, -1).reshape(-1, co)                      # noqa: E731
+    back = lambda a: np.moveaxis(a.reshape(nb, ho, wo, co), -1, 1)               # noqa: E731
+    want = back(O.requant_cpu(per_c(acc), sx, sw, so))
+    got = host(K.qconv2d(dev(x), dev(wt), padding, md, osh, K.EPI_REQUANT_CPU, **sc))
+    np.testing.assert_array_equal(got, want)
+    b32 = rng.integers(-100000, 100000, co).astype(np.int32)
+    want = back(O.requant_fixedpoint(per_c(acc), sx, sw, so, b32=b32, zo=3))
+    got = host(K.qconv2d(dev(x), dev(wt), padding, md, osh, K.EPI_REQUANT_FIXEDPOINT, bias=dev(b32),
+                         zo=3, **sc))
+    np.testing.assert_array_equal(got, want)
+    got_f = host(K.qconv2d(dev(x), dev(wt), padding, md, osh, K.EPI_REQUANT_CPU_DEQUANT_F32, **sc))
+    want_f = O.dequantize(back(O.requant_cpu(per_c(acc), sx, sw, so)), np.array([so], np.float32),
+                          np.array([0], np.int32))
+    assert np.array_equal(got_f.view(np.uint32), want_f.view(np.uint32))
+
+
 def test_qconv_known_answers(K, golden):
     for case in golden["qconv"]:
         if case["data_format"] != "NHWC":
