@@ -246,7 +246,7 @@ __global__ void __launch_bounds__(WM* WN * 64) qconv3x3_direct_kernel(const Dire
 }
 
 // ---- host side (qconv_direct.hip)
-constexpr int kNumDirectConvConfigs = 2;
+constexpr int kNumDirectConvConfigs = 3;
 
 // Tile shape of configuration `config` (0 .. kNumDirectConvConfigs - 1).
 void direct_conv_tile(int config, int* bm, int* bn);

@@ -17,7 +17,7 @@ constexpr int kStages = 4;
 struct Tile {
   int bm, bn;
 };
-const Tile kTiles[kNumDirectConvConfigs] = {{256, 64}, {128, 64}};
+const Tile kTiles[kNumDirectConvConfigs] = {{256, 64}, {128, 64}, {512, 64}};
 
 template <int BM, int BN, int WM, int WN, int EPI>
 int launch_t(const DirectConvParams& p, hipStream_t st) {
@@ -36,6 +36,7 @@ int launch_config(int config, const DirectConvParams& p, hipStream_t st) {
   switch (config) {
     case 0: return launch_t<256, 64, 4, 1, EPI>(p, st);
     case 1: return launch_t<128, 64, 2, 2, EPI>(p, st);
+    case 2: return launch_t<512, 64, 8, 1, EPI>(p, st);
   }
   return fail("direct convolution: unknown configuration");
 }

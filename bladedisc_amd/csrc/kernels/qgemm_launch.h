@@ -51,6 +51,9 @@ inline constexpr Variant kVariants[] = {
     // a quarter of the compute units idle
     {"pipe_256x192x128_w8", 256, 192, 128, 512},
     {"persist_256x192x128_w8", 256, 192, 128, 512},
+    // the third direct-convolution tile: 512 pixels on eight waves, one workgroup per compute
+    // unit (convolution only)
+    {"direct3x3_512x64", 512, 64, 128, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
@@ -59,6 +62,7 @@ constexpr int kDirectConv0 = 10;   // first of the kNumDirectConvConfigs direct 
 constexpr int kPipe256w8 = 12, kPipe128w8 = 13;
 constexpr int kPersist256 = 14, kPersist128 = 15;
 constexpr int kPipe256x192 = 16, kPersist256x192 = 17;
+constexpr int kDirectConv2 = 18;   // the third direct variant (configuration 2)
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 
