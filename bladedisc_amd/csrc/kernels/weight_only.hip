@@ -23,6 +23,7 @@
 // the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes (one dwordx4), 16
 // activations -- and feeds two MFMAs with them.
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), for M above 128;
+//  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
 //  * wo_skinny_kernel: M <= 128 rows against 32 output channels per workgroup, the k range dealt
 //    over the waves and the partial sums added through LDS (bound by the weight bytes: 1 byte
 //    per weight from HBM);
@@ -279,6 +280,73 @@ __global__ void __launch_bounds__(NW * 64) wo_skinny_kernel(const WoParams p) {
   }
 }
 
+// ---------------------------------------------------------------- M <= 16
+// 16 output channels per workgroup on v_mfma_f32_16x16x32_f16: twice as many workgroups as the
+// 32-channel form for the same weights (a 4096 x 4096 weight gives 256 instead of 128), and a
+// lane (row, g) takes the 16 consecutive k values k0 + 16 g .. of a 64-deep chunk, so a wave's
+// load covers 64 contiguous bytes of each of its 16 weight rows.
+typedef float f4v __attribute__((ext_vector_type(4)));
+
+template <typename XT, int NW>
+__global__ void __launch_bounds__(NW * 64) wo_skinny16_kernel(const WoParams p) {
+  __shared__ float red[NW - 1][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int n = min(n0 + r, p.N - 1);
+  const XT* xrow = static_cast<const XT*>(p.x) + (int64_t)min(r, p.M - 1) * p.ldx + 16 * g;
+  const uint8_t* wrow = p.w + (int64_t)n * p.w_sn + 16 * g;
+  const h2 c = centre(p, n);
+  f4v acc = {0.f, 0.f, 0.f, 0.f};
+  const u4 zero = {0, 0, 0, 0};
+  constexpr int U = 4;
+  for (int k0 = wave * 64; k0 < p.K; k0 += U * NW * 64) {
+    XFrag<XT> xf[U];
+    u4 wf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k0 + u * NW * 64;
+      const bool valid = kk + 16 * g < p.K;              // K % 16 == 0: whole 16-chunks
+      const int k = valid ? kk : 0;
+      wf[u] = valid ? *reinterpret_cast<const u4*>(wrow + k) : zero;
+      xf[u].load(xrow + k, valid);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      h8 w0, w1;
+      widen16(wf[u], p.flip, c, w0, w1);
+#pragma unroll
+      for (int part = 0; part < XFrag<XT>::kParts; ++part) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[u].step(part, 0), w0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[u].step(part, 1), w1, acc, 0, 0, 0);
+      }
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave - 1][v][lane] = acc[v];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 1; w < NW; ++w)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[v] += red[w - 1][v][lane];
+    // D of the 16x16 MFMA: column n = lane % 16, rows 4 (lane / 16) + v
+    const int nn = n0 + r;
+    if (nn < p.N) {
+      const float s = to_f32(static_cast<const XT*>(p.scale)[nn]);
+      const float b = p.bias ? to_f32(static_cast<const XT*>(p.bias)[nn]) : 0.0f;
+      XT* out = static_cast<XT*>(p.out);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = 4 * g + v;
+        if (m < p.M) out[(int64_t)m * p.ldo + nn] = (XT)(acc[v] * s + b);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- any layout, any alignment
 template <typename XT>
 __global__ void __launch_bounds__(256) wo_generic_kernel(const WoParams p) {
@@ -307,7 +375,12 @@ int launch(const WoParams& p, bool fast, hipStream_t st) {
     hipLaunchKernelGGL(wo_generic_kernel<XT>, dim3((unsigned)blocks), dim3(256), 0, st, p);
   } else if (p.M <= 128) {
     const unsigned grid = (unsigned)ceil_div(p.N, 32);
-    if (p.M <= 32)
+    // (with more than 8 rows every workgroup re-reads the activations, which then outweigh
+    // its weights: the narrow form only while the wide one would leave compute units idle)
+    if (p.M <= 8 || (p.M <= 16 && grid < 256))
+      hipLaunchKernelGGL((wo_skinny16_kernel<XT, 8>), dim3((unsigned)ceil_div(p.N, 16)), dim3(512),
+                         0, st, p);
+    else if (p.M <= 32)
       hipLaunchKernelGGL((wo_skinny_kernel<XT, 8, 1>), dim3(grid), dim3(512), 0, st, p);
     else if (p.M <= 64)
       hipLaunchKernelGGL((wo_skinny_kernel<XT, 8, 2>), dim3(grid), dim3(512), 0, st, p);
