@@ -22,7 +22,10 @@
 // the k values inside a fragment is free as long as both operands agree, so lane (row, g) takes
 // the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes (one dwordx4), 16
 // activations -- and feeds two MFMAs with them.
-//  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), for M above 128;
+//  * wo_lds_kernel: f16 activations, 128 x 128 tiles shared through LDS, once there are about a
+//    hundred of them (0.77-0.85 PFLOP/s at 4096^2 .. 8192^2 weights);
+//  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
+//    f32 activations and problems with few tiles;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
 //  * wo_skinny_kernel: M <= 128 rows against 32 output channels per workgroup, the k range dealt
 //    over the waves and the partial sums added through LDS (bound by the weight bytes: 1 byte
@@ -169,8 +172,11 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  XFrag<XT> xa[FM], xb[FM];
-  u4 wa[FN], wb[FN];
+  // D chunks of 32 in flight per wave (registers permitting: f32 activations take twice the
+  // registers of f16 ones)
+  constexpr int D = sizeof(XT) == 2 ? 4 : 2;
+  XFrag<XT> xr[D][FM];
+  u4 wr[D][FN];
   const u4 zero = {0, 0, 0, 0};
   auto load = [&](XFrag<XT>* xf, u4* wf, int k0) {
     const bool valid = k0 + 16 * g < p.K;                // K % 16 == 0: whole 16-chunks
@@ -196,19 +202,144 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
         }
       }
   };
-  // two chunks per trip, the registers of one being refilled while the other is multiplied
-  load(xa, wa, 0);
-  for (int k0 = 0; k0 < p.K; k0 += 64) {
-    load(xb, wb, k0 + 32);                               // (past K: zeros)
-    compute(xa, wa);
-    load(xa, wa, k0 + 64);
-    compute(xb, wb);
+  // a ring of D chunks: each is multiplied and at once refilled with the chunk D further on,
+  // so D - 1 loads stay in flight under every multiplication (one chunk ahead measured 16 % of
+  // the matrix rate: a wave waited out the whole load latency per chunk)
+#pragma unroll
+  for (int d = 0; d < D; ++d) load(xr[d], wr[d], d * 32);
+  for (int k0 = 0; k0 < p.K; k0 += D * 32) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      compute(xr[d], wr[d]);
+      load(xr[d], wr[d], k0 + (D + d) * 32);             // (past K: zeros)
+    }
   }
 #pragma unroll
   for (int i = 0; i < FM; ++i)
 #pragma unroll
     for (int j = 0; j < FN; ++j)
       store_frag<XT>(p, acc[i][j], m0 + i * 32, n0 + j * 32 + r, lane);
+}
+
+// ---------------------------------------------------------------- tiled kernel through LDS (f16)
+// 128 x 128 tile, 2 x 2 waves, k tiles of 64 in two LDS stages.  The register kernel above makes
+// every lane fetch its own row, 64 cache lines per load instruction, and the compute unit's
+// address path caps it at about 15 bytes per clock (0.4 PFLOP/s whatever the shape); here
+// eight lanes cover one 128-byte row segment of the activations and four one 64-byte segment of
+// the weights, the tile is shared through LDS (16-byte chunks XOR-swizzled by the row so that
+// the fragment reads spread over the banks), and the fragments are read back as ds_read_b128.
+__global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
+  constexpr int BM = 128, BN = 128, BK = 64;
+  __shared__ __attribute__((aligned(16))) uint8_t xs[2][BM * BK * 2];
+  __shared__ __attribute__((aligned(16))) uint8_t ws[2][BN * BK];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_n = (p.N + BN - 1) / BN;
+  const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+  const int r = lane & 31, g = lane >> 5;
+  const _Float16* x = static_cast<const _Float16*>(p.x);
+  const u4 zero = {0, 0, 0, 0};
+
+  // global -> LDS assignment
+  const int xc = tid & 7, wc = tid & 3;                  // 16-byte chunk of the row's k tile
+  const _Float16* xg[4];
+  int xl[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = (tid >> 3) + 32 * i;
+    xg[i] = x + (int64_t)min(m0 + row, p.M - 1) * p.ldx + 8 * xc;
+    xl[i] = row * 128 + ((xc ^ (row & 7)) << 4);
+  }
+  const uint8_t* wg[2];
+  int wl[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = (tid >> 2) + 64 * i;
+    wg[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.w_sn + 16 * wc;
+    wl[i] = row * 64 + ((wc ^ ((row >> 1) & 3)) << 4);
+  }
+  // three register sets: the loads of k tiles t + 1 .. t + 3 are in flight while tile t is
+  // multiplied (with one workgroup on a compute unit nothing else covers the load latency)
+  u4 xr[3][4], wr[3][2];
+  auto fetch = [&](u4* xq, u4* wq, int k0) {
+    const bool xv = k0 + 8 * xc < p.K, wv = k0 + 16 * wc < p.K;   // K % 16 == 0
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xq[i] = xv ? *reinterpret_cast<const u4*>(xg[i] + k0) : zero;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) wq[i] = wv ? *reinterpret_cast<const u4*>(wg[i] + k0) : zero;
+  };
+  auto park = [&](const u4* xq, const u4* wq, int stage) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u4*>(&xs[stage][xl[i]]) = xq[i];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<u4*>(&ws[stage][wl[i]]) = wq[i];
+  };
+
+  // fragment rows of this wave and the weight centres of its columns
+  int xrow[2], wrow[2];
+  h2 c[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    xrow[i] = wm * 64 + i * 32 + r;
+    wrow[i] = wn * 64 + i * 32 + r;
+    c[i] = centre(p, min(n0 + wrow[i], p.N - 1));
+  }
+  f16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  auto multiply = [&](int st) {
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    h8 a0[2], a1[2], w0[2], w1[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c0 = 4 * s + 2 * g, row = xrow[i];
+      a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ (row & 7)) << 4)]);
+      a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ (row & 7)) << 4)]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int cw = 2 * s + g, row = wrow[j];
+      const u4 q = *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 1) & 3)) << 4)]);
+      widen16(q, p.flip, c[j], w0[j], w1[j]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], w0[j], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1[i], w1[j], acc[i][j], 0, 0, 0);
+      }
+  }
+  };
+  const int KT = (p.K + BK - 1) / BK;
+  fetch(xr[0], wr[0], 0);
+  fetch(xr[1], wr[1], BK);
+  fetch(xr[2], wr[2], 2 * BK);
+  park(xr[0], wr[0], 0);
+  __syncthreads();
+  for (int t0 = 0; t0 < KT; t0 += 6) {
+#pragma unroll
+    for (int u = 0; u < 6; ++u) {
+      const int t = t0 + u;
+      if (t < KT) {                                        // (uniform over the workgroup)
+        fetch(xr[u % 3], wr[u % 3], (t + 3) * BK);         // (past K: zeros)
+        multiply(u % 2);
+        if (t + 1 < KT) park(xr[(u + 1) % 3], wr[(u + 1) % 3], (u + 1) % 2);
+        __syncthreads();
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      store_frag<_Float16>(p, acc[i][j], m0 + xrow[i] - r, n0 + wrow[j], lane);
 }
 
 // ---------------------------------------------------------------- small-M kernel, M <= 32 MT
@@ -387,9 +518,14 @@ int launch(const WoParams& p, bool fast, hipStream_t st) {
     else
       hipLaunchKernelGGL((wo_skinny_kernel<XT, 8, 4>), dim3(grid), dim3(512), 0, st, p);
   } else {
-    // 128 x 128 tiles once they fill the chip, 64 x 64 below
+    // 128 x 128 tiles through LDS once there are enough of them to put several workgroups on
+    // a compute unit (a lone workgroup's chain of load, LDS, widen and MFMA latencies is not
+    // covered: 48 tiles of a 3072-deep problem take as long through LDS as 192 small tiles
+    // through registers); the register kernel below that and for f32 activations
     const int64_t big = ceil_div(p.M, 128) * ceil_div(p.N, 128);
-    if (big >= 192) {
+    if (big >= 96 && sizeof(XT) == 2) {
+      hipLaunchKernelGGL(wo_lds_kernel, dim3((unsigned)big), dim3(256), 0, st, p);
+    } else if (big >= 192) {
       hipLaunchKernelGGL((wo_tile_kernel<XT, 2, 2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else {
       const int64_t small = ceil_div(p.M, 64) * ceil_div(p.N, 64);
