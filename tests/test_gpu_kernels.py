@@ -1088,7 +1088,10 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
     kernel without them (the reference's own test uses K = 3, N = 5)."""
     rng = np.random.default_rng(77)
     for (m, k, n) in [(2, 3, 5), (33, 48, 40), (200, 80, 136), (1, 16, 1), (70, 2064, 100),
-                      (130, 40, 260), (5, 1000, 33)]:
+                      (130, 40, 260), (5, 1000, 33),
+                      # enough 128 x 128 tiles for the kernel that stages both operands in LDS:
+                      # ragged last tiles in M and N, k depths off a multiple of 64
+                      (1500, 80, 1100), (1290, 208, 1300), (9, 4112, 40)]:
         for signed in (False, True):
             x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed)
             got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
