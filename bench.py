@@ -46,7 +46,8 @@ def parse():
     p.add_argument("--workload", default="headline",
                    help="'headline' (default), or one parity-test configuration on its own, "
                         "e.g. for a profiler: 'gemm:MxKxN' (dynamic-M sweep shape, requant to "
-                        "int8) or 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS)")
+                        "int8), 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS) or "
+                        "'wo:MxKxN' (weight-only linear, f16 x uint8)")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extra", action="store_true", help="skip the extras")
     p.add_argument("--no-two-stream", action="store_true",
@@ -645,14 +646,27 @@ def single_workload(torch, args):
         mg, kg = nb * osh[1] * osh[2], kk * kk * ci
         ops, byts = 2.0 * mg * co * kg, nb * h * w_ * ci + co * kg + mg * co + 4 * co
         name = "int8 NHWC conv %s, batch %d, requant to int8 (E1)" % (what, nb)
+    elif kind == "wo":
+        # weight-only quantized linear: f16 activations x uint8 weights [N,K]
+        m, k, n = (int(v) for v in what.split("x"))
+        wq = torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda")
+        sc = (torch.rand(n, device="cuda") * 0.02 + 0.002).half()
+        zp = torch.full((n,), 128, dtype=torch.int32, device="cuda")
+        xh = torch.randn((m, k), device="cuda").half()
+        oh = torch.empty((m, n), dtype=torch.float16, device="cuda")
+        call = lambda: K.weight_only_qgemm(xh, wq, sc, zp, out=oh)  # noqa: E731
+        ops, byts = 2.0 * m * n * k, 2.0 * m * k + n * k + 2.0 * m * n + 6.0 * n
+        name = "weight-only qgemm M=%d K=%d N=%d, f16 x uint8 (roofline against the f16 peak)" % (m, k, n)
     else:
         raise SystemExit("bench.py: unknown --workload %r" % args.workload)
     pre_launches, pre_s = prewarm(torch, call, args.prewarm_ms * 1e-3) if args.prewarm_ms > 0 \
         else (0, 0.0)
     wall, ev = time_steps(torch, call, args.steps, args.warmup)
     r = roof(ops, byts, ev / args.steps)
+    if kind == "wo":      # f16 matrix cores: 2.5 PFLOP/s
+        r["roofline_frac"] = round(max(r["TOPS"] / 2500.0, r["GB/s"] / PEAK_HBM_GBPS), 4)
     print(json.dumps({
-        "metric": "int8 TOPS", "value": round(ops * args.steps / wall / 1e12, 2), "unit": "TOPS",
+        "metric": "int8 TOPS" if kind != "wo" else "f16 TFLOP/s", "value": round(ops * args.steps / wall / 1e12, 2), "unit": "TOPS",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall / args.steps * 1e3, 5),
         "prewarm": {"ms": round(pre_s * 1e3, 1), "launches": pre_launches},

@@ -793,7 +793,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   // scratch (or with a fused residual, which has the output's layout) the generic kernel reads
   // the tensors in place.
   if (is_nchw_oihw(md) && variant != 0 && workspace != nullptr && aligned(workspace, 256) &&
-      !(post && post->residual_kind != DQ8_RESIDUAL_NONE) &&
+      !(post && post->residual_kind != DQ8_RESIDUAL_NONE) && NB <= 65535 && Co <= 65535 &&
       epilogue >= DQ8_EPI_ACC_S32 && epilogue <= DQ8_EPI_REQUANT_FIXEDPOINT) {
     const int64_t Mo = NB * out_sizes[2] * out_sizes[3];
     const int es = out_elem_size(epilogue);

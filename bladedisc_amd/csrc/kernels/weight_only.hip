@@ -248,7 +248,7 @@ __global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
   for (int i = 0; i < 4; ++i) {
     const int row = (tid >> 3) + 32 * i;
     xg[i] = x + (int64_t)min(m0 + row, p.M - 1) * p.ldx + 8 * xc;
-    xl[i] = row * 128 + ((xc ^ (row & 7)) << 4);
+    xl[i] = row * 128 + ((xc ^ ((row ^ (row >> 3)) & 7)) << 4);
   }
   const uint8_t* wg[2];
   int wl[2];
@@ -256,7 +256,7 @@ __global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
   for (int i = 0; i < 2; ++i) {
     const int row = (tid >> 2) + 64 * i;
     wg[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.w_sn + 16 * wc;
-    wl[i] = row * 64 + ((wc ^ ((row >> 1) & 3)) << 4);
+    wl[i] = row * 64 + ((wc ^ ((row >> 2) & 3)) << 4);
   }
   // three register sets: the loads of k tiles t + 1 .. t + 3 are in flight while tile t is
   // multiplied (with one workgroup on a compute unit nothing else covers the load latency)
@@ -299,13 +299,13 @@ __global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int c0 = 4 * s + 2 * g, row = xrow[i];
-      a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ (row & 7)) << 4)]);
-      a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ (row & 7)) << 4)]);
+      a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ ((row ^ (row >> 3)) & 7)) << 4)]);
+      a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ ((row ^ (row >> 3)) & 7)) << 4)]);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int cw = 2 * s + g, row = wrow[j];
-      const u4 q = *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 1) & 3)) << 4)]);
+      const u4 q = *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 2) & 3)) << 4)]);
       widen16(q, p.flip, c[j], w0[j], w1[j]);
     }
 #pragma unroll
