@@ -271,6 +271,11 @@ def config_reports(torch, K):
              FnCall(lambda: K.qgemm(xq, wq, K.EPI_REQUANT_CPU, sx=sx, sw=sw, so=so, bias=bias, out=yq)),
              FnCall(lambda: K.dequantize(yq, so, z1, out=y))]
     gpu_s = time_graph(torch, chain)
+    # the same with the trailing dequantize done in the GEMM's epilogue (bit-identical f32)
+    fused = [chain[0],
+             FnCall(lambda: K.qgemm(xq, wq, K.EPI_REQUANT_CPU_DEQUANT_F32, sx=sx, sw=sw, so=so,
+                                    bias=bias, out=y))]
+    gpu_fused_s = time_graph(torch, fused)
 
     def cpu1():
         q = O.quantize(c["x"], c["sx"], 0)
@@ -280,7 +285,8 @@ def config_reports(torch, K):
     cpu_s = cpu_time(cpu1)
     rep["1_single_linear_64x768x768_q_gemm_dq"] = {
         "gpu_us": round(gpu_s * 1e6, 2), "cpu_us": round(cpu_s * 1e6, 1),
-        "gpu_over_cpu": round(cpu_s / gpu_s, 1)}
+        "gpu_over_cpu": round(cpu_s / gpu_s, 1),
+        "gpu_us_dequantize_in_epilogue": round(gpu_fused_s * 1e6, 2)}
 
     # ---- 2: dynamic-M sweep, E1 requant, int8 out
     sweep = {}
