@@ -328,7 +328,14 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
     // the load latency: 6.3 against 7.1 us at M = 2048, 768 -> 768); with two tiles on a
     // compute unit, or a deep K, four waves (10.0 against 11.2 us at M = 2048, 768 -> 3072)
     const int64_t t128 = tiles(kPipe128);
-    if (t128 >= 120) return (K < 4096 && t128 <= cus) ? kPipe128w8 : kPipe128;
+    // (int32 / f32 results, four times the bytes to store: eight waves throughout, and the
+    // persistent form from two tiles per compute unit on -- M = 16384, 768 -> 768 with an f32
+    // result: 17.8 against 18.5 us, four waves 23.8)
+    if (t128 >= 120) {
+      if (K >= 4096) return kPipe128;
+      if (out_bytes == 1) return t128 <= cus ? kPipe128w8 : kPipe128;
+      return t128 > 2 * cus ? kPersist128 : kPipe128w8;
+    }
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
   constexpr int64_t kCus = 256;
@@ -949,8 +956,13 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     g.N = (int)Co;
     g.K = (int)Ci;
     g.epi = e;
-    const int v = Mg <= kSkinnyMaxM ? kSkinnyVariant
-                                    : pick_variant(Mg, Co, Ci, pipe_ok(256, 256, g, false), es);
+    int v = Mg <= kSkinnyMaxM ? kSkinnyVariant
+                              : pick_variant(Mg, Co, Ci, pipe_ok(256, 256, g, false), es);
+    if (fused || e.fixedpoint) {   // the persistent forms carry neither
+      if (v == kPersist256) v = kPipe256w8;
+      if (v == kPersist256x192) v = kPipe256x192;
+      if (v == kPersist128) v = kPipe128w8;
+    }
     return launch_epi<false>(v, g, epilogue, st);
   }
 
@@ -994,6 +1006,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     // on top they run out of registers)
     if (variant == kPersist256) variant = kPipe256w8;
     if (variant == kPersist256x192) variant = kPipe256x192;
+    if (variant == kPersist128) variant = kPipe128w8;
   }
   return launch_epi<true>(variant, p, epilogue, st);
 }

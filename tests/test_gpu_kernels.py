@@ -787,6 +787,37 @@ def test_qconv_fused_residual_relu_quantize(K, nb, h, w_, ci, co, k, pad):
     assert torch.equal(got, K.lut8(q, table))
 
 
+def test_qconv_1x1_with_many_tiles_keeps_the_fixed_point_stage_and_fused_operators(K):
+    """A 1x1 convolution runs as a plain GEMM over the pixels; with several rounds of tiles the
+    plain GEMM would take its persistent kernels, which carry neither the fixed-point stage nor
+    fused operators -- the dispatch has to stay on the kernels that do."""
+    rng = np.random.default_rng(5)
+    nb, h, ci, co = 32, 56, 64, 256                      # 100352 x 64 -> 256: 392 tiles of 256 x 256, two rounds
+    x = dev(rng.integers(-128, 128, (nb, h, h, ci), dtype=np.int8))
+    wt = dev(rng.integers(-128, 128, (co, 1, 1, ci), dtype=np.int8))
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    osh = [nb, h, h, co]
+    acc, _ = O.gemm_s32_fast(host(x).reshape(-1, ci), host(wt).reshape(co, ci))
+    sx, sw = make_scales(rng, co)
+    so = pick_so(acc, sx, sw)
+    sc = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so], np.float32)))
+    b32 = rng.integers(-1000, 1000, co).astype(np.int32)
+    want = O.requant_fixedpoint(acc, sx, sw, so, b32=b32, zo=1).reshape(osh)
+    got = K.qconv2d(x, wt, [0] * 4, md, osh, K.EPI_REQUANT_FIXEDPOINT, bias=dev(b32), zo=1, **sc)
+    np.testing.assert_array_equal(host(got), want)
+    table = dev(rng.integers(-128, 128, 256, dtype=np.int8))
+    q = K.qconv2d(x, wt, [0] * 4, md, osh, K.EPI_REQUANT_CPU, **sc)
+    np.testing.assert_array_equal(host(q), O.requant_cpu(acc, sx, sw, so).reshape(osh))
+    got = K.qconv2d(x, wt, [0] * 4, md, osh, K.EPI_REQUANT_CPU, **sc, post=K.make_postops(table=table))
+    assert torch.equal(got, K.lut8(q, table))
+    # the same through the GEMM entry
+    a2, w2 = x.reshape(-1, ci), wt.reshape(co, ci)
+    got = K.qgemm(a2, w2, K.EPI_REQUANT_FIXEDPOINT, bias=dev(b32), zo=1, **sc)
+    np.testing.assert_array_equal(host(got), want.reshape(-1, co))
+    got = K.qgemm(a2, w2, K.EPI_REQUANT_CPU, **sc, post=K.make_postops(table=table))
+    assert torch.equal(got, K.lut8(q, table).reshape(-1, co))
+
+
 def test_qconv_direct_random_shapes(K):
     """Seeded sweep for the kernels that keep the input patch in LDS: image sizes that make
     tiles start and end anywhere in a row, every channel count, ragged output channels,
