@@ -136,6 +136,13 @@ def test_qgemm_persistent_variants_walk_many_tiles(K, m, n, k):
         np.testing.assert_array_equal(host(K.qgemm(da, dw, K.EPI_ACC_S32, variant=v)), acc, err_msg=tag)
         got = host(K.qgemm(da, dw, K.EPI_DEQUANT_F32, sx=dsx, sw=dsw, bias=dev(bf), variant=v))
         assert np.array_equal(got.view(np.uint32), want_f32.view(np.uint32)), tag
+        # requant -> dequantize in one epilogue (f32 result) and the E2 form with its f32 bias
+        got = host(K.qgemm(da, dw, K.EPI_REQUANT_CPU_DEQUANT_F32, sx=dsx, sw=dsw, so=dso, bias=dev(bf),
+                           zo=3, variant=v))
+        want = O.dequantize(want_bias, np.array([so], np.float32), np.array([3], np.int32))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), tag
+        got = host(K.qgemm(da, dw, K.EPI_REQUANT_GPU, sx=dsx, sw=dsw, so=dso, bias=dev(bf), variant=v))
+        np.testing.assert_array_equal(got, O.requant_gpu(acc, sx, sw, so, bias_f32=bf), err_msg=tag)
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 768, 768), (1000, 768, 3072), (257, 130, 64), (5, 7, 48),
