@@ -755,7 +755,9 @@ def test_qconv_parity(K, nb, h, w_, ci, co, k, stride, pad, dil):
 
 
 @pytest.mark.parametrize("nb,h,w_,ci,co,k,pad", [(2, 14, 14, 64, 256, 1, 0), (1, 28, 28, 128, 128, 3, 1),
-                                                 (2, 9, 11, 48, 72, 3, 1), (1, 7, 7, 24, 40, 1, 0)])
+                                                 (2, 9, 11, 48, 72, 3, 1), (1, 7, 7, 24, 40, 1, 0),
+                                                 # the kernel with the input patch resident in LDS
+                                                 (64, 32, 32, 32, 32, 3, 1), (32, 56, 56, 64, 64, 3, 1)])
 def test_qconv_fused_residual_relu_quantize(K, nb, h, w_, ci, co, k, pad):
     """The tail of a ResNet block in the convolution's epilogue: dequantize -> + the block's
     int8 input (its own scale and zero point) -> ReLU -> quantize gives the bits of the
