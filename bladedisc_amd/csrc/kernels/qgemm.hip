@@ -344,6 +344,18 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
   return 3;
 }
 
+// The small-M kernel up to kSkinnyMaxM rows -- except for 17 .. 32 rows against weights large
+// enough to give the 64 x 64 tile with its k range split over two wave groups 128 workgroups
+// (M = 32, 8192 x 8192 weights: 18.5 against 24.6 us; 4096 x 4096: 9.1 against 8.5) -- and the
+// tiled kernels above.
+int pick_any(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes) {
+  if (M <= kSkinnyMaxM) {
+    if (M > 16 && pipe && K >= 2048 && ceil_div(N, 64) >= 128) return kPipe64k2;
+    return kSkinnyVariant;
+  }
+  return pick_variant(M, N, K, pipe, out_bytes);
+}
+
 // Whether a 3x3 stride-1 convolution goes to the kernel that keeps the input patch in LDS
 // (and with which tile), or to the implicit GEMM.  Measured on ResNet / VGG shaped layers
 // with batch 1 .. 128: with at most 64 input and output channels the implicit GEMM is bound
@@ -650,7 +662,7 @@ int qgemm_impl(int variant, const int8_t* A, int64_t lda, const int8_t* W, int64
   p.K = (int)K;
   p.epi = e;
   if (auto_pick)
-    variant = M <= kSkinnyMaxM ? kSkinnyVariant : pick_variant(M, N, K, pipe_ok(256, 256, p, false), es);
+    variant = pick_any(M, N, K, pipe_ok(256, 256, p, false), es);
   if (fused || e.fixedpoint) {   // the persistent forms carry neither
     DQ8_REQUIRE(auto_pick || (variant != kPersist256 && variant != kPersist256x192 && variant != kPersist128),
                 "dq8_qgemm: the persistent variants take neither fused operators nor the fixed-point stage");
@@ -956,8 +968,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     g.N = (int)Co;
     g.K = (int)Ci;
     g.epi = e;
-    int v = Mg <= kSkinnyMaxM ? kSkinnyVariant
-                              : pick_variant(Mg, Co, Ci, pipe_ok(256, 256, g, false), es);
+    int v = pick_any(Mg, Co, Ci, pipe_ok(256, 256, g, false), es);
     if (fused || e.fixedpoint) {   // the persistent forms carry neither
       if (v == kPersist256) v = kPipe256w8;
       if (v == kPersist256x192) v = kPipe256x192;
