@@ -23,7 +23,8 @@
 // the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes (one dwordx4), 16
 // activations -- and feeds two MFMAs with them.
 //  * wo_lds_kernel: f16 activations, 128 x 128 tiles shared through LDS, once there are about a
-//    hundred of them (0.77-0.85 PFLOP/s at 4096^2 .. 8192^2 weights);
+//    hundred of them (256 x 128 on eight waves once those fill the chip; 0.84-0.90 PFLOP/s at 4096^2 .. 8192^2
+//    weights, where the ROCm library's plain f16 GEMM reaches 1.16-1.49);
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
 //    f32 activations and problems with few tiles;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
@@ -222,16 +223,21 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
 }
 
 // ---------------------------------------------------------------- tiled kernel through LDS (f16)
-// 128 x 128 tile, 2 x 2 waves, k tiles of 64 in two LDS stages.  The register kernel above makes
+// (64 WM) x 128 tile, WM x 2 waves (WM = 2 or 4), k tiles of 64 in two LDS stages.  The register kernel above makes
 // every lane fetch its own row, 64 cache lines per load instruction, and the compute unit's
 // address path caps it at about 15 bytes per clock (0.4 PFLOP/s whatever the shape); here
 // eight lanes cover one 128-byte row segment of the activations and four one 64-byte segment of
 // the weights, the tile is shared through LDS (16-byte chunks XOR-swizzled by the row so that
 // the fragment reads spread over the banks), and the fragments are read back as ds_read_b128.
-__global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
-  constexpr int BM = 128, BN = 128, BK = 64;
+template <int WM, bool WIDE>
+__global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
+  constexpr int BM = WM * 64, BN = 128, BK = 64;
+  constexpr int NT = WM * 128;                           // WM x 2 waves
+  constexpr int WP = (BN * 4) / NT;                      // weight chunks per thread: 2 or 1
   __shared__ __attribute__((aligned(16))) uint8_t xs[2][BM * BK * 2];
-  __shared__ __attribute__((aligned(16))) uint8_t ws[2][BN * BK];
+  // WIDE: the weights are widened to halves once, on their way into LDS (128-byte rows like the
+  // activations'), not by every wave that reads them
+  __shared__ __attribute__((aligned(16))) uint8_t ws[2][BN * BK * (WIDE ? 2 : 1)];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_n = (p.N + BN - 1) / BN;
@@ -246,33 +252,51 @@ __global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
   int xl[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int row = (tid >> 3) + 32 * i;
+    const int row = (tid >> 3) + (NT / 8) * i;
     xg[i] = x + (int64_t)min(m0 + row, p.M - 1) * p.ldx + 8 * xc;
     xl[i] = row * 128 + ((xc ^ ((row ^ (row >> 3)) & 7)) << 4);
   }
-  const uint8_t* wg[2];
-  int wl[2];
+  const uint8_t* wg[WP];
+  int wl[WP], wl1[WP];
+  h2 cpark[WP];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = (tid >> 2) + 64 * i;
+  for (int i = 0; i < WP; ++i) {
+    const int row = (tid >> 2) + (NT / 4) * i;
     wg[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.w_sn + 16 * wc;
-    wl[i] = row * 64 + ((wc ^ ((row >> 2) & 3)) << 4);
+    if (WIDE) {
+      const int sw = (row ^ (row >> 3)) & 7;
+      wl[i] = row * 128 + (((2 * wc) ^ sw) << 4);
+      wl1[i] = row * 128 + (((2 * wc + 1) ^ sw) << 4);
+      cpark[i] = centre(p, min(n0 + row, p.N - 1));
+    } else {
+      wl[i] = row * 64 + ((wc ^ ((row >> 2) & 3)) << 4);
+      wl1[i] = 0;
+    }
   }
   // three register sets: the loads of k tiles t + 1 .. t + 3 are in flight while tile t is
   // multiplied (with one workgroup on a compute unit nothing else covers the load latency)
-  u4 xr[3][4], wr[3][2];
+  u4 xr[3][4], wr[3][WP];
   auto fetch = [&](u4* xq, u4* wq, int k0) {
     const bool xv = k0 + 8 * xc < p.K, wv = k0 + 16 * wc < p.K;   // K % 16 == 0
 #pragma unroll
     for (int i = 0; i < 4; ++i) xq[i] = xv ? *reinterpret_cast<const u4*>(xg[i] + k0) : zero;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) wq[i] = wv ? *reinterpret_cast<const u4*>(wg[i] + k0) : zero;
+    for (int i = 0; i < WP; ++i) wq[i] = wv ? *reinterpret_cast<const u4*>(wg[i] + k0) : zero;
   };
   auto park = [&](const u4* xq, const u4* wq, int stage) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) *reinterpret_cast<u4*>(&xs[stage][xl[i]]) = xq[i];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<u4*>(&ws[stage][wl[i]]) = wq[i];
+    for (int i = 0; i < WP; ++i) {
+      if (WIDE) {
+        h8 lo, hi;
+        widen16(wq[i], p.flip, cpark[i], lo, hi);
+        *reinterpret_cast<h8*>(&ws[stage][wl[i]]) = lo;
+        *reinterpret_cast<h8*>(&ws[stage][wl1[i]]) = hi;
+      } else {
+        *reinterpret_cast<u4*>(&ws[stage][wl[i]]) = wq[i];
+      }
+    }
   };
 
   // fragment rows of this wave and the weight centres of its columns
@@ -304,9 +328,16 @@ __global__ void __launch_bounds__(256) wo_lds_kernel(const WoParams p) {
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int cw = 2 * s + g, row = wrow[j];
-      const u4 q = *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 2) & 3)) << 4)]);
-      widen16(q, p.flip, c[j], w0[j], w1[j]);
+      const int row = wrow[j];
+      if (WIDE) {
+        const int c0 = 4 * s + 2 * g, sw = (row ^ (row >> 3)) & 7;
+        w0[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + ((c0 ^ sw) << 4)]);
+        w1[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + (((c0 + 1) ^ sw) << 4)]);
+      } else {
+        const int cw = 2 * s + g;
+        const u4 q = *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 2) & 3)) << 4)]);
+        widen16(q, p.flip, c[j], w0[j], w1[j]);
+      }
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -523,8 +554,11 @@ int launch(const WoParams& p, bool fast, hipStream_t st) {
     // covered: 48 tiles of a 3072-deep problem take as long through LDS as 192 small tiles
     // through registers); the register kernel below that and for f32 activations
     const int64_t big = ceil_div(p.M, 128) * ceil_div(p.N, 128);
-    if (big >= 96 && sizeof(XT) == 2) {
-      hipLaunchKernelGGL(wo_lds_kernel, dim3((unsigned)big), dim3(256), 0, st, p);
+    const int64_t big256 = ceil_div(p.M, 256) * ceil_div(p.N, 128);
+    if (big256 >= 384 && sizeof(XT) == 2) {
+      hipLaunchKernelGGL((wo_lds_kernel<4, true>), dim3((unsigned)big256), dim3(512), 0, st, p);
+    } else if (big >= 96 && sizeof(XT) == 2) {
+      hipLaunchKernelGGL((wo_lds_kernel<2, true>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else if (big >= 192) {
       hipLaunchKernelGGL((wo_tile_kernel<XT, 2, 2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else {
