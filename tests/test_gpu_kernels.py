@@ -1150,3 +1150,109 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
     _weight_only_check(got, x, w, scale, zp, bias, dtype)
     empty = K.weight_only_qgemm(dev(x[:0]), dev(w), dev(scale), dev(zp), dev(bias))
     assert tuple(empty.shape) == (0, 96)
+
+
+def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
+    """Seeded sweep over what the library's own choice of kernel depends on -- M from one row
+    to several rounds of the largest tiles, N, K, the epilogue family, fused operators -- with
+    the scalar generic kernel (variant 0, itself pinned against the oracle above) as the
+    yardstick on the same device buffers: every combination must give the same bits, whichever
+    kernel the heuristic lands on (small-M, 64 / 128 / 256-wide tiles, persistent forms)."""
+    rng = np.random.default_rng(20260101)
+    ms = [1, 7, 16, 31, 33, 100, 500, 1000, 2100, 4096, 9000, 20000]
+    cases = 0
+    for m in ms:
+        for _ in range(3):
+            n = int(rng.choice([16, 48, 64, 136, 768, 1024, 2304, 3072]))
+            k = int(rng.choice([16, 64, 144, 768, 1040, 3072]))
+            if m * n * k > 2.2e10:
+                k = 64
+            a = dev(rng.integers(-128, 128, (m, k), dtype=np.int8))
+            w = dev(rng.integers(-128, 128, (n, k), dtype=np.int8))
+            sx = dev(np.array([rng.uniform(0.01, 0.03)], np.float32))
+            sw = dev(rng.uniform(0.001, 0.05, n).astype(np.float32))
+            so = dev(np.array([float(np.sqrt(k)) * 0.02 * 0.025 * 5400 / 40.0], np.float32))
+            bf = dev((rng.standard_normal(n) * 3).astype(np.float32))
+            b32 = dev(rng.integers(-20000, 20000, n).astype(np.int32))
+            table = dev(rng.integers(-128, 128, 256, dtype=np.int8))
+            resid = dev(rng.integers(-128, 128, (m, n), dtype=np.int8))
+            rs = dev(np.array([0.05], np.float32))
+            s2 = dev(np.array([0.07], np.float32))
+            sc = dict(sx=sx, sw=sw, so=so)
+            plans = [
+                (K.EPI_ACC_S32, {}, None),
+                (K.EPI_REQUANT_CPU, dict(bias=bf, zo=2, **sc), None),
+                (K.EPI_REQUANT_GPU, dict(bias=bf, **sc), None),
+                (K.EPI_DEQUANT_F32, dict(sx=sx, sw=sw, bias=bf), None),
+                (K.EPI_REQUANT_CPU_DEQUANT_F32, dict(bias=bf, zo=2, **sc), None),
+                (K.EPI_REQUANT_FIXEDPOINT, dict(bias=b32, zo=-1, **sc), None),
+                (K.EPI_REQUANT_CPU, dict(bias=bf, **sc), dict(table=table)),
+                (K.EPI_REQUANT_GPU, dict(bias=bf, **sc),
+                 dict(residual=resid, residual_scale=rs, residual_zp=3, relu=True, out_scale=s2, out_zp=-4)),
+            ]
+            for epi, kw, post in plans:
+                if post is None:
+                    want = K.qgemm(a, w, epi, variant=0, **kw)
+                    got = K.qgemm(a, w, epi, **kw)
+                else:
+                    # (fused operators go with the library's own choice: the yardstick is the chain
+                    # of separate calls on the generic kernel's result)
+                    q = K.qgemm(a, w, epi, variant=0, **kw)
+                    if "table" in post:
+                        want = K.lut8(q, table)
+                    else:
+                        zero = torch.zeros(1, dtype=torch.int32, device="cuda")
+                        t = K.dequantize(q, so, zero) + K.dequantize(
+                            resid, rs, torch.full((1,), 3, dtype=torch.int32, device="cuda"))
+                        t = torch.where(t < 0, torch.zeros_like(t), t)
+                        want = K.quantize(t, s2, torch.full((1,), -4, dtype=torch.int32, device="cuda"))
+                    got = K.qgemm(a, w, epi, post=K.make_postops(**post), **kw)
+                assert got.dtype == want.dtype
+                same = torch.equal(got.view(torch.int32) if got.dtype == torch.float32 else got,
+                                   want.view(torch.int32) if want.dtype == torch.float32 else want)
+                assert same, (m, n, k, epi, post)
+                cases += 1
+    assert cases == len(ms) * 3 * 8
+
+
+def test_conv_dispatch_sweep_agrees_with_the_generic_kernel(K):
+    """The same for convolutions: batch, image size, channel counts (multiples of 16 and not),
+    filter, stride, padding and dilation drawn from a seeded generator; the library's choice
+    (direct 3x3 kernels, implicit GEMM tiles, 1x1 as a plain GEMM, channel padding through the
+    scratch) against the generic kernel, for the int8, int32, f32 and fixed-point results and a
+    fused table."""
+    rng = np.random.default_rng(20260102)
+    cases = 0
+    for _ in range(30):
+        nb = int(rng.choice([1, 2, 8, 32, 70]))
+        h = int(rng.choice([7, 14, 28, 33, 56]))
+        w_ = int(rng.choice([7, 14, 28, 30, 56]))
+        ci = int(rng.choice([3, 16, 24, 32, 64, 128, 256]))
+        co = int(rng.choice([16, 40, 64, 128, 256]))
+        k = int(rng.choice([1, 3, 3, 5]))
+        stride = int(rng.choice([1, 1, 2]))
+        dil = int(rng.choice([1, 1, 2]))
+        pad = int(rng.integers(0, 3))
+        ho = (h + 2 * pad - dil * (k - 1) - 1) // stride + 1
+        wo = (w_ + 2 * pad - dil * (k - 1) - 1) // stride + 1
+        if ho <= 0 or wo <= 0 or nb * ho * wo * co * k * k * ci > 6e10:
+            continue
+        x = dev(rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8))
+        wt = dev(rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8))
+        md = list(O.NHWC_OHWI_METADATA) + [stride, stride, dil, dil, 1]
+        padding, osh = [pad] * 4, [nb, ho, wo, co]
+        sc = dict(sx=dev(np.array([0.02], np.float32)), sw=dev(rng.uniform(0.001, 0.05, co).astype(np.float32)),
+                  so=dev(np.array([float(np.sqrt(k * k * ci)) * 0.02 * 0.025 * 5400 / 40.0], np.float32)))
+        b32 = dev(rng.integers(-20000, 20000, co).astype(np.int32))
+        table = dev(rng.integers(-128, 128, 256, dtype=np.int8))
+        for epi, kw in ((K.EPI_ACC_S32, {}), (K.EPI_REQUANT_CPU, dict(zo=1, **sc)),
+                        (K.EPI_REQUANT_CPU_DEQUANT_F32, sc), (K.EPI_REQUANT_FIXEDPOINT, dict(bias=b32, **sc))):
+            want = K.qconv2d(x, wt, padding, md, osh, epi, variant=0, **kw)
+            got = K.qconv2d(x, wt, padding, md, osh, epi, **kw)
+            v = (lambda t: t.view(torch.int32) if t.dtype == torch.float32 else t)
+            assert torch.equal(v(got), v(want)), (nb, h, w_, ci, co, k, stride, pad, dil, epi)
+            cases += 1
+        q = K.qconv2d(x, wt, padding, md, osh, K.EPI_REQUANT_CPU, variant=0, **sc)
+        got = K.qconv2d(x, wt, padding, md, osh, K.EPI_REQUANT_CPU, **sc, post=K.make_postops(table=table))
+        assert torch.equal(got, K.lut8(q, table)), (nb, h, w_, ci, co, k, stride, pad, dil)
+    assert cases >= 80
