@@ -376,14 +376,20 @@ template <typename XT>
 bool launch_quantize_kind(int out_kind, bool rne, const void* x, void* out, int64_t n,
                           int64_t nch, int64_t inner, int per_channel, const float* scale,
                           const int32_t* zp, float lo, float hi, hipStream_t st) {
+#define DQ8_WIDE_CASE(KIND, QT)                                                              \
+  case KIND:                                                                                 \
+    launch_quantize_wide<XT, QT>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, \
+                                 st);                                                        \
+    return true;
   switch (out_kind) {
-    case DQ8_I8: launch_quantize_wide<XT, int8_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
-    case DQ8_U8: launch_quantize_wide<XT, uint8_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
-    case DQ8_I16: launch_quantize_wide<XT, int16_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
-    case DQ8_U16: launch_quantize_wide<XT, uint16_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
-    case DQ8_I32: launch_quantize_wide<XT, int32_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
-    case DQ8_U32: launch_quantize_wide<XT, uint32_t>(rne, x, out, n, nch, inner, per_channel, scale, zp, lo, hi, st); return true;
+    DQ8_WIDE_CASE(DQ8_I8, int8_t)
+    DQ8_WIDE_CASE(DQ8_U8, uint8_t)
+    DQ8_WIDE_CASE(DQ8_I16, int16_t)
+    DQ8_WIDE_CASE(DQ8_U16, uint16_t)
+    DQ8_WIDE_CASE(DQ8_I32, int32_t)
+    DQ8_WIDE_CASE(DQ8_U32, uint32_t)
   }
+#undef DQ8_WIDE_CASE
   return false;
 }
 
@@ -622,9 +628,11 @@ extern "C" int dq8_quantize_ex(const void* x, int x_dtype, void* out, int out_ki
   const float lo = (float)qmin, hi = (float)qmax;
   hipStream_t st = (hipStream_t)stream;
   if (x_dtype == DQ8_DTYPE_F32)
-    launch_quantize_kind<float>(out_kind, rne, x, out, n, nch, inner, n_q > 1, scale, zp, lo, hi, st);
+    launch_quantize_kind<float>(out_kind, rne, x, out, n, nch, inner, n_q > 1, scale, zp, lo, hi,
+                                st);
   else
-    launch_quantize_kind<_Float16>(out_kind, rne, x, out, n, nch, inner, n_q > 1, scale, zp, lo, hi, st);
+    launch_quantize_kind<_Float16>(out_kind, rne, x, out, n, nch, inner, n_q > 1, scale, zp, lo,
+                                   hi, st);
   return dq8::check_hip(hipGetLastError(), "dq8_quantize_ex launch");
 }
 
@@ -643,11 +651,15 @@ extern "C" int dq8_dequantize_ex(const void* q, int in_kind, float* out, int64_t
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(grid_for(n, 1)), block(kThreads);
   const int pc = n_q > 1;
+#define DQ8_WIDE_CASE(QT)                                                                   \
+  hipLaunchKernelGGL(dequantize_wide<QT>, grid, block, 0, st, (const QT*)q, out, n, nch, inner, \
+                     pc, scale, zp)
   switch (in_kind) {
-    case DQ8_I16: hipLaunchKernelGGL(dequantize_wide<int16_t>, grid, block, 0, st, (const int16_t*)q, out, n, nch, inner, pc, scale, zp); break;
-    case DQ8_U16: hipLaunchKernelGGL(dequantize_wide<uint16_t>, grid, block, 0, st, (const uint16_t*)q, out, n, nch, inner, pc, scale, zp); break;
-    case DQ8_I32: hipLaunchKernelGGL(dequantize_wide<int32_t>, grid, block, 0, st, (const int32_t*)q, out, n, nch, inner, pc, scale, zp); break;
-    default: hipLaunchKernelGGL(dequantize_wide<uint32_t>, grid, block, 0, st, (const uint32_t*)q, out, n, nch, inner, pc, scale, zp); break;
+    case DQ8_I16: DQ8_WIDE_CASE(int16_t); break;
+    case DQ8_U16: DQ8_WIDE_CASE(uint16_t); break;
+    case DQ8_I32: DQ8_WIDE_CASE(int32_t); break;
+    default: DQ8_WIDE_CASE(uint32_t); break;
   }
+#undef DQ8_WIDE_CASE
   return dq8::check_hip(hipGetLastError(), "dq8_dequantize_ex launch");
 }

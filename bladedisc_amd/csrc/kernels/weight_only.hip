@@ -23,8 +23,8 @@
 // the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes (one dwordx4), 16
 // activations -- and feeds two MFMAs with them.
 //  * wo_lds_kernel: f16 activations, 128 x 128 tiles shared through LDS, once there are about a
-//    hundred of them (256 x 128 on eight waves once those fill the chip; 0.84-0.90 PFLOP/s at 4096^2 .. 8192^2
-//    weights, where the ROCm library's plain f16 GEMM reaches 1.16-1.49);
+//    hundred of them (256 x 128 on eight waves once those fill the chip; 0.84-0.90 PFLOP/s at
+//    4096^2 .. 8192^2 weights, where the ROCm library's plain f16 GEMM reaches 1.16-1.49);
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
 //    f32 activations and problems with few tiles;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
@@ -223,8 +223,8 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
 }
 
 // ---------------------------------------------------------------- tiled kernel through LDS (f16)
-// (64 WM) x 128 tile, WM x 2 waves (WM = 2 or 4), k tiles of 64 in two LDS stages.  The register kernel above makes
-// every lane fetch its own row, 64 cache lines per load instruction, and the compute unit's
+// (64 WM) x 128 tile, WM x 2 waves (WM = 2 or 4), k tiles of 64 in two LDS stages.  The
+// register kernel above makes every lane fetch its own row, 64 cache lines per load instruction, and the compute unit's
 // address path caps it at about 15 bytes per clock (0.4 PFLOP/s whatever the shape); here
 // eight lanes cover one 128-byte row segment of the activations and four one 64-byte segment of
 // the weights, the tile is shared through LDS (16-byte chunks XOR-swizzled by the row so that
@@ -323,8 +323,9 @@ __global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int c0 = 4 * s + 2 * g, row = xrow[i];
-      a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ ((row ^ (row >> 3)) & 7)) << 4)]);
-      a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ ((row ^ (row >> 3)) & 7)) << 4)]);
+      const int sx = (row ^ (row >> 3)) & 7;
+      a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ sx) << 4)]);
+      a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ sx) << 4)]);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -335,7 +336,8 @@ __global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
         w1[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + (((c0 + 1) ^ sw) << 4)]);
       } else {
         const int cw = 2 * s + g;
-        const u4 q = *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 2) & 3)) << 4)]);
+        const u4 q =
+            *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 2) & 3)) << 4)]);
         widen16(q, p.flip, c[j], w0[j], w1[j]);
       }
     }
@@ -418,8 +420,10 @@ __global__ void __launch_bounds__(NW * 64) wo_skinny_kernel(const WoParams p) {
       for (int part = 0; part < XFrag<XT>::kParts; ++part)
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[u][i].step(part, 0), w0, acc[i], 0, 0, 0);
-          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[u][i].step(part, 1), w1, acc[i], 0, 0, 0);
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[u][i].step(part, 0), w0, acc[i], 0, 0,
+                                                          0);
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[u][i].step(part, 1), w1, acc[i], 0, 0,
+                                                          0);
         }
     }
   }
