@@ -338,9 +338,11 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
     }
     return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
   }
+  // (operands the pipelined kernels cannot address: the 128 x 128 and 64 x 64 tiles of the basic
+  // kernel; its 256 x 256 form on four waves indexes 256 accumulators per lane and is kept
+  // only as a cross-check variant)
   constexpr int64_t kCus = 256;
-  for (int v = 1; v <= 3; ++v)
-    if (tiles(v) >= kCus - kCus / 8) return v;
+  if (tiles(2) >= kCus - kCus / 8) return 2;
   return 3;
 }
 

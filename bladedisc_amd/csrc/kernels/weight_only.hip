@@ -399,7 +399,7 @@ __global__ void __launch_bounds__(NW * 64) wo_skinny_kernel(const WoParams p) {
   const u4 zero = {0, 0, 0, 0};
   // chunks of 32 dealt round-robin over the waves, U in flight per wave: with one byte per
   // weight from HBM the kernel lives on the bytes it keeps in flight
-  constexpr int U = MT == 1 ? 4 : 2;
+  constexpr int U = MT == 1 ? 4 : (MT == 4 && sizeof(XT) == 4 ? 1 : 2);   // (register budget)
   for (int k0 = wave * 32; k0 < p.K; k0 += U * NW * 32) {
     XFrag<XT> xf[U][MT];
     u4 wf[U];
