@@ -27,7 +27,10 @@ inline constexpr Variant kVariants[] = {
     {"mfma_256x256x64_w2x2", 256, 256, 64, 256},
     {"mfma_128x128x64_w2x2", 128, 128, 64, 256},
     {"mfma_64x64x64_w2x2", 64, 64, 64, 256},
-    // software-pipelined kernels, operands loaded straight into LDS
+    // software-pipelined kernels, operands loaded straight into LDS (the 256 x 256 tile on four
+    // waves -- here and in the basic kernel above -- keeps 256 accumulators per lane and spills
+    // part of their indexing: superseded by the eight-wave form, kept as a cross-check variant
+    // that the library never picks by itself)
     {"pipe_256x256x128", 256, 256, 128, 256},
     {"pipe_128x128x128", 128, 128, 128, 256},
     {"pipe_64x64x128", 64, 64, 128, 256},
