@@ -16,7 +16,8 @@
 // activation (11 significant bits) and such a weight (9 bits) are exact in f32, so the only
 // rounding is the f32 accumulation.  f32 activations are split into two halves
 // x = hi + lo (hi = half(x), lo = half(x - hi)) and both are multiplied: about 22 significant
-// bits of x take part.
+// bits of x take part while lo is a normal half (|x| >= 1/8); below, lo is subnormal and the
+// error per activation is an absolute 2^-25.
 //
 // Both operands go from global memory straight into registers in MFMA layout: the order of
 // the k values inside a fragment is free as long as both operands agree, so lane (row, g) takes

@@ -324,8 +324,9 @@ int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
  * (dq8_weight_only_qgemm_workspace_bytes) on every call; a runtime does that once per constant
  * weight with dq8_transpose_s8 and passes tp_b = 1.  Without the scratch, or with K % 16 != 0
  * or rows that are not 16-byte aligned, a slower kernel without alignment rules runs.
- * Accumulation is f32; f32 activations enter the matrix cores as two halves (about 22
- * significant bits). */
+ * Accumulation is f32; f32 activations enter the matrix cores as two halves: about 22
+ * significant bits for |x| >= 1/8, an absolute 2^-25 per activation below (the low half is then
+ * a subnormal half), and |x| must stay below 65504. */
 size_t dq8_weight_only_qgemm_workspace_bytes(int64_t N, int64_t K, int tp_b);
 int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, const void* w, int w_signed,
                           int64_t ldw, int tp_b, const void* scale, const int32_t* zero_points,

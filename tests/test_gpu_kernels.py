@@ -1095,11 +1095,15 @@ def _weight_only_case(rng, m, k, n, dtype, signed):
 
 def _weight_only_check(got, x, w, scale, zp, bias, dtype):
     """|error| <= accumulation bound: products are exact in f32 (half activations; f32 ones
-    enter as two halves, 2^-21 relative), the f32 accumulation of K terms adds K * 2^-24 of
-    sum |x||w|, then one rounding to the output type."""
+    enter as two halves, 2^-21 relative -- or 2^-25 absolute per activation where the low
+    half is a subnormal half, i.e. for |x| < 1/8), the f32 accumulation of K terms adds
+    K * 2^-24 of sum |x||w|, then one rounding to the output type."""
     want, bound = O.weight_only_qgemm(x, w, scale, zp, bias)
     k = x.shape[1]
     tol = bound * (k * 2.0 ** -24 + 2.0 ** -20) + 1e-30
+    if dtype == torch.float32:
+        _, wsum = O.weight_only_qgemm(np.ones((1, k), np.float32), w, scale, zp, None)
+        tol = tol + wsum * 2.0 ** -25
     tol = tol + (np.abs(want) + bound * 2.0 ** -12) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
     err = np.abs(host(got).astype(np.float64) - want)
     assert (err <= tol).all(), "max excess %.3g at %s" % (float((err - tol).max()),
@@ -1143,6 +1147,13 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
                 _weight_only_check(got, x, w, scale, zp, None, dtype)
             got = K.weight_only_qgemm(dev(x), dev(w), dev(scale))
             _weight_only_check(got, x, w, scale, None, None, dtype)
+    # small-magnitude f32 activations: the low halves are subnormal, the absolute term of the
+    # bound takes over
+    if dtype == torch.float32:
+        x, w, scale, zp, bias = _weight_only_case(rng, 40, 256, 96, dtype, False)
+        x = (x * 1e-4).astype(np.float32)
+        got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), None)
+        _weight_only_check(got, x, w, scale, zp, None, dtype)
     # strided activations (a column slice of a wider tensor)
     x, w, scale, zp, bias = _weight_only_case(rng, 64, 64, 96, dtype, False)
     wide = dev(np.concatenate([x, x], axis=1))
