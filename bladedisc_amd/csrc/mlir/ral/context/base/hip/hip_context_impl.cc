@@ -1,5 +1,8 @@
 #include "mlir/ral/context/base/hip/hip_context_impl.h"
 
+#include <cstdlib>
+#include <cctype>
+#include <algorithm>
 #include <mutex>
 #include <sstream>
 #include <unordered_set>
@@ -372,7 +375,71 @@ bool isPersistentDeviceBuffer(ExecutionContext* ctx, const_buffer_t buffer) {
   return state->device_persistent_buffers.count(buffer) != 0;
 }
 
-void RalGlobalConstantState::onContextFinish(Context*) {
+buffer_t processLevelDeviceAlloc(size_t bytes) {
+  void* p = nullptr;
+  return hipMalloc(&p, bytes ? bytes : 1) == hipSuccess ? p : nullptr;
+}
+
+void processLevelDeviceFree(buffer_t buffer) {
+  if (buffer) (void)hipFree(buffer);
+}
+
+bool discEnableGlobalConstantStore() {
+  static const bool enabled = [] {
+    const char* env = std::getenv("DISC_USE_GLOBAL_CONST_STORE");
+    if (!env) return false;
+    std::string v = env;
+    std::transform(v.begin(), v.end(), v.begin(),
+                   [](unsigned char c) { return (char)std::tolower(c); });
+    return v == "true" || v == "1";
+  }();
+  return enabled;
+}
+
+ConstStoreRegistrar& ConstStoreRegistrar::Instance() {
+  static ConstStoreRegistrar instance;
+  return instance;
+}
+
+bool ConstStoreRegistrar::unregisterConstStore(ProcessLevelConstStore* store) {
+  std::lock_guard<std::mutex> guard(mu);
+  auto it = referenceCounter.find(store);
+  if (it == referenceCounter.end()) return false;
+  if (--it->second > 0) return false;
+  pbFile2Instance.erase(store->pb_file_path);
+  referenceCounter.erase(it);
+  return true;
+}
+
+ProcessLevelConstStore* ConstStoreRegistrar::getConstStore(const std::string& pb_file_path) {
+  std::lock_guard<std::mutex> guard(mu);
+  auto it = pbFile2Instance.find(pb_file_path);
+  if (it == pbFile2Instance.end()) {
+    std::unique_ptr<ProcessLevelConstStore> store(new ProcessLevelConstStore);
+    store->pb_file_path = pb_file_path;
+    store->state.metadata = MetadataFile::loadFromFile(pb_file_path);
+    if (!store->state.metadata) {
+      TAO_LOG(ERROR) << "failed to load metadata file from: " << pb_file_path;
+      return nullptr;
+    }
+    it = pbFile2Instance.emplace(pb_file_path, store.release()).first;
+  }
+  ++referenceCounter[it->second];
+  return it->second;
+}
+
+void RalGlobalConstantState::onContextFinish(Context* ctx) {
+  if (process_level_store) {
+    // the last context to finish releases what the shared store holds
+    ProcessLevelConstStore* store = process_level_store;
+    process_level_store = nullptr;
+    if (!ConstStoreRegistrar::Instance().unregisterConstStore(store)) return;
+    (void)ctx;
+    for (auto& kv : store->state.device_constants) processLevelDeviceFree(kv.second.first);
+    for (auto& kv : store->state.host_constants) ::operator delete(kv.second.first);
+    delete store;
+    return;
+  }
   // device constants come from alloc_persistent and go with the context state
   for (auto& kv : host_constants) ::operator delete(kv.second.first);
   host_constants.clear();
@@ -384,8 +451,13 @@ std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
   std::unique_ptr<BaseContext> ctx(new BaseContext(opt));
   ctx->getOrCreateResource(kRalGlobalConstantState, [opt]() {
     auto* state = new RalGlobalConstantState;
-    if (!opt.metadata_file_path.empty())
-      state->metadata = MetadataFile::loadFromFile(opt.metadata_file_path);
+    if (!opt.metadata_file_path.empty()) {
+      if (discEnableGlobalConstantStore())
+        state->process_level_store =
+            ConstStoreRegistrar::Instance().getConstStore(opt.metadata_file_path);
+      if (!state->process_level_store)
+        state->metadata = MetadataFile::loadFromFile(opt.metadata_file_path);
+    }
     return state;
   });
   ctx->addDriver(GPUDriver::name(), std::unique_ptr<GPUDriver>(new GPUDriver(ctx.get())));

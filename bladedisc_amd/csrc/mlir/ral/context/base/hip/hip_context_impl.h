@@ -140,15 +140,45 @@ extern const char* kRalBaseHipContextState;
 
 // Context-level store of the program's constants (ral_const): loaded lazily from the
 // metadata file named in BaseContextOption, kept for the life of the context.
+struct ProcessLevelConstStore;
 struct RalGlobalConstantState : public Context::Resource {
   using Item = std::pair<buffer_t, buffer_shape_t>;
   std::mutex mu;
   std::unordered_map<std::string, Item> host_constants;
   std::unordered_map<std::string, Item> device_constants;
   std::unique_ptr<MetadataFile> metadata;
+  // if set, the constants live in this store, shared by every context of the process that was
+  // made from the same metadata file, instead of in the maps above
+  ProcessLevelConstStore* process_level_store = nullptr;
   void onContextFinish(Context* ctx) override;
 };
 extern const char* kRalGlobalConstantState;
+
+// Process-level store of constants (reference: ral/context/common_context_impl.h:34-58,
+// 116-119; common_context_impl.cc:152-186): one per metadata file path, reference-counted by
+// the contexts that use it; its device buffers are released by the last context to finish
+// (the reference takes them from raw_alloc, i.e. from the embedding framework's allocator,
+// which outlives its contexts; here they come straight from hipMalloc).  Switched on by DISC_USE_GLOBAL_CONST_STORE=true|1
+// (common_context_impl.cc:57-64, read once per process).
+struct ProcessLevelConstStore {
+  RalGlobalConstantState state;
+  std::string pb_file_path;
+};
+struct ConstStoreRegistrar {
+  static ConstStoreRegistrar& Instance();
+  // true if the caller was the last user and now owns (and must release) the store
+  bool unregisterConstStore(ProcessLevelConstStore* store);
+  ProcessLevelConstStore* getConstStore(const std::string& pb_file_path);
+  std::mutex mu;
+  std::unordered_map<std::string, ProcessLevelConstStore*> pbFile2Instance;
+  std::unordered_map<ProcessLevelConstStore*, int> referenceCounter;
+};
+bool discEnableGlobalConstantStore();
+// Device memory of the process-level store: owned by no context (a context's own allocator
+// returns everything it handed out when the context goes away, and these buffers must
+// outlive all but the last of their users).
+buffer_t processLevelDeviceAlloc(size_t bytes);
+void processLevelDeviceFree(buffer_t buffer);
 
 // device buffers that outlive executions (alloc_persistent): true if `buffer` is one
 bool isPersistentDeviceBuffer(ExecutionContext* ctx, const_buffer_t buffer);

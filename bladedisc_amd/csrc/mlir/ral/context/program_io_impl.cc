@@ -130,6 +130,10 @@ buffer_t deviceConstant(ExecutionContext* ctx, void* stream_handle, const char* 
     ctx->signalError(Context::FAILURE, "ral_const: no constant store");
     return nullptr;
   }
+  // the process-level store, if enabled, in place of the context's own
+  // (R context/common_context_impl_cuda.cc:66-73, 119-121)
+  const bool shared = state->process_level_store != nullptr;
+  if (shared) state = &state->process_level_store->state;
   std::lock_guard<std::mutex> guard(state->mu);
   const std::string key(unique_name);
   auto it = state->device_constants.find(key);
@@ -138,7 +142,8 @@ buffer_t deviceConstant(ExecutionContext* ctx, void* stream_handle, const char* 
     std::vector<uint8_t> bytes;
     if (!constantBytes(ctx, state, key, false, &dims, &bytes)) return nullptr;
     auto* drv = ctx->getDriver<GPUDriver>(GPUDriver::name());
-    buffer_t dev = drv->alloc_persistent(ctx, bytes.empty() ? 1 : bytes.size());
+    const size_t size = bytes.empty() ? 1 : bytes.size();
+    buffer_t dev = shared ? processLevelDeviceAlloc(size) : drv->alloc_persistent(ctx, size);
     if (!dev) return nullptr;
     if (!bytes.empty()) {
       drv->h2d(ctx, stream_handle, bytes.data(), dev, bytes.size());
@@ -157,6 +162,7 @@ buffer_t hostConstant(ExecutionContext* ctx, const char* unique_name, buffer_sha
     ctx->signalError(Context::FAILURE, "ral_const: no constant store");
     return nullptr;
   }
+  if (state->process_level_store) state = &state->process_level_store->state;
   std::lock_guard<std::mutex> guard(state->mu);
   const std::string key(unique_name);
   auto it = state->host_constants.find(key);

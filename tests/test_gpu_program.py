@@ -100,6 +100,26 @@ def test_compiled_program_runs_on_the_runtime(program):
         L.disc_ral_context_destroy(C.c_void_p(ctx))
 
 
+def test_process_level_constant_store(program):
+    """DISC_USE_GLOBAL_CONST_STORE=1 (common_context_impl.cc:57-64): contexts made from one
+    metadata file share one store of constants, which outlives all but the last of them; without
+    the switch a second context has to load the file itself.  In child processes: the switch is
+    read once per process."""
+    import sys
+    lib, d = program
+    so = str(d / "libqlinear_program.so")
+    script = os.path.join(HERE, "programs", "shared_const_store_scenario.py")
+    for value, want in (("1", 0), (None, 3)):
+        env = dict(os.environ)
+        env.pop("DISC_USE_GLOBAL_CONST_STORE", None)
+        if value is not None:
+            env["DISC_USE_GLOBAL_CONST_STORE"] = value
+        r = subprocess.run([sys.executable, script, so, str(d)], env=env, capture_output=True,
+                           text=True, timeout=300)
+        assert r.returncode == want, (value, r.returncode, r.stdout[-800:], r.stderr[-800:])
+    assert "OK" in r.stdout or want == 3
+
+
 def test_program_with_an_embedded_code_object(program):
     """The same program with its dequantize replaced by a fused elementwise kernel that
     travels as a gfx950 code object, the way the compiler ships its generated kernels, and
