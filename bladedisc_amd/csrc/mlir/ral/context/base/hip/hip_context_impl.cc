@@ -1,5 +1,6 @@
 #include "mlir/ral/context/base/hip/hip_context_impl.h"
 
+#include <cstring>
 #include <cstdlib>
 #include <cctype>
 #include <algorithm>
@@ -335,6 +336,16 @@ void BaseHipExecutionContext::bindOutput(int output_idx,
   if (!state) return;
   std::lock_guard<std::mutex> guard(state->mu);
   if (state->device_persistent_buffers.count(buffer)) return;
+  auto hit = host_ptr_map.find(buffer);
+  if (hit != host_ptr_map.end()) {
+    // a host output the program took from the cpu device's `alloc`
+    if (--hit->second == 0) {
+      wrapper->set_deleter([](buffer_t data) { std::free(data); });
+      host_ptr_map.erase(hit);
+    }
+    if (outputSharedOrder[buffer] == 1) wrapper->markOwned();
+    return;
+  }
   auto dit = device_ptr_map.find(buffer);
   if (dit == device_ptr_map.end()) return;
   if (--dit->second == 0) {
@@ -365,6 +376,16 @@ BaseHipExecutionContext::~BaseHipExecutionContext() {
     }
   }
   device_ptr_map.clear();
+  auto* host = getResource<BaseHostContextState>(kRalBaseCpuContextState);
+  for (auto& kv : host_ptr_map) {
+    bool persistent = false;
+    if (host) {
+      std::lock_guard<std::mutex> guard(host->mu);
+      persistent = host->host_persistent_buffers.count(kv.first) != 0;
+    }
+    if (!persistent && !input_ptr_set.count(kv.first)) std::free(const_cast<buffer_t>(kv.first));
+  }
+  host_ptr_map.clear();
   onExecutionFinish();
 }
 
@@ -461,6 +482,7 @@ std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
     return state;
   });
   ctx->addDriver(GPUDriver::name(), std::unique_ptr<GPUDriver>(new GPUDriver(ctx.get())));
+  ctx->getOrCreateResource(kRalBaseCpuContextState, []() { return new BaseHostContextState; });
   ctx->getOrCreateResource(kRalBaseHipContextState, [opt, gpu_opt]() {
     auto* state = new BaseHipContextState;
     state->stream = gpu_opt.stream;
@@ -482,6 +504,100 @@ std::unique_ptr<BaseContext> MakeBaseHipContext(BaseContextOption& opt,
 }
 
 }  // namespace gpu
+
+// ------------------------------------------------------------ host (cpu device) memory
+// A program compiled for the gpu keeps its host-placed values (shape tensors, scalars) in
+// memory it takes from the cpu device's driver entries
+// (R context/base/cpu/cpu_context_impl.cc:105-213; names R device/cpu/cpu_driver.cc:29-35).
+namespace gpu {
+const char* kRalBaseCpuContextState = "ral_base_cpu_context_state";
+
+void BaseHostContextState::onContextFinish(Context*) {
+  std::lock_guard<std::mutex> guard(mu);
+  for (const_buffer_t b : host_persistent_buffers) std::free(const_cast<buffer_t>(b));
+  host_persistent_buffers.clear();
+}
+
+namespace cpu {
+namespace {
+buffer_t hostAlloc(size_t bytes) {
+  // 64-byte aligned, as the reference's aligned_malloc
+  const size_t n = (std::max<size_t>(bytes, 1) + 63) / 64 * 64;
+  return std::aligned_alloc(64, n);
+}
+}  // namespace
+
+buffer_t ral_base_cpu_alloc(ExecutionContext* ctx, size_t bytes) {
+  auto* exec = dynamic_cast<BaseHipExecutionContext*>(ctx);
+  if (!exec) {
+    ctx->signalError(Context::FAILURE, "alloc (cpu) needs a BaseHipExecutionContext");
+    return nullptr;
+  }
+  buffer_t ptr = hostAlloc(bytes);
+  if (!ptr) {
+    ctx->signalError(Context::FAILURE, "host allocation of " + std::to_string(bytes) + " bytes failed");
+    return nullptr;
+  }
+  exec->host_ptr_map[ptr] = 1;
+  return ptr;
+}
+
+buffer_t ral_base_cpu_alloc_persistent(ExecutionContext* ctx, size_t bytes) {
+  auto* state = ctx->getResource<BaseHostContextState>(kRalBaseCpuContextState);
+  if (!state) {
+    ctx->signalError(Context::FAILURE, "no host memory state in this context");
+    return nullptr;
+  }
+  buffer_t ptr = hostAlloc(bytes);
+  if (!ptr) {
+    ctx->signalError(Context::FAILURE, "host allocation of " + std::to_string(bytes) + " bytes failed");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(state->mu);
+  state->host_persistent_buffers.insert(ptr);
+  return ptr;
+}
+
+void ral_base_cpu_dealloc(ExecutionContext* ctx, buffer_t buffer) {
+  if (!buffer) return;
+  auto* state = ctx->getResource<BaseHostContextState>(kRalBaseCpuContextState);
+  if (state) {
+    std::lock_guard<std::mutex> guard(state->mu);
+    if (state->host_persistent_buffers.count(buffer)) return;   // persistent: ignored
+  }
+  auto* exec = dynamic_cast<BaseHipExecutionContext*>(ctx);
+  if (!exec) return;
+  auto it = exec->host_ptr_map.find(buffer);
+  if (it == exec->host_ptr_map.end()) return;
+  if (--it->second == 0) {
+    // (an alias of a program input was pinned by inc_ref: the buffer is the caller's)
+    if (!exec->input_ptr_set.count(buffer)) std::free(buffer);
+    exec->host_ptr_map.erase(it);
+  }
+}
+
+buffer_t ral_base_cpu_raw_alloc(Context*, size_t bytes) { return hostAlloc(bytes); }
+
+void ral_base_cpu_raw_dealloc(Context*, buffer_t buffer) { std::free(buffer); }
+
+void ral_base_cpu_memcpy(ExecutionContext*, buffer_t from, buffer_t to, size_t bytes) {
+  if (bytes) std::memcpy(to, from, bytes);
+}
+
+void ral_base_cpu_memset(ExecutionContext*, buffer_t buffer, int value, size_t bytes) {
+  if (bytes) std::memset(buffer, value, bytes);
+}
+
+}  // namespace cpu
+}  // namespace gpu
+
+TAO_RAL_API("alloc", "cpu", gpu::cpu::ral_base_cpu_alloc);
+TAO_RAL_API("ral_cpu_alloc_persistent", "cpu", gpu::cpu::ral_base_cpu_alloc_persistent);
+TAO_RAL_API("dealloc", "cpu", gpu::cpu::ral_base_cpu_dealloc);
+TAO_RAL_API("raw_cpu_alloc", "cpu", gpu::cpu::ral_base_cpu_raw_alloc);
+TAO_RAL_API("raw_cpu_dealloc", "cpu", gpu::cpu::ral_base_cpu_raw_dealloc);
+TAO_RAL_API("ral_cpu_memcpy", "cpu", gpu::cpu::ral_base_cpu_memcpy);
+TAO_RAL_API("ral_cpu_memset", "cpu", gpu::cpu::ral_base_cpu_memset);
 
 TAO_RAL_API(tao::ral::gpu::kRalGpuAlloc, "gpu", gpu::ral_base_hip_alloc);
 TAO_RAL_API(tao::ral::gpu::kRalGpuAllocPersistent, "gpu", gpu::ral_base_hip_alloc_persistent);

@@ -128,6 +128,9 @@ struct BaseHipExecutionContext : public ExecutionContext {
 
   // buffers handed out by `alloc` during this execution -> reference count
   std::unordered_map<const_buffer_t, int> device_ptr_map;
+  // the same for host buffers (`alloc` of the cpu device: shape tensors and other host-placed
+  // values of a program compiled for the gpu)
+  std::unordered_map<const_buffer_t, int> host_ptr_map;
   std::unordered_map<int32_t, Tensor> inputs;
   std::unordered_map<int32_t, Tensor> outputs;
   std::unordered_set<const_buffer_t> input_ptr_set;
@@ -137,6 +140,15 @@ struct BaseHipExecutionContext : public ExecutionContext {
 };
 
 extern const char* kRalBaseHipContextState;
+
+// Host memory of the cpu-device driver entries (reference: ral/context/base/cpu/
+// cpu_context_impl.cc:105-204, BaseCpuContextState): buffers that outlive executions.
+struct BaseHostContextState : public Context::Resource {
+  std::mutex mu;
+  std::unordered_set<const_buffer_t> host_persistent_buffers;
+  void onContextFinish(Context* ctx) override;
+};
+extern const char* kRalBaseCpuContextState;
 
 // Context-level store of the program's constants (ral_const): loaded lazily from the
 // metadata file named in BaseContextOption, kept for the life of the context.

@@ -299,7 +299,35 @@ void addReference(ExecutionContext* ctx, buffer_t ptr) {
     ctx->signalError(Context::FAILURE, "inc_ref: buffer is not known to this execution");
   }
 }
+
+// the same for host buffers (inc_ref on the cpu device, R context/base/cpu/
+// cpu_context_impl.cc:232-255)
+void addHostReference(ExecutionContext* ctx, buffer_t ptr) {
+  auto* exec = execOf(ctx);
+  if (!exec || !ptr) return;
+  auto it = exec->host_ptr_map.find(ptr);
+  if (it != exec->host_ptr_map.end()) {
+    ++it->second;
+    return;
+  }
+  bool persistent = false;
+  if (auto* host = ctx->getResource<BaseHostContextState>(kRalBaseCpuContextState)) {
+    std::lock_guard<std::mutex> guard(host->mu);
+    persistent = host->host_persistent_buffers.count(ptr) != 0;
+  }
+  if (exec->input_ptr_set.count(ptr) || persistent) {
+    exec->host_ptr_map[ptr] = 2;    // borrowed: never released through this alias
+  } else {
+    ctx->signalError(Context::FAILURE, "inc_ref: host buffer is not known to this execution");
+  }
+}
 }  // namespace
+
+template <typename T, int N>
+MemRefType<T, N> ral_inc_ref_host(ExecutionContext* ctx, void*, MemRefType<T, N> input) {
+  addHostReference(ctx, input.data);
+  return input;
+}
 
 template <typename T, int N>
 MemRefType<T, N> ral_inc_ref(ExecutionContext* ctx, void*, MemRefType<T, N> input) {
@@ -374,6 +402,7 @@ void ral_d2d_memref(ExecutionContext* ctx, void* stream_handle, MemRefType<T, N>
   TAO_RAL_API(tao::ral::kRalCudaConst, "gpu", gpu::io::ral_const_device<T, N>);      \
   TAO_RAL_API(tao::ral::kRalHostConst, "cpu", gpu::io::ral_const_host<T, N>);        \
   TAO_RAL_API(tao::ral::kRalBitcast, "gpu", gpu::io::ral_inc_ref<T, N>);             \
+  TAO_RAL_API(tao::ral::kRalBitcast, "cpu", gpu::io::ral_inc_ref_host<T, N>);        \
   TAO_RAL_API("h2d", "gpu", gpu::io::ral_h2d_memref<T, N>);                          \
   TAO_RAL_API("d2h", "gpu", gpu::io::ral_d2h_memref<T, N>);                          \
   TAO_RAL_API("d2d", "gpu", gpu::io::ral_d2d_memref<T, N>);

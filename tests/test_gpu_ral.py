@@ -420,6 +420,61 @@ def test_ral_quantize_dequantize_wide_types(rt, name, code, store):
         np.testing.assert_array_equal(host(f), O.dequantize(want, scale, zp, axis=1))
 
 
+def test_host_memory_entries_of_the_cpu_device(rt):
+    """What a program compiled for the gpu uses for its host-placed values (shape tensors):
+    alloc / dealloc / inc_ref on the cpu device with reference counting, persistent and raw
+    allocations, memset and memcpy (cpu_context_impl.cc:105-255, cpu_driver.cc:29-35)."""
+    import ctypes as C
+    ctx, ral, ops = rt
+
+    def call(ex, name, codes_values, ret=None):
+        a = ral.Args().ctx(ex.handle)
+        for code, v in codes_values:
+            a.scalar(code, v)
+        r = a.result_scalar(ret) if ret else None
+        ex.call(name, "cpu", a)
+        return r.value if ret else None
+
+    with ctx.execution() as ex:
+        p = call(ex, "alloc", [("i64", 64)], "pvoid")
+        q = call(ex, "alloc", [("i64", 0)], "pvoid")            # zero bytes still gives a buffer
+        assert p and q and p != q and p % 64 == 0
+        call(ex, "ral_cpu_memset", [("pvoid", p), ("i32", 7), ("i64", 64)])
+        assert bytes((C.c_uint8 * 64).from_address(p)) == b"\x07" * 64
+        src = (C.c_int64 * 4)(11, 22, 33, 44)
+        call(ex, "ral_cpu_memcpy", [("pvoid", C.addressof(src)), ("pvoid", p), ("i64", 32)])
+        assert list((C.c_int64 * 4).from_address(p)) == [11, 22, 33, 44]
+        # a second memref over the same host buffer: one more reference
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0).memref("i64", p, [4])
+        alias = a.result_memref("i64", 1)
+        ex.call("inc_ref", "cpu", a)
+        assert alias.data == p and alias.sizes[0] == 4
+        call(ex, "dealloc", [("pvoid", p)])                     # first reference
+        assert list((C.c_int64 * 4).from_address(p)) == [11, 22, 33, 44]   # still alive
+        call(ex, "dealloc", [("pvoid", p)])                     # second: released
+        call(ex, "dealloc", [("pvoid", q)])
+        call(ex, "dealloc", [("pvoid", 0)])                     # null: ignored
+        # persistent host memory survives dealloc and the execution
+        keep = call(ex, "ral_cpu_alloc_persistent", [("i64", 16)], "pvoid")
+        (C.c_int32 * 4).from_address(keep)[:] = [1, 2, 3, 4]
+        call(ex, "dealloc", [("pvoid", keep)])
+        # an alias of something the execution never saw is an error
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0).memref("i64", C.addressof(src), [4])
+        a.result_memref("i64", 1)
+        with pytest.raises(ral.RalError, match="not known"):
+            ex.call("inc_ref", "cpu", a)
+        leaked = call(ex, "alloc", [("i64", 128)], "pvoid")     # returned with the execution
+        assert leaked
+    with ctx.execution() as ex:
+        assert list((C.c_int32 * 4).from_address(keep)) == [1, 2, 3, 4]
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0).memref("i32", keep, [4])
+        a.result_memref("i32", 1)
+        ex.call("inc_ref", "cpu", a)                            # persistent: pinned, never freed
+        call(ex, "dealloc", [("pvoid", keep)])
+        call(ex, "dealloc", [("pvoid", keep)])
+        assert list((C.c_int32 * 4).from_address(keep)) == [1, 2, 3, 4]
+
+
 def test_driver_alloc_copy_roundtrip_and_pool_reuse(rt):
     ctx, ral, ops = rt
     import ctypes as C
