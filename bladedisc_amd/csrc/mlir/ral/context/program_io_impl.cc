@@ -335,7 +335,7 @@ MemRefType<T, N> ral_inc_ref(ExecutionContext* ctx, void*, MemRefType<T, N> inpu
   return input;
 }
 
-template <typename T, int N, int M, typename P = int64_t>
+template <typename T, int N, int M, bool HOST = false, typename P = int64_t>
 MemRefType<T, M> ral_inc_ref_reshape(ExecutionContext* ctx, void*, MemRefType<T, N> input,
                                      MemRefType<P, 1> shape) {
   MemRefType<T, M> out;
@@ -353,7 +353,10 @@ MemRefType<T, M> ral_inc_ref_reshape(ExecutionContext* ctx, void*, MemRefType<T,
     out.strides[i] = stride;
     stride *= out.sizes[i];
   }
-  addReference(ctx, input.data);
+  if (HOST)
+    addHostReference(ctx, input.data);
+  else
+    addReference(ctx, input.data);
   return out;
 }
 
@@ -407,8 +410,9 @@ void ral_d2d_memref(ExecutionContext* ctx, void* stream_handle, MemRefType<T, N>
   TAO_RAL_API("d2h", "gpu", gpu::io::ral_d2h_memref<T, N>);                          \
   TAO_RAL_API("d2d", "gpu", gpu::io::ral_d2d_memref<T, N>);
 
-#define RAL_IO_RESHAPE(T, N, M) \
-  TAO_RAL_API(tao::ral::kRalBitcast, "gpu", gpu::io::ral_inc_ref_reshape<T, N, M>);
+#define RAL_IO_RESHAPE(T, N, M)                                                      \
+  TAO_RAL_API(tao::ral::kRalBitcast, "gpu", gpu::io::ral_inc_ref_reshape<T, N, M>); \
+  TAO_RAL_API(tao::ral::kRalBitcast, "cpu", (gpu::io::ral_inc_ref_reshape<T, N, M, true>));
 
 #define RAL_IO_FOR_TYPE(T)                                                           \
   TAO_RAL_API(tao::ral::kRalRecvInput, "cpu", gpu::io::ral_recv_input_0d<T>);        \

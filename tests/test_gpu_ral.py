@@ -449,9 +449,17 @@ def test_host_memory_entries_of_the_cpu_device(rt):
         alias = a.result_memref("i64", 1)
         ex.call("inc_ref", "cpu", a)
         assert alias.data == p and alias.sizes[0] == 4
-        call(ex, "dealloc", [("pvoid", p)])                     # first reference
+        # ... and a reshaped one ([4] -> [2, 2], shape operand on the host): a third
+        shp = np.array([2, 2], np.int64)
+        a = ral.Args().ctx(ex.handle).scalar("pvoid", 0).memref("i64", p, [4])
+        a.host_array(shp)
+        view = a.result_memref("i64", 2)
+        ex.call("inc_ref", "cpu", a)
+        assert view.data == p and list(view.sizes) == [2, 2] and list(view.strides) == [2, 1]
+        call(ex, "dealloc", [("pvoid", p)])
+        call(ex, "dealloc", [("pvoid", p)])                     # two references gone
         assert list((C.c_int64 * 4).from_address(p)) == [11, 22, 33, 44]   # still alive
-        call(ex, "dealloc", [("pvoid", p)])                     # second: released
+        call(ex, "dealloc", [("pvoid", p)])                     # the last one: released
         call(ex, "dealloc", [("pvoid", q)])
         call(ex, "dealloc", [("pvoid", 0)])                     # null: ignored
         # persistent host memory survives dealloc and the execution
