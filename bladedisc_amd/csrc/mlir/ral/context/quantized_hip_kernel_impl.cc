@@ -874,6 +874,20 @@ void ral_qconv(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4>
   kernelFailed(ctx, st, who);
 }
 
+// The older entry without zero-point operands (R context/common_context_impl_quantization.cc:
+// 38-44, registered at :1680 as "ral_qconv_s8_s8_s8"): the same convolution.
+void ral_qconv_s8_s8_s8(ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, 4> input,
+                        MemRefType<int8_t, 4> kernel, MemRefType<int32_t, 1> padding,
+                        MemRefType<float, 0> inputScales, MemRefType<float, 1> filterScales,
+                        MemRefType<float, 0> outputScales, MemRefType<int8_t, 4> output,
+                        MemRefType<int32_t, 1> metadata) {
+  MemRefType<int32_t, 0> no_zp0 = assignMemRef_0d<int32_t>(nullptr);
+  int64_t zero[1] = {0};
+  MemRefType<int32_t, 1> no_zp1 = assignMemRef<int32_t, 1>(nullptr, zero);
+  ral_qconv(ctx, stream_handle, input, kernel, padding, inputScales, no_zp0, filterScales, no_zp1,
+            outputScales, no_zp0, output, metadata);
+}
+
 // ----------------------------------------------------------- ral_pdll_qconv2d
 // The attribute-driven convolution entry: data_format / strides / dilations / padding
 // come as custom attributes, the result is allocated here.  Weights are
@@ -1111,6 +1125,7 @@ DQ8_REGISTER_WEIGHT_ONLY(float16, 3)
 #undef DQ8_REGISTER_WEIGHT_ONLY
 
 TAO_RAL_API("ral_qconv", "gpu", gpu::q8::ral_qconv);
+TAO_RAL_API("ral_qconv_s8_s8_s8", "gpu", gpu::q8::ral_qconv_s8_s8_s8);
 TAO_RAL_API("ral_pdll_qconv2d", "gpu", gpu::q8::ral_pdll_qconv2d);
 
 #define DQ8_REGISTER_QDQ(QT, N)                                              \

@@ -158,6 +158,19 @@ def qconv(ex, x, w, padding, metadata, sx, sw_c, so, out):
     return out
 
 
+def qconv_s8_s8_s8(ex, x, w, padding, metadata, sx, sw_c, so, out):
+    """ral_qconv_s8_s8_s8: the older symmetric entry, ral_qconv without zero-point operands."""
+    a = ex.new_args().tensor(x).tensor(w)
+    a.host_array(np.asarray(padding, np.int32))
+    a.tensor(sx, rank0=True)
+    a.tensor(sw_c)
+    a.tensor(so, rank0=True)
+    a.tensor(out)
+    a.host_array(np.asarray(metadata, np.int32))
+    ex.call("ral_qconv_s8_s8_s8", "gpu", a)
+    return out
+
+
 def pdll_qconv2d(ex, x, w_ohwi, sx, sw_c, so, data_format="NHWC", strides=(1, 1, 1, 1),
                  dilations=(1, 1, 1, 1), padding="SAME", explicit_paddings=(),
                  weight_is_const=True, zo=0):

@@ -258,6 +258,10 @@ def test_ral_qconv(rt, nb, h, ci, co, k, stride, pad):
     with ctx.execution() as ex:
         ops.qconv(ex, dev(x), dev(w), padding, md, f1(sx), dev(sw), f1(so), out)
         np.testing.assert_array_equal(host(out), want)
+        # the older entry without zero-point operands gives the same bits
+        out2 = torch.empty_like(out)
+        ops.qconv_s8_s8_s8(ex, dev(x), dev(w), padding, md, f1(sx), dev(sw), f1(so), out2)
+        np.testing.assert_array_equal(host(out2), want)
 
 
 @pytest.mark.parametrize("fmt,padding,k,stride,dil", [("NHWC", "SAME", 3, 1, 1), ("NHWC", "VALID", 3, 2, 2),

@@ -15,6 +15,8 @@ GOLDEN_NAMES = [
     "ral_qgemm___gpu___pvoid_pvoid_m2di8_m2di8_m0df32_m0di32_m1df32_m1di32_m0df32_m0di32_m2di8_i1_i1_i1___void",
     # stream_executor_based_impl.cc:1831-1841,1999-2000
     "ral_qconv___gpu___pvoid_pvoid_m4di8_m4di8_m1di32_m0df32_m0di32_m1df32_m1di32_m0df32_m0di32_m4di8_m1di32___void",
+    # the older symmetric entry (common_context_impl_quantization.cc:38-44, registered for cpu at :1680) mirrored on gpu
+    "ral_qconv_s8_s8_s8___gpu___pvoid_pvoid_m4di8_m4di8_m1di32_m0df32_m1df32_m0df32_m4di8_m1di32___void",
     # quantized_gpu_kernel_impl.cc:424-475
     "ral_pdll_qgemm___gpu___pvoid_pvoid_m2di8_m2di8_m1di8_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m2di8",
     "ral_pdll_qgemm___gpu___pvoid_pvoid_m3di8_m2di8_m1di8_m0df32_m0di32_m0df32_m0di32_m0df32_m0di32_pvoid___m3di8",
