@@ -50,6 +50,7 @@ _PROTOS = {
     "dq8_mfma_probe": (_INT, [_VP] * 7),
     "dq8_lut8": (_INT, [_VP, _VP, _I64, _VP, _VP]),
     "dq8_weight_only_qgemm_workspace_bytes": (C.c_size_t, [_I64, _I64, _INT]),
+    "dq8_weight_only_qgemm_workspace_bytes_ex": (C.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "dq8_weight_only_qgemm": (_INT, [_VP, _INT, _I64, _VP, _INT, _I64, _INT, _VP, _VP, _VP, _VP,
                                      _I64, _I64, _I64, _I64, _VP, C.c_size_t, _VP]),
     "dq8_fake_quant": (_INT, [_VP, _VP, _I64, _I64, _I64, _VP, _VP, _I64, _I32, _I32, _INT, _VP]),

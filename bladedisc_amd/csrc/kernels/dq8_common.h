@@ -30,6 +30,9 @@ inline bool aligned(const void* p, size_t a) {
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// number of compute units of the current device (cached; 256 when no device answers)
+int compute_units();
+
 // Dynamic LDS above the default limit has to be allowed per kernel and per device.  `done`
 // is the kernel's bit set of devices (by ordinal) on which that has happened; two threads
 // racing on the first launch both set the attribute, which is harmless.

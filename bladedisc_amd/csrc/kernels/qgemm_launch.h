@@ -76,8 +76,6 @@ inline bool is_pipe_variant(int v) {
 }
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
-// number of compute units of the current device (cached)
-int compute_units();
 
 template <int BM, int BN, int BK, int WM, int WN, bool CONV, int EPI>
 int launch_mfma(const MainParams& p, hipStream_t st) {

@@ -34,6 +34,8 @@
 //    per weight from HBM);
 //  * wo_generic_kernel: one output per thread, any layout and alignment (also weights left as
 //    [K, N]).
+#include <algorithm>
+
 #include "dq8_common.h"
 #include "disc_q8.h"
 
@@ -48,6 +50,9 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef unsigned u4 __attribute__((ext_vector_type(4)));
 
+// gfx9 raw buffer descriptor word 3: 32-bit data format, no swizzle
+constexpr int kBufferWord3 = 0x00020000;
+
 struct WoParams {
   const void* x;        // [M, K] activations, row stride ldx elements
   const uint8_t* w;     // weights; element (n, k) at w[n * w_sn + k * w_sk]
@@ -58,6 +63,10 @@ struct WoParams {
   int64_t ldx, ldo, w_sn, w_sk;
   int M, N, K;
   unsigned flip;        // 0x80808080 for signed weights (b ^ 0x80 = b + 128 as unsigned)
+  // split k (wo_lds_kernel): workgroup (tile, y) multiplies k in [y k_split, (y + 1) k_split)
+  // and, when `partial` is set, leaves its f32 sums in partial[y][M][N] for the reduction kernel
+  float* partial;
+  int k_split;          // a multiple of 64; K when the k range is not split
 };
 
 template <typename T>
@@ -132,6 +141,18 @@ __device__ __forceinline__ void store_frag(const WoParams& p, const f16v& acc, i
   for (int v = 0; v < 16; ++v) {
     const int m = m_base + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
     if (m < p.M) out[(int64_t)m * p.ldo + n] = (XT)(acc[v] * s + b);
+  }
+}
+
+// The raw sums of one k range, for wo_splitk_reduce_kernel.
+__device__ __forceinline__ void store_partial(const WoParams& p, const f16v& acc, int split,
+                                              int m_base, int n, int lane) {
+  if (n >= p.N) return;
+  float* dst = p.partial + (int64_t)split * p.M * p.N;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int m = m_base + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+    if (m < p.M) dst[(int64_t)m * p.N + n] = acc[v];
   }
 }
 
@@ -224,90 +245,99 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
 }
 
 // ---------------------------------------------------------------- tiled kernel through LDS (f16)
-// (64 WM) x 128 tile, WM x 2 waves (WM = 2 or 4), k tiles of 64 in two LDS stages.  The
-// register kernel above makes every lane fetch its own row, 64 cache lines per load instruction, and the compute unit's
-// address path caps it at about 15 bytes per clock (0.4 PFLOP/s whatever the shape); here
-// eight lanes cover one 128-byte row segment of the activations and four one 64-byte segment of
-// the weights, the tile is shared through LDS (16-byte chunks XOR-swizzled by the row so that
-// the fragment reads spread over the banks), and the fragments are read back as ds_read_b128.
-template <int WM, bool WIDE>
+// (64 WM) x 128 tile, WM x 2 waves (WM = 1, 2 or 4), k tiles of 64 in two LDS stages.  The
+// register kernel above makes every lane fetch its own row, 64 cache lines per load
+// instruction, and the compute unit's address path caps it at about 15 bytes per clock
+// (0.4 PFLOP/s whatever the shape); here eight lanes cover one 128-byte row segment of the
+// activations and four one 64-byte segment of the weights, the tile is shared through LDS
+// (16-byte chunks XOR-swizzled by the row so that the fragment reads spread over the banks),
+// and the fragments are read back as ds_read_b128.  The weights are widened to halves once,
+// on their way into LDS (128-byte rows like the activations'), not by every wave that reads
+// them.
+//
+// Four register sets hold the k tiles t + 1 .. t + 4 on their way from memory while tile t is
+// multiplied.  The loads are buffer loads without a branch around them (a chunk past the k
+// range gets an offset past the descriptor and reads zeros) and the main loop is four k tiles
+// of straight-line code, so that the wait in front of a tile's hand-over to LDS counts the
+// loads issued after it instead of draining them all: with conditional loads in a loop of
+// guarded steps every k tile waited out a whole trip to memory (0.8 us per k tile on a
+// quiet chip, 1.5-2 us on a busy one).
+template <int WM>
 __global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
   constexpr int BM = WM * 64, BN = 128, BK = 64;
   constexpr int NT = WM * 128;                           // WM x 2 waves
-  constexpr int WP = (BN * 4) / NT;                      // weight chunks per thread: 2 or 1
+  constexpr int XP = (BM * 8) / NT;                      // activation chunks per thread: 4
+  constexpr int WP = (BN * 4) / NT;                      // weight chunks per thread: 4, 2 or 1
+  constexpr int SETS = 4;
+  constexpr int kPast = (int)0x80000000;                 // an offset no descriptor covers
+  static_assert(SETS * (XP + WP) <= 63, "vmcnt is a 6-bit counter");
   __shared__ __attribute__((aligned(16))) uint8_t xs[2][BM * BK * 2];
-  // WIDE: the weights are widened to halves once, on their way into LDS (128-byte rows like the
-  // activations'), not by every wave that reads them
-  __shared__ __attribute__((aligned(16))) uint8_t ws[2][BN * BK * (WIDE ? 2 : 1)];
+  __shared__ __attribute__((aligned(16))) uint8_t ws[2][BN * BK * 2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_n = (p.N + BN - 1) / BN;
   const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
   const int r = lane & 31, g = lane >> 5;
-  const _Float16* x = static_cast<const _Float16*>(p.x);
-  const u4 zero = {0, 0, 0, 0};
+  const int kbeg = blockIdx.y * p.k_split;               // this workgroup's k range
+  const int klen = min(p.K, kbeg + p.k_split) - kbeg;
+  // descriptors over the tile's rows from (first row, kbeg); the host has checked that the
+  // offsets below fit 31 bits
+  const int mrows = min(BM, p.M - m0), nrows = min(BN, p.N - n0);
+  const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16*>(static_cast<const _Float16*>(p.x) + (int64_t)m0 * p.ldx + kbeg), 0,
+      (int)(((int64_t)(mrows - 1) * p.ldx + klen) * 2), kBufferWord3);
+  const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(p.w + (int64_t)n0 * p.w_sn + kbeg), 0,
+      (int)((int64_t)(nrows - 1) * p.w_sn + klen), kBufferWord3);
 
-  // global -> LDS assignment
+  // global -> LDS assignment (rows past the tile's last re-read that one)
   const int xc = tid & 7, wc = tid & 3;                  // 16-byte chunk of the row's k tile
-  const _Float16* xg[4];
-  int xl[4];
+  int xo[XP], xl[XP];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < XP; ++i) {
     const int row = (tid >> 3) + (NT / 8) * i;
-    xg[i] = x + (int64_t)min(m0 + row, p.M - 1) * p.ldx + 8 * xc;
+    xo[i] = (int)((int64_t)min(row, mrows - 1) * p.ldx * 2) + 16 * xc;
     xl[i] = row * 128 + ((xc ^ ((row ^ (row >> 3)) & 7)) << 4);
   }
-  const uint8_t* wg[WP];
-  int wl[WP], wl1[WP];
+  int wo[WP], wl[WP], wl1[WP];
   h2 cpark[WP];
 #pragma unroll
   for (int i = 0; i < WP; ++i) {
     const int row = (tid >> 2) + (NT / 4) * i;
-    wg[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.w_sn + 16 * wc;
-    if (WIDE) {
-      const int sw = (row ^ (row >> 3)) & 7;
-      wl[i] = row * 128 + (((2 * wc) ^ sw) << 4);
-      wl1[i] = row * 128 + (((2 * wc + 1) ^ sw) << 4);
-      cpark[i] = centre(p, min(n0 + row, p.N - 1));
-    } else {
-      wl[i] = row * 64 + ((wc ^ ((row >> 2) & 3)) << 4);
-      wl1[i] = 0;
-    }
+    const int sw = (row ^ (row >> 3)) & 7;
+    wo[i] = (int)((int64_t)min(row, nrows - 1) * p.w_sn) + 16 * wc;
+    wl[i] = row * 128 + (((2 * wc) ^ sw) << 4);
+    wl1[i] = row * 128 + (((2 * wc + 1) ^ sw) << 4);
+    cpark[i] = centre(p, n0 + min(row, nrows - 1));
   }
-  // three register sets: the loads of k tiles t + 1 .. t + 3 are in flight while tile t is
-  // multiplied (with one workgroup on a compute unit nothing else covers the load latency)
-  u4 xr[3][4], wr[3][WP];
+  u4 xr[SETS][XP], wr[SETS][WP];
   auto fetch = [&](u4* xq, u4* wq, int k0) {
-    const bool xv = k0 + 8 * xc < p.K, wv = k0 + 16 * wc < p.K;   // K % 16 == 0
+    const bool xv = k0 + 8 * xc < klen, wv = k0 + 16 * wc < klen;   // K % 16 == 0
 #pragma unroll
-    for (int i = 0; i < 4; ++i) xq[i] = xv ? *reinterpret_cast<const u4*>(xg[i] + k0) : zero;
+    for (int i = 0; i < XP; ++i)
+      xq[i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, xv ? xo[i] + 2 * k0 : kPast, 0, 0);
 #pragma unroll
-    for (int i = 0; i < WP; ++i) wq[i] = wv ? *reinterpret_cast<const u4*>(wg[i] + k0) : zero;
+    for (int i = 0; i < WP; ++i)
+      wq[i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wv ? wo[i] + k0 : kPast, 0, 0);
   };
   auto park = [&](const u4* xq, const u4* wq, int stage) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u4*>(&xs[stage][xl[i]]) = xq[i];
+    for (int i = 0; i < XP; ++i) *reinterpret_cast<u4*>(&xs[stage][xl[i]]) = xq[i];
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
-      if (WIDE) {
-        h8 lo, hi;
-        widen16(wq[i], p.flip, cpark[i], lo, hi);
-        *reinterpret_cast<h8*>(&ws[stage][wl[i]]) = lo;
-        *reinterpret_cast<h8*>(&ws[stage][wl1[i]]) = hi;
-      } else {
-        *reinterpret_cast<u4*>(&ws[stage][wl[i]]) = wq[i];
-      }
+      h8 lo, hi;
+      widen16(wq[i], p.flip, cpark[i], lo, hi);
+      *reinterpret_cast<h8*>(&ws[stage][wl[i]]) = lo;
+      *reinterpret_cast<h8*>(&ws[stage][wl1[i]]) = hi;
     }
   };
 
-  // fragment rows of this wave and the weight centres of its columns
+  // fragment rows of this wave
   int xrow[2], wrow[2];
-  h2 c[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     xrow[i] = wm * 64 + i * 32 + r;
     wrow[i] = wn * 64 + i * 32 + r;
-    c[i] = centre(p, min(n0 + wrow[i], p.N - 1));
   }
   f16v acc[2][2];
 #pragma unroll
@@ -319,61 +349,92 @@ __global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
 
   auto multiply = [&](int st) {
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    h8 a0[2], a1[2], w0[2], w1[2];
+    for (int s = 0; s < 2; ++s) {
+      h8 a0[2], a1[2], w0[2], w1[2];
+      const int c0 = 4 * s + 2 * g;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int c0 = 4 * s + 2 * g, row = xrow[i];
-      const int sx = (row ^ (row >> 3)) & 7;
-      a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ sx) << 4)]);
-      a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ sx) << 4)]);
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int row = wrow[j];
-      if (WIDE) {
-        const int c0 = 4 * s + 2 * g, sw = (row ^ (row >> 3)) & 7;
-        w0[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + ((c0 ^ sw) << 4)]);
-        w1[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + (((c0 + 1) ^ sw) << 4)]);
-      } else {
-        const int cw = 2 * s + g;
-        const u4 q =
-            *reinterpret_cast<const u4*>(&ws[st][row * 64 + ((cw ^ ((row >> 2) & 3)) << 4)]);
-        widen16(q, p.flip, c[j], w0[j], w1[j]);
+      for (int i = 0; i < 2; ++i) {
+        const int row = xrow[i], sx = (row ^ (row >> 3)) & 7;
+        a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ sx) << 4)]);
+        a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ sx) << 4)]);
       }
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], w0[j], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1[i], w1[j], acc[i][j], 0, 0, 0);
+        const int row = wrow[j], sw = (row ^ (row >> 3)) & 7;
+        w0[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + ((c0 ^ sw) << 4)]);
+        w1[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + (((c0 + 1) ^ sw) << 4)]);
       }
-  }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], w0[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1[i], w1[j], acc[i][j], 0, 0, 0);
+        }
+    }
   };
-  const int KT = (p.K + BK - 1) / BK;
-  fetch(xr[0], wr[0], 0);
-  fetch(xr[1], wr[1], BK);
-  fetch(xr[2], wr[2], 2 * BK);
+  // k tile t: set u = t % SETS has been handed to LDS stage t % 2 and takes tile t + SETS;
+  // tile t + 1 (zeros past the last) is handed over behind the multiplication
+  // (the scheduling barriers keep a later step's arithmetic on loaded registers -- the first
+  // instructions of widening -- from being moved up to where it would wait for their loads)
+  auto step = [&](int u, int t) {
+    fetch(xr[u], wr[u], (t + SETS) * BK);
+    multiply(u % 2);
+    __builtin_amdgcn_sched_barrier(0);
+    park(xr[(u + 1) % SETS], wr[(u + 1) % SETS], (u + 1) % 2);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  const int KT = (klen + BK - 1) / BK;
+#pragma unroll
+  for (int d = 0; d < SETS; ++d) fetch(xr[d], wr[d], d * BK);
+  __builtin_amdgcn_sched_barrier(0);
   park(xr[0], wr[0], 0);
   __syncthreads();
-  for (int t0 = 0; t0 < KT; t0 += 6) {
+  __builtin_amdgcn_sched_barrier(0);
+  int t = 0;
+  for (; t + SETS <= KT; t += SETS) {
 #pragma unroll
-    for (int u = 0; u < 6; ++u) {
-      const int t = t0 + u;
-      if (t < KT) {                                        // (uniform over the workgroup)
-        fetch(xr[u % 3], wr[u % 3], (t + 3) * BK);         // (past K: zeros)
-        multiply(u % 2);
-        if (t + 1 < KT) park(xr[(u + 1) % 3], wr[(u + 1) % 3], (u + 1) % 2);
-        __syncthreads();
-      }
-    }
+    for (int u = 0; u < SETS; ++u) step(u, t + u);
   }
+#pragma unroll
+  for (int u = 0; u < SETS - 1; ++u)
+    if (t + u < KT) step(u, t + u);                        // (uniform over the workgroup)
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      store_frag<_Float16>(p, acc[i][j], m0 + xrow[i] - r, n0 + wrow[j], lane);
+      if (p.partial)
+        store_partial(p, acc[i][j], blockIdx.y, m0 + xrow[i] - r, n0 + wrow[j], lane);
+      else
+        store_frag<_Float16>(p, acc[i][j], m0 + xrow[i] - r, n0 + wrow[j], lane);
+}
+
+// out = (sum over the k ranges, in their order) * scale + bias: the second half of a split
+// launch.  VEC consecutive channels per thread.
+template <typename XT, int VEC>
+__global__ void __launch_bounds__(256) wo_splitk_reduce_kernel(const WoParams p, int splits) {
+  const int nv = p.N / VEC;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)p.M * nv) return;
+  const int m = (int)(idx / nv), n = (int)(idx % nv) * VEC;
+  const int64_t plane = (int64_t)p.M * p.N;
+  const float* src = p.partial + (int64_t)m * p.N + n;
+  float sum[VEC];
+  if constexpr (VEC == 4) {
+    f4 v = *reinterpret_cast<const f4*>(src);
+    for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const f4*>(src + s * plane);
+    sum[0] = v.x, sum[1] = v.y, sum[2] = v.z, sum[3] = v.w;
+  } else {
+    sum[0] = src[0];
+    for (int s = 1; s < splits; ++s) sum[0] += src[s * plane];
+  }
+  const XT* scale = static_cast<const XT*>(p.scale);
+  const XT* bias = static_cast<const XT*>(p.bias);
+  XT* out = static_cast<XT*>(p.out) + (int64_t)m * p.ldo + n;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e)
+    out[e] = (XT)(sum[e] * to_f32(scale[n + e]) + (bias ? to_f32(bias[n + e]) : 0.0f));
 }
 
 // ---------------------------------------------------------------- small-M kernel, M <= 32 MT
@@ -534,8 +595,69 @@ __global__ void __launch_bounds__(256) wo_generic_kernel(const WoParams p) {
   static_cast<XT*>(p.out)[(int64_t)m * p.ldo + n] = (XT)(acc * s + b);
 }
 
+// Split plan of the LDS kernel (f16 activations) for problems whose tiles would leave most of
+// the chip idle: `splits` workgroups per tile, each over k_split of the k range, and a
+// reduction kernel behind them.  splits == 1: no split.
+struct SplitPlan {
+  int wm;        // tile rows / 64: 1 or 2
+  int splits;
+  int k_split;
+};
+
+SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+  SplitPlan s = {M <= 64 ? 1 : 2, 1, (int)K};
+  // Measured (4096^2, 8192^2, 3072 x 768 and 768 x 3072 weights): up to 32 rows the skinny
+  // kernel wins; a k range below 256 per workgroup or fewer than 1024 of k is not worth the
+  // second launch; and the partial sums (splits x M x N floats, written and read once) bound
+  // the number of splits as M grows.
+  if (M <= 32 || K < 1024) return s;
+  const int64_t tiles = ceil_div(M, 64 * s.wm) * ceil_div(N, 128);
+  const int64_t splits = std::min(std::min(compute_units() / tiles, K / 256),
+                                  std::max<int64_t>(1, 4096 / M));
+  if (splits < 2) return s;
+  s.k_split = (int)(ceil_div(ceil_div(K, splits), 64) * 64);
+  s.splits = (int)ceil_div(K, s.k_split);
+  if (s.splits < 2) s.splits = 1, s.k_split = (int)K;
+  return s;
+}
+
+size_t split_bytes(const SplitPlan& s, int64_t M, int64_t N) {
+  return s.splits > 1 ? (size_t)s.splits * (size_t)(M * N) * sizeof(float) : 0;
+}
+
 template <typename XT>
-int launch(const WoParams& p, bool fast, hipStream_t st) {
+int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStream_t st) {
+  p.partial = nullptr;
+  p.k_split = p.K;
+  // (the LDS kernel addresses a tile's rows by 31-bit byte offsets from its first)
+  const bool lds_ok = sizeof(XT) == 2 && 256 * p.ldx + 2 * (int64_t)p.K + 4096 < (1LL << 31) &&
+                      128 * p.w_sn + (int64_t)p.K + 4096 < (1LL << 31);
+  if (fast && lds_ok) {
+    const SplitPlan s = plan_split(p.M, p.N, p.K);
+    if (s.splits > 1 && scratch && aligned(scratch, 16) &&
+        scratch_bytes >= split_bytes(s, p.M, p.N)) {
+      const int bm = 64 * s.wm;
+      const int sp = s.splits;
+      p.partial = static_cast<float*>(scratch);
+      p.k_split = s.k_split;
+      const dim3 grid((unsigned)(ceil_div(p.M, bm) * ceil_div(p.N, 128)), (unsigned)sp);
+      if (s.wm == 1)
+        hipLaunchKernelGGL((wo_lds_kernel<1>), grid, dim3(128), 0, st, p);
+      else
+        hipLaunchKernelGGL((wo_lds_kernel<2>), grid, dim3(256), 0, st, p);
+      if (int e = check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch")) return e;
+      const int vec = (p.N % 4 == 0 && aligned(p.out, 8) && p.ldo % 4 == 0) ? 4 : 1;
+      const int64_t blocks = ceil_div((int64_t)p.M * (p.N / vec), 256);
+      DQ8_REQUIRE(blocks < (1LL << 31), "dq8_weight_only_qgemm: problem too large");
+      if (vec == 4)
+        hipLaunchKernelGGL((wo_splitk_reduce_kernel<XT, 4>), dim3((unsigned)blocks), dim3(256), 0,
+                           st, p, sp);
+      else
+        hipLaunchKernelGGL((wo_splitk_reduce_kernel<XT, 1>), dim3((unsigned)blocks), dim3(256), 0,
+                           st, p, sp);
+      return check_hip(hipGetLastError(), "dq8_weight_only_qgemm reduction launch");
+    }
+  }
   if (!fast) {
     const int64_t blocks = ceil_div((int64_t)p.M * p.N, 256);
     DQ8_REQUIRE(blocks < (1LL << 31), "dq8_weight_only_qgemm: problem too large");
@@ -554,16 +676,25 @@ int launch(const WoParams& p, bool fast, hipStream_t st) {
     else
       hipLaunchKernelGGL((wo_skinny_kernel<XT, 8, 4>), dim3(grid), dim3(512), 0, st, p);
   } else {
-    // 128 x 128 tiles through LDS once there are enough of them to put several workgroups on
-    // a compute unit (a lone workgroup's chain of load, LDS, widen and MFMA latencies is not
-    // covered: 48 tiles of a 3072-deep problem take as long through LDS as 192 small tiles
-    // through registers); the register kernel below that and for f32 activations
+    // 128 x 128 tiles through LDS once there are enough of them (a lone workgroup's chain of
+    // load, LDS, widen and MFMA latencies is not covered: below that the register kernel,
+    // which is also the one for f32 activations).  256 x 128 tiles on eight waves where they
+    // come out cheaper by the measured time of a round of either shape at 4096 of k: 128 x 128
+    // tiles, two workgroups to a compute unit, 82 us for a full round and 45 while one
+    // workgroup has the unit to itself; 256 x 128 tiles, one to a unit, 75 us and 60 up to
+    // half a round.
     const int64_t big = ceil_div(p.M, 128) * ceil_div(p.N, 128);
     const int64_t big256 = ceil_div(p.M, 256) * ceil_div(p.N, 128);
-    if (big256 >= 384 && sizeof(XT) == 2) {
-      hipLaunchKernelGGL((wo_lds_kernel<4, true>), dim3((unsigned)big256), dim3(512), 0, st, p);
-    } else if (big >= 96 && sizeof(XT) == 2) {
-      hipLaunchKernelGGL((wo_lds_kernel<2, true>), dim3((unsigned)big), dim3(256), 0, st, p);
+    const int64_t cus = compute_units();
+    auto rounds = [](int64_t tiles, int64_t slots, int64_t half, int full_us, int part_us) {
+      const int64_t rem = tiles % slots;
+      return tiles / slots * full_us + (rem == 0 ? 0 : rem <= half ? part_us : full_us);
+    };
+    const bool wide = rounds(big256, cus, cus / 2, 75, 60) < rounds(big, 2 * cus, cus, 82, 45);
+    if (wide && lds_ok) {
+      hipLaunchKernelGGL((wo_lds_kernel<4>), dim3((unsigned)big256), dim3(512), 0, st, p);
+    } else if (big >= 64 && lds_ok) {
+      hipLaunchKernelGGL((wo_lds_kernel<2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else if (big >= 192) {
       hipLaunchKernelGGL((wo_tile_kernel<XT, 2, 2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else {
@@ -579,8 +710,26 @@ int launch(const WoParams& p, bool fast, hipStream_t st) {
 
 using namespace dq8;
 
+namespace {
+// bytes of the [N, K] copy of weights given as [K, N], kept 256-byte aligned
+size_t transposed_bytes(int64_t N, int64_t K, int tp_b) {
+  return (tp_b || N <= 0 || K <= 0) ? 0 : ((size_t)(N * K) + 255) / 256 * 256;
+}
+}  // namespace
+
 extern "C" size_t dq8_weight_only_qgemm_workspace_bytes(int64_t N, int64_t K, int tp_b) {
   return (tp_b || N <= 0 || K <= 0) ? 0 : (size_t)(N * K);
+}
+
+extern "C" size_t dq8_weight_only_qgemm_workspace_bytes_ex(int64_t M, int64_t N, int64_t K,
+                                                           int tp_b, int x_dtype) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  size_t split = 0;
+  if (x_dtype == DQ8_DTYPE_F16 && K % 16 == 0 && M < (1LL << 31) && N < (1LL << 31) &&
+      K < (1LL << 31))
+    split = split_bytes(plan_split(M, N, K), M, N);
+  if (!split) return dq8_weight_only_qgemm_workspace_bytes(N, K, tp_b);
+  return transposed_bytes(N, K, tp_b) + split;
 }
 
 extern "C" int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, const void* w,
@@ -619,6 +768,9 @@ extern "C" int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, co
   // as [K, N] are transposed into the caller's scratch first (a runtime does that once per
   // constant weight and passes the result with tp_b = 1 from then on)
   bool fast = K > 0 && K % 16 == 0 && aligned(x, 16) && (ldx * esz) % 16 == 0;
+  // what the transposed weights leave of the scratch holds the partial sums of a split launch
+  void* rest = workspace;
+  size_t rest_bytes = workspace ? workspace_bytes : 0;
   if (fast && !tp_b) {
     if (workspace && aligned(workspace, 16) && workspace_bytes >= (size_t)(N * K)) {
       if (int s = dq8_transpose_s8(static_cast<const int8_t*>(w), ldw,
@@ -627,10 +779,14 @@ extern "C" int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, co
       p.w = static_cast<const uint8_t*>(workspace);
       p.w_sn = K;
       p.w_sk = 1;
+      const size_t used = transposed_bytes(N, K, 0);
+      rest = used < workspace_bytes ? static_cast<char*>(workspace) + used : nullptr;
+      rest_bytes = used < workspace_bytes ? workspace_bytes - used : 0;
     } else {
       fast = false;
     }
   }
   fast = fast && aligned(p.w, 16) && p.w_sn % 16 == 0 && p.w_sk == 1;
-  return x_dtype == DQ8_DTYPE_F32 ? launch<float>(p, fast, st) : launch<_Float16>(p, fast, st);
+  return x_dtype == DQ8_DTYPE_F32 ? launch<float>(p, fast, rest, rest_bytes, st)
+                                  : launch<_Float16>(p, fast, rest, rest_bytes, st);
 }

@@ -784,9 +784,16 @@ MemRefType<T, N> weightOnlyQgemm(ExecutionContext* ctx, void* stream_handle,
   void* data = drv->alloc(ctx, (size_t)(m * n) * sizeof(T));
   if (!data) return result;
   result = assignMemRef<T, N>(data, sizes);
+  // (scratch for the partial sums of a launch split over k when m is small; handed back to the
+  // pool right after the launch, which later work on the same stream is ordered behind)
+  size_t ws_bytes = dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, WoDtype<T>::value);
+  void* ws = ws_bytes ? drv->alloc(ctx, ws_bytes) : nullptr;
+  if (!ws) ws_bytes = 0;                                   // (the call then runs unsplit)
   StreamTimer timer(stream);
-  const int st = dq8_weight_only_qgemm(input.data, WoDtype<T>::value, k, w_nk, 0, k, 1, scales.data,
-                                       zeroPoints.data, bias, data, n, m, n, k, nullptr, 0, stream);
+  const int st =
+      dq8_weight_only_qgemm(input.data, WoDtype<T>::value, k, w_nk, 0, k, 1, scales.data,
+                            zeroPoints.data, bias, data, n, m, n, k, ws, ws_bytes, stream);
+  if (ws) drv->dealloc(ctx, ws);
   if (timer.on() && st == 0) {
     const double ns = timer.stop();
     const int64_t bytes = (m * k + m * n) * (int64_t)sizeof(T) + k * n;

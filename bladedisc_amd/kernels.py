@@ -157,7 +157,8 @@ def weight_only_qgemm(x, w, scale, zero_points=None, bias=None, tp_b=True, out=N
     """out = x @ ((w - zero_points[:, None]) * scale[:, None]).T + bias for f16 / f32
     activations x [M,K] and 8-bit weights (uint8 or int8) w [N,K] (tp_b) or [K,N]; scale and
     bias have x's dtype, zero_points is int32.  workspace=False withholds the scratch that
-    [K,N] weights are transposed into."""
+    [K,N] weights are transposed into and that a launch split over k keeps its partial sums
+    in; a uint8 tensor is used as that scratch."""
     _need_cuda(x, w, scale, zero_points, bias)
     if x.dtype not in (torch.float32, torch.float16):
         raise TypeError("weight_only_qgemm takes f32 or f16 activations")
@@ -176,8 +177,12 @@ def weight_only_qgemm(x, w, scale, zero_points=None, bias=None, tp_b=True, out=N
     if out is None:
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
     L = _lib.lib()
-    ws_bytes = L.dq8_weight_only_qgemm_workspace_bytes(n, k, int(tp_b)) if workspace else 0
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    if isinstance(workspace, torch.Tensor):
+        ws, ws_bytes = workspace, workspace.numel() * workspace.element_size()
+    else:
+        ws_bytes = L.dq8_weight_only_qgemm_workspace_bytes_ex(
+            m, n, k, int(tp_b), 0 if x.dtype == torch.float32 else 1) if workspace else 0
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     st = L.dq8_weight_only_qgemm(_ptr(x), 0 if x.dtype == torch.float32 else 1, x.stride(0),
                                  _ptr(w), int(w.dtype == torch.int8), w.stride(0), int(tp_b),
                                  _ptr(scale), _ptr(zero_points), _ptr(bias), _ptr(out),

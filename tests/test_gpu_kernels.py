@@ -1163,6 +1163,47 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
     assert tuple(empty.shape) == (0, 96)
 
 
+def test_weight_only_qgemm_split_over_k(K):
+    """M between the skinny kernels' range and the sizes whose tiles fill the chip: the launch
+    is split over k (f32 partial sums in the scratch, a reduction launch behind the GEMM).
+    Ragged M, N and k ranges, N that is not a multiple of 4 (scalar reduction), with and
+    without the scratch (without it the unsplit kernels run), the same bits on every call, and
+    a caller-owned scratch that is reused."""
+    import bladedisc_amd._lib as _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(4242)
+    dtype = torch.float16
+    split_seen = 0
+    for (m, k, n) in [(33, 1024, 256), (64, 3072, 768), (100, 2064, 130), (128, 4096, 1024),
+                      (200, 1040, 333), (512, 2048, 640), (48, 1536, 4096)]:
+        x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed=False)
+        plain = L.dq8_weight_only_qgemm_workspace_bytes(n, k, 1)
+        need = L.dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, 1)
+        assert plain == 0 and need % (4 * m * n) == 0
+        split_seen += need > 0
+        args = (dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+        got = K.weight_only_qgemm(*args)
+        _weight_only_check(got, x, w, scale, zp, bias, dtype)
+        again = K.weight_only_qgemm(*args)
+        assert torch.equal(got, again)
+        unsplit = K.weight_only_qgemm(*args, workspace=False)
+        _weight_only_check(unsplit, x, w, scale, zp, bias, dtype)
+        if need:
+            ws = torch.empty(need + 4096, dtype=torch.uint8, device="cuda")
+            ws.fill_(0xff)                                   # (NaN patterns: nothing may leak)
+            assert torch.equal(K.weight_only_qgemm(*args, workspace=ws), got)
+            assert torch.equal(K.weight_only_qgemm(*args, workspace=ws), got)
+            # a scratch that is too small for the partial sums: the unsplit kernels
+            assert torch.equal(K.weight_only_qgemm(*args, workspace=ws[:need - 16]), unsplit)
+        # [K,N] weights: the transposed copy and the partial sums share the scratch
+        got_kn = K.weight_only_qgemm(dev(x), dev(np.ascontiguousarray(w.T)), dev(scale), dev(zp),
+                                     dev(bias), tp_b=False)
+        assert torch.equal(got_kn, got)
+    assert split_seen >= 5
+    # f32 activations are not split
+    assert L.dq8_weight_only_qgemm_workspace_bytes_ex(128, 1024, 4096, 1, 0) == 0
+
+
 def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
     """Seeded sweep over what the library's own choice of kernel depends on -- M from one row
     to several rounds of the largest tiles, N, K, the epilogue family, fused operators -- with

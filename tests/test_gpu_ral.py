@@ -205,16 +205,18 @@ def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
-@pytest.mark.parametrize("with_bias", [False, True])
-def test_ral_pdll_weight_only_qgemm(rt, dtype, with_bias):
+@pytest.mark.parametrize("with_bias,k,n", [(False, 96, 72), (True, 96, 72), (True, 1280, 200)])
+def test_ral_pdll_weight_only_qgemm(rt, dtype, with_bias, k, n):
     """The weight-only entry by its mangled name, as the pattern calls it: rank-3 activations,
     uint8 weight [K,N] with zero points 128 (quant range 0..255), per-channel scale, optional
     bias; the packed weight is cached, so a second call with other activations must agree
-    too.  Tolerance: the f32 accumulation bound of the kernel tests."""
+    too.  The deep case (80 rows, k = 1280) is one the f16 kernels split over k, with the
+    partial sums in scratch from the context's pool.  Tolerance: the f32 accumulation bound
+    of the kernel tests."""
     ctx, ral, ops = rt
-    rng = np.random.default_rng(31 + int(with_bias))
+    rng = np.random.default_rng(31 + int(with_bias) + k)
     npdt = np.float16 if dtype == torch.float16 else np.float32
-    b, s, k, n = 2, 40, 96, 72
+    b, s = 2, 40
     w = rng.integers(0, 256, (n, k), dtype=np.uint8)
     zp = np.full(n, 128, np.int32)
     scale = rng.uniform(0.002, 0.02, n).astype(npdt)
