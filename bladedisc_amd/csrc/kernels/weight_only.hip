@@ -262,17 +262,18 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
 // loads issued after it instead of draining them all: with conditional loads in a loop of
 // guarded steps every k tile waited out a whole trip to memory (0.8 us per k tile on a
 // quiet chip, 1.5-2 us on a busy one).
-template <int WM>
-__global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
-  constexpr int BM = WM * 64, BN = 128, BK = 64;
+template <int WM, int FM, int FN, int SETS>
+__global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const WoParams p) {
+  constexpr int BM = WM * FM * 32, BN = 2 * FN * 32, BK = 64;
   constexpr int NT = WM * 128;                           // WM x 2 waves
-  constexpr int XP = (BM * 8) / NT;                      // activation chunks per thread: 4
-  constexpr int WP = (BN * 4) / NT;                      // weight chunks per thread: 4, 2 or 1
-  constexpr int SETS = 4;
+  constexpr int XP = (BM * 8) / NT;                      // activation chunks per thread
+  constexpr int WP = (BN * 4) / NT;                      // weight chunks per thread
   constexpr int kPast = (int)0x80000000;                 // an offset no descriptor covers
-  static_assert(SETS * (XP + WP) <= 63, "vmcnt is a 6-bit counter");
-  __shared__ __attribute__((aligned(16))) uint8_t xs[2][BM * BK * 2];
-  __shared__ __attribute__((aligned(16))) uint8_t ws[2][BN * BK * 2];
+  static_assert(SETS % 2 == 0 && SETS * (XP + WP) <= 63, "two LDS stages; vmcnt has 6 bits");
+  // two stages of (activation tile, widened weight tile), 128 bytes per row
+  extern __shared__ __attribute__((aligned(16))) uint8_t wo_lds[];
+  uint8_t* const xs[2] = {wo_lds, wo_lds + BM * 128};
+  uint8_t* const ws[2] = {wo_lds + 2 * BM * 128, wo_lds + 2 * BM * 128 + BN * 128};
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_n = (p.N + BN - 1) / BN;
@@ -333,41 +334,69 @@ __global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
   };
 
   // fragment rows of this wave
-  int xrow[2], wrow[2];
+  int xrow[FM], wrow[FN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    xrow[i] = wm * 64 + i * 32 + r;
-    wrow[i] = wn * 64 + i * 32 + r;
-  }
-  f16v acc[2][2];
+  for (int i = 0; i < FM; ++i) xrow[i] = (wm * FM + i) * 32 + r;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int j = 0; j < FN; ++j) wrow[j] = (wn * FN + j) * 32 + r;
+  f16v acc[FM][FN];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+  // (Reading the fragments of one 16-deep k step under the MFMAs of the step before, one LDS
+  // read scheduled between every two MFMAs, changed nothing measurable: 135.2 against 137.5 us
+  // at 4096^3 on 256 x 256 tiles.)
   auto multiply = [&](int st) {
+    if constexpr (FM * FN >= 8) {
+      // eight fragments per wave: one 16-deep k step at a time (this lane's 8 halves are chunk
+      // 4 (q / 2) + 2 g + q % 2), the registers do not hold more fragments than that
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        h8 a[FM], w[FN];
+        const int c = 4 * (q >> 1) + 2 * g + (q & 1);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const int row = xrow[i], sx = (row ^ (row >> 3)) & 7;
+          a[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c ^ sx) << 4)]);
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const int row = wrow[j], sw = (row ^ (row >> 3)) & 7;
+          w[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + ((c ^ sw) << 4)]);
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      h8 a0[2], a1[2], w0[2], w1[2];
+      h8 a0[FM], a1[FM], w0[FN], w1[FN];
       const int c0 = 4 * s + 2 * g;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < FM; ++i) {
         const int row = xrow[i], sx = (row ^ (row >> 3)) & 7;
         a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ sx) << 4)]);
         a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ sx) << 4)]);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < FN; ++j) {
         const int row = wrow[j], sw = (row ^ (row >> 3)) & 7;
         w0[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + ((c0 ^ sw) << 4)]);
         w1[j] = *reinterpret_cast<const h8*>(&ws[st][row * 128 + (((c0 + 1) ^ sw) << 4)]);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < FN; ++j) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], w0[j], acc[i][j], 0, 0, 0);
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1[i], w1[j], acc[i][j], 0, 0, 0);
         }
@@ -401,9 +430,9 @@ __global__ void __launch_bounds__(WM * 128) wo_lds_kernel(const WoParams p) {
   for (int u = 0; u < SETS - 1; ++u)
     if (t + u < KT) step(u, t + u);                        // (uniform over the workgroup)
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < FN; ++j)
       if (p.partial)
         store_partial(p, acc[i][j], blockIdx.y, m0 + xrow[i] - r, n0 + wrow[j], lane);
       else
@@ -595,6 +624,17 @@ __global__ void __launch_bounds__(256) wo_generic_kernel(const WoParams p) {
   static_cast<XT*>(p.out)[(int64_t)m * p.ldo + n] = (XT)(acc * s + b);
 }
 
+template <int WM, int FM, int FN, int SETS>
+int launch_lds(dim3 grid, const WoParams& p, hipStream_t st) {
+  constexpr int lds = 2 * (WM * FM * 32 + 2 * FN * 32) * 128;
+  auto kern = wo_lds_kernel<WM, FM, FN, SETS>;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (lds > 64 * 1024)
+    if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
+  hipLaunchKernelGGL(kern, grid, dim3(WM * 128), lds, st, p);
+  return check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch");
+}
+
 // Split plan of the LDS kernel (f16 activations) for problems whose tiles would leave most of
 // the chip idle: `splits` workgroups per tile, each over k_split of the k range, and a
 // reduction kernel behind them.  splits == 1: no split.
@@ -641,11 +681,8 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
       p.partial = static_cast<float*>(scratch);
       p.k_split = s.k_split;
       const dim3 grid((unsigned)(ceil_div(p.M, bm) * ceil_div(p.N, 128)), (unsigned)sp);
-      if (s.wm == 1)
-        hipLaunchKernelGGL((wo_lds_kernel<1>), grid, dim3(128), 0, st, p);
-      else
-        hipLaunchKernelGGL((wo_lds_kernel<2>), grid, dim3(256), 0, st, p);
-      if (int e = check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch")) return e;
+      if (int e = s.wm == 1 ? launch_lds<1, 2, 2, 4>(grid, p, st) : launch_lds<2, 2, 2, 4>(grid, p, st))
+        return e;
       const int vec = (p.N % 4 == 0 && aligned(p.out, 8) && p.ldo % 4 == 0) ? 4 : 1;
       const int64_t blocks = ceil_div((int64_t)p.M * (p.N / vec), 256);
       DQ8_REQUIRE(blocks < (1LL << 31), "dq8_weight_only_qgemm: problem too large");
@@ -678,23 +715,29 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
   } else {
     // 128 x 128 tiles through LDS once there are enough of them (a lone workgroup's chain of
     // load, LDS, widen and MFMA latencies is not covered: below that the register kernel,
-    // which is also the one for f32 activations).  256 x 128 tiles on eight waves where they
-    // come out cheaper by the measured time of a round of either shape at 4096 of k: 128 x 128
-    // tiles, two workgroups to a compute unit, 82 us for a full round and 45 while one
+    // which is also the one for f32 activations).  256 x 128 and 256 x 256 tiles on eight waves
+    // (wave tiles 64 x 64 and 64 x 128: the larger the wave tile, the fewer LDS bytes per MFMA)
+    // where they come out cheaper by the measured time of a round of each shape at 4096 of k:
+    // 128 x 128 tiles, two workgroups to a compute unit, 82 us for a full round and 45 while one
     // workgroup has the unit to itself; 256 x 128 tiles, one to a unit, 75 us and 60 up to
-    // half a round.
+    // half a round; 256 x 256 tiles 135 us and 100.
     const int64_t big = ceil_div(p.M, 128) * ceil_div(p.N, 128);
     const int64_t big256 = ceil_div(p.M, 256) * ceil_div(p.N, 128);
+    const int64_t big2 = ceil_div(p.M, 256) * ceil_div(p.N, 256);
     const int64_t cus = compute_units();
     auto rounds = [](int64_t tiles, int64_t slots, int64_t half, int full_us, int part_us) {
       const int64_t rem = tiles % slots;
       return tiles / slots * full_us + (rem == 0 ? 0 : rem <= half ? part_us : full_us);
     };
-    const bool wide = rounds(big256, cus, cus / 2, 75, 60) < rounds(big, 2 * cus, cus, 82, 45);
-    if (wide && lds_ok) {
-      hipLaunchKernelGGL((wo_lds_kernel<4>), dim3((unsigned)big256), dim3(512), 0, st, p);
+    const int64_t cost128 = rounds(big, 2 * cus, cus, 82, 45);
+    const int64_t cost256x128 = rounds(big256, cus, cus / 2, 75, 60);
+    const int64_t cost256 = rounds(big2, cus, cus / 2, 135, 100);
+    if (cost256 < cost128 && cost256 <= cost256x128 && lds_ok) {
+      return launch_lds<4, 2, 4, 2>(dim3((unsigned)big2), p, st);
+    } else if (cost256x128 < cost128 && lds_ok) {
+      return launch_lds<4, 2, 2, 4>(dim3((unsigned)big256), p, st);
     } else if (big >= 64 && lds_ok) {
-      hipLaunchKernelGGL((wo_lds_kernel<2>), dim3((unsigned)big), dim3(256), 0, st, p);
+      return launch_lds<2, 2, 2, 4>(dim3((unsigned)big), p, st);
     } else if (big >= 192) {
       hipLaunchKernelGGL((wo_tile_kernel<XT, 2, 2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else {
