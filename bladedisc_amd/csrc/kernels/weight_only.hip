@@ -277,7 +277,21 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_n = (p.N + BN - 1) / BN;
-  const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+  // Workgroups go to the 8 XCDs round-robin, and each XCD has its own L2.  Where the tile grid
+  // divides, XCD x takes one compact patch of it (the grid cut 4 x 2: an activation row is
+  // twice the bytes of a weight row), so that its L2 fetches the patch's operand rows instead
+  // of every activation row (measured at 4096^3: 295 MB fetched per launch without this).
+  int tile = blockIdx.x;
+  {
+    const int tiles_m = gridDim.x / tiles_n;
+    // (launches of at least a round; the rows of a split launch are not dealt this way)
+    if (gridDim.y == 1 && gridDim.x >= 128 && tiles_m % 4 == 0 && tiles_n % 2 == 0) {
+      const int xcd = tile & 7, idx = tile >> 3;
+      const int pm = tiles_m / 4, pn = tiles_n / 2;        // the patch
+      tile = ((xcd >> 1) * pm + idx / pn) * tiles_n + (xcd & 1) * pn + idx % pn;
+    }
+  }
+  const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
   const int r = lane & 31, g = lane >> 5;
   const int kbeg = blockIdx.y * p.k_split;               // this workgroup's k range
   const int klen = min(p.K, kbeg + p.k_split) - kbeg;
