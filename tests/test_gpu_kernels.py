@@ -1135,7 +1135,10 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
                       (130, 40, 260), (5, 1000, 33),
                       # enough 128 x 128 tiles for the kernel that stages both operands in LDS:
                       # ragged last tiles in M and N, k depths off a multiple of 64
-                      (1500, 80, 1100), (1290, 208, 1300), (9, 4112, 40)]:
+                      (1500, 80, 1100), (1290, 208, 1300), (9, 4112, 40),
+                      # a full round of 256 x 256 tiles (ragged last row and column of tiles,
+                      # XCD-ordered) and of 256 x 128 tiles
+                      (4000, 144, 4090), (2000, 80, 4090)]:
         for signed in (False, True):
             x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed)
             got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
