@@ -19,15 +19,17 @@
 // bits of x take part while lo is a normal half (|x| >= 1/8); below, lo is subnormal and the
 // error per activation is an absolute 2^-25.
 //
-// Both operands go from global memory straight into registers in MFMA layout: the order of
-// the k values inside a fragment is free as long as both operands agree, so lane (row, g) takes
-// the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes (one dwordx4), 16
-// activations -- and feeds two MFMAs with them.
-//  * wo_lds_kernel: f16 activations, 128 x 128 tiles shared through LDS, once there are about a
-//    hundred of them (256 x 128 on eight waves once those fill the chip; 0.84-0.90 PFLOP/s at
-//    4096^2 .. 8192^2 weights, where the ROCm library's plain f16 GEMM reaches 1.16-1.49);
+// In the register kernels both operands go from global memory straight into registers in MFMA
+// layout: the order of the k values inside a fragment is free as long as both operands agree,
+// so lane (row, g) takes the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes
+// (one dwordx4), 16 activations -- and feeds two MFMAs with them.
+//  * wo_lds_kernel: tiles of 128 x 128, 256 x 128 or 256 x 256 shared through LDS, from 64 tiles
+//    up, and -- with several workgroups per tile, each over a part of k, and
+//    wo_splitk_reduce_kernel behind them -- for 32 < M while the tiles would not fill the chip
+//    (1.06-1.16 PFLOP/s for f16 activations at 4096^2 .. 8192^2 weights, where the ROCm
+//    library's plain f16 GEMM reaches 1.16-1.49);
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
-//    f32 activations and problems with few tiles;
+//    problems with few tiles and little k;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
 //  * wo_skinny_kernel: M <= 128 rows against 32 output channels per workgroup, the k range dealt
 //    over the waves and the partial sums added through LDS (bound by the weight bytes: 1 byte
@@ -45,6 +47,7 @@ namespace dq8 {
 namespace {
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
@@ -262,18 +265,26 @@ __global__ void __launch_bounds__(256) wo_tile_kernel(const WoParams p) {
 // loads issued after it instead of draining them all: with conditional loads in a loop of
 // guarded steps every k tile waited out a whole trip to memory (0.8 us per k tile on a
 // quiet chip, 1.5-2 us on a busy one).
-template <int WM, int FM, int FN, int SETS>
-__global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const WoParams p) {
+//
+// f32 activations (XT = float) are split on their way into LDS, x = hi + lo with hi = half(x)
+// and lo = half(x - hi), into two half tiles of the same layout; every weight fragment is
+// multiplied with both.
+template <typename XT, int WM, int FM, int FN, int SETS>
+__global__ void __launch_bounds__(WM * 128, (WM == 1 || sizeof(XT) == 4) ? 1 : 2)
+    wo_lds_kernel(const WoParams p) {
+  constexpr bool F32 = sizeof(XT) == 4;
   constexpr int BM = WM * FM * 32, BN = 2 * FN * 32, BK = 64;
   constexpr int NT = WM * 128;                           // WM x 2 waves
-  constexpr int XP = (BM * 8) / NT;                      // activation chunks per thread
+  constexpr int XL = F32 ? 16 : 8;                       // lanes (16 bytes each) per activation row
+  constexpr int XP = (BM * XL) / NT;                     // activation chunks per thread
   constexpr int WP = (BN * 4) / NT;                      // weight chunks per thread
+  constexpr int XS = BM * 128 * (F32 ? 2 : 1);           // activation bytes of a stage
   constexpr int kPast = (int)0x80000000;                 // an offset no descriptor covers
   static_assert(SETS % 2 == 0 && SETS * (XP + WP) <= 63, "two LDS stages; vmcnt has 6 bits");
-  // two stages of (activation tile, widened weight tile), 128 bytes per row
+  // two stages of (activation tile [hi, then lo], widened weight tile), 128 bytes per row
   extern __shared__ __attribute__((aligned(16))) uint8_t wo_lds[];
-  uint8_t* const xs[2] = {wo_lds, wo_lds + BM * 128};
-  uint8_t* const ws[2] = {wo_lds + 2 * BM * 128, wo_lds + 2 * BM * 128 + BN * 128};
+  uint8_t* const xs[2] = {wo_lds, wo_lds + XS};
+  uint8_t* const ws[2] = {wo_lds + 2 * XS, wo_lds + 2 * XS + BN * 128};
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_n = (p.N + BN - 1) / BN;
@@ -299,20 +310,23 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
   // offsets below fit 31 bits
   const int mrows = min(BM, p.M - m0), nrows = min(BN, p.N - n0);
   const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<_Float16*>(static_cast<const _Float16*>(p.x) + (int64_t)m0 * p.ldx + kbeg), 0,
-      (int)(((int64_t)(mrows - 1) * p.ldx + klen) * 2), kBufferWord3);
+      const_cast<XT*>(static_cast<const XT*>(p.x) + (int64_t)m0 * p.ldx + kbeg), 0,
+      (int)(((int64_t)(mrows - 1) * p.ldx + klen) * sizeof(XT)), kBufferWord3);
   const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint8_t*>(p.w + (int64_t)n0 * p.w_sn + kbeg), 0,
       (int)((int64_t)(nrows - 1) * p.w_sn + klen), kBufferWord3);
 
   // global -> LDS assignment (rows past the tile's last re-read that one)
-  const int xc = tid & 7, wc = tid & 3;                  // 16-byte chunk of the row's k tile
+  const int xc = tid & (XL - 1), wc = tid & 3;           // 16-byte chunk of the row's k tile
   int xo[XP], xl[XP];
 #pragma unroll
   for (int i = 0; i < XP; ++i) {
-    const int row = (tid >> 3) + (NT / 8) * i;
-    xo[i] = (int)((int64_t)min(row, mrows - 1) * p.ldx * 2) + 16 * xc;
-    xl[i] = row * 128 + ((xc ^ ((row ^ (row >> 3)) & 7)) << 4);
+    const int row = tid / XL + (NT / XL) * i;
+    const int sx = (row ^ (row >> 3)) & 7;
+    xo[i] = (int)((int64_t)min(row, mrows - 1) * p.ldx * sizeof(XT)) + 16 * xc;
+    // (four floats become four halves: half of the 16-byte chunk xc / 2)
+    xl[i] = F32 ? row * 128 + (((xc >> 1) ^ sx) << 4) + 8 * (xc & 1)
+                : row * 128 + ((xc ^ sx) << 4);
   }
   int wo[WP], wl[WP], wl1[WP];
   h2 cpark[WP];
@@ -327,17 +341,32 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
   }
   u4 xr[SETS][XP], wr[SETS][WP];
   auto fetch = [&](u4* xq, u4* wq, int k0) {
-    const bool xv = k0 + 8 * xc < klen, wv = k0 + 16 * wc < klen;   // K % 16 == 0
+    const bool xv = k0 + (F32 ? 4 : 8) * xc < klen, wv = k0 + 16 * wc < klen;   // K % 16 == 0
 #pragma unroll
     for (int i = 0; i < XP; ++i)
-      xq[i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, xv ? xo[i] + 2 * k0 : kPast, 0, 0);
+      xq[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          xrs, xv ? xo[i] + (int)sizeof(XT) * k0 : kPast, 0, 0);
 #pragma unroll
     for (int i = 0; i < WP; ++i)
       wq[i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wv ? wo[i] + k0 : kPast, 0, 0);
   };
   auto park = [&](const u4* xq, const u4* wq, int stage) {
 #pragma unroll
-    for (int i = 0; i < XP; ++i) *reinterpret_cast<u4*>(&xs[stage][xl[i]]) = xq[i];
+    for (int i = 0; i < XP; ++i) {
+      if constexpr (F32) {
+        const f4 v = __builtin_bit_cast(f4, xq[i]);
+        h4 hi, lo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          hi[e] = (_Float16)v[e];
+          lo[e] = (_Float16)(v[e] - (float)hi[e]);
+        }
+        *reinterpret_cast<h4*>(&xs[stage][xl[i]]) = hi;
+        *reinterpret_cast<h4*>(&xs[stage][BM * 128 + xl[i]]) = lo;
+      } else {
+        *reinterpret_cast<u4*>(&xs[stage][xl[i]]) = xq[i];
+      }
+    }
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
       h8 lo, hi;
@@ -370,12 +399,14 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
       // 4 (q / 2) + 2 g + q % 2), the registers do not hold more fragments than that
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        h8 a[FM], w[FN];
+        h8 a[FM], al[FM], w[FN];
         const int c = 4 * (q >> 1) + 2 * g + (q & 1);
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           const int row = xrow[i], sx = (row ^ (row >> 3)) & 7;
           a[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c ^ sx) << 4)]);
+          if constexpr (F32)
+            al[i] = *reinterpret_cast<const h8*>(&xs[st][BM * 128 + row * 128 + ((c ^ sx) << 4)]);
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
@@ -385,21 +416,29 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
-          for (int j = 0; j < FN; ++j)
+          for (int j = 0; j < FN; ++j) {
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], w[j], acc[i][j], 0, 0, 0);
+            if constexpr (F32)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], w[j], acc[i][j], 0, 0, 0);
+          }
         __builtin_amdgcn_sched_barrier(0);
       }
       return;
     }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      h8 a0[FM], a1[FM], w0[FN], w1[FN];
+      h8 a0[FM], a1[FM], l0[FM], l1[FM], w0[FN], w1[FN];
       const int c0 = 4 * s + 2 * g;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
         const int row = xrow[i], sx = (row ^ (row >> 3)) & 7;
         a0[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + ((c0 ^ sx) << 4)]);
         a1[i] = *reinterpret_cast<const h8*>(&xs[st][row * 128 + (((c0 + 1) ^ sx) << 4)]);
+        if constexpr (F32) {
+          l0[i] = *reinterpret_cast<const h8*>(&xs[st][BM * 128 + row * 128 + ((c0 ^ sx) << 4)]);
+          l1[i] =
+              *reinterpret_cast<const h8*>(&xs[st][BM * 128 + row * 128 + (((c0 + 1) ^ sx) << 4)]);
+        }
       }
 #pragma unroll
       for (int j = 0; j < FN; ++j) {
@@ -413,6 +452,10 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
         for (int j = 0; j < FN; ++j) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], w0[j], acc[i][j], 0, 0, 0);
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1[i], w1[j], acc[i][j], 0, 0, 0);
+          if constexpr (F32) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(l0[i], w0[j], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(l1[i], w1[j], acc[i][j], 0, 0, 0);
+          }
         }
     }
   };
@@ -450,7 +493,7 @@ __global__ void __launch_bounds__(WM * 128, WM == 1 ? 1 : 2) wo_lds_kernel(const
       if (p.partial)
         store_partial(p, acc[i][j], blockIdx.y, m0 + xrow[i] - r, n0 + wrow[j], lane);
       else
-        store_frag<_Float16>(p, acc[i][j], m0 + xrow[i] - r, n0 + wrow[j], lane);
+        store_frag<XT>(p, acc[i][j], m0 + xrow[i] - r, n0 + wrow[j], lane);
 }
 
 // out = (sum over the k ranges, in their order) * scale + bias: the second half of a split
@@ -638,10 +681,11 @@ __global__ void __launch_bounds__(256) wo_generic_kernel(const WoParams p) {
   static_cast<XT*>(p.out)[(int64_t)m * p.ldo + n] = (XT)(acc * s + b);
 }
 
-template <int WM, int FM, int FN, int SETS>
+template <typename XT, int WM, int FM, int FN, int SETS>
 int launch_lds(dim3 grid, const WoParams& p, hipStream_t st) {
-  constexpr int lds = 2 * (WM * FM * 32 + 2 * FN * 32) * 128;
-  auto kern = wo_lds_kernel<WM, FM, FN, SETS>;
+  constexpr int lds = 2 * (WM * FM * 32 * (int)(sizeof(XT) / 2) + 2 * FN * 32) * 128;
+  static_assert(lds <= 160 * 1024, "the stages fit the LDS");
+  auto kern = wo_lds_kernel<XT, WM, FM, FN, SETS>;
   static std::atomic<uint64_t> lds_allowed{0};
   if (lds > 64 * 1024)
     if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
@@ -689,7 +733,7 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
   p.partial = nullptr;
   p.k_split = p.K;
   // (the LDS kernel addresses a tile's rows by 31-bit byte offsets from its first)
-  const bool lds_ok = sizeof(XT) == 2 && 512 * p.ldx + 2 * (int64_t)p.K + 4096 < (1LL << 31) &&
+  const bool lds_ok = 512 * p.ldx + 4 * (int64_t)p.K + 4096 < (1LL << 31) &&
                       256 * p.w_sn + (int64_t)p.K + 4096 < (1LL << 31);
   if (fast && lds_ok) {
     const SplitPlan s = plan_split(p.M, p.N, p.K);
@@ -700,10 +744,12 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
       p.partial = static_cast<float*>(scratch);
       p.k_split = s.k_split;
       const dim3 grid((unsigned)(ceil_div(p.M, bm) * ceil_div(p.N, 64 * s.fn)), (unsigned)sp);
-      if (int e = s.fn == 1 ? (s.wm == 1 ? launch_lds<1, 2, 1, 4>(grid, p, st)
-                                         : launch_lds<2, 2, 1, 4>(grid, p, st))
-                            : (s.wm == 1 ? launch_lds<1, 2, 2, 4>(grid, p, st)
-                                         : launch_lds<2, 2, 2, 4>(grid, p, st)))
+      constexpr int kSets = sizeof(XT) == 2 ? 4 : 2;       // (f32 rows are twice the registers)
+      if (int e = s.fn == 1 ? (s.wm == 1 ? launch_lds<XT, 1, 2, 1, kSets>(grid, p, st)
+                                         : launch_lds<XT, 2, 2, 1, kSets>(grid, p, st))
+                            : (s.wm == 1          ? launch_lds<XT, 1, 2, 2, kSets>(grid, p, st)
+                               : sizeof(XT) == 4 ? launch_lds<XT, 4, 1, 2, kSets>(grid, p, st)
+                                                 : launch_lds<XT, 2, 2, 2, kSets>(grid, p, st)))
         return e;
       const int vec = (p.N % 4 == 0 && aligned(p.out, 8) && p.ldo % 4 == 0) ? 4 : 1;
       const int64_t blocks = ceil_div((int64_t)p.M * (p.N / vec), 256);
@@ -754,12 +800,18 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
     const int64_t cost128 = rounds(big, 2 * cus, cus, 82, 45);
     const int64_t cost256x128 = rounds(big256, cus, cus / 2, 75, 60);
     const int64_t cost256 = rounds(big2, cus, cus / 2, 135, 100);
-    if (cost256 < cost128 && cost256 <= cost256x128 && lds_ok) {
-      return launch_lds<4, 2, 4, 2>(dim3((unsigned)big2), p, st);
-    } else if (cost256x128 < cost128 && lds_ok) {
-      return launch_lds<4, 2, 2, 4>(dim3((unsigned)big256), p, st);
-    } else if (big >= 64 && lds_ok) {
-      return launch_lds<2, 2, 2, 4>(dim3((unsigned)big), p, st);
+    if constexpr (sizeof(XT) == 2) {
+      if (cost256 < cost128 && cost256 <= cost256x128 && lds_ok)
+        return launch_lds<XT, 4, 2, 4, 2>(dim3((unsigned)big2), p, st);
+      if (cost256x128 < cost128 && lds_ok)
+        return launch_lds<XT, 4, 2, 2, 4>(dim3((unsigned)big256), p, st);
+    }
+    // (f32 activations: the two half tiles of 256 rows would not leave room for a second stage)
+    if (big >= 64 && lds_ok) {
+      // (f32: the 96 KiB of stages leave one workgroup per compute unit, so it is eight waves
+      // of 32 x 64 rather than four of 64 x 64: 311 against 357 us at 4096^3)
+      if constexpr (sizeof(XT) == 4) return launch_lds<XT, 4, 1, 2, 2>(dim3((unsigned)big), p, st);
+      return launch_lds<XT, 2, 2, 2, 4>(dim3((unsigned)big), p, st);
     } else if (big >= 192) {
       hipLaunchKernelGGL((wo_tile_kernel<XT, 2, 2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else {
@@ -790,8 +842,8 @@ extern "C" size_t dq8_weight_only_qgemm_workspace_bytes_ex(int64_t M, int64_t N,
                                                            int tp_b, int x_dtype) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   size_t split = 0;
-  if (x_dtype == DQ8_DTYPE_F16 && K % 16 == 0 && M < (1LL << 31) && N < (1LL << 31) &&
-      K < (1LL << 31))
+  if ((x_dtype == DQ8_DTYPE_F16 || x_dtype == DQ8_DTYPE_F32) && K % 16 == 0 && M < (1LL << 31) &&
+      N < (1LL << 31) && K < (1LL << 31))
     split = split_bytes(plan_split(M, N, K), M, N);
   if (!split) return dq8_weight_only_qgemm_workspace_bytes(N, K, tp_b);
   return transposed_bytes(N, K, tp_b) + split;

@@ -329,7 +329,7 @@ int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
  * a subnormal half), and |x| must stay below 65504. */
 size_t dq8_weight_only_qgemm_workspace_bytes(int64_t N, int64_t K, int tp_b);
 /* The scratch that lets the call also split the k range over several workgroups per tile when
- * M is too small for the tiles to fill the chip (f16 activations: f32 partial sums and a
+ * M is too small for the tiles to fill the chip (f32 partial sums and a
  * reduction launch behind the GEMM; the sums of the k ranges are added in their order, so the
  * result does not depend on timing).  Includes the bytes of the function above; with less the
  * call still runs, unsplit. */

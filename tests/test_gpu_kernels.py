@@ -1166,7 +1166,8 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
     assert tuple(empty.shape) == (0, 96)
 
 
-def test_weight_only_qgemm_split_over_k(K):
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_weight_only_qgemm_split_over_k(K, dtype):
     """M between the skinny kernels' range and the sizes whose tiles fill the chip: the launch
     is split over k (f32 partial sums in the scratch, a reduction launch behind the GEMM).
     Ragged M, N and k ranges, N that is not a multiple of 4 (scalar reduction), with and
@@ -1175,13 +1176,13 @@ def test_weight_only_qgemm_split_over_k(K):
     import bladedisc_amd._lib as _lib
     L = _lib.lib()
     rng = np.random.default_rng(4242)
-    dtype = torch.float16
+    code = 1 if dtype == torch.float16 else 0
     split_seen = 0
     for (m, k, n) in [(33, 1024, 256), (64, 3072, 768), (100, 2064, 130), (128, 4096, 1024),
                       (200, 1040, 333), (512, 2048, 640), (48, 1536, 4096)]:
         x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed=False)
         plain = L.dq8_weight_only_qgemm_workspace_bytes(n, k, 1)
-        need = L.dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, 1)
+        need = L.dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, code)
         assert plain == 0 and need % (4 * m * n) == 0
         split_seen += need > 0
         args = (dev(x), dev(w), dev(scale), dev(zp), dev(bias))
@@ -1203,8 +1204,6 @@ def test_weight_only_qgemm_split_over_k(K):
                                      dev(bias), tp_b=False)
         assert torch.equal(got_kn, got)
     assert split_seen >= 5
-    # f32 activations are not split
-    assert L.dq8_weight_only_qgemm_workspace_bytes_ex(128, 1024, 4096, 1, 0) == 0
 
 
 def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
