@@ -703,13 +703,21 @@ struct SplitPlan {
   int fn = 2;    // tile columns / 64: 1 or 2
 };
 
-SplitPlan plan_split(int64_t M, int64_t N, int64_t K) {
+SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int esz) {
   SplitPlan s = {M <= 64 ? 1 : 2, 1, (int)K};
   // Measured (4096^2, 8192^2, 3072 x 768 and 768 x 3072 weights): up to 32 rows the skinny
-  // kernel wins; a k range below 256 per workgroup or fewer than 1024 of k is not worth the
-  // second launch; and the partial sums (splits x M x N floats, written and read once) bound
-  // the number of splits as M grows.
-  if (M <= 32 || K < 1024) return s;
+  // kernel wins; a k range below 256 per workgroup is not worth the second launch; and the
+  // partial sums (splits x M x N floats, written and read once) bound the number of splits as
+  // M grows.
+  if (M <= 32 || K < 512) return s;
+  if (K < 1024) {
+    // two or three k ranges of 256: worth it only against the kernels that gather activation
+    // rows lane by lane (all of them for f32 activations, the 65 .. 128-row one for f16) and
+    // while the tiles are few (768 .. 896 of k: M = 128, N = 3072, f16 10.6 against 13.7 us,
+    // f32 13.1 against 23.3; M = 256: 15.0 against 11.6 and 16.0 against 18.2)
+    const int64_t t128 = ceil_div(M, 64 * s.wm) * ceil_div(N, 128);
+    if (esz == 2 ? (M <= 64 || t128 > 32) : t128 > 48) return s;
+  }
   // 64-column tiles while 128-column ones are at most an eighth of the compute units: half
   // the partial sums per workgroup, so half of them in all (4096^2 weights, M = 64: 15.3
   // against 19.0 us; 3072 x 768, M = 512: 15.0 against 18.2)
@@ -736,7 +744,7 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
   const bool lds_ok = 512 * p.ldx + 4 * (int64_t)p.K + 4096 < (1LL << 31) &&
                       256 * p.w_sn + (int64_t)p.K + 4096 < (1LL << 31);
   if (fast && lds_ok) {
-    const SplitPlan s = plan_split(p.M, p.N, p.K);
+    const SplitPlan s = plan_split(p.M, p.N, p.K, (int)sizeof(XT));
     if (s.splits > 1 && scratch && aligned(scratch, 16) &&
         scratch_bytes >= split_bytes(s, p.M, p.N)) {
       const int bm = 64 * s.wm;
@@ -844,7 +852,7 @@ extern "C" size_t dq8_weight_only_qgemm_workspace_bytes_ex(int64_t M, int64_t N,
   size_t split = 0;
   if ((x_dtype == DQ8_DTYPE_F16 || x_dtype == DQ8_DTYPE_F32) && K % 16 == 0 && M < (1LL << 31) &&
       N < (1LL << 31) && K < (1LL << 31))
-    split = split_bytes(plan_split(M, N, K), M, N);
+    split = split_bytes(plan_split(M, N, K, x_dtype == DQ8_DTYPE_F32 ? 4 : 2), M, N);
   if (!split) return dq8_weight_only_qgemm_workspace_bytes(N, K, tp_b);
   return transposed_bytes(N, K, tp_b) + split;
 }
