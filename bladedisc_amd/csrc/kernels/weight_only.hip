@@ -30,6 +30,8 @@
 //    library's plain f16 GEMM reaches 1.16-1.49);
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
 //    problems with few tiles and little k;
+//  * wo_skinny_lds_kernel: 5 .. 32 rows against deep weights, 32 output channels per workgroup,
+//    both operands loaded in row segments and turned into fragments through wave-private LDS;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
 //  * wo_skinny_kernel: M <= 128 rows against 32 output channels per workgroup, the k range dealt
 //    over the waves and the partial sums added through LDS (bound by the weight bytes: 1 byte
@@ -594,6 +596,154 @@ __global__ void __launch_bounds__(NW * 64) wo_skinny_kernel(const WoParams p) {
   }
 }
 
+// ---------------------------------------------------------------- 8 < M <= 32, operands through LDS
+// 32 output channels per workgroup like wo_skinny_kernel<.., 1>, the k range dealt over the
+// waves in units of 64.  There every lane fetches its own activation row (32 rows x 32 bytes
+// per load instruction), and from nine rows on the compute unit's address path, not HBM, sets
+// the pace.  Here a wave loads each unit the way memory likes it -- eight lanes (sixteen for
+// f32) per 128-byte (256-byte) row segment of the activations, four per 64-byte segment of the
+// weights --, keeps three units in registers on their way from memory, and turns them into MFMA
+// fragments through a piece of LDS that only this wave touches (no barrier: the LDS executes a
+// wave's instructions in order).  f32 activations are split into hi and lo half tiles there.
+// MR: rows staged (16 or 32).
+template <typename XT, int NW, int MR>
+__global__ void __launch_bounds__(NW * 64) wo_skinny_lds_kernel(const WoParams p) {
+  constexpr bool F32 = sizeof(XT) == 4;
+  constexpr int XL = F32 ? 16 : 8;                       // lanes per activation row of a unit
+  constexpr int XP = MR * XL / 64;                       // activation loads per lane and unit
+  constexpr int XBYTES = MR * 128 * (F32 ? 2 : 1);       // [hi, then lo] half tiles
+  constexpr int WBYTES = 32 * 64;
+  constexpr int D = 3;                                   // units in registers
+  static_assert(D * (XP + 2) <= 63, "vmcnt is a 6-bit counter");
+  extern __shared__ __attribute__((aligned(16))) uint8_t wo_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const int n0 = blockIdx.x * 32;
+  const int nrows = min(32, p.N - n0), mrows = min(MR, p.M);
+  uint8_t* const xs = wo_lds + wave * (XBYTES + WBYTES);
+  uint8_t* const ws = xs + XBYTES;
+  // descriptors over the activation rows and this workgroup's weight rows; the host has
+  // checked that the byte offsets fit 31 bits
+  const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void*>(p.x), 0, (int)(((int64_t)(mrows - 1) * p.ldx + p.K) * sizeof(XT)),
+      kBufferWord3);
+  const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(p.w + (int64_t)n0 * p.w_sn), 0,
+      (int)((int64_t)(nrows - 1) * p.w_sn + p.K), kBufferWord3);
+  constexpr int kPast = (int)0x80000000;                 // an offset no descriptor covers
+
+  // global -> LDS assignment
+  const int xc = lane & (XL - 1), wc = lane & 3;
+  int xo[XP], xl[XP];
+  bool xok[XP];
+#pragma unroll
+  for (int i = 0; i < XP; ++i) {
+    const int row = lane / XL + (64 / XL) * i;
+    const int sx = (row ^ (row >> 3)) & 7;
+    xok[i] = row < mrows;                                // (rows past M are never stored)
+    xo[i] = (int)((int64_t)min(row, mrows - 1) * p.ldx * sizeof(XT)) + 16 * xc;
+    xl[i] = F32 ? row * 128 + (((xc >> 1) ^ sx) << 4) + 8 * (xc & 1)
+                : row * 128 + ((xc ^ sx) << 4);
+  }
+  int wo[2], wl[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = (lane >> 2) + 16 * i;
+    wo[i] = (int)((int64_t)min(row, nrows - 1) * p.w_sn) + 16 * wc;
+    wl[i] = row * 64 + ((wc ^ ((row >> 2) & 3)) << 4);
+  }
+  const h2 c = centre(p, n0 + min(r, nrows - 1));
+  u4 xr[D][XP], wr[D][2];
+  auto fetch = [&](u4* xq, u4* wq, int k0) {
+    const bool xv = k0 + (F32 ? 4 : 8) * xc < p.K, wv = k0 + 16 * wc < p.K;   // K % 16 == 0
+#pragma unroll
+    for (int i = 0; i < XP; ++i)
+      xq[i] = __builtin_amdgcn_raw_buffer_load_b128(
+          xrs, xv && xok[i] ? xo[i] + (int)sizeof(XT) * k0 : kPast, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      wq[i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wv ? wo[i] + k0 : kPast, 0, 0);
+  };
+  auto park = [&](const u4* xq, const u4* wq) {
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+      if constexpr (F32) {
+        const f4 v = __builtin_bit_cast(f4, xq[i]);
+        h4 hi, lo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          hi[e] = (_Float16)v[e];
+          lo[e] = (_Float16)(v[e] - (float)hi[e]);
+        }
+        *reinterpret_cast<h4*>(&xs[xl[i]]) = hi;
+        *reinterpret_cast<h4*>(&xs[MR * 128 + xl[i]]) = lo;
+      } else {
+        *reinterpret_cast<u4*>(&xs[xl[i]]) = xq[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *reinterpret_cast<u4*>(&ws[wl[i]]) = wq[i];
+  };
+  f16v acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  // this lane's fragment rows (activation rows past the staged ones re-read a staged one:
+  // their results are not stored)
+  const int xrow = r & (MR - 1), sxr = (xrow ^ (xrow >> 3)) & 7, swr = (r >> 2) & 3;
+  auto multiply = [&]() {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {                          // the unit's two 32-deep chunks
+      const int cx = 4 * q + 2 * g;
+      const h8 a0 = *reinterpret_cast<const h8*>(&xs[xrow * 128 + ((cx ^ sxr) << 4)]);
+      const h8 a1 = *reinterpret_cast<const h8*>(&xs[xrow * 128 + (((cx + 1) ^ sxr) << 4)]);
+      const u4 wq = *reinterpret_cast<const u4*>(&ws[r * 64 + (((2 * q + g) ^ swr) << 4)]);
+      h8 w0, w1;
+      widen16(wq, p.flip, c, w0, w1);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, w0, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, w1, acc, 0, 0, 0);
+      if constexpr (F32) {
+        const h8 l0 =
+            *reinterpret_cast<const h8*>(&xs[MR * 128 + xrow * 128 + ((cx ^ sxr) << 4)]);
+        const h8 l1 =
+            *reinterpret_cast<const h8*>(&xs[MR * 128 + xrow * 128 + (((cx + 1) ^ sxr) << 4)]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(l0, w0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(l1, w1, acc, 0, 0, 0);
+      }
+    }
+  };
+  // units wave, wave + NW, ... of 64 of k; set u holds unit i + u on its way from memory
+  // (past K: zeros, no memory touched).  The scheduling barriers keep a later step's arithmetic
+  // on loaded registers from being moved up to where it would wait for their loads.
+  const int w64 = __builtin_amdgcn_readfirstlane(wave) * 64;
+#pragma unroll
+  for (int d = 0; d < D; ++d) fetch(xr[d], wr[d], w64 + d * NW * 64);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int k0 = w64; k0 < p.K; k0 += D * NW * 64) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      park(xr[u], wr[u]);
+      fetch(xr[u], wr[u], k0 + (D + u) * NW * 64);
+      multiply();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // partial sums of the waves through LDS (all waves are done with their pieces of it)
+  __syncthreads();
+  float* const red = reinterpret_cast<float*>(wo_lds);   // [NW - 1][16][64]
+  if (wave > 0) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[((wave - 1) * 16 + v) * 64 + lane] = acc[v];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 1; w < NW; ++w)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[v] += red[((w - 1) * 16 + v) * 64 + lane];
+    store_frag<XT>(p, acc, 0, n0 + r, lane);
+  }
+}
+
 // ---------------------------------------------------------------- M <= 16
 // 16 output channels per workgroup on v_mfma_f32_16x16x32_f16: twice as many workgroups as the
 // 32-channel form for the same weights (a 4096 x 4096 weight gives 256 instead of 128), and a
@@ -693,6 +843,18 @@ int launch_lds(dim3 grid, const WoParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch");
 }
 
+template <typename XT, int MR>
+int launch_skinny_lds(const WoParams& p, hipStream_t st) {
+  constexpr int lds = 8 * (MR * 128 * (int)(sizeof(XT) / 2) + 32 * 64);
+  static_assert(lds >= 7 * 16 * 64 * 4, "the partial sums of the waves fit");
+  auto kern = wo_skinny_lds_kernel<XT, 8, MR>;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (lds > 64 * 1024)
+    if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
+  hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(p.N, 32)), dim3(512), lds, st, p);
+  return check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch");
+}
+
 // Split plan of the LDS kernel (f16 activations) for problems whose tiles would leave most of
 // the chip idle: `splits` workgroups per tile, each over k_split of the k range, and a
 // reduction kernel behind them.  splits == 1: no split.
@@ -779,6 +941,16 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
     const unsigned grid = (unsigned)ceil_div(p.N, 32);
     // (with more than 8 rows every workgroup re-reads the activations, which then outweigh
     // its weights: the narrow form only while the wide one would leave compute units idle)
+    // (the staged kernel addresses activation and weight rows by 31-bit byte offsets)
+    const bool staged_ok =
+        ((int64_t)(p.M - 1) * p.ldx + p.K) * (int64_t)sizeof(XT) + 65536 < (1LL << 31) &&
+        32 * p.w_sn + (int64_t)p.K + 65536 < (1LL << 31);
+    // (it needs several 64-deep units per wave to run its pipeline: measured against the two
+    // kernels below it wins from 12 rows on at 3072 and 4096 of k -- 4096^2 weights, f16, M = 32:
+    // 10.7 against 14.9 us -- and from 5 rows on at 8192 -- M = 16: 16.8 against 22.5 us --, and
+    // loses about a microsecond at 768 or 1040 of k)
+    if (staged_ok && p.M <= 32 && ((p.K >= 2048 && p.M >= 12) || (p.K >= 6144 && p.M >= 5)))
+      return p.M <= 16 ? launch_skinny_lds<XT, 16>(p, st) : launch_skinny_lds<XT, 32>(p, st);
     if (p.M <= 8 || (p.M <= 16 && grid < 256))
       hipLaunchKernelGGL((wo_skinny16_kernel<XT, 8>), dim3((unsigned)ceil_div(p.N, 16)), dim3(512),
                          0, st, p);

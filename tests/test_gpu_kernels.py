@@ -1167,6 +1167,24 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_weight_only_qgemm_small_m_staged_through_lds(K, dtype):
+    """5 .. 32 rows against deep weights: the kernel that stages both operands through
+    wave-private LDS (16 and 32 staged rows; k depths that end inside a unit of 64 and inside
+    a group of three units; N that ends inside a workgroup's 32 channels; signed weights)."""
+    rng = np.random.default_rng(99)
+    for (m, k, n, signed) in [(12, 2048, 96, False), (16, 3072, 768, False), (17, 2064, 100, True),
+                              (32, 4096, 330, False), (5, 6160, 72, True), (9, 8192, 64, False),
+                              (31, 2048 + 16 * 9, 40, False)]:
+        x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed)
+        got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+        _weight_only_check(got, x, w, scale, zp, bias, dtype)
+        # strided activations and no bias / zero points
+        wide = dev(np.concatenate([x, x], axis=1))
+        got = K.weight_only_qgemm(wide[:, :k], dev(w), dev(scale))
+        _weight_only_check(got, x, w, scale, None, None, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_weight_only_qgemm_split_over_k(K, dtype):
     """M between the skinny kernels' range and the sizes whose tiles fill the chip: the launch
     is split over k (f32 partial sums in the scratch, a reduction launch behind the GEMM).
