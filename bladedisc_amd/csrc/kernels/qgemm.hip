@@ -298,8 +298,9 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) {
   auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
   if (pipe) {
-    if (N <= 64 && M >= 256 * 64) return kPipe256x64;
     const int64_t cus = compute_units();
+    // (256 x 64 tiles for a narrow N once they occupy three quarters of the compute units)
+    if (N <= 64 && 4 * tiles(kPipe256x64) >= 3 * cus) return kPipe256x64;
     const int64_t t256 = tiles(kPipe256w8);
     const int64_t rounds = ceil_div(t256, cus);
     const bool big256 = t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * cus * rounds) &&
@@ -374,8 +375,14 @@ int pick_direct_conv(int64_t images, int64_t pixels_per_image, int64_t Ci, int64
   const int64_t cus = compute_units();
   const int64_t wg512 = images * ceil_div(pixels_per_image, bm) * ceil_div(Co, bn);
   if (wg512 <= cus && 4 * wg512 >= 3 * cus) return 2;
-  direct_conv_tile(0, &bm, &bn);
-  return images * ceil_div(pixels_per_image, bm) * ceil_div(Co, bn) >= 256 ? 0 : -1;
+  // else the largest of the 256- and 128-pixel tiles that still occupies three quarters of
+  // the compute units (batch 8 of the same layer: 200 workgroups of 128 pixels 6.5 us, 104 of
+  // 256 pixels 7.8, the implicit GEMM's 256 x 64 tiles 9.4)
+  for (int config : {0, 1}) {
+    direct_conv_tile(config, &bm, &bn);
+    if (4 * images * ceil_div(pixels_per_image, bm) * ceil_div(Co, bn) >= 3 * cus) return config;
+  }
+  return -1;
 }
 
 int elem_size(int epilogue) {
