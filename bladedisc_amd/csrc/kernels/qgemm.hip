@@ -151,6 +151,48 @@ int transpose_batched(const void* src, void* dst, int64_t B, int64_t R, int64_t 
   return check_hip(hipGetLastError(), "layout change launch");
 }
 
+// Space to depth for stride-2 convolutions of images with at most 4 channels (the stem of a
+// vision network: 7 x 7, stride 2, 3 channels).  src: [B, H, W, C] with C <= 4; the element
+// at padded position (2 by + dy, 2 bx + dx), channel c goes to dst[b][by][bx][(2 dy + dx) C + c]
+// of [B, Hb, Wb, 16]; positions in the padding frame and the channels past 4 C are zero.  A
+// K x K stride-2 convolution of src is then a ceil(K / 2)^2 stride-1 convolution of dst.  With
+// H = Kh, W = Kw, no padding and B = Co the same kernel re-lays out the weights.  One 16-byte
+// store per thread.
+__global__ void __launch_bounds__(256)
+space_to_depth2_s8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, int64_t B,
+                          int H, int W, int C, int Hb, int Wb, int pad_t, int pad_l) {
+  const int64_t total = B * Hb * Wb;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * 256) {
+    const int bx = (int)(idx % Wb);
+    const int by = (int)((idx / Wb) % Hb);
+    const int64_t b = idx / ((int64_t)Wb * Hb);
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int iy = 2 * by + (q >> 1) - pad_t, ix = 2 * bx + (q & 1) - pad_l;
+      if ((unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W) {
+        const int8_t* px = src + ((b * H + iy) * W + ix) * C;
+        for (int c = 0; c < C; ++c) {
+          const int e = q * C + c;
+          w[e >> 2] |= (uint32_t)(uint8_t)px[c] << (8 * (e & 3));
+        }
+      }
+    }
+    *reinterpret_cast<v4i*>(dst + idx * 16) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  }
+}
+
+int space_to_depth2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t H, int64_t W,
+                       int64_t C, int64_t Hb, int64_t Wb, int pad_t, int pad_l, hipStream_t st) {
+  const int64_t total = B * Hb * Wb;
+  if (total == 0) return 0;
+  const int64_t blocks = std::min<int64_t>(ceil_div(total, 256), 1 << 20);
+  hipLaunchKernelGGL(space_to_depth2_s8_kernel, dim3((unsigned)blocks), dim3(256), 0, st, src,
+                     dst, B, (int)H, (int)W, (int)C, (int)Hb, (int)Wb, pad_t, pad_l);
+  return check_hip(hipGetLastError(), "space-to-depth launch");
+}
+
 // int8 [R, C] (row stride ld, any alignment) -> [R, ldd], ldd % 16 == 0 and dst 16-byte
 // aligned, columns C .. ldd-1 zero.  One 16-byte store per thread and step.
 __global__ void __launch_bounds__(256)
@@ -852,6 +894,38 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     }
   }
 
+  // Stride 2 on an image of at most 4 channels (NHWC x OHWI, no dilation): with scratch, the
+  // image goes through space to depth -- 2 x 2 pixels become the 16 channels of one, the
+  // padding frame is written out -- and the weights likewise, and the convolution runs as a
+  // ceil(K / 2)^2 stride-1 one on 16 channels.  Padding the 3 channels of a 7 x 7 stem to 16
+  // instead costs 784 of k per output where this costs 256 (measured, batch 32 of 224 x 224:
+  // 62-65 us that way).
+  if (variant == -1 && is_nhwc_ohwi(md) && Ci >= 1 && Ci <= 4 && sh == 2 && sw_ == 2 &&
+      dh == 1 && dw == 1 && workspace != nullptr && aligned(workspace, 256) && Ho > 0 && Wo > 0 &&
+      NB > 0 && Co > 0 && in && w && out && H < (1 << 30) && Wd < (1 << 30)) {
+    const int64_t kbh = (Kh + 1) / 2, kbw = (Kw + 1) / 2;
+    const int64_t Hb = Ho + kbh - 1, Wb = Wo + kbw - 1;
+    const size_t in_b = pad256(NB * Hb * Wb * 16), w_b = pad256(Co * kbh * kbw * 16);
+    if (workspace_bytes >= in_b + w_b) {
+      hipStream_t st0 = (hipStream_t)stream;
+      int8_t* in_t = static_cast<int8_t*>(workspace);
+      int8_t* w_t = in_t + in_b;
+      if (int s = space_to_depth2_s8(in, in_t, NB, H, Wd, Ci, Hb, Wb, padding[0], padding[2], st0))
+        return s;
+      if (int s = space_to_depth2_s8(w, w_t, Co, Kh, Kw, Ci, kbh, kbw, 0, 0, st0)) return s;
+      const int64_t in2[4] = {NB, Hb, Wb, 16}, w2[4] = {Co, kbh, kbw, 16};
+      const int32_t pad2[4] = {0, 0, 0, 0};
+      int32_t md2[17];
+      for (int i = 0; i < 17; ++i) md2[i] = md[i];
+      md2[12] = md2[13] = 1;
+      const size_t used = in_b + w_b;
+      return qconv2d_impl(variant, in_t, in2, w_t, w2, pad2, md2, out, out_sizes, epilogue, bias,
+                          bias_kind, sx, sw, n_sw, so, zo,
+                          static_cast<uint8_t*>(workspace) + used, workspace_bytes - used, stream,
+                          post);
+    }
+  }
+
   // requant -> dequantize in one epilogue, as in dq8_qgemm
   int requant = 0;
   if (epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || epilogue == DQ8_EPI_REQUANT_GPU_DEQUANT_F32) {
@@ -1054,8 +1128,17 @@ extern "C" size_t dq8_qconv2d_workspace_bytes_ex(const int64_t in_sizes[4],
   const int64_t ci = in_sizes[3];
   if (ci % 16 == 0) return 0;
   const int64_t cip = (ci + 15) / 16 * 16;
-  return pad256(in_sizes[0] * in_sizes[1] * in_sizes[2] * cip) +
-         pad256(w_sizes[0] * w_sizes[1] * w_sizes[2] * cip);
+  size_t need = pad256(in_sizes[0] * in_sizes[1] * in_sizes[2] * cip) +
+                pad256(w_sizes[0] * w_sizes[1] * w_sizes[2] * cip);
+  // (the space-to-depth copies of a stride-2 convolution with at most 4 channels; smaller
+  // than the padded copies except for images of a few pixels)
+  if (ci <= 4 && out_sizes && metadata[12] == 2 && metadata[13] == 2) {
+    const int64_t kbh = (w_sizes[1] + 1) / 2, kbw = (w_sizes[2] + 1) / 2;
+    const size_t s2d = pad256(in_sizes[0] * (out_sizes[1] + kbh - 1) * (out_sizes[2] + kbw - 1) * 16) +
+                       pad256(w_sizes[0] * kbh * kbw * 16);
+    if (s2d > need) need = s2d;
+  }
+  return need;
 }
 
 extern "C" size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const int64_t w_sizes[4],

@@ -937,6 +937,40 @@ def test_qconv_nchw_oihw_on_the_mfma_path(K, nb, ci, h, w_, co, k, stride, pad, 
     assert np.array_equal(got_f.view(np.uint32), want_f.view(np.uint32))
 
 
+@pytest.mark.parametrize("nb,ci,h,w_,co,k,pads", [(2, 3, 32, 32, 64, 7, (3, 3, 3, 3)), (1, 3, 17, 23, 20, 7, (3, 2, 2, 3)),
+                                                 (3, 1, 12, 12, 16, 3, (1, 1, 1, 1)), (2, 4, 15, 14, 33, 5, (2, 2, 2, 2)),
+                                                 (1, 2, 9, 9, 8, 2, (0, 0, 0, 0)), (2, 3, 8, 8, 64, 3, (0, 1, 0, 1)),
+                                                 (1, 3, 4, 4, 8, 7, (3, 3, 3, 3))])
+def test_qconv_stride2_few_channels_space_to_depth(K, nb, ci, h, w_, co, k, pads):
+    """Stride-2 convolutions of images with at most 4 channels (the 7 x 7 stem of a vision
+    network): with scratch they run as a stride-1 convolution of the space-to-depth image on
+    the MFMA kernels -- the same bits as the oracle and as the path without scratch; odd and
+    even filter sizes, asymmetric padding, odd image sizes, an image so small that the
+    space-to-depth copy is larger than the padded one, NCHW x OIHW on top."""
+    rng = np.random.default_rng(ci * 100 + k + h)
+    x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+    wt = rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8)
+    ho = (h + pads[0] + pads[1] - k) // 2 + 1
+    wo = (w_ + pads[2] + pads[3] - k) // 2 + 1
+    md = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
+    padding, osh = list(pads), [nb, ho, wo, co]
+    acc = O.conv_s32(x, wt, padding, md, osh)
+    for ws in (True, False):
+        got = host(K.qconv2d(dev(x), dev(wt), padding, md, osh, K.EPI_ACC_S32, workspace=ws))
+        np.testing.assert_array_equal(got, acc)
+    sx, sw = make_scales(rng, co)
+    so = pick_so(acc, sx, sw)
+    sc = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so], np.float32)))
+    want = O.requant_cpu(acc.reshape(-1, co), sx, sw, so).reshape(osh)
+    got = host(K.qconv2d(dev(x), dev(wt), padding, md, osh, K.EPI_REQUANT_CPU, **sc))
+    np.testing.assert_array_equal(got, want)
+    # the PyTorch layouts: NCHW x OIHW -> NCHW
+    md_t = [0, 1, 2, 3, 1, 0, 2, 3, 0, 1, 2, 3, 2, 2, 1, 1, 1]
+    x_t, w_t = np.ascontiguousarray(np.moveaxis(x, -1, 1)), np.ascontiguousarray(np.moveaxis(wt, -1, 1))
+    got = host(K.qconv2d(dev(x_t), dev(w_t), padding, md_t, [nb, co, ho, wo], K.EPI_REQUANT_CPU, **sc))
+    np.testing.assert_array_equal(got, np.moveaxis(want, -1, 1))
+
+
 def test_qconv_known_answers(K, golden):
     for case in golden["qconv"]:
         if case["data_format"] != "NHWC":
