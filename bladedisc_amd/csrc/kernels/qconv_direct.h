@@ -1,4 +1,4 @@
-// int8 NHWC 3x3 stride-1 convolution with the input patch resident in LDS.
+// int8 NHWC stride-1 convolution (3x3 in the first place) with the input patch resident in LDS.
 //
 // As an implicit GEMM a 3x3 convolution pulls every input pixel through the CU's
 // address unit nine times (once per tap), and at 64 or 128 channels that, not the MFMAs,
@@ -20,7 +20,11 @@
 //    in and out, a k loop without waits or barriers -- was measured: the k loop gets 12 %
 //    shorter, the launch no faster.  Eight waves instead of four on the 256 x 64 tile:
 //    slower at 64 channels, 9.75 against 10.7 us at 128, where the implicit GEMM is used.)
-// Requires Ci in {32, 64, 128, 256}, 16-byte aligned tensors, dilation 1, stride 1.
+// Requires Ci in {32, 64, 128, 256}, 16-byte aligned tensors, dilation 1, stride 1.  Other
+// filter sizes up to 7 x 7 run the same way (k runs over (kh, kw, ci), the patch has Kh - 1
+// and Kw - 1 extra rows and columns), and so do 16 channels with an even filter width: the 32
+// bytes of k of an MFMA step are then two taps next to each other in a filter row, i.e. two
+// neighbouring patch pixels -- the stride-1 form of a stem convolution after space to depth.
 #ifndef DQ8_QCONV_DIRECT_H_
 #define DQ8_QCONV_DIRECT_H_
 
@@ -30,14 +34,16 @@ namespace dq8 {
 
 struct DirectConvParams {
   const int8_t* in;     // [NB, H, W, Ci]
-  const int8_t* w;      // [Co, 3, 3, Ci]
+  const int8_t* w;      // [Co, Kh, Kw, Ci]
   int NB, H, Wd, Ci, Co, Ho, Wo;
+  int Kh, Kw;
+  int kw_inv;           // ceil(65536 / Kw): tap / Kw == (tap * kw_inv) >> 16 for tap < 64
   int pad_t, pad_l;
   int log2_ci;          // Ci = 1 << log2_ci
   int tiles_per_image;  // ceil(Ho * Wo / BM)
   int tiles_n;          // ceil(Co / BN)
-  int patch_bytes;      // LDS reserved for the patch: (most rows a tile spans + 2) *
-                        // (Wo + 2) * Ci, rounded up to 1 KiB
+  int patch_bytes;      // LDS reserved for the patch: (most rows a tile spans + Kh - 1) *
+                        // (Wo + Kw - 1) * Ci, rounded up to 1 KiB
   int64_t in_bytes;
   EpiParams epi;
 };
@@ -78,8 +84,9 @@ __global__ void __launch_bounds__(WM* WN * 64) qconv3x3_direct_kernel(const Dire
   const int p0 = tp * BM;                                  // first output pixel of the tile
   const int p_last = min(p0 + BM, hw) - 1;
   const int y_base = p0 / p.Wo;
-  const int rows = p_last / p.Wo - y_base + 1 + 2;         // patch rows in use
-  const int PW = p.Wo + 2;                                 // patch width
+  const int rows = p_last / p.Wo - y_base + p.Kh;          // patch rows in use
+  const int PW = p.Wo + p.Kw - 1;                          // patch width
+  const int taps = p.Kh * p.Kw;
   const int CP = p.Ci >> 4;                                // 16-byte chunks per pixel
   // LDS swizzle: chunk c of patch pixel q is stored in slot c ^ f(q) of the pixel.  A
   // 16-byte-per-lane LDS read is served 16 lanes (256 bytes, all 64 banks) at a time; the
@@ -89,11 +96,11 @@ __global__ void __launch_bounds__(WM* WN * 64) qconv3x3_direct_kernel(const Dire
   // f(q) = (q >> fshift) & fmask.
   const int fshift = p.log2_ci >= 8 ? 0 : 8 - p.log2_ci;
   const int fmask = CP - 1;
-  const int KT = (9 * p.Ci + BK - 1) / BK;
+  const int KT = (taps * p.Ci + BK - 1) / BK;
 
   const v4i in_rsrc = make_rsrc(p.in, p.in_bytes);
-  const int8_t* w_base = p.w + (int64_t)n0 * 9 * p.Ci;
-  const int64_t w_valid = (int64_t)(p.Co - n0) * 9 * p.Ci;
+  const int8_t* w_base = p.w + (int64_t)n0 * taps * p.Ci;
+  const int64_t w_valid = (int64_t)(p.Co - n0) * taps * p.Ci;
   const v4i w_rsrc = make_rsrc(w_base, w_valid < 0x7fffffff ? w_valid : 0x7fffffff);
   const unsigned lds_base =
       (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(size_t)(lds_void_t*)smem);
@@ -137,11 +144,11 @@ __global__ void __launch_bounds__(WM* WN * 64) qconv3x3_direct_kernel(const Dire
 #pragma unroll
   for (int i = 0; i < B_LD; ++i) {
     const int qb = wave + i * NW;
-    b_off[i] = (qb * 8 + lr) * 9 * p.Ci + kc;
+    b_off[i] = (qb * 8 + lr) * taps * p.Ci + kc;
     b_lds[i] = __builtin_amdgcn_readfirstlane(p.patch_bytes + qb * 1024);
   }
   auto issue_weights = [&](int kt, int st) {
-    const bool in = kt < KT && kt * BK + kc < 9 * p.Ci;
+    const bool in = kt < KT && kt * BK + kc < taps * p.Ci;
     const unsigned base = (unsigned)__builtin_amdgcn_readfirstlane((int)(lds_base + st * B_BYTES));
 #pragma unroll
     for (int i = 0; i < B_LD; ++i)
@@ -179,11 +186,12 @@ __global__ void __launch_bounds__(WM* WN * 64) qconv3x3_direct_kernel(const Dire
   // Fragments are read one k-step ahead of their MFMAs, into two alternating sets.
   v4i fa[2][FM], fb[2][FN];
   auto load_frags = [&](int set, int kt, int st, int ks) {
-    // the 32 bytes of k of a step lie in one tap (Ci is a multiple of 32)
+    // the 32 bytes of k of a step lie in one tap (Ci a multiple of 32) or in two taps next to
+    // each other in a filter row (Ci = 16, even Kw: chunk 1 of a 16-byte pixel is the next one)
     const int koff = kt * BK + ks * 32;
     int tap = koff >> p.log2_ci;
-    tap = tap < 9 ? tap : 8;                               // past K: the weights are zeros
-    const int kh = (tap * 11) >> 5, kw = tap - 3 * kh;
+    tap = tap < taps ? tap : taps - 1;                     // past K: the weights are zeros
+    const int kh = (tap * p.kw_inv) >> 16, kw = tap - p.Kw * kh;
     const int c = ((koff & (p.Ci - 1)) >> 4) + (lane >> 5);
     const int shift = kh * PW + kw;
 #pragma unroll
@@ -251,8 +259,9 @@ constexpr int kNumDirectConvConfigs = 3;
 // Tile shape of configuration `config` (0 .. kNumDirectConvConfigs - 1).
 void direct_conv_tile(int config, int* bm, int* bn);
 
-// Whether configuration `config` can run the problem: 3x3 filter, Ci in {32, 64, 128, 256},
-// 32-bit buffer offsets, and the patch plus the weight stages fit the LDS.  Fills the
+// Whether configuration `config` can run the problem: filter up to 7 x 7 (p->Kh, p->Kw), Ci in
+// {32, 64, 128, 256} or 16 with an even Kw, 32-bit buffer offsets, and the patch plus the weight
+// stages fit the LDS.  Fills the
 // launch geometry of `p` (tiles_per_image, tiles_n, patch_bytes, log2_ci).
 bool direct_conv_plan(int config, DirectConvParams* p);
 

@@ -53,12 +53,14 @@ bool direct_conv_plan(int config, DirectConvParams* p) {
   const int bm = kTiles[config].bm, bn = kTiles[config].bn;
   int log2_ci = 0;
   while ((1 << log2_ci) < p->Ci) ++log2_ci;
-  if ((1 << log2_ci) != p->Ci || p->Ci < 32 || p->Ci > 256) return false;
+  if ((1 << log2_ci) != p->Ci || p->Ci < 16 || p->Ci > 256) return false;
+  if (p->Kh < 1 || p->Kw < 1 || p->Kh > 7 || p->Kw > 7) return false;
+  if (p->Ci == 16 && p->Kw % 2 != 0) return false;
   if (p->NB <= 0 || p->Ho <= 0 || p->Wo <= 0 || p->Co <= 0) return false;
   const int64_t in_bytes = (int64_t)p->NB * p->H * p->Wd * p->Ci;
   if (in_bytes >= (1LL << 31)) return false;
   // byte offset of the last weight chunk a block may address, from its first row
-  if ((int64_t)(bn + 8) * 9 * p->Ci + 4 * 128 >= (1LL << 31)) return false;
+  if ((int64_t)(bn + 8) * p->Kh * p->Kw * p->Ci + 4 * 128 >= (1LL << 31)) return false;
   const int hw = p->Ho * p->Wo;
   const int tiles = (hw + bm - 1) / bm;
   int span = 0;
@@ -66,11 +68,13 @@ bool direct_conv_plan(int config, DirectConvParams* p) {
     const int first = t * bm, last = std::min(first + bm, hw) - 1;
     span = std::max(span, last / p->Wo - first / p->Wo + 1);
   }
-  const int64_t patch = ((int64_t)(span + 2) * (p->Wo + 2) * p->Ci + 1023) / 1024 * 1024;
+  const int64_t patch =
+      ((int64_t)(span + p->Kh - 1) * (p->Wo + p->Kw - 1) * p->Ci + 1023) / 1024 * 1024;
   if (patch + (int64_t)kStages * bn * 128 > kLdsBytes) return false;
   // (the epilogue's staging -- 8 bytes per channel plus at most bm * bn bytes -- fits in the
   // weight stages alone: 4 * 128 * bn bytes)
   p->log2_ci = log2_ci;
+  p->kw_inv = (65536 + p->Kw - 1) / p->Kw;
   p->tiles_per_image = tiles;
   p->tiles_n = (p->Co + bn - 1) / bn;
   p->patch_bytes = (int)patch;

@@ -1081,13 +1081,17 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   d.NB = (int)NB; d.H = (int)H; d.Wd = (int)Wd; d.Ci = (int)Ci; d.Co = (int)Co;
   d.Ho = (int)Ho; d.Wo = (int)Wo;
   d.pad_t = padding[0]; d.pad_l = padding[2];
+  d.Kh = (int)(Kh < 64 ? Kh : 64); d.Kw = (int)(Kw < 64 ? Kw : 64);
   d.epi = e;
-  const bool direct_shape = Kh == 3 && Kw == 3 && sh == 1 && sw_ == 1 && dh == 1 && dw == 1;
+  // (3 x 3 in the first place; any filter up to 7 x 7 with more than one tap runs the same way)
+  const bool direct_shape = Kh * Kw > 1 && Kh <= 7 && Kw <= 7 && sh == 1 && sw_ == 1 && dh == 1 &&
+                            dw == 1 && padding[0] < Kh && padding[2] < Kw;
   if ((variant >= kDirectConv0 && variant < kDirectConv0 + 2) || variant == kDirectConv2) {
     const int config = variant == kDirectConv2 ? 2 : variant - kDirectConv0;
     DQ8_REQUIRE(direct_shape && direct_conv_plan(config, &d),
-                "dq8_qconv2d: the direct variants need a 3x3 filter with stride and dilation "
-                "1, Ci in {32, 64, 128, 256} and a patch that fits the LDS");
+                "dq8_qconv2d: the direct variants need a filter of 2 to 7 x 7 taps with stride and "
+                "dilation 1, Ci in {32, 64, 128, 256} (or 16 with an even filter width) and a "
+                "patch that fits the LDS");
     return launch_direct_conv(config, epilogue, d, st);
   }
   if (auto_pick) {

@@ -862,9 +862,57 @@ def test_qconv_direct_random_shapes(K):
             np.testing.assert_array_equal(got, want, err_msg=tag + " variant %d" % v)
 
 
+def test_qconv_direct_other_filter_sizes(K):
+    """The same kernels on filters other than 3 x 3 (up to 7 x 7, rectangular ones too) and on
+    16 channels with an even filter width, where an MFMA step's 32 bytes of k are two
+    neighbouring patch pixels (the stride-1 form of a stem convolution after space to depth):
+    bit-exact against the oracle for every tile shape that accepts the problem."""
+    rng = np.random.default_rng(20260303)
+    names = K.variant_names()
+    direct = [i for i, nm in enumerate(names) if nm.startswith("direct3x3_")]
+    ran = 0
+    for (nb, h, w_, ci, co, kh, kw, pad) in [
+            (2, 20, 30, 32, 64, 5, 5, [2, 2, 2, 2]), (1, 16, 16, 64, 40, 7, 7, [3, 3, 3, 3]),
+            (2, 12, 25, 32, 64, 1, 3, [0, 0, 1, 1]), (1, 18, 18, 128, 17, 2, 2, [0, 1, 0, 1]),
+            (2, 35, 35, 16, 64, 4, 4, [0, 0, 0, 0]), (3, 19, 40, 16, 48, 2, 2, [1, 0, 0, 1]),
+            (1, 60, 115, 16, 64, 4, 4, [0, 0, 0, 0]), (1, 14, 14, 16, 8, 3, 6, [1, 1, 2, 3])]:
+        ho, wo = h + pad[0] + pad[1] - kh + 1, w_ + pad[2] + pad[3] - kw + 1
+        x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, kh, kw, ci), dtype=np.int8)
+        md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+        out_shape = [nb, ho, wo, co]
+        acc = O.conv_s32(x, wt, pad, md, out_shape)
+        sx, sw = make_scales(rng, co)
+        so = pick_so(acc, sx, sw)
+        want = O.requant_cpu(acc.reshape(-1, co), sx, sw, so).reshape(out_shape)
+        tag = "%dx%dx%dx%d -> %d, %dx%d pad %s" % (nb, h, w_, ci, co, kh, kw, pad)
+        for v in direct:
+            try:
+                got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_ACC_S32, variant=v))
+            except RuntimeError as exc:
+                assert "fits the LDS" in str(exc), (tag, names[v], exc)
+                continue
+            ran += 1
+            np.testing.assert_array_equal(got, acc, err_msg=tag + " " + names[v])
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU,
+                                 sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])),
+                                 variant=v))
+            np.testing.assert_array_equal(got, want, err_msg=tag + " " + names[v])
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_ACC_S32))
+        np.testing.assert_array_equal(got, acc, err_msg=tag + " auto")
+    assert ran >= 20
+    # 16 channels and an odd filter width: no layout for that
+    x = rng.integers(-128, 128, (1, 8, 8, 16), dtype=np.int8)
+    wt = rng.integers(-128, 128, (8, 3, 3, 16), dtype=np.int8)
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    for v in direct:
+        with pytest.raises(RuntimeError, match="direct variants"):
+            K.qconv2d(dev(x), dev(wt), [1] * 4, md, [1, 8, 8, 8], K.EPI_ACC_S32, variant=v)
+
+
 def test_qconv_direct_variants_refuse_what_they_cannot_run(K):
     """A named direct-convolution variant fails with an error, not a wrong result, on a
-    filter that is not 3x3 stride 1, on a channel count it has no layout for, and on an image
+    filter of a single tap or a stride other than 1, on a channel count it has no layout for, and on an image
     row too wide for its patch to fit the LDS; the automatic choice runs all of them."""
     names = K.variant_names()
     direct = [i for i, nm in enumerate(names) if nm.startswith("direct3x3_")]
