@@ -572,6 +572,25 @@ def extras(torch, steps, warmup, which="all"):
                 "roofline_frac": round(max(byts / t / 1e9 / PEAK_HBM_GBPS,
                                            flops / t / 1e12 / 2500.0), 4)}
     out["weight_only_qgemm_f16_u8"] = wo
+    # the same with f32 activations, the type of the reference's own test of the pattern: they
+    # enter the f16 matrix cores as hi + lo halves, twice the MFMAs (the fraction is of the
+    # nominal flops against the f16 peak)
+    wo32 = {}
+    k, n = 4096, 4096
+    wq = torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda")
+    sc = torch.rand(n, device="cuda") * 0.02 + 0.002
+    zp = torch.full((n,), 128, dtype=torch.int32, device="cuda")
+    for m in (16, 128, 4096):
+        xf = torch.randn((m, k), device="cuda")
+        of = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        t = time_graph(torch, [FnCall(lambda: K.weight_only_qgemm(xf, wq, sc, zp, out=of))])
+        byts, flops = 4.0 * m * k + n * k + 4.0 * m * n + 8.0 * n, 2.0 * m * n * k
+        wo32["M%d_K%d_N%d" % (m, k, n)] = {
+            "us": round(t * 1e6, 2), "us_fastest_replay": round(t.fastest * 1e6, 2),
+            "GB/s": round(byts / t / 1e9, 1), "TFLOP/s": round(flops / t / 1e12, 1),
+            "roofline_frac": round(max(byts / t / 1e9 / PEAK_HBM_GBPS,
+                                       flops / t / 1e12 / 2500.0), 4)}
+    out["weight_only_qgemm_f32_u8"] = wo32
     out["configs"] = config_reports(torch, K)
     # yardstick: the ROCm library int8 GEMM behind torch._int_mm (int32 output, no
     # epilogue) on the headline shape and data distribution -- a library, not the reference
