@@ -32,6 +32,8 @@
 //    problems with few tiles and little k;
 //  * wo_skinny_lds_kernel: 5 .. 32 rows against deep weights, 32 output channels per workgroup,
 //    both operands loaded in row segments and turned into fragments through wave-private LDS;
+//  * wo_gemv_kernel: one or two rows, a wave per output channel streaming its weight row on the
+//    vector ALUs;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
 //  * wo_skinny_kernel: M <= 128 rows against 32 output channels per workgroup, the k range dealt
 //    over the waves and the partial sums added through LDS (bound by the weight bytes: 1 byte
@@ -596,6 +598,87 @@ __global__ void __launch_bounds__(NW * 64) wo_skinny_kernel(const WoParams p) {
   }
 }
 
+// ---------------------------------------------------------------- M <= 2: matrix times one or two vectors
+// One wave per output channel streams that channel's weight row from end to end -- 64 lanes x
+// 16 bytes = 1 KiB contiguous per load instruction, U of them in flight -- and multiplies it
+// with the activation rows, which the workgroup keeps in LDS (f32 ones as hi and lo halves),
+// on the vector ALUs (v_dot2_f32_f16: the matrix cores have nothing to gain on one or two
+// rows, and a row read linearly keeps one DRAM page open where 16 rows read side by side keep
+// 16).  The lanes' partial sums meet in a butterfly of cross-lane shuffles.
+template <typename XT, int NW, int MR, int U>
+__global__ void __launch_bounds__(NW * 64) wo_gemv_kernel(const WoParams p) {
+  constexpr bool F32 = sizeof(XT) == 4;
+  extern __shared__ __attribute__((aligned(16))) uint8_t wo_lds[];   // [MR][hi | lo][K] halves
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * NW + __builtin_amdgcn_readfirstlane(wave);
+  const int kpad = (p.K + 7) & ~7;                       // (K % 16 == 0 anyway)
+  // the activation rows into LDS, 8 elements per thread and step
+  for (int i = threadIdx.x; i < MR * (kpad >> 3); i += NW * 64) {
+    const int m = i / (kpad >> 3), k = (i - m * (kpad >> 3)) << 3;
+    const XT* src = static_cast<const XT*>(p.x) + (int64_t)min(m, p.M - 1) * p.ldx + k;
+    h8 hi, lo;
+    if constexpr (F32) {
+      const f4 a = *reinterpret_cast<const f4*>(src), b = *reinterpret_cast<const f4*>(src + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float v = e < 4 ? a[e] : b[e - 4];
+        hi[e] = (_Float16)v;
+        lo[e] = (_Float16)(v - (float)hi[e]);
+      }
+      *reinterpret_cast<h8*>(&wo_lds[((2 * m + 1) * kpad + k) * 2]) = lo;
+      *reinterpret_cast<h8*>(&wo_lds[((2 * m) * kpad + k) * 2]) = hi;
+    } else {
+      *reinterpret_cast<h8*>(&wo_lds[(m * kpad + k) * 2]) = *reinterpret_cast<const h8*>(src);
+    }
+  }
+  __syncthreads();
+  if (n >= p.N) return;                                  // (no barrier below)
+  const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(p.w + (int64_t)n * p.w_sn), 0, p.K, kBufferWord3);
+  const h2 c = centre(p, n);
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.0f;
+  for (int k0 = 16 * lane; k0 < p.K; k0 += U * 1024) {
+    u4 wq[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)                          // (past K: zeros, no memory touched)
+      wq[u] = __builtin_amdgcn_raw_buffer_load_b128(wrs, k0 + u * 1024, 0, 0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * 1024;
+      if (k < p.K) {
+        h8 w0, w1;
+        widen16(wq[u], p.flip, c, w0, w1);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+#pragma unroll
+          for (int part = 0; part < (F32 ? 2 : 1); ++part) {
+            const uint8_t* xs = &wo_lds[(((F32 ? 2 * m + part : m) * kpad) + k) * 2];
+            const h8 x0 = *reinterpret_cast<const h8*>(xs), x1 = *reinterpret_cast<const h8*>(xs + 16);
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+              acc[m] = __builtin_amdgcn_fdot2((h2){x0[e], x0[e + 1]}, (h2){w0[e], w0[e + 1]}, acc[m], false);
+              acc[m] = __builtin_amdgcn_fdot2((h2){x1[e], x1[e + 1]}, (h2){w1[e], w1[e + 1]}, acc[m], false);
+            }
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    float v = acc[m];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (lane == 0 && m < p.M) {
+      const float sc = to_f32(static_cast<const XT*>(p.scale)[n]);
+      const float b = p.bias ? to_f32(static_cast<const XT*>(p.bias)[n]) : 0.0f;
+      static_cast<XT*>(p.out)[(int64_t)m * p.ldo + n] = (XT)(v * sc + b);
+    }
+  }
+}
+
 // ---------------------------------------------------------------- 8 < M <= 32, operands through LDS
 // 32 output channels per workgroup like wo_skinny_kernel<.., 1>, the k range dealt over the
 // waves in units of 64.  There every lane fetches its own activation row (32 rows x 32 bytes
@@ -843,6 +926,16 @@ int launch_lds(dim3 grid, const WoParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch");
 }
 
+template <typename XT, int MR, int U>
+int launch_gemv(const WoParams& p, hipStream_t st) {
+  const int lds = MR * ((p.K + 7) & ~7) * (int)sizeof(XT);
+  auto kern = wo_gemv_kernel<XT, 8, MR, U>;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, &lds_allowed)) return s;
+  hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(p.N, 8)), dim3(512), lds, st, p);
+  return check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch");
+}
+
 template <typename XT, int MR>
 int launch_skinny_lds(const WoParams& p, hipStream_t st) {
   constexpr int lds = 8 * (MR * 128 * (int)(sizeof(XT) / 2) + 32 * 64);
@@ -949,6 +1042,16 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
     // kernels below it wins from 12 rows on at 3072 and 4096 of k -- 4096^2 weights, f16, M = 32:
     // 10.7 against 14.9 us -- and from 5 rows on at 8192 -- M = 16: 16.8 against 22.5 us --, and
     // loses about a microsecond at 768 or 1040 of k)
+    // one row, or two where it was measured faster (f32 activations; f16 from 2048 to 8192 of
+    // k), while the rows fit 64 KiB of LDS: the row-streaming kernel on the vector ALUs (4096^2
+    // weights, M = 1: f16 4.3 against 5.8 us, f32 4.5 against 7.5; 8192^2: 13.5 against 15.2 us,
+    // 5.0 TB/s; three and four rows are slower that way than on the matrix cores)
+    if ((p.M == 1 || (p.M == 2 && (sizeof(XT) == 4 || (p.K >= 2048 && p.K <= 8192)))) &&
+        (int64_t)p.M * p.K * (int64_t)sizeof(XT) <= 64 * 1024) {
+      const bool deep = p.K > 4096;
+      if (p.M == 1) return deep ? launch_gemv<XT, 1, 8>(p, st) : launch_gemv<XT, 1, 4>(p, st);
+      return deep ? launch_gemv<XT, 2, 8>(p, st) : launch_gemv<XT, 2, 4>(p, st);
+    }
     if (staged_ok && p.M <= 32 && ((p.K >= 2048 && p.M >= 12) || (p.K >= 6144 && p.M >= 5)))
       return p.M <= 16 ? launch_skinny_lds<XT, 16>(p, st) : launch_skinny_lds<XT, 32>(p, st);
     if (p.M <= 8 || (p.M <= 16 && grid < 256))
