@@ -137,9 +137,26 @@ int launch_skinny_t(const MainParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_skinny launch");
 }
 
+template <int MR, int U, int EPI>
+int launch_gemv_t(const MainParams& p, hipStream_t st) {
+  auto kern = qgemm_gemv_kernel<8, MR, U, EPI>;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), 160 * 1024, &lds_allowed)) return s;
+  hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(p.N, 8)), dim3(512), MR * p.K, st, p);
+  return check_hip(hipGetLastError(), "qgemm_gemv launch");
+}
+
 // rows per workgroup grow with M (fewer passes over W), waves with the depth of K
 template <int EPI>
 int launch_skinny(const MainParams& p, hipStream_t st) {
+  // one or two rows against rows of at least 2048 of k (two steps of a wave): the
+  // row-streaming kernel (M = 1, 3072 -> 768: 3.1 against 4.0 us; 4096^2: 3.8 against 5.0;
+  // 8192^2: 12.7 against 14.2 us, 5.3 TB/s; at 768 of k, and from three rows on, it is slower)
+  if (p.M <= 2 && p.K >= 2048 && (int64_t)2 * p.K <= 64 * 1024) {
+    const bool deep8 = p.K > 4096;
+    if (p.M == 1) return deep8 ? launch_gemv_t<1, 8, EPI>(p, st) : launch_gemv_t<1, 4, EPI>(p, st);
+    return deep8 ? launch_gemv_t<2, 8, EPI>(p, st) : launch_gemv_t<2, 4, EPI>(p, st);
+  }
   const bool deep = p.K >= 1024;
   if (p.M <= 16) return deep ? launch_skinny_t<8, 1, EPI>(p, st) : launch_skinny_t<4, 1, EPI>(p, st);
   if (p.M <= 32) return deep ? launch_skinny_t<8, 2, EPI>(p, st) : launch_skinny_t<4, 2, EPI>(p, st);

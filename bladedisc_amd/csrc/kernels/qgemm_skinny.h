@@ -88,6 +88,67 @@ __global__ void __launch_bounds__(NW * 64) qgemm_skinny_kernel(const MainParams 
   }
 }
 
+// One or two rows: a matrix times a vector or two.  One wave per output channel streams that
+// channel's weight row from end to end -- 64 lanes x 16 bytes = 1 KiB contiguous per load
+// instruction, U of them in flight -- and multiplies it with the activation rows, which the
+// workgroup keeps in LDS, on the vector ALUs (v_dot4_i32_i8); the lanes' sums meet in a
+// butterfly of cross-lane shuffles.  A row read linearly keeps one DRAM page open where 16
+// rows read side by side keep 16, and every output channel is a wave of its own instead of a
+// sixteenth of a workgroup.  Integer sums: the same bits as every other kernel.
+// Needs K % 16 == 0, 16-byte aligned k-contiguous rows and MR * K bytes of LDS.
+template <int NW, int MR, int U, int EPI>
+__global__ void __launch_bounds__(NW * 64) qgemm_gemv_kernel(const MainParams p) {
+  extern __shared__ __attribute__((aligned(16))) int8_t gemv_lds[];      // [MR][K]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * NW + __builtin_amdgcn_readfirstlane(wave);
+  for (int i = threadIdx.x; i < MR * (p.K >> 4); i += NW * 64) {
+    const int m = i / (p.K >> 4), k = (i - m * (p.K >> 4)) << 4;
+    *(v4i*)(gemv_lds + m * p.K + k) =
+        *(const v4i*)(p.A + (int64_t)(m < p.M ? m : p.M - 1) * p.lda + k);
+  }
+  __syncthreads();
+  if (n >= p.N) return;                                    // (no barrier below)
+  const int8_t* wp = p.W + (int64_t)n * p.ldw;
+  int acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0;
+  const v4i zero = {0, 0, 0, 0};
+  for (int k0 = 16 * lane; k0 < p.K; k0 += U * 1024) {
+    v4i wq[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) wq[u] = k0 + u * 1024 < p.K ? *(const v4i*)(wp + k0 + u * 1024) : zero;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * 1024;
+      if (k < p.K) {
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+          const v4i a = *(const v4i*)(gemv_lds + m * p.K + k);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[m] = __builtin_amdgcn_sdot4(a[e], wq[u][e], acc[m], false);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MR; ++m) {
+    int sum = acc[m];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0 && m < p.M) {
+      const EpiParams& ep = p.epi;
+      const ColParams c = col_params<EPI>(ep, n);
+      const int64_t off = (int64_t)m * ep.ldo + n;
+      if (EPI == DQ8_EPI_ACC_S32)
+        ((int32_t*)ep.out)[off] = sum;
+      else if (EPI == DQ8_EPI_DEQUANT_F32)
+        ((float*)ep.out)[off] = finish_f32(ep, dequant_one_any(ep, c, sum, dequant_so(ep)), m, n);
+      else
+        ((int8_t*)ep.out)[off] = (int8_t)finish_s8(ep, requant_one<EPI>(ep, c, sum), m, n);
+    }
+  }
+}
+
 }  // namespace dq8
 
 #endif  // DQ8_QGEMM_SKINNY_H_

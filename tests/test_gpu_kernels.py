@@ -1329,14 +1329,19 @@ def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
     to several rounds of the largest tiles, N, K, the epilogue family, fused operators -- with
     the scalar generic kernel (variant 0, itself pinned against the oracle above) as the
     yardstick on the same device buffers: every combination must give the same bits, whichever
-    kernel the heuristic lands on (small-M, 64 / 128 / 256-wide tiles, persistent forms)."""
+    kernel the heuristic lands on (row-streaming for one or two rows against deep weights,
+    small-M, 64 / 128 / 256-wide tiles, persistent forms)."""
     rng = np.random.default_rng(20260101)
     ms = [1, 7, 16, 31, 33, 100, 500, 1000, 2100, 4096, 9000, 20000]
     cases = 0
-    for m in ms:
-        for _ in range(3):
-            n = int(rng.choice([16, 48, 64, 136, 768, 1024, 2304, 3072]))
-            k = int(rng.choice([16, 64, 144, 768, 1040, 3072]))
+    # (m, n, k): three random (n, k) per m, then one and two rows against rows of 2048 of k and
+    # more, with k ending inside a wave's step and N inside a workgroup's channels
+    shapes = [(m, None, None) for m in ms for _ in range(3)] + \
+             [(1, 100, 3072), (2, 9, 2048), (1, 40, 8208), (2, 130, 4112)]
+    for m, n_fixed, k_fixed in shapes:
+        if True:
+            n = n_fixed or int(rng.choice([16, 48, 64, 136, 768, 1024, 2304, 3072]))
+            k = k_fixed or int(rng.choice([16, 64, 144, 768, 1040, 3072]))
             if m * n * k > 2.2e10:
                 k = 64
             a = dev(rng.integers(-128, 128, (m, k), dtype=np.int8))
@@ -1384,7 +1389,7 @@ def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
                                    want.view(torch.int32) if want.dtype == torch.float32 else want)
                 assert same, (m, n, k, epi, post)
                 cases += 1
-    assert cases == len(ms) * 3 * 8
+    assert cases == len(shapes) * 8
 
 
 def test_conv_dispatch_sweep_agrees_with_the_generic_kernel(K):
