@@ -375,7 +375,10 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
     // persistent form from two tiles per compute unit on -- M = 16384, 768 -> 768 with an f32
     // result: 17.8 against 18.5 us, four waves 23.8)
     if (t128 >= 120) {
-      if (K >= 4096) return kPipe128;
+      // (deep K: four waves; while the 128 x 128 tiles leave compute units idle and the 64 x 64
+      // ones come to at most two per unit, those with the k range split over two wave groups --
+      // M = 256, 8192^2 weights: 28.5 against 33.1 us; M = 512, 4096^2: 16.4 against 18.0)
+      if (K >= 4096) return (t128 < cus && tiles(kPipe64) <= 2 * cus) ? kPipe64k2 : kPipe128;
       if (out_bytes == 1) return t128 <= cus ? kPipe128w8 : kPipe128;
       return t128 > 2 * cus ? kPersist128 : kPipe128w8;
     }
