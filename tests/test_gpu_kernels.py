@@ -1324,6 +1324,55 @@ def test_weight_only_qgemm_split_over_k(K, dtype):
     assert split_seen >= 5
 
 
+def test_multi_kernel_paths_replay_from_a_captured_graph(K):
+    """The paths that are several launches -- a weight-only GEMM split over k (GEMM, then the
+    reduction), a stem convolution through space to depth (two re-layouts, then the
+    convolution) -- captured into one HIP graph with caller-owned scratch and replayed with
+    other work in between: every replay gives the eager result, also after the inputs change."""
+    import bladedisc_amd._lib as _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(808)
+    m, k, n = 128, 2048, 512
+    x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, torch.float16, False)
+    xd, wd, sd, zd, bd = dev(x), dev(w), dev(scale), dev(zp), dev(bias)
+    need = L.dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, 1)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    ci, co, h = 3, 32, 40
+    cx = dev(rng.integers(-128, 128, (2, h, h, ci), dtype=np.int8))
+    cw = dev(rng.integers(-128, 128, (co, 7, 7, ci), dtype=np.int8))
+    md = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
+    osh = [2, h // 2, h // 2, co]
+    cout = torch.empty(tuple(osh), dtype=torch.int32, device="cuda")
+
+    def run():
+        K.weight_only_qgemm(xd, wd, sd, zd, bd, out=out, workspace=ws)
+        K.qconv2d(cx, cw, [3, 3, 3, 3], md, osh, K.EPI_ACC_S32, out=cout)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run()
+    for rep in range(4):
+        if rep == 2:                                       # new inputs in the captured buffers
+            xd.copy_(dev(rng.standard_normal((m, k)).astype(np.float16)))
+            cx.copy_(dev(rng.integers(-128, 128, (2, h, h, ci), dtype=np.int8)))
+        out.zero_()
+        cout.zero_()
+        ws.fill_(0xff)
+        graph.replay()
+        torch.cuda.synchronize()
+        got, cgot = out.clone(), cout.clone()
+        want = K.weight_only_qgemm(xd, wd, sd, zd, bd)
+        cwant = K.qconv2d(cx, cw, [3, 3, 3, 3], md, osh, K.EPI_ACC_S32)
+        assert torch.equal(got, want), rep
+        assert torch.equal(cgot, cwant), rep
+
+
 def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
     """Seeded sweep over what the library's own choice of kernel depends on -- M from one row
     to several rounds of the largest tiles, N, K, the epilogue family, fused operators -- with
