@@ -741,8 +741,10 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     // MODE 0: float stage with its additive terms, 1: without them, 2: fixed-point stage
     auto store_all = [&](auto mode_c) {
       constexpr int MODE = decltype(mode_c)::value;
-#pragma unroll
-      for (int j = 0; j < FN; ++j) {
+      // (static_for: with 16 fragments a loop this size is past what "#pragma unroll" unrolls,
+      // and an accumulator array indexed by a loop variable lives in scratch memory)
+      static_for<FN>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
         const int cl0 = wn_off + j * 32 + 4 * (lane >> 5);
         ColParams c[4][4];
 #pragma unroll
@@ -756,8 +758,8 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
           c[g][2] = {p23[0], p23[1], sh[2]};
           c[g][3] = {p23[2], p23[3], sh[3]};
         }
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
+        static_for<FM>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
           uint32_t w[4];
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
@@ -835,8 +837,8 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
             held[kHook ? i : 0][kHook ? j : 0] = v;
           else
             store_frag(v, i, j);
-        }
-      }
+        });
+      });
     };
     if (fixedpoint)
       store_all(IntC<2>());
@@ -936,28 +938,28 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
   }
 
   // direct stores: 4 consecutive channels of one row per accumulator quad
-#pragma unroll
-  for (int j = 0; j < FN; ++j) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
+  static_for<FN>([&](auto jc) {
+    constexpr int j = decltype(jc)::value;
+    static_for<4>([&](auto gc) {
+      constexpr int g = decltype(gc)::value;
       const int cl = wn_off + j * 32 + 8 * g + 4 * (lane >> 5);
       const int n = n_blk0 + cl;
-      if (n >= e.N) continue;
+      if (n >= e.N) return;
       const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl]);
       const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl + 2]);
       v4i sh = {0, 0, 0, 0};
       if (fixedpoint) sh = *reinterpret_cast<const v4i*>(&cps[cl]);
       const ColParams c[4] = {{p01[0], p01[1], sh[0]}, {p01[2], p01[3], sh[1]},
                               {p23[0], p23[1], sh[2]}, {p23[2], p23[3], sh[3]}};
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
+      static_for<FM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
         const int m = m_wave0 + i * 32 + (lane & 31);
         if (m < m_end)
           store_group4<EPI>(e, m, n, c, acc[i][j][4 * g + 0], acc[i][j][4 * g + 1],
                             acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-      }
-    }
-  }
+      });
+    });
+  });
 }
 
 }  // namespace dq8
