@@ -23,13 +23,13 @@
 // layout: the order of the k values inside a fragment is free as long as both operands agree,
 // so lane (row, g) takes the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes
 // (one dwordx4), 16 activations -- and feeds two MFMAs with them.
-//  * wo_lds_kernel: tiles of 128 x 128, 256 x 128 or 256 x 256 shared through LDS, from 64 tiles
-//    up, and -- with several workgroups per tile, each over a part of k, and
-//    wo_splitk_reduce_kernel behind them -- for 32 < M while the tiles would not fill the chip
-//    (1.06-1.16 PFLOP/s for f16 activations at 4096^2 .. 8192^2 weights, where the ROCm
-//    library's plain f16 GEMM reaches 1.16-1.49);
+//  * wo_lds_kernel: tiles shared through LDS, everything above 32 rows: 64 x 64 or 128 x 128
+//    tiles while the problem is a few rounds of them -- with several workgroups per tile, each
+//    over a part of k, and wo_splitk_reduce_kernel behind them, where that is estimated
+//    cheaper --, 256 x 128 and 256 x 256 tiles beyond (1.06-1.16 PFLOP/s for f16 activations
+//    at 4096^2 .. 8192^2 weights, where the ROCm library's plain f16 GEMM reaches 1.16-1.49);
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
-//    problems with few tiles and little k;
+//    operands too large for the LDS kernel's 31-bit offsets;
 //  * wo_skinny_lds_kernel: 5 .. 32 rows against deep weights, 32 output channels per workgroup,
 //    both operands loaded in row segments and turned into fragments through wave-private LDS;
 //  * wo_gemv_kernel: one or two rows, a wave per output channel streaming its weight row on the
@@ -948,47 +948,125 @@ int launch_skinny_lds(const WoParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "dq8_weight_only_qgemm launch");
 }
 
-// Split plan of the LDS kernel (f16 activations) for problems whose tiles would leave most of
-// the chip idle: `splits` workgroups per tile, each over k_split of the k range, and a
-// reduction kernel behind them.  splits == 1: no split.
+// The small tile forms of the LDS kernel, for problems whose tiles would leave most of the chip
+// idle.  A lone workgroup on a compute unit runs its k tiles as a chain of latencies (LDS
+// reads, MFMAs, hand-over of the next tile, barrier): 0.4 us per k tile with two 32 x 32
+// fragments per wave, 0.27 us with one -- so below a few rounds of tiles the 64 x 64 tile on
+// four waves beats every larger one, although it moves the most bytes per MFMA.
+enum { kForm64x64w2 = 0, kForm128x64, kForm64x128w2, kForm128x128, kForm64x64, kNumForms };
+struct TileForm { int bm, bn; };
+constexpr TileForm kForms[kNumForms] = {{64, 64}, {128, 64}, {64, 128}, {128, 128}, {64, 64}};
+
+// Plan: `splits` workgroups per tile of form `form`, each over k_split of the k range, and
+// (splits > 1) a reduction kernel behind them.  `us`: the estimate it was chosen by.
 struct SplitPlan {
-  int wm;        // tile rows / 64: 1 or 2
+  int form;
   int splits;
   int k_split;
-  int fn = 2;    // tile columns / 64: 1 or 2
+  float us;
 };
 
-SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int esz) {
-  SplitPlan s = {M <= 64 ? 1 : 2, 1, (int)K};
-  // Measured (4096^2, 8192^2, 3072 x 768 and 768 x 3072 weights): up to 32 rows the skinny
-  // kernel wins; a k range below 256 per workgroup is not worth the second launch; and the
-  // partial sums (splits x M x N floats, written and read once) bound the number of splits as
-  // M grows.
-  if (M <= 32 || K < 512) return s;
-  if (K < 1024) {
-    // two or three k ranges of 256: worth it only against the kernels that gather activation
-    // rows lane by lane (all of them for f32 activations, the 65 .. 128-row one for f16) and
-    // while the tiles are few (768 .. 896 of k: M = 128, N = 3072, f16 10.6 against 13.7 us,
-    // f32 13.1 against 23.3; M = 256: 15.0 against 11.6 and 16.0 against 18.2)
-    const int64_t t128 = ceil_div(M, 64 * s.wm) * ceil_div(N, 128);
-    if (esz == 2 ? (M <= 64 || t128 > 32) : t128 > 48) return s;
+// Estimated time of a plan in microseconds, fitted (least squares on relative error, median
+// error 4 %, 90th percentile 10 %) to 3300 timed launches of the 64 x 64 and 128 x 128 forms:
+// M = 40 .. 3072, nine weight shapes from 768 x 768 to 8192 x 8192, 1 .. 16 k ranges.
+//   t = c0 + kt (c1 + c2 (r - 1)) + c3 (r - 1) + [splits > 1] (c4 + c5 M N splits / 1e6)
+// kt: 64-deep k tiles per workgroup; r: workgroups per compute unit, rounded up.
+struct FormCost { float c0, c1, c2, c3, c4, c5; };
+constexpr FormCost kCost64x64[2] = {{4.272f, 0.274f, 0.177f, 0.472f, 2.347f, 1.649f},     // f16
+                                    {5.805f, 0.456f, 0.334f, 0.613f, 1.023f, 1.731f}};    // f32
+constexpr FormCost kCost128x128[2] = {{7.616f, 0.569f, 0.484f, -0.948f, 1.629f, 1.696f},
+                                      {8.471f, 0.919f, 1.175f, -1.589f, -1.035f, 2.310f}};
+
+// The cheapest of the 64 x 64 and 128 x 128 forms with 1, 2, 3, 4, 6 or 8 k ranges of at
+// least 192 (one range only unless `may_split`).  Choosing by this estimate comes within
+// 1.2 % (geometric mean; worst case 14 %) of the best timed plan of each of those problems.
+SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int esz, bool may_split = true) {
+  SplitPlan best = {kForm128x128, 1, (int)K, 0.0f};
+  const int64_t cus = compute_units();
+  for (int form : {(int)kForm64x64, (int)kForm128x128}) {
+    const FormCost& c = (form == kForm64x64 ? kCost64x64 : kCost128x128)[esz == 4];
+    const int64_t tiles = ceil_div(M, kForms[form].bm) * ceil_div(N, kForms[form].bn);
+    for (int want : {1, 2, 3, 4, 6, 8}) {
+      if (want > 1 && (!may_split || K / want < 192)) break;
+      const int64_t k_split = ceil_div(ceil_div(K, (int64_t)want), 64) * 64;
+      const int64_t splits = ceil_div(K, k_split);
+      const float kt = (float)(k_split / 64), r = (float)(ceil_div(tiles * splits, cus) - 1);
+      float us = c.c0 + kt * (c.c1 + c.c2 * r) + c.c3 * r;
+      if (splits > 1) us += c.c4 + c.c5 * (float)((double)(M * N * splits) * 1e-6);
+      if (best.us == 0.0f || us < best.us)
+        best = {form, (int)splits, splits > 1 ? (int)k_split : (int)K, us};
+    }
   }
-  // 64-column tiles while 128-column ones are at most an eighth of the compute units: half
-  // the partial sums per workgroup, so half of them in all (4096^2 weights, M = 64: 15.3
-  // against 19.0 us; 3072 x 768, M = 512: 15.0 against 18.2)
-  if (ceil_div(M, 64 * s.wm) * ceil_div(N, 128) * 8 <= compute_units()) s.fn = 1;
-  const int64_t tiles = ceil_div(M, 64 * s.wm) * ceil_div(N, 64 * s.fn);
-  const int64_t splits = std::min(std::min(compute_units() / tiles, K / 256),
-                                  std::max<int64_t>(1, 4096 / M));
-  if (splits < 2) return s;
-  s.k_split = (int)(ceil_div(ceil_div(K, splits), 64) * 64);
-  s.splits = (int)ceil_div(K, s.k_split);
-  if (s.splits < 2) s.splits = 1, s.k_split = (int)K;
+  return best;
+}
+
+// The 256-row tiles of f16 activations (eight waves, wave tiles 64 x 64 and 64 x 128: the
+// larger the wave tile, the fewer LDS bytes per MFMA) against 128 x 128 ones, by the measured
+// time of a round of each at 4096 of k: 128 x 128 tiles, two workgroups to a compute unit,
+// 82 us for a full round and 45 while one workgroup has the unit to itself; 256 x 128 tiles,
+// one to a unit, 75 us and 60 up to half a round; 256 x 256 tiles 135 us and 100.
+struct BigTiles {
+  int64_t n256x128, n256;     // tiles of the two shapes
+  int64_t cost128, cost256x128, cost256;
+  bool take256() const { return cost256 < cost128 && cost256 <= cost256x128; }
+  bool take256x128() const { return !take256() && cost256x128 < cost128; }
+};
+BigTiles big_tiles(int64_t M, int64_t N) {
+  const int64_t cus = compute_units();
+  auto rounds = [](int64_t tiles, int64_t slots, int64_t half, int full_us, int part_us) {
+    const int64_t rem = tiles % slots;
+    return tiles / slots * full_us + (rem == 0 ? 0 : rem <= half ? part_us : full_us);
+  };
+  BigTiles b;
+  b.n256x128 = ceil_div(M, 256) * ceil_div(N, 128);
+  b.n256 = ceil_div(M, 256) * ceil_div(N, 256);
+  b.cost128 = rounds(ceil_div(M, 128) * ceil_div(N, 128), 2 * cus, cus, 82, 45);
+  b.cost256x128 = rounds(b.n256x128, cus, cus / 2, 75, 60);
+  b.cost256 = rounds(b.n256, cus, cus / 2, 135, 100);
+  return b;
+}
+
+// Estimated time of whichever 256-row tile big_tiles prefers to 128 x 128: 8 us + 0.85 x its
+// rounds scaled to K (fitted to 70 timed launches, median error 9 %); 0 where it prefers none.
+float big_tile_us(int64_t M, int64_t N, int64_t K) {
+  const BigTiles b = big_tiles(M, N);
+  const int64_t cost = b.take256() ? b.cost256 : b.take256x128() ? b.cost256x128 : 0;
+  return cost ? 8.0f + 0.85f * (float)cost * (float)K / 4096.0f : 0.0f;
+}
+
+// The plan for M x N x K, or form = -1 where the small forms are not the choice: up to 32
+// rows the kernels for few rows, and the 256-row tiles where they are estimated cheaper.
+SplitPlan choose_small(int64_t M, int64_t N, int64_t K, int esz, bool may_split) {
+  const SplitPlan none = {-1, 1, (int)K, 0.0f};
+  if (M <= 32) return none;
+  const SplitPlan s = plan_split(M, N, K, esz, may_split);
+  if (esz == 2 && M > 128) {
+    const float big = big_tile_us(M, N, K);
+    if (big > 0.0f && big < s.us) return none;
+  }
   return s;
 }
 
 size_t split_bytes(const SplitPlan& s, int64_t M, int64_t N) {
   return s.splits > 1 ? (size_t)s.splits * (size_t)(M * N) * sizeof(float) : 0;
+}
+
+// one launch of a small tile form over the whole k range (splits == 1) or its split
+template <typename XT>
+int launch_form(int form, int splits, const WoParams& p, hipStream_t st) {
+  constexpr int kSets = sizeof(XT) == 2 ? 4 : 2;         // (f32 rows are twice the registers)
+  const dim3 grid((unsigned)(ceil_div(p.M, kForms[form].bm) * ceil_div(p.N, kForms[form].bn)),
+                  (unsigned)splits);
+  switch (form) {
+    case kForm64x64w2: return launch_lds<XT, 1, 2, 1, kSets>(grid, p, st);
+    case kForm128x64: return launch_lds<XT, 2, 2, 1, kSets>(grid, p, st);
+    case kForm64x128w2: return launch_lds<XT, 1, 2, 2, kSets>(grid, p, st);
+    case kForm128x128:
+      if constexpr (sizeof(XT) == 4) return launch_lds<XT, 4, 1, 2, kSets>(grid, p, st);
+      return launch_lds<XT, 2, 2, 2, kSets>(grid, p, st);
+    case kForm64x64: return launch_lds<XT, 2, 1, 1, kSets>(grid, p, st);
+  }
+  return fail("dq8_weight_only_qgemm: unknown tile form");
 }
 
 template <typename XT>
@@ -999,21 +1077,15 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
   const bool lds_ok = 512 * p.ldx + 4 * (int64_t)p.K + 4096 < (1LL << 31) &&
                       256 * p.w_sn + (int64_t)p.K + 4096 < (1LL << 31);
   if (fast && lds_ok) {
-    const SplitPlan s = plan_split(p.M, p.N, p.K, (int)sizeof(XT));
-    if (s.splits > 1 && scratch && aligned(scratch, 16) &&
-        scratch_bytes >= split_bytes(s, p.M, p.N)) {
-      const int bm = 64 * s.wm;
+    const bool have = scratch && aligned(scratch, 16);
+    SplitPlan s = choose_small(p.M, p.N, p.K, (int)sizeof(XT), have);
+    if (s.splits > 1 && scratch_bytes < split_bytes(s, p.M, p.N))
+      s = choose_small(p.M, p.N, p.K, (int)sizeof(XT), false);
+    if (s.form >= 0 && s.splits > 1) {
       const int sp = s.splits;
       p.partial = static_cast<float*>(scratch);
       p.k_split = s.k_split;
-      const dim3 grid((unsigned)(ceil_div(p.M, bm) * ceil_div(p.N, 64 * s.fn)), (unsigned)sp);
-      constexpr int kSets = sizeof(XT) == 2 ? 4 : 2;       // (f32 rows are twice the registers)
-      if (int e = s.fn == 1 ? (s.wm == 1 ? launch_lds<XT, 1, 2, 1, kSets>(grid, p, st)
-                                         : launch_lds<XT, 2, 2, 1, kSets>(grid, p, st))
-                            : (s.wm == 1          ? launch_lds<XT, 1, 2, 2, kSets>(grid, p, st)
-                               : sizeof(XT) == 4 ? launch_lds<XT, 4, 1, 2, kSets>(grid, p, st)
-                                                 : launch_lds<XT, 2, 2, 2, kSets>(grid, p, st)))
-        return e;
+      if (int e = launch_form<XT>(s.form, sp, p, st)) return e;
       const int vec = (p.N % 4 == 0 && aligned(p.out, 8) && p.ldo % 4 == 0) ? 4 : 1;
       const int64_t blocks = ceil_div((int64_t)p.M * (p.N / vec), 256);
       DQ8_REQUIRE(blocks < (1LL << 31), "dq8_weight_only_qgemm: problem too large");
@@ -1025,6 +1097,7 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
                            st, p, sp);
       return check_hip(hipGetLastError(), "dq8_weight_only_qgemm reduction launch");
     }
+    if (s.form >= 0) return launch_form<XT>(s.form, 1, p, st);
   }
   if (!fast) {
     const int64_t blocks = ceil_div((int64_t)p.M * p.N, 256);
@@ -1064,38 +1137,17 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
     else
       hipLaunchKernelGGL((wo_skinny_kernel<XT, 8, 4>), dim3(grid), dim3(512), 0, st, p);
   } else {
-    // 128 x 128 tiles through LDS once there are enough of them (a lone workgroup's chain of
-    // load, LDS, widen and MFMA latencies is not covered: below that the register kernel,
-    // which is also the one for f32 activations).  256 x 128 and 256 x 256 tiles on eight waves
-    // (wave tiles 64 x 64 and 64 x 128: the larger the wave tile, the fewer LDS bytes per MFMA)
-    // where they come out cheaper by the measured time of a round of each shape at 4096 of k:
-    // 128 x 128 tiles, two workgroups to a compute unit, 82 us for a full round and 45 while one
-    // workgroup has the unit to itself; 256 x 128 tiles, one to a unit, 75 us and 60 up to
-    // half a round; 256 x 256 tiles 135 us and 100.
-    const int64_t big = ceil_div(p.M, 128) * ceil_div(p.N, 128);
-    const int64_t big256 = ceil_div(p.M, 256) * ceil_div(p.N, 128);
-    const int64_t big2 = ceil_div(p.M, 256) * ceil_div(p.N, 256);
-    const int64_t cus = compute_units();
-    auto rounds = [](int64_t tiles, int64_t slots, int64_t half, int full_us, int part_us) {
-      const int64_t rem = tiles % slots;
-      return tiles / slots * full_us + (rem == 0 ? 0 : rem <= half ? part_us : full_us);
-    };
-    const int64_t cost128 = rounds(big, 2 * cus, cus, 82, 45);
-    const int64_t cost256x128 = rounds(big256, cus, cus / 2, 75, 60);
-    const int64_t cost256 = rounds(big2, cus, cus / 2, 135, 100);
+    // (here: the plan above preferred a 256-row tile, or the LDS kernel cannot address the
+    // operands and the register kernel takes the problem)
     if constexpr (sizeof(XT) == 2) {
-      if (cost256 < cost128 && cost256 <= cost256x128 && lds_ok)
-        return launch_lds<XT, 4, 2, 4, 2>(dim3((unsigned)big2), p, st);
-      if (cost256x128 < cost128 && lds_ok)
-        return launch_lds<XT, 4, 2, 2, 4>(dim3((unsigned)big256), p, st);
+      const BigTiles b = big_tiles(p.M, p.N);
+      if (b.take256() && lds_ok)
+        return launch_lds<XT, 4, 2, 4, 2>(dim3((unsigned)b.n256), p, st);
+      if (b.take256x128() && lds_ok)
+        return launch_lds<XT, 4, 2, 2, 4>(dim3((unsigned)b.n256x128), p, st);
     }
-    // (f32 activations: the two half tiles of 256 rows would not leave room for a second stage)
-    if (big >= 64 && lds_ok) {
-      // (f32: the 96 KiB of stages leave one workgroup per compute unit, so it is eight waves
-      // of 32 x 64 rather than four of 64 x 64: 311 against 357 us at 4096^3)
-      if constexpr (sizeof(XT) == 4) return launch_lds<XT, 4, 1, 2, 2>(dim3((unsigned)big), p, st);
-      return launch_lds<XT, 2, 2, 2, 4>(dim3((unsigned)big), p, st);
-    } else if (big >= 192) {
+    const int64_t big = ceil_div(p.M, 128) * ceil_div(p.N, 128);
+    if (big >= 192) {
       hipLaunchKernelGGL((wo_tile_kernel<XT, 2, 2>), dim3((unsigned)big), dim3(256), 0, st, p);
     } else {
       const int64_t small = ceil_div(p.M, 64) * ceil_div(p.N, 64);
@@ -1127,7 +1179,7 @@ extern "C" size_t dq8_weight_only_qgemm_workspace_bytes_ex(int64_t M, int64_t N,
   size_t split = 0;
   if ((x_dtype == DQ8_DTYPE_F16 || x_dtype == DQ8_DTYPE_F32) && K % 16 == 0 && M < (1LL << 31) &&
       N < (1LL << 31) && K < (1LL << 31))
-    split = split_bytes(plan_split(M, N, K, x_dtype == DQ8_DTYPE_F32 ? 4 : 2), M, N);
+    split = split_bytes(choose_small(M, N, K, x_dtype == DQ8_DTYPE_F32 ? 4 : 2, true), M, N);
   if (!split) return dq8_weight_only_qgemm_workspace_bytes(N, K, tp_b);
   return transposed_bytes(N, K, tp_b) + split;
 }

@@ -1324,6 +1324,30 @@ def test_weight_only_qgemm_split_over_k(K, dtype):
     assert split_seen >= 5
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_weight_only_qgemm_few_rounds_of_small_tiles(K, dtype):
+    """Above 32 rows while the tiles are a few rounds of the chip: 64 x 64 tiles on four waves
+    (or 128 x 128), over the whole k range where a split is not estimated to pay -- shallow k,
+    ragged M and N, a k range that is not a multiple of the 64-deep tile, M on both sides of
+    the tile sizes."""
+    import bladedisc_amd._lib as _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(5151)
+    code = 1 if dtype == torch.float16 else 0
+    unsplit_seen = 0
+    for (m, k, n) in [(33, 16, 64), (40, 256, 1024), (64, 272, 100), (65, 768, 3072),
+                      (128, 768, 768), (129, 528, 200), (300, 1024, 4096), (700, 784, 1000),
+                      (1000, 768, 3072)]:
+        x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed=bool(m & 1))
+        unsplit_seen += L.dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, code) == 0
+        args = (dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+        got = K.weight_only_qgemm(*args)
+        _weight_only_check(got, x, w, scale, zp, bias, dtype)
+        assert torch.equal(K.weight_only_qgemm(*args), got)
+        _weight_only_check(K.weight_only_qgemm(*args, workspace=False), x, w, scale, zp, bias, dtype)
+    assert unsplit_seen >= 5
+
+
 def test_multi_kernel_paths_replay_from_a_captured_graph(K):
     """The paths that are several launches -- a weight-only GEMM split over k (GEMM, then the
     reduction), a stem convolution through space to depth (two re-layouts, then the
