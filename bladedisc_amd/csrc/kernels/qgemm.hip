@@ -371,6 +371,20 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
     // the load latency: 6.3 against 7.1 us at M = 2048, 768 -> 768); with two tiles on a
     // compute unit, or a deep K, four waves (10.0 against 11.2 us at M = 2048, 768 -> 3072)
     const int64_t t128 = tiles(kPipe128);
+    // 128 x 128 tiles, two to a compute unit, that end in a round of a few tiles (at most a
+    // quarter of a round) pay a whole k loop for them: the larger tiles, whichever the estimate
+    // prefers, although they leave compute units idle (M = 768, 4096 -> 11008: 516 tiles of
+    // 128 x 128 55.1 us, 174 of 256 x 192 38.4)
+    if (out_bytes == 1 && t128 > 2 * cus && t128 % (2 * cus) != 0 && t128 % (2 * cus) <= cus / 2) {
+      const double kt = (double)ceil_div(K, 128);
+      auto one_round = [&](int64_t t, double per_k, double fixed) {
+        const double busy = (double)(t < cus ? t : cus) / (double)cus;
+        return (double)ceil_div(t, cus) * (kt * per_k * (1.0 + 0.65 * busy * std::sqrt(busy)) / 1.65 + fixed);
+      };
+      const int64_t t192 = tiles(kPipe256x192);
+      if (t256 <= cus && t192 <= cus)
+        return one_round(t192, 1.27, 4.7) < one_round(t256, 1.6, 5.4) ? kPipe256x192 : kPipe256w8;
+    }
     // (int32 / f32 results, four times the bytes to store: eight waves throughout, and the
     // persistent form from two tiles per compute unit on -- M = 16384, 768 -> 768 with an f32
     // result: 17.8 against 18.5 us, four waves 23.8)
@@ -382,7 +396,9 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
       if (out_bytes == 1) return t128 <= cus ? kPipe128w8 : kPipe128;
       return t128 > 2 * cus ? kPersist128 : kPipe128w8;
     }
-    return (K >= 2048 && tiles(kPipe64) <= 256) ? kPipe64k2 : kPipe64;
+    // (64 x 64 tiles: the k range split over two wave groups while they come to at most one per
+    // compute unit, from 4096 of k on at most two -- M = 384, 11008 -> 4096: 37.0 against 40.1 us)
+    return (K >= 2048 && tiles(kPipe64) <= (K >= 4096 ? 2 * cus : cus)) ? kPipe64k2 : kPipe64;
   }
   // (operands the pipelined kernels cannot address: the 128 x 128 and 64 x 64 tiles of the basic
   // kernel; its 256 x 256 form on four waves indexes 256 accumulators per lane and is kept
