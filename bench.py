@@ -557,11 +557,12 @@ def extras(torch, steps, warmup, which="all"):
     # weight-only quantized linear (f16 activations x uint8 weights, per-channel scale and zero
     # point): bound by the weight bytes for small M, by the f16 matrix cores (2.5 PFLOP/s) above
     wo = {}
-    for (k, n) in ((768, 3072), (4096, 4096)):
+    for (k, n, ms) in ((768, 3072, (1, 16, 128, 1024, 4096)), (4096, 4096, (1, 16, 64, 128, 1024, 4096)),
+                       (8192, 8192, (1, 16, 64))):
         wq = torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda")
         sc = (torch.rand(n, device="cuda") * 0.02 + 0.002).half()
         zp = torch.full((n,), 128, dtype=torch.int32, device="cuda")
-        for m in (1, 16, 128, 1024, 4096):
+        for m in ms:
             xh = torch.randn((m, k), device="cuda").half()
             oh = torch.empty((m, n), dtype=torch.float16, device="cuda")
             t = time_graph(torch, [FnCall(lambda: K.weight_only_qgemm(xh, wq, sc, zp, out=oh))])
