@@ -361,7 +361,8 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
       const int64_t t192 = tiles(kPipe256x192);
       bool p256 = false, p192 = false;
       const double e256 = big256 ? estimate(t256, 1.6, 5.4, &p256) : 1e30;
-      const double e192 = t192 >= 200 ? estimate(t192, 1.27, 4.7, &p192) : 1e30;
+      // (from 180 tiles: M = 1152, 2048 -> 7424, 195 tiles: 24.3 against 27.2 us on 145 of 256 x 256)
+      const double e192 = t192 >= 180 ? estimate(t192, 1.27, 4.7, &p192) : 1e30;
       if (e192 < e256) return p192 ? kPersist256x192 : kPipe256x192;
       if (big256) return p256 ? kPersist256 : kPipe256w8;
     } else if (big256) {
