@@ -992,7 +992,7 @@ SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int esz, bool may_split = 
       const int64_t splits = ceil_div(K, k_split);
       const float kt = (float)(k_split / 64), r = (float)(ceil_div(tiles * splits, cus) - 1);
       float us = c.c0 + kt * (c.c1 + c.c2 * r) + c.c3 * r;
-      if (splits > 1) us += c.c4 + c.c5 * (float)((double)(M * N * splits) * 1e-6);
+      if (splits > 1) us += c.c4 + c.c5 * (float)((double)M * (double)N * (double)splits * 1e-6);
       if (best.us == 0.0f || us < best.us)
         best = {form, (int)splits, splits > 1 ? (int)k_split : (int)K, us};
     }
