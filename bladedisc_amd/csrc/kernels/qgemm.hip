@@ -409,13 +409,19 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
   return 3;
 }
 
-// The small-M kernel up to kSkinnyMaxM rows -- except for 17 .. 32 rows against weights large
-// enough to give the 64 x 64 tile with its k range split over two wave groups 128 workgroups
-// (M = 32, 8192 x 8192 weights: 18.5 against 24.6 us; 4096 x 4096: 9.1 against 8.5) -- and the
-// tiled kernels above.
+// The small-M kernel up to kSkinnyMaxM rows -- except against weights wide enough to give the
+// 64 x 64 tile with its k range split over two wave groups a workgroup for every second compute
+// unit or more: its time hardly depends on M, the small-M kernel's grows with it.  From 17 rows
+// at 128 tiles (M = 32, 8192 x 8192 weights: 18.5 against 24.6 us; 4096 x 4096: 9.1 against
+// 8.5), from 9 rows at 144 (M = 16, 4096 -> 11008: 12.0 against 14.2 us; at 128 tiles, 8192^2,
+// 18.7 against 17.9), from 3 rows at 224 (M = 4, 4096 -> 16384: 13.2 against 15.1 us; M = 16,
+// 8192 -> 16384: 22.0 against 32.0) -- and the tiled kernels above.
 int pick_any(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes) {
   if (M <= kSkinnyMaxM) {
-    if (M > 16 && pipe && K >= 2048 && ceil_div(N, 64) >= 128) return kPipe64k2;
+    const int64_t t64 = ceil_div(N, 64);
+    if (pipe && K >= 2048 &&
+        ((M > 16 && t64 >= 128) || (M >= 9 && t64 >= 144) || (M >= 3 && t64 >= 224)))
+      return kPipe64k2;
     return kSkinnyVariant;
   }
   return pick_variant(M, N, K, pipe, out_bytes);

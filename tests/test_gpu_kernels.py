@@ -1408,9 +1408,11 @@ def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
     ms = [1, 7, 16, 31, 33, 100, 500, 1000, 2100, 4096, 9000, 20000]
     cases = 0
     # (m, n, k): three random (n, k) per m, then one and two rows against rows of 2048 of k and
-    # more, with k ending inside a wave's step and N inside a workgroup's channels
+    # more, with k ending inside a wave's step and N inside a workgroup's channels, then few
+    # rows against weights wide enough for the tiled kernel to take them
     shapes = [(m, None, None) for m in ms for _ in range(3)] + \
-             [(1, 100, 3072), (2, 9, 2048), (1, 40, 8208), (2, 130, 4112)]
+             [(1, 100, 3072), (2, 9, 2048), (1, 40, 8208), (2, 130, 4112),
+              (3, 14400, 2048), (9, 9250, 2064), (16, 9216, 2048), (8, 9216, 2048)]
     for m, n_fixed, k_fixed in shapes:
         if True:
             n = n_fixed or int(rng.choice([16, 48, 64, 136, 768, 1024, 2304, 3072]))
