@@ -23,15 +23,16 @@
 // layout: the order of the k values inside a fragment is free as long as both operands agree,
 // so lane (row, g) takes the 16 consecutive k values k0 + 16 g .. of its row -- 16 weight bytes
 // (one dwordx4), 16 activations -- and feeds two MFMAs with them.
-//  * wo_lds_kernel: tiles shared through LDS, everything above 32 rows: 64 x 64 or 128 x 128
+//  * wo_lds_kernel: tiles shared through LDS, everything above 32 rows (16 for f32): 64 x 64 or 128 x 128
 //    tiles while the problem is a few rounds of them -- with several workgroups per tile, each
 //    over a part of k, and wo_splitk_reduce_kernel behind them, where that is estimated
 //    cheaper --, 256 x 128 and 256 x 256 tiles beyond (1.06-1.16 PFLOP/s for f16 activations
 //    at 4096^2 .. 8192^2 weights, where the ROCm library's plain f16 GEMM reaches 1.16-1.49);
 //  * wo_tile_kernel: 2 x 2 waves, wave tile (32 FM) x (32 FN), operands straight into registers:
 //    operands too large for the LDS kernel's 31-bit offsets;
-//  * wo_skinny_lds_kernel: 5 .. 32 rows against deep weights, 32 output channels per workgroup,
-//    both operands loaded in row segments and turned into fragments through wave-private LDS;
+//  * wo_skinny_lds_kernel: 5 .. 32 rows (16 for f32 activations) against deep or wide weights,
+//    32 output channels per workgroup, both operands loaded in row segments and turned into
+//    fragments through wave-private LDS;
 //  * wo_gemv_kernel: one or two rows, a wave per output channel streaming its weight row on the
 //    vector ALUs;
 //  * wo_skinny16_kernel: M <= 16 rows against 16 output channels per workgroup (16x16x32 MFMA);
@@ -1035,10 +1036,12 @@ float big_tile_us(int64_t M, int64_t N, int64_t K) {
 }
 
 // The plan for M x N x K, or form = -1 where the small forms are not the choice: up to 32
-// rows the kernels for few rows, and the 256-row tiles where they are estimated cheaper.
+// rows (16 for f32 activations, whose staged kernel pays for two half tiles: M = 32,
+// 4096 -> 11008: 25.5 against 33.5 us; 4096^2: 15.7 against 17.9; 8192^2: 33.1 against 31.2) the
+// kernels for few rows, and the 256-row tiles where they are estimated cheaper.
 SplitPlan choose_small(int64_t M, int64_t N, int64_t K, int esz, bool may_split) {
   const SplitPlan none = {-1, 1, (int)K, 0.0f};
-  if (M <= 32) return none;
+  if (M <= (esz == 4 ? 16 : 32)) return none;
   const SplitPlan s = plan_split(M, N, K, esz, may_split);
   if (esz == 2 && M > 128) {
     const float big = big_tile_us(M, N, K);
@@ -1125,7 +1128,11 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
       if (p.M == 1) return deep ? launch_gemv<XT, 1, 8>(p, st) : launch_gemv<XT, 1, 4>(p, st);
       return deep ? launch_gemv<XT, 2, 8>(p, st) : launch_gemv<XT, 2, 4>(p, st);
     }
-    if (staged_ok && p.M <= 32 && ((p.K >= 2048 && p.M >= 12) || (p.K >= 6144 && p.M >= 5)))
+    // (and from 5 rows on against weights of at least 8192 channels, where its 32-channel
+    // workgroups fill the chip: 4096 -> 16384, M = 8: f16 17.7 against 19.6 us, f32 23.7
+    // against 30.5)
+    if (staged_ok && p.M <= 32 &&
+        ((p.K >= 2048 && p.M >= 12) || (p.M >= 5 && (p.K >= 6144 || (p.K >= 2048 && p.N >= 8192)))))
       return p.M <= 16 ? launch_skinny_lds<XT, 16>(p, st) : launch_skinny_lds<XT, 32>(p, st);
     if (p.M <= 8 || (p.M <= 16 && grid < 256))
       hipLaunchKernelGGL((wo_skinny16_kernel<XT, 8>), dim3((unsigned)ceil_div(p.N, 16)), dim3(512),

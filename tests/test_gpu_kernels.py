@@ -1270,11 +1270,13 @@ def test_weight_only_qgemm_one_or_two_rows(K, dtype):
 def test_weight_only_qgemm_small_m_staged_through_lds(K, dtype):
     """5 .. 32 rows against deep weights: the kernel that stages both operands through
     wave-private LDS (16 and 32 staged rows; k depths that end inside a unit of 64 and inside
-    a group of three units; N that ends inside a workgroup's 32 channels; signed weights)."""
+    a group of three units; N that ends inside a workgroup's 32 channels; signed weights; few
+    rows against 8192 channels and more, where it starts at five rows whatever the depth).
+    With f32 activations it ends at 16 rows and the tiled kernel takes the rest."""
     rng = np.random.default_rng(99)
     for (m, k, n, signed) in [(12, 2048, 96, False), (16, 3072, 768, False), (17, 2064, 100, True),
                               (32, 4096, 330, False), (5, 6160, 72, True), (9, 8192, 64, False),
-                              (31, 2048 + 16 * 9, 40, False)]:
+                              (31, 2048 + 16 * 9, 40, False), (7, 2048, 8200, False)]:
         x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed)
         got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
         _weight_only_check(got, x, w, scale, zp, bias, dtype)
