@@ -1131,6 +1131,13 @@ int launch(WoParams& p, bool fast, void* scratch, size_t scratch_bytes, hipStrea
     // (and from 5 rows on against weights of at least 8192 channels, where its 32-channel
     // workgroups fill the chip: 4096 -> 16384, M = 8: f16 17.7 against 19.6 us, f32 23.7
     // against 30.5)
+    // (three and four rows that way only against narrow weights, where a workgroup per 16
+    // channels leaves most compute units idle: 3072 -> 768, M = 4: f16 5.3 against 5.5 us, f32
+    // 6.1 against 7.8; 8192 -> 1024: 8.0 against 9.5 and 10.2 against 13.0; at 4096 channels
+    // and more the matrix cores win)
+    if (p.M >= 3 && p.M <= 4 && p.N <= 1024 && p.K >= 2048 &&
+        (int64_t)4 * p.K * (int64_t)sizeof(XT) <= 128 * 1024)
+      return p.K > 4096 ? launch_gemv<XT, 4, 8>(p, st) : launch_gemv<XT, 4, 4>(p, st);
     if (staged_ok && p.M <= 32 &&
         ((p.K >= 2048 && p.M >= 12) || (p.M >= 5 && (p.K >= 6144 || (p.K >= 2048 && p.N >= 8192)))))
       return p.M <= 16 ? launch_skinny_lds<XT, 16>(p, st) : launch_skinny_lds<XT, 32>(p, st);

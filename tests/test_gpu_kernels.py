@@ -1250,14 +1250,17 @@ def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_weight_only_qgemm_one_or_two_rows(K, dtype):
-    """One or two activation rows: the row-streaming kernel on the vector ALUs (k depths that
-    end inside a wave's 1 KiB step and inside a group of steps, N that ends inside a
-    workgroup's 8 channels, signed weights, strided activations, no bias / zero points), and a
-    k depth whose rows do not fit the LDS, which the matrix-core kernels take."""
+    """One or two activation rows (three or four against narrow weights): the row-streaming
+    kernel on the vector ALUs (k depths that end inside a wave's 1 KiB step and inside a group
+    of steps, N that ends inside a workgroup's 8 channels, signed weights, strided activations,
+    no bias / zero points), and a k depth whose rows do not fit the LDS, which the matrix-core
+    kernels take."""
     rng = np.random.default_rng(1234)
     for (m, k, n, signed) in [(1, 16, 1, False), (1, 768, 3072, False), (1, 4096, 100, True),
                               (2, 2064, 77, False), (1, 8192 + 48, 19, False), (2, 8192, 64, True),
-                              (1, 1024 * 5 + 16, 9, False), (1, 40000, 24, False), (2, 20000, 24, False)]:
+                              (1, 1024 * 5 + 16, 9, False), (1, 40000, 24, False), (2, 20000, 24, False),
+                              (3, 3072, 768, False), (4, 2064, 77, True), (4, 8192 + 48, 1024, False),
+                              (3, 16384, 20, False), (4, 2048, 1030, False)]:
         x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed)
         got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
         _weight_only_check(got, x, w, scale, zp, bias, dtype)
