@@ -337,6 +337,15 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
 //    only 6-10 % from 256 tiles of 256x192 and not the 25 % its idle quarter suggests.  The
 //    persistent form saves the first-tile latency and the hand-over (1.5 us per tile) from
 //    the second tile of a workgroup on and costs about 1 us per launch.
+// 64 x 64 tiles with the k range split inside the workgroup: over two wave groups, and over
+// four from 8192 of k on while there is at most a tile per compute unit (M = 128,
+// 11008 -> 4096: 20.8 against 23.4 us; M = 32, 8192^2: 17.1 against 18.8; M = 256, 16384 -> 1024:
+// 25.4 against 30.7; at 3072 of k the wider reduction costs more than the shorter loop saves)
+int pick_k_split64(int64_t M, int64_t N, int64_t K) {
+  const int64_t t64 = ceil_div(M, 64) * ceil_div(N, 64);
+  return (K >= 8192 && t64 <= compute_units()) ? kPipe64k4 : kPipe64k2;
+}
+
 int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) {
   auto tiles = [&](int v) { return ceil_div(M, kVariants[v].bm) * ceil_div(N, kVariants[v].bn); };
   if (pipe) {
@@ -393,13 +402,15 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
       // (deep K: four waves; while the 128 x 128 tiles leave compute units idle and the 64 x 64
       // ones come to at most two per unit, those with the k range split over two wave groups --
       // M = 256, 8192^2 weights: 28.5 against 33.1 us; M = 512, 4096^2: 16.4 against 18.0)
-      if (K >= 4096) return (t128 < cus && tiles(kPipe64) <= 2 * cus) ? kPipe64k2 : kPipe128;
+      if (K >= 4096)
+        return (t128 < cus && tiles(kPipe64) <= 2 * cus) ? pick_k_split64(M, N, K) : kPipe128;
       if (out_bytes == 1) return t128 <= cus ? kPipe128w8 : kPipe128;
       return t128 > 2 * cus ? kPersist128 : kPipe128w8;
     }
     // (64 x 64 tiles: the k range split over two wave groups while they come to at most one per
     // compute unit, from 4096 of k on at most two -- M = 384, 11008 -> 4096: 37.0 against 40.1 us)
-    return (K >= 2048 && tiles(kPipe64) <= (K >= 4096 ? 2 * cus : cus)) ? kPipe64k2 : kPipe64;
+    return (K >= 2048 && tiles(kPipe64) <= (K >= 4096 ? 2 * cus : cus)) ? pick_k_split64(M, N, K)
+                                                                        : kPipe64;
   }
   // (operands the pipelined kernels cannot address: the 128 x 128 and 64 x 64 tiles of the basic
   // kernel; its 256 x 256 form on four waves indexes 256 accumulators per lane and is kept
@@ -421,7 +432,7 @@ int pick_any(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes) {
     const int64_t t64 = ceil_div(N, 64);
     if (pipe && K >= 2048 &&
         ((M > 16 && t64 >= 128) || (M >= 9 && t64 >= 144) || (M >= 3 && t64 >= 224)))
-      return kPipe64k2;
+      return pick_k_split64(M, N, K);
     return kSkinnyVariant;
   }
   return pick_variant(M, N, K, pipe, out_bytes);

@@ -57,6 +57,8 @@ inline constexpr Variant kVariants[] = {
     // the third direct-convolution tile: 512 pixels on eight waves, one workgroup per compute
     // unit (convolution only)
     {"direct3x3_512x64", 512, 64, 128, 512},
+    // 64x64 with the k tiles split over 4 groups of waves (sixteen waves, 128 KiB LDS)
+    {"pipe_64x64x128_k4", 64, 64, 128, 1024},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
@@ -66,12 +68,13 @@ constexpr int kPipe256w8 = 12, kPipe128w8 = 13;
 constexpr int kPersist256 = 14, kPersist128 = 15;
 constexpr int kPipe256x192 = 16, kPersist256x192 = 17;
 constexpr int kDirectConv2 = 18;   // the third direct variant (configuration 2)
+constexpr int kPipe64k4 = 19;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 
 inline bool is_pipe_variant(int v) {
   return v == kPipe256 || v == kPipe128 || v == kPipe64 || v == kPipe256x64 || v == kPipe64k2 ||
-         v == kPipe256w8 || v == kPipe128w8 || v == kPersist256 ||
+         v == kPipe64k4 || v == kPipe256w8 || v == kPipe128w8 || v == kPersist256 ||
          v == kPersist128 || v == kPipe256x192 || v == kPersist256x192;
 }
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -177,6 +180,7 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
     case kPipe64: return launch_pipe<64, 64, 2, 2, 1, CONV, EPI>(p, st);
     case kPipe256x64: return launch_pipe<256, 64, 4, 1, 1, CONV, EPI>(p, st);
     case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, CONV, EPI>(p, st);
+    case kPipe64k4: return launch_pipe<64, 64, 2, 2, 4, CONV, EPI>(p, st);
     case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, CONV, EPI>(p, st);
     case kPipe128w8: return launch_pipe<128, 128, 2, 4, 1, CONV, EPI>(p, st);
     case kPipe256x192: return launch_pipe<256, 192, 4, 2, 1, CONV, EPI>(p, st);
