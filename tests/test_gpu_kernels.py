@@ -1414,10 +1414,12 @@ def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
     cases = 0
     # (m, n, k): three random (n, k) per m, then one and two rows against rows of 2048 of k and
     # more, with k ending inside a wave's step and N inside a workgroup's channels, then few
-    # rows against weights wide enough for the tiled kernel to take them
+    # rows against weights wide enough for the tiled kernel to take them, then k deep enough
+    # for the split over four wave groups
     shapes = [(m, None, None) for m in ms for _ in range(3)] + \
              [(1, 100, 3072), (2, 9, 2048), (1, 40, 8208), (2, 130, 4112),
-              (3, 14400, 2048), (9, 9250, 2064), (16, 9216, 2048), (8, 9216, 2048)]
+              (3, 14400, 2048), (9, 9250, 2064), (16, 9216, 2048), (8, 9216, 2048),
+              (40, 1000, 8192), (100, 520, 8208)]
     for m, n_fixed, k_fixed in shapes:
         if True:
             n = n_fixed or int(rng.choice([16, 48, 64, 136, 768, 1024, 2304, 3072]))
