@@ -1353,6 +1353,24 @@ def test_weight_only_qgemm_few_rounds_of_small_tiles(K, dtype):
     assert unsplit_seen >= 5
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_weight_only_qgemm_strided_rows_in_and_out(K, dtype):
+    """Activation and result rows that are slices of wider buffers (ldx > K, ldo > N), one shape
+    per kernel family (row-streaming, 16-channel, staged, 64 x 64 tiles unsplit and split over
+    k, 128-row and 256-row tiles): right results, and nothing written outside the slice."""
+    rng = np.random.default_rng(5)
+    for (m, k, n) in [(1, 4096, 100), (4, 3072, 768), (8, 768, 200), (8, 2048, 8200),
+                      (24, 2064, 300), (40, 4096, 520), (100, 784, 200), (300, 1024, 1000),
+                      (64, 8192, 264), (1000, 768, 3072), (2100, 256, 520)]:
+        x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, False)
+        wide = dev(np.concatenate([x, x], axis=1))
+        frame = torch.full((m, n + 24), 7.0, dtype=dtype, device="cuda")
+        out = frame[:, 8:8 + n]
+        K.weight_only_qgemm(wide[:, :k], dev(w), dev(scale), dev(zp), dev(bias), out=out)
+        _weight_only_check(out, x, w, scale, zp, bias, dtype)
+        assert bool((frame[:, :8] == 7).all()) and bool((frame[:, 8 + n:] == 7).all())
+
+
 def test_multi_kernel_paths_replay_from_a_captured_graph(K):
     """The paths that are several launches -- a weight-only GEMM split over k (GEMM, then the
     reduction), a stem convolution through space to depth (two re-layouts, then the
