@@ -1036,12 +1036,15 @@ float big_tile_us(int64_t M, int64_t N, int64_t K) {
 }
 
 // The plan for M x N x K, or form = -1 where the small forms are not the choice: up to 32
-// rows (16 for f32 activations, whose staged kernel pays for two half tiles: M = 32,
-// 4096 -> 11008: 25.5 against 33.5 us; 4096^2: 15.7 against 17.9; 8192^2: 33.1 against 31.2) the
-// kernels for few rows, and the 256-row tiles where they are estimated cheaper.
+// rows (16 for f32 activations from 2048 of k on, where the staged kernel pays for two half
+// tiles: M = 32, 4096 -> 11008: 25.5 against 33.5 us; 4096^2: 15.7 against 17.9; 8192^2: 33.1
+// against 31.2) the kernels for few rows, and the 256-row tiles where they are estimated
+// cheaper.
 SplitPlan choose_small(int64_t M, int64_t N, int64_t K, int esz, bool may_split) {
   const SplitPlan none = {-1, 1, (int)K, 0.0f};
-  if (M <= (esz == 4 ? 16 : 32)) return none;
+  // (f32, between: 1536 x 1536 weights, M = 24: 10.0 against 11.2 us, M = 17: 9.5 against 9.2;
+  // 768 -> 3072, M = 24: 8.7 against 7.6)
+  if (M <= (esz == 4 && K >= 2048 ? 16 : esz == 4 && K >= 1280 ? 23 : 32)) return none;
   const SplitPlan s = plan_split(M, N, K, esz, may_split);
   if (esz == 2 && M > 128) {
     const float big = big_tile_us(M, N, K);
