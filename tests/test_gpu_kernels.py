@@ -1371,6 +1371,32 @@ def test_weight_only_qgemm_strided_rows_in_and_out(K, dtype):
         assert bool((frame[:, :8] == 7).all()) and bool((frame[:, 8 + n:] == 7).all())
 
 
+def test_weight_only_dispatch_sweep_stays_within_the_accumulation_bound(K):
+    """Seeded sweep over what the launcher's choice depends on -- rows from 1 to several rounds
+    of tiles, k from one 16-chunk to 9000, narrow to wide weights, both activation types,
+    signed and unsigned weights: whichever kernel the rules and the cost estimate land on,
+    the result stays within the accumulation bound of the oracle."""
+    rng = np.random.default_rng(20260202)
+    ms = [1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256,
+          300, 512, 700, 1100]
+    cases = []
+    for m in ms:
+        for _ in range(2):
+            k = 16 * int(rng.integers(1, 560))
+            n = int(rng.integers(1, 3000))
+            while m * k * n > 1.2e9:
+                n = max(1, n // 2)
+            cases.append((m, k, n))
+    # few rows against wide weights, deep k against narrow ones
+    cases += [(5, 2048, 8200), (11, 2064, 9000), (24, 2048, 8192), (4, 8192, 1000),
+              (3, 2048, 1024), (24, 1536, 1536), (40, 8192, 520), (2100, 256, 4100)]
+    for i, (m, k, n) in enumerate(cases):
+        dtype = torch.float16 if i % 2 == 0 else torch.float32
+        x, w, scale, zp, bias = _weight_only_case(rng, m, k, n, dtype, signed=bool(i % 3 == 0))
+        got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+        _weight_only_check(got, x, w, scale, zp, bias, dtype)
+
+
 def test_multi_kernel_paths_replay_from_a_captured_graph(K):
     """The paths that are several launches -- a weight-only GEMM split over k (GEMM, then the
     reduction), a stem convolution through space to depth (two re-layouts, then the
