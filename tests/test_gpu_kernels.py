@@ -1526,6 +1526,7 @@ def test_conv_dispatch_sweep_agrees_with_the_generic_kernel(K):
     fused table."""
     rng = np.random.default_rng(20260102)
     cases = 0
+    shapes = []
     for _ in range(30):
         nb = int(rng.choice([1, 2, 8, 32, 70]))
         h = int(rng.choice([7, 14, 28, 33, 56]))
@@ -1536,6 +1537,10 @@ def test_conv_dispatch_sweep_agrees_with_the_generic_kernel(K):
         stride = int(rng.choice([1, 1, 2]))
         dil = int(rng.choice([1, 1, 2]))
         pad = int(rng.integers(0, 3))
+        shapes.append((nb, h, w_, ci, co, k, stride, dil, pad))
+    # k deep enough for the 64 x 64 tiles to split it over four wave groups
+    shapes += [(8, 7, 7, 1024, 256, 3, 1, 1, 1), (1, 10, 10, 1040, 70, 3, 1, 1, 0)]
+    for (nb, h, w_, ci, co, k, stride, dil, pad) in shapes:
         ho = (h + 2 * pad - dil * (k - 1) - 1) // stride + 1
         wo = (w_ + 2 * pad - dil * (k - 1) - 1) // stride + 1
         if ho <= 0 or wo <= 0 or nb * ho * wo * co * k * k * ci > 6e10:
