@@ -1184,6 +1184,30 @@ namespace {
 size_t transposed_bytes(int64_t N, int64_t K, int tp_b) {
   return (tp_b || N <= 0 || K <= 0) ? 0 : ((size_t)(N * K) + 255) / 256 * 256;
 }
+// Undoes the byte permutation the reference's compiler applies to a constant [K, N] ui8 weight
+// (R tao_compiler/mlir/disc/transforms/disc_transform_weight_data_layout_for_weight_only_gemm.cc
+// :54-300 as composed at :362-370: rows permuted in blocks of 16, transpose, column pairs
+// interleaved in tiles of 64 rows, bytes 1 and 2 of every word swapped).  Composed, the 16
+// bytes W^T[n, 16 j .. 16 j + 15] sit in one 16-byte group of the reordered buffer, at byte
+//   (n / 2) * 2 K + (16 j / 64) * 128 + (n % 2) * 64 + (16 j) % 64,
+// even bytes of the group = the first eight k, odd bytes = the last eight.  One thread per
+// group: a 16-byte load, four byte permutes, a 16-byte store into the kernels' [N, K] layout.
+__global__ void __launch_bounds__(256)
+wo_undo_compiler_layout_kernel(const u4* __restrict__ src, u4* __restrict__ dst, int N, int K16) {
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= (int64_t)N * K16) return;
+  const int n = (int)(g / K16), j = (int)(g % K16);
+  const int64_t off16 = (int64_t)(n >> 1) * (2 * K16) + (j >> 2) * 8 + (n & 1) * 4 + (j & 3);
+  const u4 v = __builtin_nontemporal_load(src + off16);
+  u4 r;
+  // v_perm_b32 selector bytes: 0-3 pick from the second operand, 4-7 from the first
+  r.x = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u);   // k 0..3  = bytes 0,2 of words 0,1
+  r.y = __builtin_amdgcn_perm(v.w, v.z, 0x06040200u);   // k 4..7  = bytes 0,2 of words 2,3
+  r.z = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);   // k 8..11 = bytes 1,3 of words 0,1
+  r.w = __builtin_amdgcn_perm(v.w, v.z, 0x07050301u);   // k 12..15
+  dst[g] = r;
+}
+
 }  // namespace
 
 extern "C" size_t dq8_weight_only_qgemm_workspace_bytes(int64_t N, int64_t K, int tp_b) {
@@ -1199,6 +1223,27 @@ extern "C" size_t dq8_weight_only_qgemm_workspace_bytes_ex(int64_t M, int64_t N,
     split = split_bytes(choose_small(M, N, K, x_dtype == DQ8_DTYPE_F32 ? 4 : 2, true), M, N);
   if (!split) return dq8_weight_only_qgemm_workspace_bytes(N, K, tp_b);
   return transposed_bytes(N, K, tp_b) + split;
+}
+
+extern "C" int dq8_weight_only_undo_compiler_layout(const uint8_t* reordered, uint8_t* w_nk,
+                                                    int64_t K, int64_t N, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(K >= 0 && N >= 0 && K < (1LL << 31) && N < (1LL << 31),
+              "dq8_weight_only_undo_compiler_layout: bad shape");
+  // (outside these shapes the compiler's pass reads and writes out of bounds: not a permutation)
+  DQ8_REQUIRE(K % 64 == 0 && N % 4 == 0,
+              "dq8_weight_only_undo_compiler_layout: the compiler's weight layout is defined for "
+              "K % 64 == 0 and N % 4 == 0 only");
+  if (K == 0 || N == 0) return 0;
+  DQ8_REQUIRE(reordered && w_nk, "dq8_weight_only_undo_compiler_layout: null pointer");
+  DQ8_REQUIRE(aligned(reordered, 16) && aligned(w_nk, 16),
+              "dq8_weight_only_undo_compiler_layout: buffers must be 16-byte aligned");
+  DQ8_REQUIRE(reordered != w_nk, "dq8_weight_only_undo_compiler_layout: not in place");
+  const int64_t groups = N * (K / 16);
+  hipLaunchKernelGGL(wo_undo_compiler_layout_kernel, dim3((unsigned)ceil_div(groups, 256)),
+                     dim3(256), 0, (hipStream_t)stream, reinterpret_cast<const u4*>(reordered),
+                     reinterpret_cast<u4*>(w_nk), (int)N, (int)(K / 16));
+  return check_hip(hipGetLastError(), "dq8_weight_only_undo_compiler_layout launch");
 }
 
 extern "C" int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, const void* w,

@@ -390,10 +390,18 @@ BaseHipExecutionContext::~BaseHipExecutionContext() {
 }
 
 bool isPersistentDeviceBuffer(ExecutionContext* ctx, const_buffer_t buffer) {
-  auto* state = ctx->getResource<BaseHipContextState>(kRalBaseHipContextState);
-  if (!state) return false;
-  std::lock_guard<std::mutex> guard(state->mu);
-  return state->device_persistent_buffers.count(buffer) != 0;
+  if (auto* state = ctx->getResource<BaseHipContextState>(kRalBaseHipContextState)) {
+    std::lock_guard<std::mutex> guard(state->mu);
+    if (state->device_persistent_buffers.count(buffer) != 0) return true;
+  }
+  // constants of the process-level store come from hipMalloc, not from this context
+  if (auto* consts = ctx->getResource<RalGlobalConstantState>(kRalGlobalConstantState)) {
+    if (ProcessLevelConstStore* store = consts->process_level_store) {
+      std::lock_guard<std::mutex> guard(store->state.mu);
+      return store->state.device_constant_buffers.count(buffer) != 0;
+    }
+  }
+  return false;
 }
 
 buffer_t processLevelDeviceAlloc(size_t bytes) {

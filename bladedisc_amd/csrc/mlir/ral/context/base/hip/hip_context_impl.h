@@ -158,6 +158,9 @@ struct RalGlobalConstantState : public Context::Resource {
   std::mutex mu;
   std::unordered_map<std::string, Item> host_constants;
   std::unordered_map<std::string, Item> device_constants;
+  // addresses of the device constants above (what isPersistentDeviceBuffer consults for the
+  // process-level store, whose buffers belong to no context's allocator)
+  std::unordered_set<const_buffer_t> device_constant_buffers;
   std::unique_ptr<MetadataFile> metadata;
   // if set, the constants live in this store, shared by every context of the process that was
   // made from the same metadata file, instead of in the maps above
@@ -192,7 +195,8 @@ bool discEnableGlobalConstantStore();
 buffer_t processLevelDeviceAlloc(size_t bytes);
 void processLevelDeviceFree(buffer_t buffer);
 
-// device buffers that outlive executions (alloc_persistent): true if `buffer` is one
+// device buffers that outlive executions (alloc_persistent, and the constants of the
+// process-level store): true if `buffer` is one
 bool isPersistentDeviceBuffer(ExecutionContext* ctx, const_buffer_t buffer);
 
 }  // namespace gpu

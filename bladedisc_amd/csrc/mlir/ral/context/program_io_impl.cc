@@ -151,6 +151,7 @@ buffer_t deviceConstant(ExecutionContext* ctx, void* stream_handle, const char* 
     }
     state->metadata->releaseDeviceConstant(key);
     it = state->device_constants.emplace(key, std::make_pair(dev, dims)).first;
+    state->device_constant_buffers.insert(dev);
   }
   *shape = &it->second.second;
   return it->second.first;

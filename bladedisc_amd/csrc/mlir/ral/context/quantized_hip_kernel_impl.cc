@@ -45,6 +45,7 @@
 #include <unordered_map>
 
 #include "disc_q8.h"
+#include "mlir/ral/context/base/hip/hip_context_impl.h"
 #include "mlir/ral/context/context_util.h"
 #include "mlir/ral/context/conv_attr_util.h"
 #include "mlir/ral/context/pdll_util.h"
@@ -145,15 +146,21 @@ GPUDriver* driverOf(ExecutionContext* ctx) {
 // [K,N] constant weights are turned into the kernels' [N,K] layout once and kept
 // for the life of the context, keyed by the weight buffer's address and shape.
 struct PackedWeightState : public Context::Resource {
+  // how the bytes at `ptr` are laid out: plain [K,N], or [K,N] after the compiler's
+  // weight-only layout pass
+  enum Layout { kPlainKN = 0, kCompilerReorderedKN = 1 };
   struct Key {
     const void* ptr;
     int64_t k, n;
-    bool operator==(const Key& o) const { return ptr == o.ptr && k == o.k && n == o.n; }
+    int layout = kPlainKN;
+    bool operator==(const Key& o) const {
+      return ptr == o.ptr && k == o.k && n == o.n && layout == o.layout;
+    }
   };
   struct Hash {
     size_t operator()(const Key& k) const {
       return std::hash<const void*>()(k.ptr) ^ (std::hash<int64_t>()(k.k) * 1000003u) ^
-             (std::hash<int64_t>()(k.n) * 998244353u);
+             (std::hash<int64_t>()(k.n) * 998244353u) ^ (size_t)k.layout;
     }
   };
   std::mutex mu;
@@ -697,12 +704,18 @@ MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_s32_per_tensor(
 // f16 [..., K], weight ui8 [K, N] (the pattern transposes the [N, K] constant), [bias [N],]
 // per-channel scale [N] and zero point [N], all on the device; result [..., N] in the
 // activation type.  The reference tree has no implementation of this entry to compare with.
-// custom_attrs: `weight_should_be_reordered` -- true as the pattern emits it: the runtime may
-// put the weight into whatever layout its kernel wants, which here is [N, K], done once per
-// weight buffer and cached for the life of the context.  false means the compiler's CUDA
-// layout pass (R tao_compiler/mlir/disc/transforms/
-// disc_transform_weight_data_layout_for_weight_only_gemm.cc:305) has already interleaved the
-// bytes for NVIDIA tensor-core fragments; that layout has no meaning here and is refused.
+// custom_attrs: `weight_should_be_reordered`.
+//  * false: the compiler's layout pass (R tao_compiler/mlir/disc/transforms/
+//    disc_transform_weight_data_layout_for_weight_only_gemm.cc:305-410, run unconditionally from
+//    R tao_compiler/mlir/disc/disc_compiler.cc:257-258) has matched, i.e. the weight is a rank-2
+//    ui8 *constant* (:322-338) whose bytes it has permuted for NVIDIA tensor-core fragments
+//    (:362-370).  The permutation is undone once per weight buffer into the kernels' [N,K]
+//    layout and kept for the life of the context (the buffer is a constant by construction).
+//  * true (what the pattern emits and the pass leaves when it does not match): the weight is
+//    plain [K,N] and may be the result of another operator (the reference's test IR feeds it
+//    from an mhlo.transpose), whose buffer the allocator reuses for other contents.  The
+//    [N,K] copy is therefore cached only for buffers known to outlive executions (constants
+//    served by ral_const); any other weight is transposed on every call, into pool scratch.
 namespace {
 
 template <typename T>
@@ -724,6 +737,7 @@ MemRefType<T, N> weightOnlyQgemm(ExecutionContext* ctx, void* stream_handle,
   static const char* who = "ral_pdll_weight_only_qgemm";
   int64_t sizes[N] = {0};
   MemRefType<T, N> result = assignMemRef<T, N>(nullptr, sizes);
+  bool reordered_by_compiler = false;
   if (customAttrs) {
     PDLAttr* attr = getOrParsePDLAttr(ctx, customAttrs, who);
     if (!attr || attr->getType() != "dict") {
@@ -731,15 +745,17 @@ MemRefType<T, N> weightOnlyQgemm(ExecutionContext* ctx, void* stream_handle,
       return result;
     }
     auto& dict = attr->as<DictPDLAttr>();
-    if (dict.hasKey("weight_should_be_reordered") &&
-        dict.get("weight_should_be_reordered").getType() == "bool" &&
-        !dict.get("weight_should_be_reordered").as<BoolPDLAttr>().getValue()) {
-      fail(ctx, std::string(who) + ": a weight already reordered by the compiler's CUDA layout "
-                                   "pass cannot be used on this device");
-      return result;
-    }
+    reordered_by_compiler = dict.hasKey("weight_should_be_reordered") &&
+                            dict.get("weight_should_be_reordered").getType() == "bool" &&
+                            !dict.get("weight_should_be_reordered").as<BoolPDLAttr>().getValue();
   }
   const int64_t k = weight.sizes[0], n = weight.sizes[1];
+  if (reordered_by_compiler && (k % 64 != 0 || n % 4 != 0)) {
+    // (the pass indexes out of bounds there; what it leaves is not a permutation of the weight)
+    fail(ctx, std::string(who) + ": weight_should_be_reordered = false needs K % 64 == 0 and "
+                                 "N % 4 == 0, the shapes the compiler's layout pass is defined for");
+    return result;
+  }
   if (input.sizes[N - 1] != k && !isEmptyMemref(input)) {
     fail(ctx, std::string(who) + ": mismatch contraction dim");
     return result;
@@ -762,37 +778,48 @@ MemRefType<T, N> weightOnlyQgemm(ExecutionContext* ctx, void* stream_handle,
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return result;
   void* stream = drv->asCUStream(ctx, stream_handle);
-  // [K,N] -> [N,K], once per weight buffer
+  // The kernels' [N,K] layout, cached per weight buffer where the buffer is known to be a
+  // constant; a [K,N] weight that is not goes through scratch on every call.
   const uint8_t* w_nk = nullptr;
-  if (k > 0) {
+  const bool cacheable =
+      k > 0 && (reordered_by_compiler || gpu::isPersistentDeviceBuffer(ctx, weight.data));
+  if (cacheable) {
     auto* state = ctx->getOrCreateResource<PackedWeightState>(
         kPackedWeightState, [] { return new PackedWeightState; });
     if (!state) return result;
     std::lock_guard<std::mutex> guard(state->mu);
-    PackedWeightState::Key key{weight.data, k, n};
+    PackedWeightState::Key key{weight.data, k, n,
+                               reordered_by_compiler ? PackedWeightState::kCompilerReorderedKN
+                                                     : PackedWeightState::kPlainKN};
     auto it = state->packed.find(key);
     if (it == state->packed.end()) {
       auto* nk = static_cast<int8_t*>(drv->alloc_persistent(ctx, (size_t)(n * k)));
       if (!nk) return result;
-      if (kernelFailed(ctx, dq8_transpose_s8(reinterpret_cast<const int8_t*>(weight.data), n, nk,
-                                             k, n, stream), who))
-        return result;
+      const int st =
+          reordered_by_compiler
+              ? dq8_weight_only_undo_compiler_layout(weight.data, reinterpret_cast<uint8_t*>(nk), k,
+                                                     n, stream)
+              : dq8_transpose_s8(reinterpret_cast<const int8_t*>(weight.data), n, nk, k, n, stream);
+      if (kernelFailed(ctx, st, who)) return result;
       it = state->packed.emplace(key, nk).first;
     }
     w_nk = reinterpret_cast<const uint8_t*>(it->second);
   }
+  const int tp_b = w_nk ? 1 : 0;
   void* data = drv->alloc(ctx, (size_t)(m * n) * sizeof(T));
   if (!data) return result;
   result = assignMemRef<T, N>(data, sizes);
-  // (scratch for the partial sums of a launch split over k when m is small; handed back to the
-  // pool right after the launch, which later work on the same stream is ordered behind)
-  size_t ws_bytes = dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, 1, WoDtype<T>::value);
+  // (scratch for the transposed copy of a weight that is not cached and for the partial sums of
+  // a launch split over k when m is small; handed back to the pool right after the launch,
+  // which later work on the same stream is ordered behind)
+  size_t ws_bytes = dq8_weight_only_qgemm_workspace_bytes_ex(m, n, k, tp_b, WoDtype<T>::value);
   void* ws = ws_bytes ? drv->alloc(ctx, ws_bytes) : nullptr;
   if (!ws) ws_bytes = 0;                                   // (the call then runs unsplit)
   StreamTimer timer(stream);
-  const int st =
-      dq8_weight_only_qgemm(input.data, WoDtype<T>::value, k, w_nk, 0, k, 1, scales.data,
-                            zeroPoints.data, bias, data, n, m, n, k, ws, ws_bytes, stream);
+  const int st = dq8_weight_only_qgemm(input.data, WoDtype<T>::value, k,
+                                       w_nk ? static_cast<const void*>(w_nk) : weight.data, 0,
+                                       tp_b ? k : n, tp_b, scales.data, zeroPoints.data, bias, data,
+                                       n, m, n, k, ws, ws_bytes, stream);
   if (ws) drv->dealloc(ctx, ws);
   if (timer.on() && st == 0) {
     const double ns = timer.stop();
@@ -801,6 +828,10 @@ MemRefType<T, N> weightOnlyQgemm(ExecutionContext* ctx, void* stream_handle,
                   << "\tm = " << m << "\n"
                   << "\tn = " << n << "\n"
                   << "\tk = " << k << "\n"
+                  << "\tweight = "
+                  << (reordered_by_compiler ? "compiler layout, cached"
+                                            : (w_nk ? "[K,N] constant, cached" : "[K,N], per call"))
+                  << "\n"
                   << "\tMath Ops = " << 2 * m * n * k << "\n"
                   << "\tBytes = " << bytes << "\n"
                   << "\tElapsed = " << ns / 1e3 << " us\n"

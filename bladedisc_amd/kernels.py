@@ -191,6 +191,20 @@ def weight_only_qgemm(x, w, scale, zero_points=None, bias=None, tp_b=True, out=N
     return out
 
 
+def weight_only_undo_compiler_layout(reordered_kn):
+    """[K,N] uint8 bytes as the reference's compiler leaves a constant weight-only weight
+    (`weight_should_be_reordered = false`) -> the dense [N,K] weight matrix."""
+    _need_cuda(reordered_kn)
+    if reordered_kn.dtype != torch.uint8 or reordered_kn.dim() != 2:
+        raise TypeError("weight_only_undo_compiler_layout takes a uint8 [K,N] tensor")
+    r = reordered_kn.contiguous()
+    k, n = r.shape
+    out = torch.empty((n, k), dtype=torch.uint8, device=r.device)
+    st = _lib.lib().dq8_weight_only_undo_compiler_layout(_ptr(r), _ptr(out), k, n, _stream())
+    _lib.check(st, "dq8_weight_only_undo_compiler_layout")
+    return out
+
+
 def activation_table(fn, s_in, z_in, s_out, z_out, in_dtype=torch.int8, out_dtype=torch.int8,
                      device="cuda"):
     """The table of  q -> quantize(fn(dequantize(q, s_in, z_in)), s_out, z_out)  for every

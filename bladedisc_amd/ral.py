@@ -273,6 +273,14 @@ class RalExecution:
         a = Args().ctx(self.handle).scalar("pvoid", ptr)
         self.call("dealloc", "gpu", a)
 
+    def alloc_persistent(self, nbytes):
+        """Device memory that outlives executions and goes with the context, as a program's
+        constants do."""
+        a = Args().ctx(self.handle).scalar("i64", nbytes)
+        r = a.result_scalar("pvoid")
+        self.call("ral_gpu_alloc_persistent", "gpu", a)
+        return r.value
+
     def sync(self):
         a = Args().ctx(self.handle).scalar("pvoid", 0)
         self.call("sync_on_stream", "gpu", a)

@@ -340,6 +340,19 @@ int dq8_weight_only_qgemm(const void* x, int x_dtype, int64_t ldx, const void* w
                           const void* bias, void* out, int64_t ldo, int64_t M, int64_t N,
                           int64_t K, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The compiler's constant-weight layout, undone.  The reference's pipeline rewrites every
+ * rank-2 ui8 *constant* weight [K,N] of a `ral_pdll_weight_only_qgemm` call with a byte
+ * permutation meant for NVIDIA tensor-core fragments and sets `weight_should_be_reordered =
+ * false` (R tao_compiler/mlir/disc/transforms/
+ * disc_transform_weight_data_layout_for_weight_only_gemm.cc:54-300, composed at :362-370, run
+ * from R tao_compiler/mlir/disc/disc_compiler.cc:257-258).  This puts such a buffer
+ * (`reordered`, K*N bytes) back in order, as the dense [N,K] matrix dq8_weight_only_qgemm takes
+ * with tp_b = 1 (`w_nk`, K*N bytes, must not overlap).  The pass is a permutation only for
+ * K % 64 == 0 and N % 4 == 0 (elsewhere it indexes out of bounds); other shapes are refused.
+ * Both buffers 16-byte aligned.  A runtime does this once per constant. */
+int dq8_weight_only_undo_compiler_layout(const uint8_t* reordered, uint8_t* w_nk, int64_t K,
+                                         int64_t N, void* stream);
+
 /* ---- int8 convolution (rank 4) ---------------------------------------- */
 
 /* Implicit-GEMM convolution.  Layouts are described exactly as ral_qconv's

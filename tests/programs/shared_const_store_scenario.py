@@ -74,8 +74,35 @@ def main():
         L.disc_ral_execution_context_destroy(C.c_void_p(ex))
         return True
 
+    def alias_of_a_constant(ctx_h):
+        """inc_ref (a reshape) of a constant, then dealloc of the alias, as compiled graphs do:
+        a constant of the process-level store must count as persistent although no context's
+        allocator made it."""
+        class _Ctx:                      # the little of ral.RalContext that RalExecution uses
+            handle, _L, _names = ctx_h, L, {}
+            _name = ral.RalContext._name
+            last_error = ral.RalContext.last_error
+            clear_error = ral.RalContext.clear_error
+
+        ex = ral.RalExecution(_Ctx())
+        name = C.create_string_buffer(b"b0_f32_768")
+        a = ex.new_args().scalar("pvoid", C.addressof(name)).scalar("i32", 1)
+        cst = a.result_memref("f32", 1)
+        ex.call("ral_const", "gpu", a)
+        a = ex.new_args().memref("f32", cst.data, [768]).host_array(np.array([2, 384], np.int64))
+        alias = a.result_memref("f32", 2)
+        ex.call("inc_ref", "gpu", a)
+        assert alias.data == cst.data and [alias.sizes[0], alias.sizes[1]] == [2, 384]
+        ex.dealloc(alias.data)
+        ex.sync()
+        got = ral.device_view(cst.data, (768,), torch.float32).cpu().numpy()
+        np.testing.assert_array_equal(got, c["bias"])
+        ex.close()
+
     a = create()
     assert run(a, 8)
+    alias_of_a_constant(a)
+    assert run(a, 8)                      # the constant is intact after its alias was dropped
     os.remove(meta)                       # from here on only an already loaded store can serve
     b = L.disc_ral_context_create_for_program(C.c_void_p(stream), 0, None, None, None, 1, meta)
     if not b or not run(b, 5):

@@ -1206,6 +1206,25 @@ def test_weight_only_qgemm_bert_linears(K, m, k, n, dtype):
     _weight_only_check(got, x, w, scale, zp, bias, dtype)
 
 
+@pytest.mark.parametrize("k,n", [(64, 4), (128, 8), (192, 20), (1280, 200), (4096, 4096),
+                                 (11008, 4096)])
+def test_weight_only_undo_compiler_layout(K, k, n):
+    """The inverse of the compiler's constant-weight permutation
+    (R tao_compiler/mlir/disc/transforms/disc_transform_weight_data_layout_for_weight_only_gemm.cc
+    :54-300, :362-370), bit for bit against the oracle's restatement of the four functions."""
+    from oracle import weight_layout_oracle as WL
+    w_kn = np.random.default_rng(k + n).integers(0, 256, (k, n), dtype=np.uint8)
+    got = K.weight_only_undo_compiler_layout(dev(WL.forward(w_kn)))
+    assert tuple(got.shape) == (n, k)
+    np.testing.assert_array_equal(host(got), w_kn.T)
+
+
+def test_weight_only_undo_compiler_layout_refuses_shapes_outside_the_pass_domain(K):
+    for k, n in [(96, 8), (64, 6)]:
+        with pytest.raises(RuntimeError, match="K % 64 == 0"):
+            K.weight_only_undo_compiler_layout(torch.zeros((k, n), dtype=torch.uint8, device="cuda"))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_weight_only_qgemm_layouts_and_ragged_shapes(K, dtype):
     """[K,N] weights as the custom call passes them (with and without the scratch for the

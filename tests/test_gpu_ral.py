@@ -19,9 +19,6 @@ def rt():
     ctx.close()
 
 
-_CONSTANT_WEIGHTS = []
-
-
 def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
@@ -204,15 +201,30 @@ def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
             ex.call("ral_pdll_qgemm", "gpu", a)
 
 
+def _wo_tolerance(want, bound, k, dtype):
+    return bound * (k * 2.0 ** -24 + 2.0 ** -20) + \
+        (np.abs(want) + bound * 2.0 ** -12) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
+
+
+def _persistent(ral, ex, a):
+    """A device buffer from the context's alloc_persistent holding `a`: what ral_const hands a
+    program for a constant."""
+    a = np.ascontiguousarray(a)
+    ptr = ex.alloc_persistent(a.nbytes)
+    t = ral.device_view(ptr, a.shape, torch.uint8)
+    t.copy_(torch.from_numpy(a))
+    return t
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("with_bias,k,n", [(False, 96, 72), (True, 96, 72), (True, 1280, 200)])
 def test_ral_pdll_weight_only_qgemm(rt, dtype, with_bias, k, n):
     """The weight-only entry by its mangled name, as the pattern calls it: rank-3 activations,
     uint8 weight [K,N] with zero points 128 (quant range 0..255), per-channel scale, optional
-    bias; the packed weight is cached, so a second call with other activations must agree
-    too.  The deep case (80 rows, k = 1280) is one the f16 kernels split over k, with the
-    partial sums in scratch from the context's pool.  Tolerance: the f32 accumulation bound
-    of the kernel tests."""
+    bias.  The weight is a constant of the context (alloc_persistent), so its [N,K] copy is
+    cached: a second call with other activations must agree too.  The deep case (80 rows,
+    k = 1280) is one the f16 kernels split over k, with the partial sums in scratch from the
+    context's pool.  Tolerance: the f32 accumulation bound of the kernel tests."""
     ctx, ral, ops = rt
     rng = np.random.default_rng(31 + int(with_bias) + k)
     npdt = np.float16 if dtype == torch.float16 else np.float32
@@ -221,24 +233,105 @@ def test_ral_pdll_weight_only_qgemm(rt, dtype, with_bias, k, n):
     zp = np.full(n, 128, np.int32)
     scale = rng.uniform(0.002, 0.02, n).astype(npdt)
     bias = rng.standard_normal(n).astype(npdt) if with_bias else None
-    w_kn = dev(np.ascontiguousarray(w.T))
-    # (the entry caches the re-laid-out weight by buffer address for the life of the context, as
-    # for a program's constants: the buffer must not be freed and reused while `rt` lives)
-    _CONSTANT_WEIGHTS.append(w_kn)
     with ctx.execution() as ex:
+        w_kn = _persistent(ral, ex, w.T)
         for rep in range(2):
             x = rng.standard_normal((b, s, k)).astype(npdt)
             got = ops.pdll_weight_only_qgemm(ex, dev(x), w_kn, dev(scale), dev(zp),
                                              dev(bias) if with_bias else None)
             assert got.dtype == dtype and tuple(got.shape) == (b, s, n)
             want, bound = O.weight_only_qgemm(x.reshape(-1, k), w, scale, zp, bias)
-            tol = bound * (k * 2.0 ** -24 + 2.0 ** -20) + \
-                (np.abs(want) + bound * 2.0 ** -12) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
             err = np.abs(host(got).astype(np.float64).reshape(-1, n) - want)
-            assert (err <= tol).all(), rep
-        # a weight the compiler's CUDA layout pass has already interleaved is refused
-        with pytest.raises(ral.RalError, match="reordered"):
-            ops.pdll_weight_only_qgemm(ex, dev(x), w_kn, dev(scale), dev(zp), None, reorder=False)
+            assert (err <= _wo_tolerance(want, bound, k, dtype)).all(), rep
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("m,k,n", [(80, 1280, 200), (3, 64, 4), (300, 256, 1024)])
+def test_ral_pdll_weight_only_qgemm_takes_the_compiler_reordered_constant(rt, dtype, m, k, n):
+    """What the unchanged compiler emits for a constant ui8 weight: the bytes permuted by its
+    layout pass and `weight_should_be_reordered = false`
+    (R tao_compiler/mlir/disc/transforms/disc_transform_weight_data_layout_for_weight_only_gemm.cc
+    :362-410).  The result must be bit-identical to the plain [K,N] weight with the attribute
+    true, cached (constant) or not."""
+    from oracle import weight_layout_oracle as WL
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(5 * m + k + n)
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    w_kn = rng.integers(0, 256, (k, n), dtype=np.uint8)
+    reordered = WL.forward(w_kn)
+    zp = rng.integers(100, 156, n).astype(np.int32)
+    scale = rng.uniform(0.002, 0.02, n).astype(npdt)
+    bias = rng.standard_normal(n).astype(npdt)
+    x = dev(rng.standard_normal((1, m, k)).astype(npdt))
+    with ctx.execution() as ex:
+        plain_const = _persistent(ral, ex, w_kn)
+        reordered_const = _persistent(ral, ex, reordered)
+        args = (dev(scale), dev(zp), dev(bias))
+        for rep in range(2):                                        # second call: from the cache
+            got = host(ops.pdll_weight_only_qgemm(ex, x, reordered_const, *args, reorder=False))
+            want = host(ops.pdll_weight_only_qgemm(ex, x, plain_const, *args, reorder=True))
+            np.testing.assert_array_equal(got.view(np.uint8), want.view(np.uint8))
+        # the same weight as the result of another operator (pool memory: not cached)
+        want2 = host(ops.pdll_weight_only_qgemm(ex, x, dev(w_kn), *args, reorder=True))
+        np.testing.assert_array_equal(want2.view(np.uint8), want.view(np.uint8))
+        ref, bound = O.weight_only_qgemm(host(x).reshape(-1, k), np.ascontiguousarray(w_kn.T),
+                                         scale, zp, bias)
+        err = np.abs(got.astype(np.float64).reshape(-1, n) - ref)
+        assert (err <= _wo_tolerance(ref, bound, k, dtype)).all()
+
+
+def test_ral_pdll_weight_only_qgemm_reordered_shape_outside_the_pass_domain(rt):
+    """K % 64 != 0 or N % 4 != 0: the compiler's pass indexes out of bounds there, so what it
+    would leave is not a permutation of the weight; the entry says so."""
+    ctx, ral, ops = rt
+    with ctx.execution() as ex:
+        x = torch.zeros((1, 4, 96), dtype=torch.float16, device="cuda")
+        w = torch.zeros((96, 72), dtype=torch.uint8, device="cuda")
+        sc = torch.ones(72, dtype=torch.float16, device="cuda")
+        zp = torch.zeros(72, dtype=torch.int32, device="cuda")
+        with pytest.raises(ral.RalError, match="K % 64 == 0"):
+            ops.pdll_weight_only_qgemm(ex, x, w, sc, zp, None, reorder=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_ral_pdll_weight_only_qgemm_weight_that_is_not_a_constant(rt, dtype):
+    """`weight_should_be_reordered = true` reaches the runtime exactly when the weight is not a
+    constant the layout pass could match -- e.g. the result of an mhlo.transpose, in memory the
+    allocator reuses.  Two same-shaped weights at one address, one after the other (the buffer
+    rewritten in place, and a buffer freed to the context's pool and handed out again), must each
+    give their own result."""
+    ctx, ral, ops = rt
+    rng = np.random.default_rng(77)
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    m, k, n = 48, 192, 136
+    scale = dev(rng.uniform(0.002, 0.02, n).astype(npdt))
+    zp = dev(np.full(n, 128, np.int32))
+    x = rng.standard_normal((1, m, k)).astype(npdt)
+    ws = [rng.integers(0, 256, (k, n), dtype=np.uint8) for _ in range(3)]
+
+    def check(got, w_kn):
+        want, bound = O.weight_only_qgemm(x.reshape(-1, k), np.ascontiguousarray(w_kn.T),
+                                          host(scale), host(zp), None)
+        err = np.abs(host(got).astype(np.float64).reshape(-1, n) - want)
+        assert (err <= _wo_tolerance(want, bound, k, dtype)).all()
+
+    with ctx.execution() as ex:
+        buf = dev(ws[0])
+        check(ops.pdll_weight_only_qgemm(ex, dev(x), buf, scale, zp), ws[0])
+        buf.copy_(torch.from_numpy(ws[1]))                       # same address, new contents
+        check(ops.pdll_weight_only_qgemm(ex, dev(x), buf, scale, zp), ws[1])
+        # a pool buffer released and handed out again for the next layer's weight
+        addrs = []
+        for w_kn in ws[1:]:
+            ptr = ex.alloc(k * n)
+            addrs.append(ptr)
+            t = ral.device_view(ptr, (k, n), torch.uint8)
+            t.copy_(torch.from_numpy(w_kn))
+            got = ops.pdll_weight_only_qgemm(ex, dev(x), t, scale, zp)
+            check(got, w_kn)
+            torch.cuda.synchronize()
+            ex.dealloc(ptr)
+        assert addrs[0] == addrs[1], "the pool was expected to hand the same buffer out again"
 
 
 @pytest.mark.parametrize("nb,h,ci,co,k,stride,pad", [(2, 14, 64, 64, 3, 1, 1), (2, 7, 256, 128, 1, 1, 0),
