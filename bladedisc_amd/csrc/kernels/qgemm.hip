@@ -893,6 +893,32 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   DQ8_REQUIRE(Ho == out_len(H, padding[0], padding[1], Kh, dh, sh) &&
                   Wo == out_len(Wd, padding[2], padding[3], Kw, dw, sw_),
               "dq8_qconv2d: output spatial size inconsistent with padding/stride/dilation");
+  // Everything that can refuse the call is checked before any re-layout kernel is enqueued
+  // (the re-layout branches below launch into the caller's scratch and then come back here
+  // through a recursive call, which repeats these checks on its own arguments).
+  {
+    int ep = epilogue, rq = 0;
+    if (ep == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || ep == DQ8_EPI_REQUANT_GPU_DEQUANT_F32) {
+      rq = 1;
+      ep = ep == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 ? DQ8_EPI_REQUANT_CPU : DQ8_EPI_REQUANT_GPU;
+    }
+    if (ep == DQ8_EPI_REQUANT_FIXEDPOINT) {
+      DQ8_REQUIRE(bias_kind == DQ8_BIAS_NONE || bias_kind == DQ8_BIAS_S32,
+                  "dq8_qconv2d: the fixed-point stage takes an s32 bias or none");
+      ep = DQ8_EPI_REQUANT_CPU;
+    }
+    if (int s = check_epilogue("dq8_qconv2d", ep, bias, bias_kind, sx, sw, so, 1, n_sw, 1, Co))
+      return s;
+    DQ8_REQUIRE(zo == 0 || ep == DQ8_EPI_REQUANT_CPU,
+                "dq8_qconv2d: an output zero point needs the REQUANT_CPU epilogue");
+    EpiParams dry = {};
+    if (int s = apply_postops("dq8_qconv2d", post, !rq && elem_size(ep) == 1 && ep != DQ8_EPI_ACC_S32,
+                              rq != 0, 1, Co, &dry))
+      return s;
+    DQ8_REQUIRE(!dry.resid_kind || is_nhwc_ohwi(md) || dry.ldr == Co,
+                "dq8_qconv2d: a fused residual has the layout of the output");
+  }
+
   // NCHW x OIHW -> NCHW (the PyTorch layouts): with scratch, the input and the weights are
   // re-laid out as NHWC / OHWI, the convolution runs on the MFMA kernels into an NHWC scratch
   // result, and that is turned back into NCHW -- what the reference's GPU path does around its

@@ -205,6 +205,44 @@ void ral_base_hip_raw_dealloc(Context* ctx, buffer_t buffer) {
   state->gpu_allocator->dealloc(buffer);
 }
 
+namespace {
+// True if the image at `blob` carries device code for gfx950: an AMDGPU ELF whose e_flags name
+// that processor, or a clang offload bundle with an entry whose target ends in it.  Only the
+// headers are read (a launch receives its images without their sizes).
+bool codeObjectIsForGfx950(const void* blob) {
+  const unsigned char* b = static_cast<const unsigned char*>(blob);
+  auto u16 = [&](size_t o) { return (uint32_t)b[o] | ((uint32_t)b[o + 1] << 8); };
+  auto u64 = [&](size_t o) {
+    uint64_t v = 0;
+    for (int i = 7; i >= 0; --i) v = (v << 8) | b[o + i];
+    return v;
+  };
+  if (b[0] == 0x7f && b[1] == 'E' && b[2] == 'L' && b[3] == 'F') {
+    constexpr uint32_t kEmAmdgpu = 224, kMachGfx950 = 0x4f;   // EF_AMDGPU_MACH: e_flags & 0xff
+    return b[4] == 2 /* ELFCLASS64 */ && u16(18) == kEmAmdgpu && b[48] == kMachGfx950;
+  }
+  static const char kBundle[] = "__CLANG_OFFLOAD_BUNDLE__";
+  if (std::memcmp(b, kBundle, 24) == 0) {
+    // magic[24], u64 entries, then per entry u64 offset, u64 size, u64 triple length, triple
+    const uint64_t entries = u64(24);
+    size_t o = 32;
+    for (uint64_t e = 0; e < entries && e < 64; ++e) {
+      const uint64_t size = u64(o + 8), len = u64(o + 16);
+      if (len > 256) return false;
+      const std::string triple(reinterpret_cast<const char*>(b + o + 24), (size_t)len);
+      o += 24 + (size_t)len;
+      if (size == 0 || triple.compare(0, 4, "host") == 0) continue;
+      // "hipv4-amdgcn-amd-amdhsa--gfx950" with optional ":feature" suffixes
+      const size_t at = triple.rfind("gfx950");
+      if (at != std::string::npos && at > 0 && triple[at - 1] == '-' &&
+          (at + 6 == triple.size() || triple[at + 6] == ':'))
+        return true;
+    }
+  }
+  return false;
+}
+}  // namespace
+
 void ral_base_hip_launch(ExecutionContext* ctx, void** blobs, size_t num_blobs,
                          const char* kernel_name, intptr_t gridX, intptr_t gridY,
                          intptr_t gridZ, intptr_t blockX, intptr_t blockY,
@@ -217,8 +255,22 @@ void ral_base_hip_launch(ExecutionContext* ctx, void** blobs, size_t num_blobs,
     ctx->signalError(Context::FAILURE, "ral_kernel_launch: no code object");
     return;
   }
-  // a DISC build for this runtime carries one gfx950 code object per kernel
+  // One blob is taken as it is; of several (the reference's builds for NVIDIA carry one image
+  // per compute capability and pick by the device's, R context/base/cuda/
+  // cuda_context_impl.cc:375-392) the first that holds gfx950 code.
   void* blob = blobs[0];
+  if (num_blobs > 1) {
+    blob = nullptr;
+    for (size_t i = 0; i < num_blobs && !blob; ++i)
+      if (blobs[i] && codeObjectIsForGfx950(blobs[i])) blob = blobs[i];
+    if (!blob) {
+      ctx->signalError(Context::FAILURE, "ral_kernel_launch: none of the " +
+                                             std::to_string(num_blobs) +
+                                             " code objects of kernel " + kernel_name +
+                                             " is built for gfx950");
+      return;
+    }
+  }
   hipFunction_t fn = nullptr;
   {
     std::lock_guard<std::mutex> guard(state->mu);

@@ -320,7 +320,9 @@ int dq8_transpose_s8(const int8_t* src, int64_t ld, int8_t* dst, int64_t rows,
  * x, out, scale, bias: x_dtype (DQ8_DTYPE_*), rows ldx / ldo elements apart; bias and
  * zero_points may be NULL; w: uint8 (w_signed = 0) or int8 (1), [N,K] with rows ldw bytes
  * apart if tp_b, else [K,N] as the custom call passes it.  Zero points must lie in
- * [-1024, 1024].  [K,N] weights are transposed into `workspace`
+ * [-1024, 1024] for uint8 weights and in [-1152, 896] for int8 weights (the kernels subtract
+ * the half 1024 + zp, + 128 for int8, which holds integers exactly only up to 2048; they are
+ * device data and not checked).  [K,N] weights are transposed into `workspace`
  * (dq8_weight_only_qgemm_workspace_bytes) on every call; a runtime does that once per constant
  * weight with dq8_transpose_s8 and passes tp_b = 1.  Without the scratch, or with K % 16 != 0
  * or rows that are not 16-byte aligned, a slower kernel without alignment rules runs.

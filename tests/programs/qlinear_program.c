@@ -142,8 +142,14 @@ void disc_program_main(void** ctx_struct) {
 /* The same program with the dequantize replaced by a fused elementwise kernel that the
  * compiler would have generated and embedded as a code object:
  * y = relu(dequantize(yq)) + x, launched through ral_kernel_launch (N must equal K). */
-static const void* g_code_object = 0;
-void disc_program_set_code_object(const void* blob) { g_code_object = blob; }
+static const void* g_code_objects[8] = {0};
+static int64_t g_num_code_objects = 0;
+void disc_program_set_code_object(const void* blob) { g_code_objects[0] = blob; g_num_code_objects = 1; }
+/* Several images for one kernel, as a build for more than one processor carries them. */
+void disc_program_set_code_objects(const void** blobs, int64_t n) {
+  g_num_code_objects = n < 8 ? n : 8;
+  for (int64_t i = 0; i < g_num_code_objects; ++i) g_code_objects[i] = blobs[i];
+}
 
 void disc_program_main_fused(void** ctx_struct) {
   Front f; run_front(ctx_struct, &f);
@@ -152,7 +158,8 @@ void disc_program_main_fused(void** ctx_struct) {
   MemRef2 y = {0};
   y.base = y.data = gpu_alloc(call, exec, M * N * 4);
   y.sizes[0] = M; y.sizes[1] = N; y.strides[0] = N; y.strides[1] = 1;
-  { void* blobs[1] = {(void*)g_code_object}; void** blobs_p = blobs; int64_t num_blobs = 1;
+  { void* blobs[8]; for (int i = 0; i < 8; ++i) blobs[i] = (void*)g_code_objects[i];
+    void** blobs_p = blobs; int64_t num_blobs = g_num_code_objects;
     const char* name = "fused_dequant_relu_residual";
     int64_t total = M * N;
     int64_t gx = (total + 255) / 256, gy = 1, gz = 1, bx = 256, by = 1, bz = 1;

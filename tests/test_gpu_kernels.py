@@ -1206,6 +1206,25 @@ def test_weight_only_qgemm_bert_linears(K, m, k, n, dtype):
     _weight_only_check(got, x, w, scale, zp, bias, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("signed", [False, True])
+@pytest.mark.parametrize("m", [2, 24, 200])
+def test_weight_only_qgemm_zero_points_at_the_documented_extremes(K, dtype, signed, m):
+    """Zero points at both ends of the documented range (uint8 weights [-1024, 1024], int8
+    weights [-1152, 896]), odd values next to the ends included: the kernels' half 1024 + zp
+    (+ 128) is exact there, so the usual accumulation bound holds."""
+    k, n = 256, 96
+    rng = np.random.default_rng(m + int(signed))
+    x, w, scale, _, bias = _weight_only_case(rng, m, k, n, dtype, signed)
+    lo, hi = (-1152, 896) if signed else (-1024, 1024)
+    ends = np.array([lo, lo + 1, lo + 3, hi - 3, hi - 1, hi], np.int32)
+    zp = ends[rng.integers(0, len(ends), n)]
+    zp[:len(ends)] = ends
+    scale = (scale / 8).astype(scale.dtype)              # keeps f16 results finite
+    got = K.weight_only_qgemm(dev(x), dev(w), dev(scale), dev(zp), dev(bias))
+    _weight_only_check(got, x, w, scale, zp, bias, dtype)
+
+
 @pytest.mark.parametrize("k,n", [(64, 4), (128, 8), (192, 20), (1280, 200), (4096, 4096),
                                  (11008, 4096)])
 def test_weight_only_undo_compiler_layout(K, k, n):

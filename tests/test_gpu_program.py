@@ -120,11 +120,27 @@ def test_process_level_constant_store(program):
     assert "OK" in r.stdout or want == 3
 
 
-def test_program_with_an_embedded_code_object(program):
+def _decoy_code_objects():
+    """Images a multi-target build could carry next to the gfx950 one: PTX text, and the ELF
+    header of a code object for another AMD processor (EM_AMDGPU = 224, e_flags mach 0x4c)."""
+    import struct
+    ptx = b"//\n// Generated by NVIDIA NVVM Compiler\n.version 7.8\n.target sm_80\n" + b" " * 64
+    elf = bytearray(64)
+    elf[:7] = b"\x7fELF\x02\x01\x01"
+    struct.pack_into("<HHI", elf, 16, 1, 224, 1)
+    struct.pack_into("<I", elf, 48, 0x54c)
+    return ptx, bytes(elf)
+
+
+@pytest.mark.parametrize("images", ["one", "three", "none_for_this_device"])
+def test_program_with_an_embedded_code_object(program, images):
     """The same program with its dequantize replaced by a fused elementwise kernel that
     travels as a gfx950 code object, the way the compiler ships its generated kernels, and
     is launched through ral_kernel_launch: y = relu(dequantize(qgemm(...))) + x.  Two
-    executions (the second finds the loaded module cached), checked bit for bit."""
+    executions (the second finds the loaded module cached), checked bit for bit.  With
+    several images per kernel (R context/base/cuda/cuda_context_impl.cc:375-392 picks by
+    compute capability) the launch takes the one built for this device, and says so when
+    there is none."""
     lib, d = program
     hsaco = os.path.join(HERE, "programs", "fused_dequant_relu_residual.hsaco")
     if not os.path.exists(hsaco):        # normally built beforehand by __graft_entry__.build()
@@ -132,7 +148,14 @@ def test_program_with_an_embedded_code_object(program):
         b.build_test_code_objects()
     blob = open(hsaco, "rb").read()
     blob_buf = C.create_string_buffer(blob, len(blob))      # lives as long as the context
-    lib.disc_program_set_code_object(C.cast(blob_buf, C.c_void_p))
+    ptx, other_elf = _decoy_code_objects()
+    decoys = [C.create_string_buffer(ptx, len(ptx)), C.create_string_buffer(other_elf, len(other_elf))]
+    if images == "one":
+        lib.disc_program_set_code_object(C.cast(blob_buf, C.c_void_p))
+    else:
+        bufs = [decoys[0], decoys[1]] + ([blob_buf] if images == "three" else [])
+        arr = (C.c_void_p * len(bufs))(*[C.cast(b, C.c_void_p).value for b in bufs])
+        lib.disc_program_set_code_objects(arr, len(bufs))
     from bladedisc_amd import baseline_configs as cfg
     from bladedisc_amd import ral
     L = ral.lib()
@@ -162,6 +185,12 @@ def test_program_with_an_embedded_code_object(program):
                                                    (C.c_int64 * 2)(m, 768), 2) == 0
             lib.disc_program_main_fused((C.c_void_p * 2)(ex, call_impl))
             msg = C.c_char_p()
+            if images == "none_for_this_device":
+                assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) != 0
+                assert b"is built for gfx950" in msg.value
+                L.tao_ral_clear_error(C.c_void_p(ctx))
+                L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+                break
             assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) == 0, msg.value
             out = L.disc_ral_execution_take_output(C.c_void_p(ex), 0)
             assert out

@@ -80,3 +80,52 @@ def test_static_scratch_folds_into_running_state_and_rejects_oversize():
     assert b"more than the built-in" in L.dq8_last_error()
     torch.cuda.synchronize()
     assert lo.item() == -7.0 and hi.item() == 3.0
+
+
+def test_static_scratch_under_graph_capture_and_without_allocation():
+    """The callers this entry is for: code under HIP graph capture.  After one warm call (the
+    per-device address lookup), the call is captured into a graph and replayed on fresh data
+    several times, with eager work and synchronisations in between, each replay against
+    dq8_minmax; and a call leaves the device's free memory as it found it."""
+    from bladedisc_amd import _lib
+    L = _lib.lib()
+    p = lambda t: C.c_void_p(t.data_ptr())  # noqa: E731
+    outer, nch, inner = 300, 64, 257
+    rng = np.random.default_rng(5)
+    x = torch.zeros(outer * nch * inner, device="cuda")
+    lo, hi = _state(nch)
+    warm = torch.from_numpy(rng.standard_normal(x.numel()).astype(np.float32)).cuda()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert L.dq8_minmax_static(p(warm), outer, nch, inner, p(lo), p(hi), st) == 0   # warm the lookup
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    assert L.dq8_minmax_static(p(warm), outer, nch, inner, p(lo), p(hi), st) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        g.capture_begin()
+        rc = L.dq8_minmax_static(p(x), outer, nch, inner, p(lo), p(hi), C.c_void_p(side.cuda_stream))
+        g.capture_end()
+    assert rc == 0, L.dq8_last_error()
+    torch.cuda.synchronize()
+    need = L.dq8_minmax_workspace_bytes(outer, nch, inner)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
+    for rep in range(3):
+        data = rng.standard_normal(x.numel()).astype(np.float32) * (rep + 1)
+        x.copy_(torch.from_numpy(data))
+        lo.fill_(float("inf"))
+        hi.fill_(float("-inf"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        lo_ref, hi_ref = _state(nch)
+        assert L.dq8_minmax(p(x), outer, nch, inner, p(lo_ref), p(hi_ref), p(ws), need, st) == 0
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(lo.cpu().numpy(), lo_ref.cpu().numpy())
+        np.testing.assert_array_equal(hi.cpu().numpy(), hi_ref.cpu().numpy())
+        v = data.reshape(outer, nch, inner)
+        np.testing.assert_array_equal(lo.cpu().numpy(), v.min(axis=(0, 2)))
