@@ -24,11 +24,26 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA peak, 5.0 POP/s
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, 8 TB/s
 
-# Bytes the L2s exchange with the memory side per launch of the headline kernel, from
-# two rocprofv3 --pmc passes over this script (FETCH_SIZE, WRITE_SIZE; summary and
-# commands in profiles/qgemm_4096_requant_hbm_traffic.md).  Counters cannot be read
-# from inside the run, so the figure is recorded here for the size it was measured on.
-MEASURED_TRAFFIC_BYTES = {4096: (98660 + 16384) * 1024}
+def measured_traffic(size, kernel_name):
+    """(bytes, note): what the L2s exchange with the memory side per launch of the headline
+    kernel, from the record written next to the rocprofv3 --pmc summary of this command
+    (profiles/qgemm_4096_requant_hbm_traffic.{md,json}: FETCH_SIZE and WRITE_SIZE in KiB per
+    dispatch, each with the factor a kernel of known size reads under the same counter).
+    Counters cannot be read from inside the run, so the figure is only reported when the record
+    is for this size and for the kernel configuration the library picks now."""
+    path = os.path.join(ROOT, "profiles", "qgemm_%d_requant_hbm_traffic.json" % size)
+    if not os.path.exists(path):
+        return None, "no counter record for this size under profiles/"
+    with open(path) as f:
+        rec = json.load(f)
+    if rec.get("size") != size or rec.get("kernel") != kernel_name:
+        return None, ("the counter record %s is for kernel %r, the library now picks %r: "
+                      "re-measure" % (os.path.basename(path), rec.get("kernel"), kernel_name))
+    byts = int((rec["fetch_size_kib_per_dispatch"] * rec["fetch_size_factor"]
+                + rec["write_size_kib_per_dispatch"] * rec["write_size_factor"]) * 1024)
+    return byts, ("recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over this command "
+                  "(%s, kernel %s); counters cannot be read from inside the run"
+                  % (rec.get("summary", path), rec.get("kernel_symbol", kernel_name)))
 
 
 def parse():
@@ -744,6 +759,10 @@ def main():
     o = out.cpu().numpy()
     sat_frac = float(((o == 127) | (o == -128)).mean())
 
+    from bladedisc_amd import _lib
+    kernel_name = _lib.lib().dq8_qgemm_kernel_name(size, size, size, 1).decode()
+    traffic, traffic_note = measured_traffic(size, kernel_name)
+
     result = {
         "metric": "int8 qgemm TOPS (M=%d,K=N=%d)" % (size, size),
         "value": round(tops, 2),
@@ -773,10 +792,9 @@ def main():
             "peak": PEAK_INT8_TOPS,
             "unit": "TOP/s",
             "frac": round(achieved / PEAK_INT8_TOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(size),
-            "traffic_source": "recorded: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes over "
-                              "this command (profiles/qgemm_4096_requant_hbm_traffic.md); "
-                              "counters cannot be read from inside the run",
+            "traffic": traffic,
+            "traffic_source": traffic_note,
+            "kernel": kernel_name,
             "algorithmic_bytes": 3 * size * size + 8 * size,
             "kernel_us": round(kernel_s * 1e6, 2),
             "ops_per_launch": ops,
@@ -795,6 +813,15 @@ def main():
         result["cpu_baseline"] = None
     if not args.no_extra:
         result["extra"] = extras(torch, args.steps, args.warmup, args.extras)
+        # the second size BASELINE's roofline configuration names, next to the headline
+        big = result["extra"].get("configs", {}).get("3_large_square_8192_fused_bias_requant")
+        if big:
+            result["headline_8192"] = {
+                "metric": "int8 qgemm TOPS (M=8192,K=N=8192)", "value": big["TOPS"],
+                "unit": "TOPS", "kernel_us": big["us"],
+                "roofline": {"bound": "mfma", "achieved": big["TOPS"], "peak": PEAK_INT8_TOPS,
+                             "unit": "TOP/s", "frac": round(big["TOPS"] / PEAK_INT8_TOPS, 4)},
+                "kernel": _lib.lib().dq8_qgemm_kernel_name(8192, 8192, 8192, 1).decode()}
     print(json.dumps(result))
 
 

@@ -415,8 +415,8 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
   // (operands the pipelined kernels cannot address: the 128 x 128 and 64 x 64 tiles of the basic
   // kernel; its 256 x 256 form on four waves indexes 256 accumulators per lane and is kept
   // only as a cross-check variant)
-  constexpr int64_t kCus = 256;
-  if (tiles(2) >= kCus - kCus / 8) return 2;
+  const int64_t cus = compute_units();
+  if (tiles(2) >= cus - cus / 8) return 2;
   return 3;
 }
 
@@ -794,6 +794,18 @@ int qgemm_impl(int variant, const int8_t* A, int64_t lda, const int8_t* W, int64
   return launch_epi<false>(variant, p, epilogue, st);
 }
 }  // namespace
+
+extern "C" const char* dq8_qgemm_kernel_name(int64_t M, int64_t N, int64_t K, int out_bytes) {
+  if (M <= 0 || N <= 0 || K <= 0 || M >= (1LL << 31) || N >= (1LL << 31) || K >= (1LL << 31))
+    return "";
+  if (K % 16 != 0) return kVariants[0].name;
+  MainParams p = {};
+  p.lda = p.ldw = K;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  return kVariants[pick_any(M, N, K, pipe_ok(256, 256, p, false), out_bytes == 1 ? 1 : 4)].name;
+}
 
 extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                                  const int8_t* W, int64_t ldw, void* out, int64_t ldo,

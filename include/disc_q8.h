@@ -300,6 +300,14 @@ int dq8_qgemm_fused(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, 
                     int32_t zx, int32_t zw, int32_t zo, void* workspace, size_t workspace_bytes,
                     const dq8_postops_t* post, void* stream);
 
+/* Name of the kernel configuration dq8_qgemm chooses on the current device for dense,
+ * 16-byte aligned, k-contiguous operands of this shape without zero points or fused operators
+ * and an output element of `out_bytes` bytes (1: int8, 4: int32 / f32), e.g.
+ * "pipe_256x256x128_w8"; "" for an empty or oversized problem.  For logs and profiles (the
+ * counterpart of the algorithm the reference prints with DISC_GPU_ENABLE_PROFILE,
+ * R ral/context/stream_executor_based_impl.cc:427-483); the returned string is static. */
+const char* dq8_qgemm_kernel_name(int64_t M, int64_t N, int64_t K, int out_bytes);
+
 /* dst[c, r] = src[r, c] for an int8 matrix src [rows, cols] with row stride ld;
  * dst is dense [cols, rows].  Used to put [K,N] weights into the kernels' [N,K]
  * layout once (the reference's counterpart is oneDNN's weight pre-packing,
