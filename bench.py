@@ -291,6 +291,11 @@ def config_reports(torch, K):
              FnCall(lambda: K.qgemm(xq, wq, K.EPI_REQUANT_CPU_DEQUANT_F32, sx=sx, sw=sw, so=so,
                                     bias=bias, out=y))]
     gpu_fused_s = time_graph(torch, fused)
+    # the whole chain as one launch: the activations are quantized on their way into the
+    # matrix cores (dq8_qlinear_f32), the dequantize runs in the epilogue (bit-identical f32)
+    one = [FnCall(lambda: K.qlinear_f32(x, wq, K.EPI_REQUANT_CPU_DEQUANT_F32, sx, sw, so,
+                                        bias=bias, out=y))]
+    gpu_one_s = time_graph(torch, one)
 
     def cpu1():
         q = O.quantize(c["x"], c["sx"], 0)
@@ -301,7 +306,9 @@ def config_reports(torch, K):
     rep["1_single_linear_64x768x768_q_gemm_dq"] = {
         "gpu_us": round(gpu_s * 1e6, 2), "cpu_us": round(cpu_s * 1e6, 1),
         "gpu_over_cpu": round(cpu_s / gpu_s, 1),
-        "gpu_us_dequantize_in_epilogue": round(gpu_fused_s * 1e6, 2)}
+        "gpu_us_dequantize_in_epilogue": round(gpu_fused_s * 1e6, 2),
+        "gpu_us_one_launch": round(gpu_one_s * 1e6, 2),
+        "gpu_one_launch_over_cpu": round(cpu_s / gpu_one_s, 1)}
 
     # ---- 2: dynamic-M sweep, E1 requant, int8 out
     sweep = {}

@@ -53,6 +53,9 @@ _PROTOS = {
     "dq8_weight_only_qgemm_workspace_bytes_ex": (C.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "dq8_weight_only_qgemm": (_INT, [_VP, _INT, _I64, _VP, _INT, _I64, _INT, _VP, _VP, _VP, _VP,
                                      _I64, _I64, _I64, _I64, _VP, C.c_size_t, _VP]),
+    "dq8_qlinear_f32_fused_max_rows": (_I64, [_I64, _I64]),
+    "dq8_qlinear_f32": (_INT, [_VP, _I64, _VP, _I64, _VP, _I64, _I64, _I64, _I64, _INT, _VP, _INT,
+                               _VP, _VP, _I64, _VP, _I64, _I32, _INT, _VP]),
     "dq8_qgemm_kernel_name": (C.c_char_p, [_I64, _I64, _I64, _INT]),
     "dq8_weight_only_undo_compiler_layout": (_INT, [_VP, _VP, _I64, _I64, _VP]),
     "dq8_fake_quant": (_INT, [_VP, _VP, _I64, _I64, _I64, _VP, _VP, _I64, _I32, _I32, _INT, _VP]),

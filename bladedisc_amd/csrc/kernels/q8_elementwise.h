@@ -28,6 +28,56 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
          ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
 }
 
+// mhlo_disc.quantize of one element (R disc/transforms/disc_lower_quantize_and_dequantize.cc
+// :77-94): divide, add the zero point, round, clamp, convert -- each a separately rounded f32
+// operation (every file that includes this is compiled with -ffp-contract=off), the division
+// a true IEEE division.  ROUND: 1 = half to even, 0 = half away from zero.
+template <int ROUND>
+__device__ __forceinline__ int quant_one(float x, float s, float z, float lo, float hi) {
+  float t0 = x / s;
+  float t1 = t0 + z;
+  float t2 = ROUND == 1 ? rintf(t1) : roundf(t1);
+  float t3 = fminf(fmaxf(t2, lo), hi);  // clamp; NaN -> lo like the CPU loop
+  return (int)t3;
+}
+
+// Four quotients x / s for a divisor that is the same for a whole kernel, from its reciprocal
+// y = 1.0f / s (a true division, done once): q0 = x y, r = fma(-q0, s, x), q = fma(r, y, q0).
+// With y correctly rounded and q0 within an ulp of the quotient, r is exact and q is the
+// correctly rounded x / s (Markstein's correction step) as long as nothing under- or
+// overflows; the caller guarantees 2^-40 <= |s| <= 2^40, and an infinite or NaN x, or a q0
+// that overflows, ends as NaN, in which case the four are divided for real.  Checked against
+// x / s on the CPU for every one of the 2^32 values of x and 18 divisors (powers of two, all-ones
+// and 1 + ulp significands, negative, 2^-23 .. 2^23): the same bits wherever 1/8 <= |x / s| <=
+// 1024 and the same int8 after rounding (either mode) and clamping everywhere else
+// (tests/native/div_by_constant_check.c runs a sample of that).
+__device__ __forceinline__ float4 div4_by_constant(const float4& x, float s, float y) {
+  float4 q;
+  {
+    const float a = x.x * y, b = x.y * y, c = x.z * y, d = x.w * y;
+    q.x = __builtin_fmaf(__builtin_fmaf(-a, s, x.x), y, a);
+    q.y = __builtin_fmaf(__builtin_fmaf(-b, s, x.y), y, b);
+    q.z = __builtin_fmaf(__builtin_fmaf(-c, s, x.z), y, c);
+    q.w = __builtin_fmaf(__builtin_fmaf(-d, s, x.w), y, d);
+  }
+  const float probe = (q.x + q.y) + (q.z + q.w);   // NaN if any is NaN (or +inf meets -inf)
+  if (__builtin_expect(!(probe == probe) || __builtin_fabsf(probe) == __builtin_inff(), 0)) {
+    q.x = x.x / s;
+    q.y = x.y / s;
+    q.z = x.z / s;
+    q.w = x.w / s;
+  }
+  return q;
+}
+
+// quant_one from the quotient on (zero point 0)
+template <int ROUND>
+__device__ __forceinline__ int quant_from_quotient(float t0, float lo, float hi) {
+  float t2 = ROUND == 1 ? rintf(t0) : roundf(t0);
+  float t3 = fminf(fmaxf(t2, lo), hi);
+  return (int)t3;
+}
+
 template <bool SIGNED>
 __device__ __forceinline__ int4 unpack4(uint32_t w) {
   if (SIGNED)

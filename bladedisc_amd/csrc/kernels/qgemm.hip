@@ -270,7 +270,8 @@ mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* 
 // (qgemm_launch.h; every launch_variant<CONV, EPI> is instantiated in a qgemm_launch_*.hip)
 }  // namespace
 #define DQ8_DECLARE_LAUNCH(CONV, EPI) \
-  extern template int launch_variant<CONV, EPI>(int, MainParams&, hipStream_t);
+  extern template int launch_variant<CONV, EPI>(int, MainParams&, hipStream_t); \
+  extern template int launch_f32a<CONV, EPI>(const MainParams&, hipStream_t);
 DQ8_DECLARE_LAUNCH(false, DQ8_EPI_ACC_S32)
 DQ8_DECLARE_LAUNCH(false, DQ8_EPI_REQUANT_CPU)
 DQ8_DECLARE_LAUNCH(false, DQ8_EPI_REQUANT_GPU)
@@ -842,6 +843,91 @@ extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t 
   return dq8_qgemm_variant(-1, A, lda, W, ldw, out, ldo, M, N, K, tp_a, tp_b, epilogue,
                            bias, bias_kind, sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo,
                            workspace, workspace_bytes, stream);
+}
+
+// ---- quantize -> qgemm as one operator ---------------------------------------------------
+extern "C" int64_t dq8_qlinear_f32_fused_max_rows(int64_t N, int64_t K) {
+  // A workgroup takes 16 rows x 16 channels, and every workgroup along N quantizes its 16 rows
+  // again.  That is cheaper than a quantize launch of its own (about 2.2 us) while the
+  // workgroups come to at most one and a half per compute unit: measured against
+  // dq8_quantize + dq8_qgemm (launches replayed from a graph), 64 x 768 -> 768: 5.4 against
+  // 7.9 us; 128 rows: 7.5 against 8.1; 256 rows: 10.3 against 8.3; 64 x 768 -> 3072: 10.3
+  // against 8.0; 64 x 3072 -> 768: 9.9 against 11.4.
+  if (N <= 0 || N >= (1LL << 31) || K < 16 || K % 16 != 0) return 0;
+  const int64_t blocks = (3 * (int64_t)compute_units() / 2) / ceil_div(N, 16);
+  return std::min<int64_t>(16 * blocks, 256);
+}
+
+extern "C" int dq8_qlinear_f32(const float* X, int64_t ldx, const int8_t* W, int64_t ldw, void* out,
+                               int64_t ldo, int64_t M, int64_t N, int64_t K, int epilogue,
+                               const void* bias, int bias_kind, const float* sx, const float* sw,
+                               int64_t n_sw, const float* so, int64_t n_so, int32_t zo,
+                               int round_mode, void* stream) {
+  clear_error();
+  DQ8_REQUIRE(M >= 0 && N >= 0 && K >= 0, "dq8_qlinear_f32: negative size");
+  DQ8_REQUIRE(M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31), "dq8_qlinear_f32: 2^31 limit");
+  DQ8_REQUIRE(round_mode == DQ8_ROUND_HALF_TO_EVEN || round_mode == DQ8_ROUND_HALF_AWAY_FROM_ZERO,
+              "dq8_qlinear_f32: unknown round_mode");
+  DQ8_REQUIRE(epilogue != DQ8_EPI_REQUANT_FIXEDPOINT,
+              "dq8_qlinear_f32: the fixed-point stage is not offered here");
+  if (M == 0 || N == 0) return 0;
+  DQ8_REQUIRE(X && sx, "dq8_qlinear_f32: null activations or scale");
+  DQ8_REQUIRE(ldx >= K, "dq8_qlinear_f32: leading dimension smaller than the row length");
+  hipStream_t st = (hipStream_t)stream;
+  DQ8_REQUIRE(M <= dq8_qlinear_f32_fused_max_rows(N, K),
+              "dq8_qlinear_f32: more rows than dq8_qlinear_f32_fused_max_rows() (or K % 16 != 0): "
+              "run dq8_quantize and dq8_qgemm");
+  DQ8_REQUIRE(aligned(X, 16) && ldx % 4 == 0 && aligned(W, 16) && ldw % 16 == 0,
+              "dq8_qlinear_f32: rows of X and W must be 16-byte aligned");
+  // the same validation and epilogue set-up as dq8_qgemm
+  int requant = 0;
+  if (epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 || epilogue == DQ8_EPI_REQUANT_GPU_DEQUANT_F32) {
+    requant = epilogue == DQ8_EPI_REQUANT_CPU_DEQUANT_F32 ? 1 : 2;
+    epilogue = requant == 1 ? DQ8_EPI_REQUANT_CPU : DQ8_EPI_REQUANT_GPU;
+  }
+  if (int s = check_epilogue("dq8_qlinear_f32", epilogue, bias, bias_kind, sx, sw, so, 1, n_sw,
+                             n_so, N))
+    return s;
+  DQ8_REQUIRE(zo == 0 || epilogue == DQ8_EPI_REQUANT_CPU,
+              "dq8_qlinear_f32: an output zero point needs the REQUANT_CPU epilogue");
+  if (requant) epilogue = DQ8_EPI_DEQUANT_F32;
+  DQ8_REQUIRE(out != nullptr && W != nullptr, "dq8_qlinear_f32: null pointer");
+  DQ8_REQUIRE(ldw >= K && ldo >= N, "dq8_qlinear_f32: leading dimension smaller than the row length");
+  MainParams p = {};
+  p.A = reinterpret_cast<const int8_t*>(X);
+  p.W = W;
+  p.lda = ldx;
+  p.ldw = ldw;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.K = (int)K;
+  p.a_scale = sx;
+  p.a_round_even = round_mode == DQ8_ROUND_HALF_TO_EVEN;
+  EpiParams& e = p.epi;
+  e.out = out;
+  e.ldo = ldo;
+  e.M = (int)M;
+  e.N = (int)N;
+  e.bias = bias;
+  e.bias_kind = bias_kind;
+  e.sx = sx;
+  e.sw = sw;
+  e.so = so;
+  e.sx_stride = 0;
+  e.sw_stride = n_sw > 1;
+  e.so_stride = n_so > 1;
+  e.zo = zo;
+  e.requant = requant;
+  const int es = elem_size(epilogue);
+  e.vec_store = aligned(out, 4 * es) && (ldo % 4 == 0);
+  e.vec_store16 = aligned(out, 16) && (ldo % 16 == 0);
+  switch (epilogue) {
+    case DQ8_EPI_ACC_S32: return launch_f32a<false, DQ8_EPI_ACC_S32>(p, st);
+    case DQ8_EPI_REQUANT_CPU: return launch_f32a<false, DQ8_EPI_REQUANT_CPU>(p, st);
+    case DQ8_EPI_REQUANT_GPU: return launch_f32a<false, DQ8_EPI_REQUANT_GPU>(p, st);
+    case DQ8_EPI_DEQUANT_F32: return launch_f32a<false, DQ8_EPI_DEQUANT_F32>(p, st);
+  }
+  return fail("dq8_qlinear_f32: unknown epilogue");
 }
 
 namespace {

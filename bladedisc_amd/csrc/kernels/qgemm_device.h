@@ -86,6 +86,11 @@ struct MainParams {
   // output (m, n) starts at corr_n[n] + corr_m[m] instead of 0.
   const int32_t* corr_n;
   const int32_t* corr_m;
+  // f32 activations quantized on their way into the matrix cores (qgemm_skinny_f32a_kernel):
+  // A then points to floats, lda counts floats, and a row is quantized per tensor with
+  // a_scale[0] (device), zero point 0, to [-128, 127] with the given rounding
+  const float* a_scale;
+  int a_round_even;
   EpiParams epi;
 };
 

@@ -166,6 +166,22 @@ int launch_skinny(const MainParams& p, hipStream_t st) {
   return deep ? launch_skinny_t<8, 4, EPI>(p, st) : launch_skinny_t<4, 4, EPI>(p, st);
 }
 
+// f32 activations quantized on load (GEMM only)
+template <bool CONV, int EPI>
+int launch_f32a(const MainParams& p, hipStream_t st) {
+  if constexpr (CONV) {
+    return fail("f32 activations: GEMM only");
+  } else {
+    const dim3 grid((unsigned)ceil_div(p.N, 16), (unsigned)ceil_div(p.M, 16));
+    DQ8_REQUIRE(grid.y <= 65535, "qgemm with f32 activations: too many rows for this kernel");
+    if (p.a_round_even)
+      hipLaunchKernelGGL((qgemm_skinny_f32a_kernel<8, EPI, 1>), grid, dim3(512), 0, st, p);
+    else
+      hipLaunchKernelGGL((qgemm_skinny_f32a_kernel<8, EPI, 0>), grid, dim3(512), 0, st, p);
+    return check_hip(hipGetLastError(), "qgemm_skinny_f32a launch");
+  }
+}
+
 template <bool CONV, int EPI>
 int launch_variant(int variant, MainParams& p, hipStream_t st) {
   const Variant& v = kVariants[variant];
@@ -200,6 +216,7 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
 #define DQ8_INSTANTIATE_LAUNCH(CONV, EPI) \
   namespace dq8 {                          \
   template int launch_variant<CONV, EPI>(int, MainParams&, hipStream_t); \
+  template int launch_f32a<CONV, EPI>(const MainParams&, hipStream_t);   \
   }
 
 #endif  // DQ8_QGEMM_LAUNCH_H_

@@ -13,6 +13,7 @@
 #ifndef DQ8_QGEMM_SKINNY_H_
 #define DQ8_QGEMM_SKINNY_H_
 
+#include "q8_elementwise.h"
 #include "qgemm_device.h"
 
 namespace dq8 {
@@ -85,6 +86,106 @@ __global__ void __launch_bounds__(NW * 64) qgemm_skinny_kernel(const MainParams 
       ((float*)ep.out)[off] = finish_f32(ep, dequant_one_any(ep, c, sum, dequant_so(ep)), m, n);
     else
       ((int8_t*)ep.out)[off] = (int8_t)finish_s8(ep, requant_one<EPI>(ep, c, sum), m, n);
+  }
+}
+
+// The same for f32 activations: mhlo_disc.quantize (per tensor, zero point 0, int8) runs on the
+// activations on their way from memory into the MFMA operand registers, so that a quantized
+// linear on a few dozen rows is one launch and the int8 activations never exist in memory.
+// 16 rows x 16 output channels per workgroup (every workgroup along N quantizes its 16 rows
+// again: the kernel is for a handful of row blocks, where that costs less than a launch);
+// a lane's 16 k-values are 64 contiguous bytes of its row.  The arithmetic is quant_one's,
+// element for element, so the result equals dq8_quantize followed by the int8 kernel.
+template <int NW, int EPI, int ROUND>
+__global__ void __launch_bounds__(NW * 64) qgemm_skinny_f32a_kernel(const MainParams p) {
+  constexpr int U = 2;  // k-steps in flight per wave (64 f32 registers of activations)
+  __shared__ int red[NW][256];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int m0 = blockIdx.y * 16;
+  const int KS = (p.K + 63) / 64;
+
+  const bool w_ok = n0 + r < p.N;
+  const int8_t* wp = p.W + (int64_t)(w_ok ? n0 + r : 0) * p.ldw + g * 16;
+  const bool a_ok = m0 + r < p.M;
+  const float* ap = reinterpret_cast<const float*>(p.A) + (int64_t)(a_ok ? m0 + r : 0) * p.lda + g * 16;
+  const float s = p.a_scale[0];
+  // (kernel-uniform) the division by the scale through its reciprocal, see div4_by_constant
+  const float y = 1.0f / s;
+  const bool fast = __builtin_fabsf(s) >= 0x1p-40f && __builtin_fabsf(s) <= 0x1p40f;
+
+  // the output this thread finishes after the reduction, and its per-channel factors, fetched
+  // now so that they arrive behind the operands instead of after the barrier
+  const int e_m = m0 + ((threadIdx.x & 255) >> 4), e_n = n0 + (threadIdx.x & 15);
+  const ColParams e_c = col_params<EPI>(p.epi, e_n < p.N ? e_n : p.N - 1);
+  const float e_so = EPI == DQ8_EPI_DEQUANT_F32 ? dequant_so(p.epi) : 0.0f;
+
+  v4i acc = {0, 0, 0, 0};
+  const v4i zero = {0, 0, 0, 0};
+  for (int ks0 = wave; ks0 < KS; ks0 += NW * U) {
+    // Loads are unconditional (a branch around each would serialise them): a lane whose chunk
+    // lies past K, or whose row lies past M / N, reads a valid address instead -- chunk 0 of
+    // its (clamped) row -- and its operand is zeroed afterwards.
+    v4i wf[U];
+    float4 xf[U][4];
+    bool in[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = (ks0 + u * NW) * 64;
+      in[u] = k + g * 16 < p.K;              // K % 16 == 0: a lane's 16 k are all in or all out
+      const int kk = in[u] ? k : -g * 16;
+      wf[u] = *(const v4i*)(wp + kk);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) xf[u][c] = *(const float4*)(ap + kk + 4 * c);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      using elementwise::pack4;
+      using elementwise::quant_one;
+      v4i af;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float4 v = xf[u][c];
+        if (fast) {
+          using elementwise::quant_from_quotient;
+          const float4 t = elementwise::div4_by_constant(v, s, y);
+          af[c] = (int)pack4(quant_from_quotient<ROUND>(t.x, -128.f, 127.f),
+                             quant_from_quotient<ROUND>(t.y, -128.f, 127.f),
+                             quant_from_quotient<ROUND>(t.z, -128.f, 127.f),
+                             quant_from_quotient<ROUND>(t.w, -128.f, 127.f));
+        } else {
+          af[c] = (int)pack4(quant_one<ROUND>(v.x, s, 0.f, -128.f, 127.f),
+                             quant_one<ROUND>(v.y, s, 0.f, -128.f, 127.f),
+                             quant_one<ROUND>(v.z, s, 0.f, -128.f, 127.f),
+                             quant_one<ROUND>(v.w, s, 0.f, -128.f, 127.f));
+        }
+      }
+      if (!(in[u] && a_ok)) af = zero;
+      if (!(in[u] && w_ok)) wf[u] = zero;
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u], af, acc, 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[wave][r * 16 + 4 * g + v] = acc[v];
+  __syncthreads();
+
+  if (threadIdx.x < 256 && e_m < p.M && e_n < p.N) {
+    const int e = threadIdx.x;
+    int sum = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += red[w][e];
+    const EpiParams& ep = p.epi;
+    const int64_t off = (int64_t)e_m * ep.ldo + e_n;
+    if (EPI == DQ8_EPI_ACC_S32)
+      ((int32_t*)ep.out)[off] = sum;
+    else if (EPI == DQ8_EPI_DEQUANT_F32)
+      ((float*)ep.out)[off] = finish_f32(ep, dequant_one_any(ep, e_c, sum, e_so), e_m, e_n);
+    else
+      ((int8_t*)ep.out)[off] = (int8_t)finish_s8(ep, requant_one<EPI>(ep, e_c, sum), e_m, e_n);
   }
 }
 

@@ -26,16 +26,6 @@ namespace {
 
 using namespace dq8::elementwise;
 
-template <int ROUND>
-__device__ __forceinline__ int quant_one(float x, float s, float z, float lo,
-                                         float hi) {
-  float t0 = x / s;
-  float t1 = t0 + z;
-  float t2 = ROUND == DQ8_ROUND_HALF_TO_EVEN ? rintf(t1) : roundf(t1);
-  float t3 = fminf(fmaxf(t2, lo), hi);  // clamp; NaN -> lo like the CPU loop
-  return (int)t3;
-}
-
 // ---------------------------------------------------------------- per tensor
 // One unit per thread and a grid that covers the tensor in one sweep (the loop only
 // runs again beyond 2^30 units): on this part a linear sweep by many small workgroups

@@ -313,6 +313,39 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
     return out
 
 
+def qlinear_f32_fused_max_rows(n, k):
+    return int(_lib.lib().dq8_qlinear_f32_fused_max_rows(n, k))
+
+
+def qlinear_f32(x, w, epilogue, sx, sw=None, so=None, bias=None, zo=0,
+                round_mode=ROUND_HALF_TO_EVEN, out=None):
+    """quantize(x; sx, zero point 0) -> qgemm(., w [N,K]) with the given epilogue, one launch,
+    for a few rows of f32 activations x [M,K]; the same bits as quantize followed by qgemm."""
+    _need_cuda(x, w, bias)
+    L = _lib.lib()
+    if x.dim() != 2 or x.stride(1) != 1:
+        x = x.reshape(-1, x.shape[-1]).contiguous()
+    if w.dim() != 2 or w.stride(1) != 1:
+        w = w.contiguous()
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k:
+        raise ValueError("mismatch contraction dim")
+    dev = x.device
+    if out is None:
+        out = torch.empty((m, n), dtype=_OUT_DTYPE[epilogue], device=dev)
+    sx = _scale(sx, dev)
+    sw = _scale(sw, dev) if sw is not None else None
+    so = _scale(so, dev) if so is not None else None
+    bias_kind = BIAS_NONE if bias is None else _BIAS_KIND[bias.dtype]
+    st = L.dq8_qlinear_f32(_ptr(x), max(x.stride(0), k), _ptr(w), max(w.stride(0), k), _ptr(out),
+                           out.stride(0) if m else n, m, n, k, epilogue, _ptr(bias), bias_kind,
+                           _ptr(sx), _ptr(sw), sw.numel() if sw is not None else 0,
+                           _ptr(so), so.numel() if so is not None else 0, zo, round_mode, _stream())
+    _lib.check(st, "dq8_qlinear_f32")
+    return out
+
+
 NHWC_OHWI = (0, 3, 1, 2, 3, 0, 1, 2, 0, 3, 1, 2)
 
 

@@ -261,6 +261,26 @@ int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
               const float* so, int64_t n_so, int32_t zx, int32_t zw, int32_t zo,
               void* workspace, size_t workspace_bytes, void* stream);
 
+/* A quantized linear on a few rows of f32 activations in ONE launch:
+ *   xq  = dq8_quantize(X; scale sx[0], zero point 0, [-128, 127], round_mode)
+ *   out = dq8_qgemm(xq, W [N,K], ..., epilogue, ...)                       bit for bit,
+ * the fused mhlo_disc.quantize in front of quantized_dot_general (R disc/transforms/
+ * disc_lower_quantize_and_dequantize.cc:77-94 emits the quantize as elementwise ops that the
+ * compiler's fusion then merges with neighbours; here it is merged into the GEMM): the
+ * activations are quantized on their way into the matrix cores and the int8 tensor is never
+ * written.  X: device f32 [M,K], row stride ldx floats; W: device int8 [N,K], row stride ldw;
+ * sx: one device f32 (also the GEMM's input scale); epilogues, bias, sw, so, zo as for
+ * dq8_qgemm (all but REQUANT_FIXEDPOINT; with REQUANT_*_DEQUANT_F32 the whole
+ * quantize -> linear -> dequantize chain is one launch).  Every workgroup along N quantizes
+ * its rows again, so this pays only for M <= dq8_qlinear_f32_fused_max_rows(N, K) (0 when
+ * K % 16 != 0); more rows are an error: run the two operators.  Rows of X and W 16-byte
+ * aligned. */
+int64_t dq8_qlinear_f32_fused_max_rows(int64_t N, int64_t K);
+int dq8_qlinear_f32(const float* X, int64_t ldx, const int8_t* W, int64_t ldw, void* out,
+                    int64_t ldo, int64_t M, int64_t N, int64_t K, int epilogue, const void* bias,
+                    int bias_kind, const float* sx, const float* sw, int64_t n_sw,
+                    const float* so, int64_t n_so, int32_t zo, int round_mode, void* stream);
+
 /* Operators the compiler fuses behind a quantized GEMM or convolution (its elementwise
  * fusion around quantized_dot_general / quantized_conv, next to the graph rewrites of
  * R disc/transforms/disc_quantized_dot_merge.cc:155-456): done in the producing kernel's

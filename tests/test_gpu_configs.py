@@ -53,6 +53,13 @@ def test_config1_single_quantized_linear(K, C):
     np.testing.assert_allclose(y, ref_y, rtol=REL_TOL_F32, atol=0)
     # and it approximates the fp32 linear to quantisation accuracy
     assert np.abs(y - c["y_fp32"]).max() < 4 * float(c["so"])
+    # the whole chain as one launch (quantize on load, dequantize in the epilogue): the same bits
+    y1 = K.qlinear_f32(dev(c["x"]), dev(c["w_q"]), K.EPI_REQUANT_CPU_DEQUANT_F32, f1(c["sx"]),
+                       dev(c["sw"]), f1(c["so"]), bias=dev(c["bias"])).cpu().numpy()
+    np.testing.assert_array_equal(y1, ref_y)
+    yq1 = K.qlinear_f32(dev(c["x"]), dev(c["w_q"]), K.EPI_REQUANT_CPU, f1(c["sx"]), dev(c["sw"]),
+                        f1(c["so"]), bias=dev(c["bias"])).cpu().numpy()
+    np.testing.assert_array_equal(yq1, ref_yq)
     # E3: int32 accumulators dequantized directly, against a float64 closed form
     y3 = K.qgemm(x_q, dev(c["w_q"]), K.EPI_DEQUANT_F32, sx=f1(c["sx"]), sw=dev(c["sw"]),
                  bias=dev(c["bias"])).cpu().numpy()

@@ -1161,6 +1161,72 @@ def test_bad_arguments_fail_loudly(K):
     assert st != 0 and b"negative" in L.dq8_last_error()
 
 
+@pytest.mark.parametrize("m,k,n", [(64, 768, 768), (1, 768, 768), (16, 768, 3072), (33, 3072, 768),
+                                   (128, 768, 768), (7, 80, 24), (50, 1024, 200), (32, 768, 2304)])
+@pytest.mark.parametrize("epi_name", ["REQUANT_CPU", "REQUANT_GPU", "REQUANT_CPU_DEQUANT_F32",
+                                      "DEQUANT_F32", "ACC_S32"])
+def test_qlinear_f32_equals_quantize_then_qgemm(K, m, k, n, epi_name):
+    """The one-launch quantized linear on f32 activations against the oracle's quantize ->
+    gemm -> epilogue and against the library's own two operators: the same bits.  Activations
+    include exact rounding ties (multiples of scale / 2), values beyond the int8 range, zeros,
+    and infinities; both rounding modes.  (A NaN activation is compared between the two forms of
+    the library only: the reference leaves its quantized value undefined.)"""
+    rng = np.random.default_rng(m + k + n)
+    sx = np.float32(rng.uniform(0.01, 0.05))
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    ties = rng.integers(-300, 300, x.shape).astype(np.float32) * np.float32(0.5) * sx
+    x = np.where(rng.random(x.shape) < 0.1, ties, x).astype(np.float32)
+    x.flat[0] = 0.0
+    if x.size > 8:
+        x.flat[3], x.flat[4] = np.inf, -np.inf
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    sw = rng.uniform(0.001, 0.05, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    epi = getattr(K, "EPI_" + epi_name)
+    for round_mode in (K.ROUND_HALF_TO_EVEN, K.ROUND_HALF_AWAY_FROM_ZERO):
+        xq = O.quantize(x, sx, 0, round_mode=round_mode)
+        acc = O.gemm_s32(xq, w, tp_b=True)
+        so = pick_so(acc, sx, sw)
+        b = None if epi_name == "ACC_S32" else bias
+        got = K.qlinear_f32(dev(x), dev(w), epi, dev(np.array([sx])), dev(sw), dev(np.array([so])),
+                            bias=dev(b) if b is not None else None, round_mode=round_mode)
+        dxq = K.quantize(dev(x), dev(np.array([sx])), dev(np.zeros(1, np.int32)), round_mode=round_mode)
+        np.testing.assert_array_equal(host(dxq), xq)
+        two = K.qgemm(dxq, dev(w), epi, sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])),
+                      bias=dev(b) if b is not None else None)
+        np.testing.assert_array_equal(host(got).view(np.uint8), host(two).view(np.uint8))
+        if x.size > 8:
+            xn = x.copy()
+            xn.flat[6] = np.nan
+            args = (dev(w), epi, dev(np.array([sx])), dev(sw), dev(np.array([so])))
+            got_n = K.qlinear_f32(dev(xn), *args, bias=dev(b) if b is not None else None,
+                                  round_mode=round_mode)
+            xnq = K.quantize(dev(xn), dev(np.array([sx])), dev(np.zeros(1, np.int32)), round_mode=round_mode)
+            two_n = K.qgemm(xnq, dev(w), epi, sx=args[2], sw=args[3], so=args[4],
+                            bias=dev(b) if b is not None else None)
+            np.testing.assert_array_equal(host(got_n).view(np.uint8), host(two_n).view(np.uint8))
+        if epi_name == "REQUANT_CPU":
+            want = O.requant_cpu(acc, sx, sw, so, b32=O.bias_f32_to_s32(bias, sx, sw))
+        elif epi_name == "REQUANT_GPU":
+            want = O.requant_gpu(acc, sx, sw, so, bias_f32=bias)
+        elif epi_name == "ACC_S32":
+            want = acc
+        else:
+            continue
+        np.testing.assert_array_equal(host(got), want)
+
+
+def test_qlinear_f32_refuses_more_rows_than_it_pays_for(K):
+    n, k = 768, 768
+    rows = K.qlinear_f32_fused_max_rows(n, k)
+    assert 64 <= rows <= 256 and K.qlinear_f32_fused_max_rows(n, 100) == 0
+    x = torch.zeros((rows + 1, k), device="cuda")
+    w = torch.zeros((n, k), dtype=torch.int8, device="cuda")
+    one = torch.ones(1, device="cuda")
+    with pytest.raises(RuntimeError, match="fused_max_rows"):
+        K.qlinear_f32(x, w, K.EPI_ACC_S32, one)
+
+
 def _weight_only_case(rng, m, k, n, dtype, signed):
     npdt = np.float16 if dtype == torch.float16 else np.float32
     x = rng.standard_normal((m, k)).astype(npdt)

@@ -28,3 +28,17 @@ def test_parsers_under_asan_ubsan(tmp_path):
     run = subprocess.run([exe, str(scratch)], capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stdout + run.stderr
     assert run.stdout.strip().endswith("ok"), run.stdout + run.stderr
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="needs gcc")
+def test_division_by_a_kernel_constant_matches_true_division(tmp_path):
+    """The quotient the one-launch quantized linear forms from the scale's reciprocal and two
+    fused multiply-adds (tests/native/div_by_constant_check.c restates it) against x / s: a
+    strided sample of all x, every x around the rounding ties of the int8 result, 40 divisors."""
+    exe = str(tmp_path / "div_by_constant_check")
+    build = subprocess.run(["gcc", "-O2", "-fopenmp", "-ffp-contract=off", "-o", exe,
+                            os.path.join(ROOT, "tests", "native", "div_by_constant_check.c"), "-lm"],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([exe, "2053"], capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0 and run.stdout.strip() == "ok", run.stdout + run.stderr
