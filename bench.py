@@ -430,12 +430,12 @@ def config_reports(torch, K):
         # GELU -> quantize between the FFN linears as one 256-entry table lookup on the int8
         # tensor; with each trailing dequantize done in its GEMM's epilogue as well; and with
         # the table and both residual additions in the epilogues too (all bit-identical)
-        def replay_us(**flags):
+        def replay_us(layer=layer, stream=None, **flags):
             saved = {k: getattr(layer, k) for k in flags}
             try:
                 for k, v in flags.items():
                     setattr(layer, k, v)
-                replay, _, _ = layer.capture(h)
+                replay, _, _ = layer.capture(h, stream=stream)
                 for _ in range(3):
                     replay()
                 torch.cuda.synchronize()
@@ -459,6 +459,22 @@ def config_reports(torch, K):
         fused_us = replay_us(fuse_gelu=True)
         fused2_us = replay_us(fuse_gelu=True, fuse_dequant=True)
         fused3_us = replay_us(fuse_gelu=True, fuse_dequant=True, fuse_epilogue=True)
+        # the same through the RAL entries (the plugin path): results from the context's pool,
+        # the fused forms as ral_pdll_qgemm_fused
+        from bladedisc_amd import ral
+        rstream = torch.cuda.Stream()
+        rctx = ral.RalContext(stream=rstream.cuda_stream)
+        rex = rctx.execution()
+        try:
+            rlayer = B.QuantBertLayer(weights, B.RalBackend(rex))
+            rlayer.calibrate(h)
+            ral_graph_us = replay_us(layer=rlayer, stream=rstream)
+            ral_fused3_us = replay_us(layer=rlayer, stream=rstream, fuse_gelu=True,
+                                      fuse_dequant=True, fuse_epilogue=True)
+        finally:
+            torch.cuda.synchronize()
+            rex.close()
+            rctx.close()
         bert["seq%d" % seq] = {"linears_q_gemm_dq": per,
                                "quantized_ops_gpu_us": round(gpu_sum * 1e6, 2),
                                "quantized_ops_cpu_us": round(cpu_sum * 1e6, 1),
@@ -466,7 +482,9 @@ def config_reports(torch, K):
                                "layer_graph_replay_us": graph_us,
                                "layer_graph_replay_fused_gelu_table_us": fused_us,
                                "layer_graph_replay_fused_gelu_table_and_dequantize_us": fused2_us,
-                               "layer_graph_replay_fused_epilogues_us": fused3_us}
+                               "layer_graph_replay_fused_epilogues_us": fused3_us,
+                               "layer_graph_replay_ral_entries_us": ral_graph_us,
+                               "layer_graph_replay_ral_entries_fused_epilogues_us": ral_fused3_us}
     rep["5_bert_base_layer_batch8"] = bert
     return rep
 

@@ -78,6 +78,18 @@ class RalBackend:
         return ral_ops.pdll_qgemm_cpu_style(self.ex, x_q, w_q, bias, sx, sw, so,
                                             transpose_b=True, weight_is_const=True)
 
+    def qlinear_dequantized(self, x_q, w_q, bias, sx, sw, so):
+        return ral_ops.pdll_qgemm_fused(self.ex, x_q, w_q, bias, sx, sw, so, transpose_b=True,
+                                        weight_is_const=True)
+
+    def qlinear_table(self, x_q, w_q, bias, sx, sw, so, table):
+        return ral_ops.pdll_qgemm_fused(self.ex, x_q, w_q, bias, sx, sw, so, transpose_b=True,
+                                        weight_is_const=True, table=table)
+
+    def qlinear_dequantized_residual(self, x_q, w_q, bias, sx, sw, so, residual):
+        return ral_ops.pdll_qgemm_fused(self.ex, x_q, w_q, bias, sx, sw, so, transpose_b=True,
+                                        weight_is_const=True, residual=residual)
+
     def lut8(self, q, table):
         # a compiled program would carry this as one of its own generated kernels; the
         # runtime has no entry for it
@@ -93,13 +105,13 @@ class QuantBertLayer:
 
     def __init__(self, weights, backend, heads=12, device="cuda", fuse_gelu=False,
                  fuse_dequant=False, fuse_epilogue=False):
-        """fuse_dequant (raw backend): a linear whose int8 result is only dequantized writes
+        """fuse_dequant: a linear whose int8 result is only dequantized writes
         the dequantized f32 from the GEMM's epilogue (same bits, no int8 round trip).
         fuse_gelu: run dequantize -> GELU -> quantize between the two FFN linears as one
         256-entry table lookup on the int8 tensor (what the compiler's fusion of those three
         elementwise operators amounts to); the result is bit-identical to the three separate
         operators because the table is built by running exactly them on all 256 inputs.
-        fuse_epilogue (raw backend): the operators behind three of the linears run in the
+        fuse_epilogue: the operators behind three of the linears run in the
         GEMM's epilogue -- the residual additions behind the attention output and FFN2
         (dequantize + add, f32 out) and the GELU table behind FFN1 -- again the same bits."""
         self.fuse_gelu = fuse_gelu or fuse_epilogue
@@ -233,21 +245,37 @@ class QuantBertLayer:
             rec["ffn2"] = dict(x_q=x2_q, y_q=y2_q, y=y2)
         return y2.reshape(*shape[:-1], y2.shape[-1])
 
-    def capture(self, h):
+    def capture(self, h, stream=None):
         """Records one forward pass on `h`'s shape into a HIP graph and returns
         (replay, static_input, static_output): copy new activations into static_input,
         call replay(), read static_output.  A BERT layer at small batch x seq is a few
         dozen short kernels, and launching them one by one from the host takes longer
-        than running them; a graph replays them back to back.  Only the raw backend can be
-        captured (its kernels take preallocated outputs; the RAL entries allocate theirs)."""
-        if not isinstance(self.be, RawBackend):
-            raise RuntimeError("graph capture needs the raw backend")
+        than running them; a graph replays them back to back.  With the RAL backend the
+        context must be bound to `stream` (pass the stream it was created on): its entries
+        allocate their results from the context's pool, which the warm-up passes fill, so
+        nothing is allocated from the device while capturing; the execution must stay open
+        for as long as the graph is replayed (it owns the buffers the graph writes)."""
         static_in = h.clone()
-        side = torch.cuda.Stream()
+        if isinstance(self.be, RalBackend) and stream is None:
+            raise RuntimeError("capture with the RAL backend needs the stream its context is bound to")
+        side = stream if stream is not None else torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):        # warm-up on the capture stream
-            for _ in range(2):
-                self.forward(static_in)
+            if isinstance(self.be, RalBackend):
+                # in an execution of its own: when it ends, its buffers go back to the
+                # context's pool, where the captured pass finds them
+                keep = self.be.ex
+                self.be.ex = keep.ctx.execution()
+                try:
+                    for _ in range(2):
+                        self.forward(static_in)
+                    side.synchronize()
+                finally:
+                    self.be.ex.close()
+                    self.be.ex = keep
+            else:
+                for _ in range(2):
+                    self.forward(static_in)
         torch.cuda.current_stream().wait_stream(side)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
@@ -260,8 +288,6 @@ class QuantBertLayer:
         qkv = self._qlinear("qkv", h, record)
         ctx = self.attention(qkv)
         if self.fuse_epilogue:
-            if not isinstance(self.be, RawBackend):
-                raise RuntimeError("fused epilogues need the raw backend")
             pre1 = self._qlinear_residual("out", ctx, h, record)
             h1 = _layer_norm(pre1, self.f["ln1_g"], self.f["ln1_b"])
             pre2 = self._ffn_fused(h1, record)       # h1 + ffn2(gelu(ffn1(h1)))

@@ -192,7 +192,7 @@ struct Epilogue {
 // Launches the GEMM, providing scratch (or the cached packed weight) for
 // operands that are not k-contiguous.
 void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const Epilogue& e,
-             int8_t* out, const char* who) {
+             void* out, const char* who, const dq8_postops_t* post = nullptr) {
   GPUDriver* drv = driverOf(ctx);
   if (!drv) return;
   void* stream = drv->asCUStream(ctx, stream_handle);
@@ -227,9 +227,9 @@ void runGemm(ExecutionContext* ctx, void* stream_handle, GemmOperands op, const 
     if (!ws) return;
   }
   StreamTimer timer(stream);
-  int st = dq8_qgemm(op.a, lda, op.w, ldw, out, op.n, op.m, op.n, op.k, op.tp_a, op.tp_b,
-                     e.mode, e.bias, e.bias_kind, e.sx, e.n_sx, e.sw, e.n_sw, e.so, e.n_so,
-                     op.zx, op.zw, e.zo, ws, ws_bytes, stream);
+  int st = dq8_qgemm_fused(op.a, lda, op.w, ldw, out, op.n, op.m, op.n, op.k, op.tp_a, op.tp_b,
+                           e.mode, e.bias, e.bias_kind, e.sx, e.n_sx, e.sw, e.n_sw, e.so, e.n_so,
+                           op.zx, op.zw, e.zo, ws, ws_bytes, post, stream);
   if (timer.on() && st == 0) {
     const double ns = timer.stop();
     const int64_t bytes = op.m * op.k + op.k * op.n + op.m * op.n;
@@ -369,9 +369,9 @@ namespace {
 // Flattens the leading dims of a rank-N input into M and allocates the result
 // through the driver.  Returns false (with `result` describing a null buffer of
 // the right shape) when there is nothing to compute.
-template <int N>
-bool prepareResult(ExecutionContext* ctx, const MemRefType<int8_t, N>& input, int64_t n,
-                   int64_t* m, MemRefType<int8_t, N>* result) {
+template <int N, typename InT = int8_t, typename OutT = int8_t>
+bool prepareResult(ExecutionContext* ctx, const MemRefType<InT, N>& input, int64_t n,
+                   int64_t* m, MemRefType<OutT, N>* result) {
   int64_t sizes[N];
   *m = 1;
   for (int i = 0; i < N - 1; ++i) {
@@ -380,16 +380,16 @@ bool prepareResult(ExecutionContext* ctx, const MemRefType<int8_t, N>& input, in
   }
   sizes[N - 1] = n;
   if (*m == 0 || n == 0) {
-    *result = assignMemRef<int8_t, N>(nullptr, sizes);
+    *result = assignMemRef<OutT, N>(nullptr, sizes);
     return false;
   }
   GPUDriver* drv = driverOf(ctx);
   if (!drv) {
-    *result = assignMemRef<int8_t, N>(nullptr, sizes);
+    *result = assignMemRef<OutT, N>(nullptr, sizes);
     return false;
   }
-  void* data = drv->alloc(ctx, (size_t)(*m * n));
-  *result = assignMemRef<int8_t, N>(data, sizes);
+  void* data = drv->alloc(ctx, (size_t)(*m * n) * sizeof(OutT));
+  *result = assignMemRef<OutT, N>(data, sizes);
   return data != nullptr;
 }
 
@@ -520,21 +520,30 @@ namespace {
 
 struct NoBias {};
 
-template <int N>
-MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_handle,
-                                        MemRefType<int8_t, N> input,
-                                        MemRefType<int8_t, 2> weight, const void* bias,
-                                        int64_t n_bias, int bias_kind,
-                                        MemRefType<float, 0> inputScales,
-                                        MemRefType<int32_t, 0> inputZeroPoints,
-                                        MemRefType<float, 1> weightScales,
-                                        MemRefType<int32_t, 1> weightZeroPoints,
-                                        MemRefType<float, 0> resultScales,
-                                        MemRefType<int32_t, 0> resultZeroPoints,
-                                        void* customAttrs, int stage = DQ8_EPI_REQUANT_CPU) {
+// What a fused entry adds behind the requantisation (ral_pdll_qgemm_fused below).
+struct FusedTail {
+  const float* residual = nullptr;   // f32, the result's shape; null = none
+  int64_t residual_elems = 0;
+  const uint8_t* table = nullptr;    // 256 entries; null = none
+};
+
+template <int N, typename OutT = int8_t>
+MemRefType<OutT, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_handle,
+                                      MemRefType<int8_t, N> input,
+                                      MemRefType<int8_t, 2> weight, const void* bias,
+                                      int64_t n_bias, int bias_kind,
+                                      MemRefType<float, 0> inputScales,
+                                      MemRefType<int32_t, 0> inputZeroPoints,
+                                      MemRefType<float, 1> weightScales,
+                                      MemRefType<int32_t, 1> weightZeroPoints,
+                                      MemRefType<float, 0> resultScales,
+                                      MemRefType<int32_t, 0> resultZeroPoints,
+                                      void* customAttrs, int stage = DQ8_EPI_REQUANT_CPU,
+                                      const FusedTail* tail = nullptr) {
   static const char* who = "ral_pdll_qgemm";
   int64_t zeros[N] = {0};
-  MemRefType<int8_t, N> result = assignMemRef<int8_t, N>(nullptr, zeros);
+  MemRefType<OutT, N> result = assignMemRef<OutT, N>(nullptr, zeros);
+  bool relu = false;
   bool tp_a = false, tp_b = false, weight_is_const = false;
   if (customAttrs) {
     PDLAttr* attr = getOrParsePDLAttr(ctx, customAttrs, "ral_pdll_qgemm_gpu_cpu_style");
@@ -550,6 +559,7 @@ MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_hand
     tp_a = flag("transpose_a");
     tp_b = flag("transpose_b");
     weight_is_const = flag("weight_is_const");
+    relu = flag("relu");
   }
   if (tp_a) {
     fail(ctx, "ral_pdll_qgemm: transpose_a is not supported on gpu");
@@ -562,7 +572,7 @@ MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_hand
     fail(ctx, "mismatch contraction dim for ral_pdll_qgemm");
     return result;
   }
-  if (!prepareResult<N>(ctx, input, op.n, &op.m, &result)) return result;
+  if (!prepareResult<N, int8_t, OutT>(ctx, input, op.n, &op.m, &result)) return result;
   // One input zero point and one weight zero point, as oneDNN takes them from the
   // reference's CPU entries (ideep matmul.hpp:516-517, 548-549; the reference silently uses
   // element 0 of a weight zero-point vector -- a vector that is not uniform is refused here).
@@ -597,11 +607,208 @@ MemRefType<int8_t, N> pdllQgemmCpuStyle(ExecutionContext* ctx, void* stream_hand
   e.n_sw = weightScales.sizes[0];
   e.so = resultScales.data;
   e.zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
-  runGemm(ctx, stream_handle, op, e, result.data, who);
+  dq8_postops_t post = {};
+  if (tail) {
+    if (tail->residual) {
+      if (tail->residual_elems != op.m * op.n) {
+        fail(ctx, "ral_pdll_qgemm_fused: the residual must have the result's shape");
+        return result;
+      }
+      post.residual = tail->residual;
+      post.residual_kind = DQ8_RESIDUAL_F32;
+      post.ldr = op.n;
+      post.relu = relu ? 1 : 0;
+    }
+    post.table = tail->table;
+  }
+  runGemm(ctx, stream_handle, op, e, result.data, who, tail ? &post : nullptr);
   return result;
 }
 
 }  // namespace
+
+// ---- ral_pdll_qgemm_fused: operators the compiler's elementwise fusion leaves next to a
+// quantized GEMM, taken into the call.  No counterpart among the reference's entries (there the
+// fused elementwise kernel is generated code next to the custom call); a pattern set for this
+// runtime rewrites  dequantize(ral_pdll_qgemm(...))  [+ residual, relu]  or
+// quantize(f(dequantize(ral_pdll_qgemm(...))))  into one of these.  Operands up to
+// customAttrs are those of the CPU-style ral_pdll_qgemm with an f32 bias
+// (R context/common_context_impl_quantization.cc:1268-1423); the results are bit for bit what
+// the separate operators give.
+//   (..., attrs)                   -> f32   dequantize of the int8 result, in the epilogue
+//   (..., residual f32, attrs)     -> f32   the same + residual [, relu per attr `relu`]
+//   (..., table ui8[256], attrs)   -> int8  table[(uint8) q]: any dequantize -> f -> quantize
+template <int N>
+MemRefType<float, N> ral_pdll_qgemm_fused_dequant(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 1> bias, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, void* customAttrs) {
+  return pdllQgemmCpuStyle<N, float>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0],
+                                     DQ8_BIAS_F32, inputScales, inputZeroPoints, weightScales,
+                                     weightZeroPoints, resultScales, resultZeroPoints, customAttrs,
+                                     DQ8_EPI_REQUANT_CPU_DEQUANT_F32);
+}
+
+template <int N>
+MemRefType<float, N> ral_pdll_qgemm_fused_dequant_residual(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 1> bias, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, MemRefType<float, N> residual, void* customAttrs) {
+  int64_t zeros[N] = {0};
+  if (!isContiguous(residual)) {
+    ctx->signalError(Context::FAILURE, "ral_pdll_qgemm_fused: residual must be a dense memref");
+    return assignMemRef<float, N>(nullptr, zeros);
+  }
+  FusedTail tail;
+  tail.residual = residual.data;
+  tail.residual_elems = 1;
+  for (int i = 0; i < N; ++i) tail.residual_elems *= residual.sizes[i];
+  return pdllQgemmCpuStyle<N, float>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0],
+                                     DQ8_BIAS_F32, inputScales, inputZeroPoints, weightScales,
+                                     weightZeroPoints, resultScales, resultZeroPoints, customAttrs,
+                                     DQ8_EPI_REQUANT_CPU_DEQUANT_F32, &tail);
+}
+
+template <int N>
+MemRefType<int8_t, N> ral_pdll_qgemm_fused_table(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<int8_t, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 1> bias, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, MemRefType<uint8_t, 1> table, void* customAttrs) {
+  int64_t zeros[N] = {0};
+  if (table.sizes[0] != 256 || !table.data) {
+    ctx->signalError(Context::FAILURE, "ral_pdll_qgemm_fused: the table must have 256 entries");
+    return assignMemRef<int8_t, N>(nullptr, zeros);
+  }
+  FusedTail tail;
+  tail.table = table.data;
+  return pdllQgemmCpuStyle<N, int8_t>(ctx, stream_handle, input, weight, bias.data, bias.sizes[0],
+                                      DQ8_BIAS_F32, inputScales, inputZeroPoints, weightScales,
+                                      weightZeroPoints, resultScales, resultZeroPoints, customAttrs,
+                                      DQ8_EPI_REQUANT_CPU, &tail);
+}
+
+// ---- ral_pdll_qlinear: quantize -> ral_pdll_qgemm -> dequantize on f32 activations, the whole
+// quantized linear as one call (no counterpart among the reference's entries; a pattern set for
+// this runtime rewrites the chain the reference's patterns leave,  dequantize(ral_pdll_qgemm(
+// quantize(x), ...)),  into it).  Operands: those of the CPU-style ral_pdll_qgemm with an f32
+// bias, the input f32; the input is quantized with inputScales, zero point 0 (others are
+// refused), to int8, rounding per attr `round_mode` (0 half away from zero, 1 half to even,
+// default 1).  A few rows run as one launch (dq8_qlinear_f32); more as quantize + GEMM with the
+// int8 activations in pool scratch.  Bit for bit the three operators' result.
+template <int N>
+MemRefType<float, N> ral_pdll_qlinear(
+    ExecutionContext* ctx, void* stream_handle, MemRefType<float, N> input,
+    MemRefType<int8_t, 2> weight, MemRefType<float, 1> bias, MemRefType<float, 0> inputScales,
+    MemRefType<int32_t, 0> inputZeroPoints, MemRefType<float, 1> weightScales,
+    MemRefType<int32_t, 1> weightZeroPoints, MemRefType<float, 0> resultScales,
+    MemRefType<int32_t, 0> resultZeroPoints, void* customAttrs) {
+  static const char* who = "ral_pdll_qlinear";
+  int64_t zeros[N] = {0};
+  MemRefType<float, N> result = assignMemRef<float, N>(nullptr, zeros);
+  bool tp_b = false, weight_is_const = false;
+  int round_mode = DQ8_ROUND_HALF_TO_EVEN;
+  if (customAttrs) {
+    PDLAttr* attr = getOrParsePDLAttr(ctx, customAttrs, who);
+    if (!attr || attr->getType() != "dict") {
+      fail(ctx, "fail to parse custom_attrs\n");
+      return result;
+    }
+    auto& dict = attr->as<DictPDLAttr>();
+    auto flag = [&](const char* key) {
+      return dict.hasKey(key) && dict.get(key).getType() == "bool" &&
+             dict.get(key).as<BoolPDLAttr>().getValue();
+    };
+    if (flag("transpose_a")) {
+      fail(ctx, std::string(who) + ": transpose_a is not supported on gpu");
+      return result;
+    }
+    tp_b = flag("transpose_b");
+    weight_is_const = flag("weight_is_const");
+    if (dict.hasKey("round_mode") && dict.get("round_mode").getType() == "int")
+      round_mode = (int)dict.get("round_mode").as<IntPDLAttr>().getValue();
+  }
+  if ((inputZeroPoints.data && inputZeroPoints.data[0] != 0)) {
+    fail(ctx, std::string(who) + ": a non-zero input zero point is not supported; run "
+                                 "ral_quantize and ral_pdll_qgemm");
+    return result;
+  }
+  for (int64_t i = 0; weightZeroPoints.data && i < weightZeroPoints.sizes[0]; ++i)
+    if (weightZeroPoints.data[i] != 0) {
+      fail(ctx, std::string(who) + ": non-zero weight zero points are not supported; run "
+                                   "ral_quantize and ral_pdll_qgemm");
+      return result;
+    }
+  const int64_t k = tp_b ? weight.sizes[1] : weight.sizes[0];
+  const int64_t n = tp_b ? weight.sizes[0] : weight.sizes[1];
+  if (input.sizes[N - 1] != k && !isEmptyMemref(input)) {
+    fail(ctx, std::string(who) + ": mismatch contraction dim");
+    return result;
+  }
+  if ((weightScales.sizes[0] != 1 && weightScales.sizes[0] != n) || bias.sizes[0] != n) {
+    fail(ctx, std::string(who) + ": weight scale must have 1 or N entries, bias N");
+    return result;
+  }
+  int64_t m = 0;
+  if (!prepareResult<N, float, float>(ctx, input, n, &m, &result)) return result;
+  if (!requireContiguous(ctx, input, who, "input") ||
+      !requireContiguous(ctx, weight, who, "weight"))
+    return result;
+  GPUDriver* drv = driverOf(ctx);
+  if (!drv) return result;
+  void* stream = drv->asCUStream(ctx, stream_handle);
+  const int32_t zo = resultZeroPoints.data ? resultZeroPoints.data[0] : 0;
+  // one launch: a few rows against [N,K] weights
+  if (tp_b && k > 0 && m <= dq8_qlinear_f32_fused_max_rows(n, k) &&
+      reinterpret_cast<uintptr_t>(input.data) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(weight.data) % 16 == 0) {
+    kernelFailed(ctx,
+                 dq8_qlinear_f32(input.data, k, weight.data, k, result.data, n, m, n, k,
+                                 DQ8_EPI_REQUANT_CPU_DEQUANT_F32, bias.data, DQ8_BIAS_F32,
+                                 inputScales.data, weightScales.data, weightScales.sizes[0],
+                                 resultScales.data, 1, zo, round_mode, stream),
+                 who);
+    return result;
+  }
+  // quantize into pool scratch (the zero point 0 it needs on the device sits behind the data)
+  const size_t xq_bytes = ((size_t)(m * k) + 255) / 256 * 256;
+  auto* xq = static_cast<int8_t*>(drv->alloc(ctx, xq_bytes + 256));
+  if (!xq) return result;
+  int32_t* zero_zp = reinterpret_cast<int32_t*>(xq + xq_bytes);
+  if (kernelFailed(ctx, dq8_fill(zero_zp, 0, 4, stream), who) ||
+      kernelFailed(ctx,
+                   dq8_quantize(input.data, xq, DQ8_I8, 1, 1, m * k, inputScales.data, zero_zp, 1,
+                                -128, 127, round_mode, stream),
+                   who)) {
+    drv->dealloc(ctx, xq);
+    return result;
+  }
+  GemmOperands op;
+  op.a = xq;
+  op.w = weight.data;
+  op.m = m;
+  op.n = n;
+  op.k = k;
+  op.tp_b = tp_b;
+  op.weight_is_const = weight_is_const;
+  Epilogue e;
+  e.mode = DQ8_EPI_REQUANT_CPU_DEQUANT_F32;
+  e.bias = bias.data;
+  e.bias_kind = DQ8_BIAS_F32;
+  e.sx = inputScales.data;
+  e.sw = weightScales.data;
+  e.n_sw = weightScales.sizes[0];
+  e.so = resultScales.data;
+  e.zo = zo;
+  runGemm(ctx, stream_handle, op, e, result.data, who);
+  drv->dealloc(ctx, xq);   // (later work on the stream is ordered behind the GEMM)
+  return result;
+}
 
 template <int N>
 MemRefType<int8_t, N> ral_pdll_qgemm_s8_s8_s8_f32_per_channel(
@@ -1147,6 +1354,15 @@ TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channe
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_channel<4>);
 
 // the AArch64 build's per-tensor signatures (fixed-point output stage)
+// (fused forms: no counterpart among the reference's entries)
+TAO_RAL_API("ral_pdll_qgemm_fused", "gpu", gpu::q8::ral_pdll_qgemm_fused_dequant<2>);
+TAO_RAL_API("ral_pdll_qgemm_fused", "gpu", gpu::q8::ral_pdll_qgemm_fused_dequant<3>);
+TAO_RAL_API("ral_pdll_qgemm_fused", "gpu", gpu::q8::ral_pdll_qgemm_fused_dequant_residual<2>);
+TAO_RAL_API("ral_pdll_qgemm_fused", "gpu", gpu::q8::ral_pdll_qgemm_fused_dequant_residual<3>);
+TAO_RAL_API("ral_pdll_qgemm_fused", "gpu", gpu::q8::ral_pdll_qgemm_fused_table<2>);
+TAO_RAL_API("ral_pdll_qgemm_fused", "gpu", gpu::q8::ral_pdll_qgemm_fused_table<3>);
+TAO_RAL_API("ral_pdll_qlinear", "gpu", gpu::q8::ral_pdll_qlinear<2>);
+TAO_RAL_API("ral_pdll_qlinear", "gpu", gpu::q8::ral_pdll_qlinear<3>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<2>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<3>);
 TAO_RAL_API("ral_pdll_qgemm", "gpu", gpu::q8::ral_pdll_qgemm_s8_s8_s8_per_tensor<4>);

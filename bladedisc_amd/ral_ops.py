@@ -100,6 +100,49 @@ def pdll_qgemm_cpu_style(ex, x, w, bias, sx, sw_n, so, zo=0, transpose_b=False,
     return ral.memref_to_tensor(res, torch.int8)
 
 
+def _cpu_style_operands(ex, x, w, bias, sx, sw_n, so, zo):
+    a = ex.new_args().tensor(x).tensor(w).tensor(bias)
+    a.tensor(sx, rank0=True)
+    a.host_array(np.array([0], np.int32), rank0=True)
+    a.tensor(sw_n)
+    a.host_array(np.zeros(sw_n.numel(), np.int32))
+    a.tensor(so, rank0=True)
+    a.host_array(np.array([zo], np.int32), rank0=True)
+    return a
+
+
+def pdll_qgemm_fused(ex, x, w, bias, sx, sw_n, so, zo=0, transpose_b=False, weight_is_const=True,
+                     residual=None, relu=False, table=None):
+    """ral_pdll_qgemm_fused: the CPU-style ral_pdll_qgemm (f32 bias) with the operators that
+    follow it taken into the call -- dequantize (f32 result), dequantize + f32 residual
+    [+ relu], or a 256-entry table on the int8 result (int8 result)."""
+    a = _cpu_style_operands(ex, x, w, bias, sx, sw_n, so, zo)
+    if residual is not None:
+        a.tensor(residual)
+    elif table is not None:
+        a.tensor(table.view(torch.uint8))
+    a.blob(ral.encode_attr({"transpose_a": False, "transpose_b": bool(transpose_b),
+                            "weight_is_const": bool(weight_is_const), "bias_is_const": True,
+                            "relu": bool(relu)}))
+    int8_out = table is not None
+    res = a.result_memref("i8" if int8_out else "f32", x.dim())
+    ex.call("ral_pdll_qgemm_fused", "gpu", a)
+    return ral.memref_to_tensor(res, torch.int8 if int8_out else torch.float32)
+
+
+def pdll_qlinear(ex, x_f32, w, bias, sx, sw_n, so, zo=0, transpose_b=False, weight_is_const=True,
+                 round_mode=1):
+    """ral_pdll_qlinear: quantize -> ral_pdll_qgemm -> dequantize of f32 activations as one
+    call; f32 result."""
+    a = _cpu_style_operands(ex, x_f32, w, bias, sx, sw_n, so, zo)
+    a.blob(ral.encode_attr({"transpose_a": False, "transpose_b": bool(transpose_b),
+                            "weight_is_const": bool(weight_is_const), "bias_is_const": True,
+                            "round_mode": int(round_mode)}))
+    res = a.result_memref("f32", x_f32.dim())
+    ex.call("ral_pdll_qlinear", "gpu", a)
+    return ral.memref_to_tensor(res, torch.float32)
+
+
 def pdll_qgemm_per_tensor(ex, x, w, bias_s32, sx, sw, so, zo=0, transpose_b=False,
                           weight_is_const=True):
     """ral_pdll_qgemm with the AArch64 patterns' per-tensor signature on the gpu device

@@ -250,23 +250,52 @@ def test_config5_bert_layer_operators_in_the_gemm_epilogues_are_bit_identical(C,
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
 
 
+@pytest.mark.parametrize("backend", ["raw", "ral"])
 @pytest.mark.parametrize("fused", [False, True, "epilogue"])
-def test_config5_bert_layer_graph_replays_match_eager(C, fused):
+def test_config5_bert_layer_graph_replays_match_eager(C, fused, backend):
     """The captured layer against eager execution: several replays, with eager work and
     synchronisations in between, each compared bit for bit; also with the GELU table and the
-    dequantize-in-epilogue forms switched on."""
+    dequantize-in-epilogue forms switched on.  Through the RAL entries as well (the plugin
+    path): their results come from the context's pool, so nothing is allocated while
+    capturing, and the fused forms are the ral_pdll_qgemm_fused entries."""
     from bladedisc_amd import bert_layer as B
-    layer = B.QuantBertLayer(C.config5_weights(), B.RawBackend(), fuse_gelu=bool(fused),
-                             fuse_dequant=bool(fused), fuse_epilogue=fused == "epilogue")
-    h0 = layer.embed(C.config5_tokens(8, 32))
-    layer.calibrate(h0)
-    replay, static_in, static_out = layer.capture(h0)
-    for i in range(4):
-        h = layer.embed(C.config5_tokens(8, 32) if i == 0 else
-                        np.roll(C.config5_tokens(8, 32), i, axis=1))
-        want = layer.forward(h)                       # eager work between the replays
+    from bladedisc_amd import ral
+    ctx = ex = ex2 = stream = None
+    if backend == "ral":
+        stream = torch.cuda.Stream()
+        ctx = ral.RalContext(stream=stream.cuda_stream)
+        ex = ctx.execution()
+        be = B.RalBackend(ex)
+    else:
+        be = B.RawBackend()
+    try:
+        layer = B.QuantBertLayer(C.config5_weights(), be, fuse_gelu=bool(fused),
+                                 fuse_dequant=bool(fused), fuse_epilogue=fused == "epilogue")
+        h0 = layer.embed(C.config5_tokens(8, 32))
+        layer.calibrate(h0)
+        replay, static_in, static_out = layer.capture(h0, stream=stream)
+        if backend == "ral":          # eager passes from here on run in another execution
+            ex2 = ctx.execution()
+            be.ex = ex2
+        for i in range(4):
+            h = layer.embed(C.config5_tokens(8, 32) if i == 0 else
+                            np.roll(C.config5_tokens(8, 32), i, axis=1))
+            if stream is not None:
+                stream.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(stream):
+                    want = layer.forward(h)               # eager work between the replays
+            else:
+                want = layer.forward(h)
+            torch.cuda.synchronize()
+            static_in.copy_(h)
+            torch.cuda.synchronize()
+            replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_out, want), "replay %d differs from eager" % i
+    finally:
         torch.cuda.synchronize()
-        static_in.copy_(h)
-        replay()
-        torch.cuda.synchronize()
-        assert torch.equal(static_out, want), "replay %d differs from eager" % i
+        for e in (ex2, ex):
+            if e is not None:
+                e.close()
+        if ctx is not None:
+            ctx.close()

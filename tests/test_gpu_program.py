@@ -100,6 +100,87 @@ def test_compiled_program_runs_on_the_runtime(program):
         L.disc_ral_context_destroy(C.c_void_p(ctx))
 
 
+def test_compiled_program_captured_into_a_graph(program):
+    """A serving loop replays a compiled program from a HIP graph.  After one ordinary
+    execution (constants loaded, the context's pool holds buffers of every size the program
+    asks for) a second execution of `main` runs under stream capture -- no entry on the way may
+    allocate device memory, synchronise or copy through the host -- and the graph is replayed
+    three times on new input contents, with eager work and synchronisations in between; every
+    replay must give the oracle's bits."""
+    lib, d = program
+    from bladedisc_amd import baseline_configs as cfg
+    from bladedisc_amd import ral
+    L = ral.lib()
+    c = cfg.config1()
+    names = ["w0_i8_768x768", "b0_f32_768", "sw0_f32_768", "sx0_f32_", "so0_f32_", "z0_i32_"]
+    values = [hexstr(c["w_q"]), hexstr(c["bias"]), hexstr(c["sw"]),
+              hexstr(np.array([c["sx"]], np.float32)), hexstr(np.array([c["so"]], np.float32)),
+              hexstr(np.array([0], np.int32))]
+    meta = str(d / "captured.metadata").encode()
+    n = len(names)
+    L.disc_ral_metadata_emit.restype = C.c_int
+    assert L.disc_ral_metadata_emit(meta, n, (C.c_uint8 * n)(*([0] * n)),
+                                    (C.c_char_p * n)(*[s.encode() for s in names]),
+                                    (C.c_char_p * n)(*[v.encode() for v in values])) == 0
+    L.disc_ral_context_create_for_program.restype = C.c_void_p
+    L.disc_ral_execution_take_output.restype = C.c_void_p
+    L.disc_ral_output_data.restype = C.c_void_p
+    side = torch.cuda.Stream()
+    ctx = L.disc_ral_context_create_for_program(C.c_void_p(side.cuda_stream), 0, None, None, None,
+                                                1, meta)
+    assert ctx
+    call_impl = C.cast(L.tao_ral_call_impl, C.c_void_p).value
+    m = 48
+    x = torch.zeros((m, 768), device="cuda")
+
+    def run_main():
+        ex = L.disc_ral_execution_context_create(C.c_void_p(ctx))
+        assert L.disc_ral_execution_bind_input(C.c_void_p(ex), 0, C.c_void_p(x.data_ptr()),
+                                               (C.c_int64 * 2)(m, 768), 2) == 0
+        lib.disc_program_main((C.c_void_p * 2)(ex, call_impl))
+        msg = C.c_char_p()
+        assert L.tao_ral_last_error(C.c_void_p(ctx), C.byref(msg)) == 0, msg.value
+        out = L.disc_ral_execution_take_output(C.c_void_p(ex), 0)
+        fwd = L.disc_ral_execution_take_output(C.c_void_p(ex), 1)
+        L.disc_ral_output_destroy(C.c_void_p(fwd))
+        L.disc_ral_execution_context_destroy(C.c_void_p(ex))
+        return out
+
+    def want(xs):
+        xq = O.quantize(xs, c["sx"], 0)
+        acc = O.gemm_s32(xq, c["w_q"], tp_b=True)
+        b32 = O.bias_f32_to_s32(c["bias"], float(c["sx"]), c["sw"])
+        return O.dequantize(O.requant_cpu(acc, float(c["sx"]), c["sw"], float(c["so"]), b32=b32),
+                            c["so"], 0)
+
+    try:
+        x.copy_(torch.from_numpy(np.ascontiguousarray(c["x"][:m])))
+        side.wait_stream(torch.cuda.current_stream())
+        warm = run_main()                                   # ordinary execution: warms everything
+        side.synchronize()
+        L.disc_ral_output_destroy(C.c_void_p(warm))         # its result goes back to the pool
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            g.capture_begin()
+            out = run_main()
+            g.capture_end()
+        y = ral.device_view(L.disc_ral_output_data(C.c_void_p(out)), (m, 768), torch.float32)
+        rng = np.random.default_rng(11)
+        for rep in range(3):
+            xs = (rng.standard_normal((m, 768)) * (rep + 1)).astype(np.float32)
+            x.copy_(torch.from_numpy(xs))
+            y.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(y.cpu().numpy(), want(xs))
+        del g
+        L.disc_ral_output_destroy(C.c_void_p(out))
+    finally:
+        torch.cuda.synchronize()
+        L.disc_ral_context_destroy(C.c_void_p(ctx))
+
+
 def test_process_level_constant_store(program):
     """DISC_USE_GLOBAL_CONST_STORE=1 (common_context_impl.cc:57-64): contexts made from one
     metadata file share one store of constants, which outlives all but the last of them; without

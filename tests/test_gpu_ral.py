@@ -201,6 +201,60 @@ def test_ral_pdll_qgemm_rejects_nonzero_input_zero_point(rt):
             ex.call("ral_pdll_qgemm", "gpu", a)
 
 
+@pytest.mark.parametrize("rank", [2, 3])
+@pytest.mark.parametrize("tp_b", [True, False])
+def test_ral_pdll_qgemm_fused_and_qlinear(rt, rank, tp_b):
+    """The fused entries (they have no counterpart among the reference's): each must give, bit
+    for bit, what the separate entries give -- ral_pdll_qgemm then ral_dequantize [then an f32
+    add and a clamp at zero], a table lookup on the int8 result, and ral_quantize ->
+    ral_pdll_qgemm -> ral_dequantize for ral_pdll_qlinear, in its one-launch form (few rows) and
+    its two-launch form (many).  (The weights here are torch tensors whose addresses torch hands
+    out again, so they are not declared constants: a [K,N] weight is re-laid out per call.)"""
+    ctx, ral, ops = rt
+    from bladedisc_amd import kernels as K
+    for m, n, k in ((48, 96, 256), (600, 768, 768)):
+        rng, a, w, acc, sx, sw, so = problem(900 + m + rank, m, n, k)
+        bias = rng.standard_normal(n).astype(np.float32)
+        shape = (m,) if rank == 2 else (2, m // 2)
+        xq = dev(a.reshape(*shape, k))
+        wd = dev(w if tp_b else np.ascontiguousarray(w.T))
+        z1 = dev(np.zeros(1, np.int32))
+        with ctx.execution() as ex:
+            base_q = ops.pdll_qgemm_cpu_style(ex, xq, wd, dev(bias), f1(sx), dev(sw), f1(so),
+                                              transpose_b=tp_b, weight_is_const=False)
+            want_q = O.requant_cpu(acc, sx, sw, so, b32=O.bias_f32_to_s32(bias, sx, sw))
+            np.testing.assert_array_equal(host(base_q).reshape(m, n), want_q)
+            base_f = ops.dequantize(ex, base_q, f1(so), z1)
+            got = ops.pdll_qgemm_fused(ex, xq, wd, dev(bias), f1(sx), dev(sw), f1(so), transpose_b=tp_b, weight_is_const=False)
+            assert got.dtype == torch.float32 and tuple(got.shape) == shape + (n,)
+            np.testing.assert_array_equal(host(got), host(base_f))
+            np.testing.assert_array_equal(host(got).reshape(m, n), O.dequantize(want_q, so, 0))
+            resid = dev(rng.standard_normal(shape + (n,)).astype(np.float32))
+            for relu in (False, True):
+                got = ops.pdll_qgemm_fused(ex, xq, wd, dev(bias), f1(sx), dev(sw), f1(so),
+                                           transpose_b=tp_b, weight_is_const=False, residual=resid, relu=relu)
+                want = host(base_f) + host(resid)
+                if relu:
+                    want = np.where(want < 0, np.float32(0), want)
+                np.testing.assert_array_equal(host(got), want)
+            table = K.activation_table(torch.nn.functional.gelu, f1(so), z1, f1(np.float32(0.02)), z1)
+            got = ops.pdll_qgemm_fused(ex, xq, wd, dev(bias), f1(sx), dev(sw), f1(so),
+                                       transpose_b=tp_b, weight_is_const=False, table=table)
+            assert got.dtype == torch.int8
+            np.testing.assert_array_equal(host(got), host(K.lut8(base_q, table)))
+            # quantize -> qgemm -> dequantize on f32 activations
+            x = (a.astype(np.float32) * sx + rng.uniform(-0.4, 0.4, a.shape).astype(np.float32) * sx)
+            x = x.reshape(*shape, k)
+            xq2 = ops.quantize(ex, dev(x), f1(sx), z1)
+            want2 = ops.dequantize(ex, ops.pdll_qgemm_cpu_style(ex, xq2, wd, dev(bias), f1(sx), dev(sw),
+                                                                f1(so), transpose_b=tp_b, weight_is_const=False), f1(so), z1)
+            got2 = ops.pdll_qlinear(ex, dev(x), wd, dev(bias), f1(sx), dev(sw), f1(so), transpose_b=tp_b, weight_is_const=False)
+            np.testing.assert_array_equal(host(got2), host(want2))
+            acc2 = O.gemm_s32(O.quantize(x.reshape(m, k), sx, 0), w, tp_b=True)
+            ref2 = O.dequantize(O.requant_cpu(acc2, sx, sw, so, b32=O.bias_f32_to_s32(bias, sx, sw)), so, 0)
+            np.testing.assert_array_equal(host(got2).reshape(m, n), ref2)
+
+
 def _wo_tolerance(want, bound, k, dtype):
     return bound * (k * 2.0 ** -24 + 2.0 ** -20) + \
         (np.abs(want) + bound * 2.0 ** -12) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -22)
