@@ -7,8 +7,12 @@ import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "libdisc_q8_ral.so")
+# the same library plus the tests' entry points (tests/dq8_test_hooks.h): kernel variant
+# selection and the MFMA layout probe, which the product library does not carry
+HOOKS_LIB_PATH = os.path.join(_PKG, "libdisc_q8_testhooks.so")
 
 _lib = None
+_hooks = None
 
 _I64, _I32, _INT, _VP, _SZ = C.c_int64, C.c_int32, C.c_int, C.c_void_p, C.c_size_t
 _F32 = C.c_float
@@ -85,6 +89,33 @@ class PostOps(C.Structure):
                 ("out_scale", _VP), ("out_zp", _I32), ("table", _VP)]
 
 
+_HOOKS = ("dq8_qgemm_variant", "dq8_qgemm_num_variants", "dq8_qgemm_variant_name",
+          "dq8_qconv2d_variant", "dq8_mfma_probe")
+
+
+def _bind(L, skip=()):
+    for name, (res, args) in _PROTOS.items():
+        if name in skip:
+            continue
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    return L
+
+
+def hooks():
+    """libdisc_q8_testhooks.so: every entry of the product library (a second copy of the
+    kernels, with its own state and its own dq8_last_error) plus the tests' hooks."""
+    global _hooks
+    if _hooks is None:
+        if not os.path.exists(HOOKS_LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -m bladedisc_amd.build` "
+                "(there is no CPU fallback)" % HOOKS_LIB_PATH)
+        _hooks = _bind(C.CDLL(HOOKS_LIB_PATH))
+    return _hooks
+
+
 def lib():
     global _lib
     if _lib is None:
@@ -92,15 +123,11 @@ def lib():
             raise RuntimeError(
                 "%s is missing: build it with `python -m bladedisc_amd.build` "
                 "(there is no CPU fallback)" % LIB_PATH)
-        _lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
-        for name, (res, args) in _PROTOS.items():
-            fn = getattr(_lib, name)
-            fn.restype = res
-            fn.argtypes = args
+        _lib = _bind(C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL), skip=_HOOKS)
     return _lib
 
 
-def check(status, what):
+def check(status, what, L=None):
     if status != 0:
-        msg = lib().dq8_last_error().decode()
+        msg = (L or lib()).dq8_last_error().decode()
         raise RuntimeError("%s failed: %s" % (what, msg))

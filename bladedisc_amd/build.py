@@ -13,6 +13,12 @@ ROOT = os.path.dirname(PKG)
 CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(PKG, "build")
 LIB = os.path.join(PKG, "libdisc_q8_ral.so")
+# The same library plus the entry points of tests/dq8_test_hooks.h (kernel variant selection,
+# the MFMA layout probe): what the tests and tuning scripts load when they force a variant.
+# The product library carries none of them.
+HOOKS_LIB = os.path.join(PKG, "libdisc_q8_testhooks.so")
+HOOKS_SRC = os.path.join(CSRC, "kernels", "qgemm.hip")     # compiled a second time with the hooks
+EXPORTS = os.path.join(CSRC, "exports.map")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -52,13 +58,14 @@ def _headers_mtime():
     return m
 
 
-def _compile(src, force, hdr_m):
+def _compile(src, force, hdr_m, hooks=False):
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
-    obj = os.path.join(OBJ, rel + ".o")
+    obj = os.path.join(OBJ, rel + (".hooks.o" if hooks else ".o"))
     if (not force and os.path.exists(obj)
             and os.path.getmtime(obj) > max(os.path.getmtime(src), hdr_m)):
         return obj, ""
-    cmd = [HIPCC] + COMMON + DEVICE + ["-x", "hip", "-c", src, "-o", obj]
+    cmd = [HIPCC] + COMMON + DEVICE + (["-DDQ8_TEST_HOOKS"] if hooks else []) + \
+        ["-x", "hip", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     log = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
                     if "packed-fp32-ops" not in l)
@@ -89,18 +96,31 @@ def build(force=False, verbose=False, jobs=8):
     srcs = sources()
     hdr_m = _headers_mtime()
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        hooks_job = ex.submit(_compile, HOOKS_SRC, force, hdr_m, True)
         results = list(ex.map(lambda s: _compile(s, force, hdr_m), srcs))
-    objs = [o for o, _ in results]
+        hooks_obj, hooks_log = hooks_job.result()
+    results.append((None, hooks_log))
+    objs = [o for o, _ in results if o]
     if verbose:
         for _, log in results:
             if log.strip():
                 print(log)
     newest = max(os.path.getmtime(o) for o in objs)
+    newest = max(newest, os.path.getmtime(EXPORTS))
     if force or not os.path.exists(LIB) or os.path.getmtime(LIB) < newest:
-        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs
+        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950",
+               "-Wl,--version-script=" + EXPORTS, "-o", LIB] + objs
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
+    newest = max(newest, os.path.getmtime(hooks_obj))
+    if force or not os.path.exists(HOOKS_LIB) or os.path.getmtime(HOOKS_LIB) < newest:
+        plain = os.path.join(OBJ, os.path.relpath(HOOKS_SRC, CSRC).replace(os.sep, "_") + ".o")
+        cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", HOOKS_LIB] + \
+            [o for o in objs if o != plain] + [hooks_obj]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link of the test-hooks library failed:\n" + r.stdout + r.stderr)
     return LIB
 
 

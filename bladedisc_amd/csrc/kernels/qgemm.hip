@@ -236,6 +236,7 @@ rowsum_s8_kernel(const int8_t* __restrict__ X, int64_t ld, int rows, int K, int 
   if (lane == 0) out[row] = mul * s + add;
 }
 
+#ifdef DQ8_TEST_HOOKS
 // one MFMA of each shape, operands straight from global memory
 __global__ void __launch_bounds__(64)
 mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* a16,
@@ -265,6 +266,7 @@ mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* 
     }
   }
 }
+#endif
 
 // ------------------------------------------------------------- tile variants
 // (qgemm_launch.h; every launch_variant<CONV, EPI> is instantiated in a qgemm_launch_*.hip)
@@ -553,12 +555,14 @@ int launch_generic_epi(void (*k0)(const P), void (*k1)(const P), void (*k2)(cons
 
 using namespace dq8;
 
+#ifdef DQ8_TEST_HOOKS   // (tests/dq8_test_hooks.h; compiled into libdisc_q8_testhooks.so only)
 extern "C" int dq8_qgemm_num_variants(void) { return kNumVariants; }
 
 extern "C" const char* dq8_qgemm_variant_name(int variant) {
   if (variant < 0 || variant >= kNumVariants) return "";
   return kVariants[variant].name;
 }
+#endif
 
 extern "C" size_t dq8_qgemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int tp_a,
                                             int tp_b) {
@@ -808,6 +812,7 @@ extern "C" const char* dq8_qgemm_kernel_name(int64_t M, int64_t N, int64_t K, in
   return kVariants[pick_any(M, N, K, pipe_ok(256, 256, p, false), out_bytes == 1 ? 1 : 4)].name;
 }
 
+#ifdef DQ8_TEST_HOOKS
 extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                                  const int8_t* W, int64_t ldw, void* out, int64_t ldo,
                                  int64_t M, int64_t N, int64_t K, int tp_a, int tp_b,
@@ -820,6 +825,7 @@ extern "C" int dq8_qgemm_variant(int variant, const int8_t* A, int64_t lda,
                     bias_kind, sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo, workspace,
                     workspace_bytes, nullptr, stream);
 }
+#endif
 
 extern "C" int dq8_qgemm_fused(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
                                void* out, int64_t ldo, int64_t M, int64_t N, int64_t K, int tp_a,
@@ -840,9 +846,9 @@ extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t 
                          int64_t n_sw, const float* so, int64_t n_so, int32_t zx,
                          int32_t zw, int32_t zo, void* workspace, size_t workspace_bytes,
                          void* stream) {
-  return dq8_qgemm_variant(-1, A, lda, W, ldw, out, ldo, M, N, K, tp_a, tp_b, epilogue,
-                           bias, bias_kind, sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo,
-                           workspace, workspace_bytes, stream);
+  return qgemm_impl(-1, A, lda, W, ldw, out, ldo, M, N, K, tp_a, tp_b, epilogue, bias, bias_kind,
+                    sx, n_sx, sw, n_sw, so, n_so, zx, zw, zo, workspace, workspace_bytes, nullptr,
+                    stream);
 }
 
 // ---- quantize -> qgemm as one operator ---------------------------------------------------
@@ -1311,6 +1317,7 @@ extern "C" size_t dq8_qconv2d_workspace_bytes(const int64_t in_sizes[4], const i
   return dq8_qconv2d_workspace_bytes_ex(in_sizes, w_sizes, nullptr, metadata);
 }
 
+#ifdef DQ8_TEST_HOOKS
 extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t in_sizes[4],
                                    const int8_t* w, const int64_t w_sizes[4],
                                    const int32_t padding[4], const int32_t md[17],
@@ -1322,6 +1329,7 @@ extern "C" int dq8_qconv2d_variant(int variant, const int8_t* in, const int64_t 
   return qconv2d_impl(variant, in, in_sizes, w, w_sizes, padding, md, out, out_sizes, epilogue,
                       bias, bias_kind, sx, sw, n_sw, so, zo, workspace, workspace_bytes, stream);
 }
+#endif
 
 extern "C" int dq8_qconv2d_ws(const int8_t* in, const int64_t in_sizes[4], const int8_t* w,
                               const int64_t w_sizes[4], const int32_t padding[4],
@@ -1355,6 +1363,7 @@ extern "C" int dq8_qconv2d(const int8_t* in, const int64_t in_sizes[4], const in
                       bias, bias_kind, sx, sw, n_sw, so, zo, nullptr, 0, stream);
 }
 
+#ifdef DQ8_TEST_HOOKS
 extern "C" int dq8_mfma_probe(const int8_t* a, const int8_t* b, int32_t* d32,
                               const int8_t* a16, const int8_t* b16, int32_t* d16,
                               void* stream) {
@@ -1364,3 +1373,4 @@ extern "C" int dq8_mfma_probe(const int8_t* a, const int8_t* b, int32_t* d32,
                      a16, b16, d16);
   return check_hip(hipGetLastError(), "dq8_mfma_probe launch");
 }
+#endif

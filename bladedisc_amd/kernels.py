@@ -45,7 +45,8 @@ def _scale(t, device):
 
 
 def variant_names():
-    L = _lib.lib()
+    """Names of the kernel variants a test can force (from the test-hooks library)."""
+    L = _lib.hooks()
     return [L.dq8_qgemm_variant_name(i).decode() for i in range(L.dq8_qgemm_num_variants())]
 
 
@@ -307,9 +308,12 @@ def qgemm(a, w, epilogue, sx=None, sw=None, so=None, bias=None, tp_a=False, tp_b
             raise ValueError("fused operators go with the library's own choice of kernel")
         po, keep = post if isinstance(post, tuple) else (post, None)
         st = L.dq8_qgemm_fused(*args, C.byref(po), _stream())
-    else:
+    elif variant == -1:
+        st = L.dq8_qgemm(*args, _stream())
+    else:       # a forced kernel variant: the tests' entry point, in the test-hooks library
+        L = _lib.hooks()
         st = L.dq8_qgemm_variant(variant, *args, _stream())
-    _lib.check(st, "dq8_qgemm")
+    _lib.check(st, "dq8_qgemm", L)
     return out
 
 
@@ -378,16 +382,19 @@ def qconv2d(x, w, padding, metadata, out_shape, epilogue, sx=None, sw=None, so=N
             raise ValueError("fused operators go with the library's own choice of kernel")
         po, keep = post if isinstance(post, tuple) else (post, None)
         st = L.dq8_qconv2d_fused(*args, C.byref(po), _stream())
-    else:
+    elif variant == -1:
+        st = L.dq8_qconv2d_ws(*args, _stream())
+    else:       # a forced kernel variant: the tests' entry point, in the test-hooks library
+        L = _lib.hooks()
         st = L.dq8_qconv2d_variant(variant, *args, _stream())
-    _lib.check(st, "dq8_qconv2d")
+    _lib.check(st, "dq8_qconv2d", L)
     return out
 
 
 def mfma_probe(a32, b32, a16, b16):
     d32 = torch.empty((32, 32), dtype=torch.int32, device=a32.device)
     d16 = torch.empty((16, 16), dtype=torch.int32, device=a32.device)
-    st = _lib.lib().dq8_mfma_probe(_ptr(a32), _ptr(b32), _ptr(d32), _ptr(a16), _ptr(b16),
-                                   _ptr(d16), _stream())
-    _lib.check(st, "dq8_mfma_probe")
+    st = _lib.hooks().dq8_mfma_probe(_ptr(a32), _ptr(b32), _ptr(d32), _ptr(a16), _ptr(b16),
+                                     _ptr(d16), _stream())
+    _lib.check(st, "dq8_mfma_probe", _lib.hooks())
     return d32, d16
