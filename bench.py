@@ -63,6 +63,11 @@ def parse():
                         "e.g. for a profiler: 'gemm:MxKxN' (dynamic-M sweep shape, requant to "
                         "int8), 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS) or "
                         "'wo:MxKxN' (weight-only linear, f16 x uint8)")
+    p.add_argument("--operands", choices=("config", "uniform", "ones", "zeros"), default="config",
+                   help="with --workload gemm:MxKxN: the operand bytes -- the benchmark "
+                        "configuration's quantized normals (default), uniform integers in "
+                        "[-127,127], all ones or all zeros (the same instructions and traffic; "
+                        "what differs is the switching power the data causes)")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extra", action="store_true", help="skip the extras")
     p.add_argument("--no-two-stream", action="store_true",
@@ -691,10 +696,17 @@ def single_workload(torch, args):
         m, k, n = (int(v) for v in what.split("x"))
         c = cfg.config2(m, k, n)
         o = torch.empty((m, n), dtype=torch.int8, device="cuda")
-        call = GemmCall(torch, dev(c["a_q"]), dev(c["w_q"]), f1(c["sx"]), dev(c["sw"]), f1(c["so"]),
-                        None, 1, 0, o)
+        a_q, w_q = dev(c["a_q"]), dev(c["w_q"])
+        if args.operands == "uniform":
+            a_q = torch.randint(-127, 128, (m, k), dtype=torch.int8, device="cuda")
+            w_q = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+        elif args.operands in ("ones", "zeros"):
+            fill = 1 if args.operands == "ones" else 0
+            a_q = torch.full((m, k), fill, dtype=torch.int8, device="cuda")
+            w_q = torch.full((n, k), fill, dtype=torch.int8, device="cuda")
+        call = GemmCall(torch, a_q, w_q, f1(c["sx"]), dev(c["sw"]), f1(c["so"]), None, 1, 0, o)
         ops, byts = 2.0 * m * n * k, m * k + n * k + m * n + 4 * n
-        name = "int8 qgemm M=%d K=%d N=%d, requant to int8 (E1)" % (m, k, n)
+        name = "int8 qgemm M=%d K=%d N=%d, requant to int8 (E1), operands: %s" % (m, k, n, args.operands)
     elif kind == "conv":
         conv = {c["name"]: c for c in cfg.RESNET_CONVS}[what]
         c = cfg.config4(conv)
