@@ -61,8 +61,9 @@ def parse():
     p.add_argument("--workload", default="headline",
                    help="'headline' (default), or one parity-test configuration on its own, "
                         "e.g. for a profiler: 'gemm:MxKxN' (dynamic-M sweep shape, requant to "
-                        "int8), 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS) or "
-                        "'wo:MxKxN' (weight-only linear, f16 x uint8)")
+                        "int8), 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS), "
+                        "'wo:MxKxN' (weight-only linear, f16 x uint8) or 'qlinear:MxKxN' "
+                        "(quantize -> qgemm -> dequantize of f32 activations in one launch)")
     p.add_argument("--operands", choices=("config", "uniform", "ones", "zeros"), default="config",
                    help="with --workload gemm:MxKxN: the operand bytes -- the benchmark "
                         "configuration's quantized normals (default), uniform integers in "
@@ -735,6 +736,19 @@ def single_workload(torch, args):
         call = lambda: K.weight_only_qgemm(xh, wq, sc, zp, out=oh)  # noqa: E731
         ops, byts = 2.0 * m * n * k, 2.0 * m * k + n * k + 2.0 * m * n + 6.0 * n
         name = "weight-only qgemm M=%d K=%d N=%d, f16 x uint8 (roofline against the f16 peak)" % (m, k, n)
+    elif kind == "qlinear":
+        # quantize -> qgemm (E1, f32 bias) -> dequantize of f32 activations as one launch
+        m, k, n = (int(v) for v in what.split("x"))
+        x = torch.randn((m, k), device="cuda")
+        wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, device="cuda")
+        sx, so = f1(0.03), f1(0.5)
+        sw = torch.rand(n, device="cuda") * 0.05 + 0.001
+        bias = torch.randn(n, device="cuda")
+        o = torch.empty((m, n), device="cuda")
+        call = lambda: K.qlinear_f32(x, wq, K.EPI_REQUANT_CPU_DEQUANT_F32, sx, sw, so,  # noqa: E731
+                                     bias=bias, out=o)
+        ops, byts = 2.0 * m * n * k, 4.0 * m * k + n * k + 4.0 * m * n + 8 * n
+        name = "quantized linear on f32 activations, one launch, M=%d K=%d N=%d" % (m, k, n)
     else:
         raise SystemExit("bench.py: unknown --workload %r" % args.workload)
     pre_launches, pre_s = prewarm(torch, call, args.prewarm_ms * 1e-3) if args.prewarm_ms > 0 \

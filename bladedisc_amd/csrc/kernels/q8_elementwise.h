@@ -78,6 +78,34 @@ __device__ __forceinline__ int quant_from_quotient(float t0, float lo, float hi)
   return (int)t3;
 }
 
+// Four quotients -> four int8 in one word, half-to-even rounding: clamp first (for integer
+// bounds clamp(rne(t)) = rne(clamp(t)); v_med3_f32 returns the smaller bound for a NaN, as
+// quant_one's fmaxf / fminf pair does), then one addition of 1.5 * 2^23 per value rounds to the
+// nearest-even integer and leaves its two's-complement int8 in the low byte of the sum, which
+// the sub-dword form of the add writes straight into its byte of the word.
+__device__ __forceinline__ uint32_t quant4_pack_rne(const float4& t) {
+  const float c0 = __builtin_amdgcn_fmed3f(t.x, -128.0f, 127.0f);
+  const float c1 = __builtin_amdgcn_fmed3f(t.y, -128.0f, 127.0f);
+  const float c2 = __builtin_amdgcn_fmed3f(t.z, -128.0f, 127.0f);
+  const float c3 = __builtin_amdgcn_fmed3f(t.w, -128.0f, 127.0f);
+  const float magic = 12582912.0f;
+  uint32_t word = __float_as_uint(c0 + magic);   // byte 0; bytes 1 .. 3 are replaced below
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(word) : "v"(c1), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(word) : "v"(c2), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(word) : "v"(c3), "v"(magic));
+#else
+  word &= 0xffu;
+  word |= (__float_as_uint(c1 + magic) & 0xffu) << 8;
+  word |= (__float_as_uint(c2 + magic) & 0xffu) << 16;
+  word |= (__float_as_uint(c3 + magic) & 0xffu) << 24;
+#endif
+  return word;
+}
+
 template <bool SIGNED>
 __device__ __forceinline__ int4 unpack4(uint32_t w) {
   if (SIGNED)

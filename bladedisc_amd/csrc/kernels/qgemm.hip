@@ -2,6 +2,7 @@
 // (any layout, any alignment, zero points) scalar kernels, and the MFMA layout
 // probe.  The tile shape is chosen at run time from the dynamic M.
 #include <algorithm>
+#include <cstdlib>
 #include <cmath>
 
 #include "dq8_common.h"
@@ -438,6 +439,7 @@ int pick_any(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes) {
       return pick_k_split64(M, N, K);
     return kSkinnyVariant;
   }
+  if (skinny_takes_rows(M, N, K)) return kSkinnyVariant;
   return pick_variant(M, N, K, pipe, out_bytes);
 }
 
@@ -855,13 +857,16 @@ extern "C" int dq8_qgemm(const int8_t* A, int64_t lda, const int8_t* W, int64_t 
 extern "C" int64_t dq8_qlinear_f32_fused_max_rows(int64_t N, int64_t K) {
   // A workgroup takes 16 rows x 16 channels, and every workgroup along N quantizes its 16 rows
   // again.  That is cheaper than a quantize launch of its own (about 2.2 us) while the
-  // workgroups come to at most one and a half per compute unit: measured against
-  // dq8_quantize + dq8_qgemm (launches replayed from a graph), 64 x 768 -> 768: 5.4 against
-  // 7.9 us; 128 rows: 7.5 against 8.1; 256 rows: 10.3 against 8.3; 64 x 768 -> 3072: 10.3
-  // against 8.0; 64 x 3072 -> 768: 9.9 against 11.4.
+  // workgroups come to at most three per compute unit (one per compute unit from 3072 of k
+  // on).  Measured against dq8_quantize + dq8_qgemm with the dequantize in its epilogue
+  // (launches replayed from a graph, us): 768 -> 768: 16 rows 4.1 against 5.4, 64 rows 4.2 / 7.9,
+  // 256 rows 6.0 / 8.3, 512 rows 9.4 / 8.3; 768 -> 2304: 64 rows 6.0 / 8.0, 128 rows 8.3 / 8.2;
+  // 768 -> 3072: 64 rows 6.1 / 8.1, 128 rows 9.4 / 8.1; 3072 -> 768: 64 rows 6.5 / 11.4, 256 rows
+  // 11.2 / 12.3, 512 rows 21.3 / 13.0; 4096 -> 4096: 16 rows 9.1 / 9.2, 32 rows 12.3 / 11.4.
   if (N <= 0 || N >= (1LL << 31) || K < 16 || K % 16 != 0) return 0;
-  const int64_t blocks = (3 * (int64_t)compute_units() / 2) / ceil_div(N, 16);
-  return std::min<int64_t>(16 * blocks, 256);
+  const int64_t cus = compute_units();
+  const int64_t blocks = (K <= 3072 ? 3 * cus : cus) / ceil_div(N, 16);
+  return std::min<int64_t>(16 * blocks, 4096);
 }
 
 extern "C" int dq8_qlinear_f32(const float* X, int64_t ldx, const int8_t* W, int64_t ldw, void* out,

@@ -5,6 +5,8 @@
 #ifndef DQ8_QGEMM_LAUNCH_H_
 #define DQ8_QGEMM_LAUNCH_H_
 
+#include <cstdlib>
+
 #include "dq8_common.h"
 #include "disc_q8.h"
 #include "qgemm_device.h"
@@ -71,6 +73,18 @@ constexpr int kDirectConv2 = 18;   // the third direct variant (configuration 2)
 constexpr int kPipe64k4 = 19;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
+// Above that many rows the small-M kernel still beats the 64 x 64 tiles while its workgroups
+// (16 rows x 16 channels, each over all of k) are few: up to 256 rows and
+// ceil(M / 16) ceil(N / 16) ceil(K / 768) <= 1024, or 3072 from 2048 of k on, where the tiles'
+// k loop is long (us per launch, small-M kernel against tiles: M = 64, 768 -> 768: 3.2 / 4.8;
+// M = 256: 4.1 / 4.7; M = 64, 768 -> 3072: 4.1 / 4.6; M = 128: 5.1 / 4.9; M = 64, 3072 -> 768:
+// 4.3 / 7.7; M = 256: 6.5 / 7.8; M = 64, 4096^2: 8.7 / 9.2; M = 128: 13.6 / 9.2).
+inline bool skinny_takes_rows(int64_t M, int64_t N, int64_t K) {
+  if (M <= kSkinnyMaxM) return true;
+  if (M > 256) return false;
+  const int64_t units = ceil_div(M, 16) * ceil_div(N, 16) * ceil_div(K, 768);
+  return units <= (K >= 2048 ? 3072 : 1024);
+}
 
 inline bool is_pipe_variant(int v) {
   return v == kPipe256 || v == kPipe128 || v == kPipe64 || v == kPipe256x64 || v == kPipe64k2 ||
@@ -160,9 +174,18 @@ int launch_skinny(const MainParams& p, hipStream_t st) {
     if (p.M == 1) return deep8 ? launch_gemv_t<1, 8, EPI>(p, st) : launch_gemv_t<1, 4, EPI>(p, st);
     return deep8 ? launch_gemv_t<2, 8, EPI>(p, st) : launch_gemv_t<2, 4, EPI>(p, st);
   }
+  // Waves: four, eight from 1024 of k on (M = 16, 3072 -> 768: 4.1 against 4.3 us).  Row tiles
+  // of 16 per workgroup: one, i.e. as many workgroups as possible, while the weights, which
+  // every block of rows streams again, stay below about 20 MB over all its passes; else two or
+  // four (us per launch, graph replays, for (waves, row tiles) = (4,1) (4,2) (4,4) / (8,1) (8,2)
+  // (8,4): M = 64, 768 -> 768: 3.2 3.9 4.9; M = 256, 768 -> 3072: 7.3 7.0 7.5; M = 32, 4096^2:
+  // 7.2 6.3 7.3 (eight waves); M = 64, 4096^2: 10.7 9.4 8.7; M = 128, 3072 -> 768: 5.7 5.0 6.8).
   const bool deep = p.K >= 1024;
-  if (p.M <= 16) return deep ? launch_skinny_t<8, 1, EPI>(p, st) : launch_skinny_t<4, 1, EPI>(p, st);
-  if (p.M <= 32) return deep ? launch_skinny_t<8, 2, EPI>(p, st) : launch_skinny_t<4, 2, EPI>(p, st);
+  const int64_t weight_bytes = (int64_t)p.N * p.K;
+  int mt = 1;
+  while (mt < 4 && ceil_div(p.M, 16 * mt) * weight_bytes > (20LL << 20)) mt *= 2;
+  if (mt == 1) return deep ? launch_skinny_t<8, 1, EPI>(p, st) : launch_skinny_t<4, 1, EPI>(p, st);
+  if (mt == 2) return deep ? launch_skinny_t<8, 2, EPI>(p, st) : launch_skinny_t<4, 2, EPI>(p, st);
   return deep ? launch_skinny_t<8, 4, EPI>(p, st) : launch_skinny_t<4, 4, EPI>(p, st);
 }
 
