@@ -1567,7 +1567,11 @@ def test_dispatch_sweep_agrees_with_the_generic_kernel(K):
     shapes = [(m, None, None) for m in ms for _ in range(3)] + \
              [(1, 100, 3072), (2, 9, 2048), (1, 40, 8208), (2, 130, 4112),
               (3, 14400, 2048), (9, 9250, 2064), (16, 9216, 2048), (8, 9216, 2048),
-              (40, 1000, 8192), (100, 520, 8208)]
+              (40, 1000, 8192), (100, 520, 8208),
+              # the small-M kernel's range above 32 rows: one, two and four row tiles per
+              # workgroup, ragged N and k, partial last row tile
+              (64, 776, 784), (130, 40, 3088), (256, 768, 768), (200, 24, 2064),
+              (64, 4096, 4096), (33, 4104, 4096), (250, 72, 1040)]
     for m, n_fixed, k_fixed in shapes:
         if True:
             n = n_fixed or int(rng.choice([16, 48, 64, 136, 768, 1024, 2304, 3072]))
