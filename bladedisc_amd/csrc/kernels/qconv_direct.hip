@@ -1,5 +1,6 @@
 // Host launchers of the 3x3 convolution kernels that keep the input patch in LDS.
 #include "qconv_direct.h"
+#include "qconv_stream.h"
 
 #include <algorithm>
 
@@ -80,6 +81,77 @@ bool direct_conv_plan(int config, DirectConvParams* p) {
   p->patch_bytes = (int)patch;
   p->in_bytes = in_bytes;
   return true;
+}
+
+bool stream_conv_plan(DirectConvParams* p) {
+  if (p->Ci != 64 || p->Kh != 3 || p->Kw != 3) return false;   // the instantiated filter
+  if (p->NB <= 0 || p->Ho <= 0 || p->Wo <= 1 || p->Co <= 0) return false;
+  constexpr int K = 3 * 3 * 64;
+  const int64_t in_bytes = (int64_t)p->NB * p->H * p->Wd * p->Ci;
+  if (in_bytes >= (1LL << 31) || (int64_t)(p->Co + 64) * K >= (1LL << 31)) return false;
+  const int64_t hw = (int64_t)p->Ho * p->Wo;
+  if (hw >= (1 << 24) || hw * p->Wo >= (1LL << 31)) return false;   // (exact umulhi division)
+  const int64_t pitch = (p->Wo + 2 + 15) / 16 * 16;
+  const int64_t tiles_n = ceil_div(p->Co, 64);
+  const int64_t cus = compute_units();
+  const int fixed = kLdsBytes - stream_conv_weight_lds(K) - kStreamConvCpBytes;
+  // Time of a launch in units of one block of 32 pixels on one SIMD: rounds of workgroups x
+  // (blocks of the busiest SIMD -- it runs waves 0 and 4, which take blocks 0, 8, ... and
+  // 4, 12, ... -- plus about three block times of loading and of the last epilogue).
+  int64_t best_cost = -1, best_tpi = 0, best_patch = 0;
+  for (int64_t tpi = 1; tpi <= ceil_div(hw, 32); ++tpi) {
+    const int64_t tile = ceil_div(hw, tpi);
+    if (ceil_div(hw, tile) != tpi) continue;               // the same tiling as a smaller tpi
+    int64_t span = 0;
+    for (int64_t t = 0; t < tpi; ++t) {
+      const int64_t first = t * tile, last = std::min(first + tile, hw) - 1;
+      span = std::max(span, last / p->Wo - first / p->Wo + 1);
+    }
+    const int64_t patch = ((span + 2) * pitch * 64 + 1023) / 1024 * 1024;
+    if (patch > fixed) continue;
+    const int64_t blocks = ceil_div(tile, 32);
+    const int64_t simd0 = ceil_div(blocks, 8) + (blocks > 4 ? ceil_div(blocks - 4, 8) : 0);
+    const int64_t wgs = (int64_t)p->NB * tpi * tiles_n;
+    const int64_t cost = ceil_div(wgs, cus) * (simd0 + 3);
+    if (best_cost < 0 || cost < best_cost || (cost == best_cost && wgs <= cus)) {
+      best_cost = cost;
+      best_tpi = tpi;
+      best_patch = patch;
+    }
+  }
+  if (best_cost < 0) return false;
+  if ((int64_t)p->NB * best_tpi * tiles_n >= (1LL << 31)) return false;
+  p->log2_ci = 6;
+  p->kw_inv = 0;
+  p->tile_px = (int)ceil_div(hw, best_tpi);
+  p->patch_pitch = (int)pitch;
+  p->wo_inv = (unsigned)((1ULL << 32) / (uint64_t)p->Wo + 1);
+  p->tiles_per_image = (int)best_tpi;
+  p->tiles_n = (int)tiles_n;
+  p->patch_bytes = (int)best_patch;
+  p->in_bytes = in_bytes;
+  return true;
+}
+
+namespace {
+template <int EPI>
+int launch_stream_t(const DirectConvParams& p, hipStream_t st) {
+  const int lds = p.patch_bytes + stream_conv_weight_lds(3 * 3 * 64) + kStreamConvCpBytes;
+  auto kern = qconv_stream_kernel<3, 3, 64, EPI>;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLdsBytes, &lds_allowed)) return s;
+  const int64_t grid = (int64_t)p.NB * p.tiles_per_image * p.tiles_n;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, st, p);
+  return check_hip(hipGetLastError(), "qconv_stream launch");
+}
+}  // namespace
+
+int launch_stream_conv(int epilogue, const DirectConvParams& p, hipStream_t st) {
+  switch (epilogue) {
+    case DQ8_EPI_REQUANT_CPU: return launch_stream_t<DQ8_EPI_REQUANT_CPU>(p, st);
+    case DQ8_EPI_REQUANT_GPU: return launch_stream_t<DQ8_EPI_REQUANT_GPU>(p, st);
+  }
+  return fail("the streaming convolution kernel has int8 results only");
 }
 
 int launch_direct_conv(int config, int epilogue, const DirectConvParams& p, hipStream_t st) {

@@ -1,0 +1,290 @@
+// int8 NHWC stride-1 convolution with the whole filter in registers ("streaming" form), for
+// filters whose 64-channel slice fits there: Kh * Kw * Ci <= 576 (3 x 3 x 64 in the first place).
+//
+// Where the time of such a layer goes in the LDS-tiled kernels (32 x 56 x 56 x 64 -> 64, 9 us):
+// every workgroup loads, then multiplies, then requantises and stores, all in the same phase, so
+// the matrix pipe idles while operands arrive and while the epilogue's VALU chain runs (a wave
+// issues about one VALU instruction per 5 cycles; 64 results per lane are 1.3 us of it), and the
+// k loop itself is paced by barriers and by LDS reads of both operands.  Here
+//  * a workgroup (8 waves, one per compute unit) takes `tile_px` consecutive output pixels of one
+//    image x 64 output channels; the input rows they touch, with the filter's frame, are loaded
+//    into LDS once (as in qconv_direct.h, same swizzle);
+//  * the 64 x K weight slice is loaded into LDS once and from there into registers: every wave
+//    holds all of it in MFMA operand layout (K / 4 registers: 144 for 3 x 3 x 64), so the main
+//    loop reads only the pixel operand from LDS -- 1 KiB per two MFMAs -- and has no barrier;
+//  * a wave walks blocks of 32 pixels: K / 32 steps of two MFMAs (channels 0-31, 32-63), then
+//    requantises and stores that block's 32 x 64 results from registers and goes on to its next
+//    block.  The two waves of a SIMD drift apart by themselves (the older wave wins the matrix
+//    pipe), so one wave's epilogue runs under the other's MFMAs.
+// The weights go to LDS before the patch and are copied to registers while the patch is still
+// arriving.  int8 results only (REQUANT_CPU / REQUANT_GPU), 16-byte aligned output rows.
+#ifndef DQ8_QCONV_STREAM_H_
+#define DQ8_QCONV_STREAM_H_
+
+#include "qconv_direct.h"
+
+// Per-wave timeline hook for profiling builds, like DQ8_TRACE_POINT: stage i of the calling wave
+// (0 entry, 1 weights in LDS, 2 weights in registers, 3 patch landed, 4 + 2 k / 5 + 2 k: MFMAs /
+// stores of the wave's k-th block done).  Expands to nothing in the library.
+#ifndef DQ8_TRACE_WAVE
+#define DQ8_TRACE_WAVE(i)
+#endif
+
+namespace dq8 {
+
+// LDS bytes the kernel needs on top of the patch: the padded weight slice (rows of K + 16
+// bytes, rounded up to the 8 KiB the eight waves' equal shares of load instructions cover) and
+// the per-channel (scale, addend) pairs.
+constexpr int stream_conv_weight_lds(int K) {
+  return ((64 * (K / 16 + 1) + 511) / 512) * 512 * 16;
+}
+constexpr int kStreamConvCpBytes = 64 * 8;
+
+template <int KH, int KW, int CI, int EPI>
+__global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  static_assert(EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU, "int8 results only");
+  static_assert(CI == 32 || CI == 64 || CI == 128 || CI == 256, "channels per pixel");
+  constexpr int NW = 8;
+  constexpr int K = KH * KW * CI;
+  constexpr int KS = K / 32;                 // MFMA steps per block
+  constexpr int ROWC = K / 16 + 1;           // 16-byte chunks per weight row in LDS (one of padding)
+  constexpr int W_INSTR = (64 * ROWC + 63) / 64;           // 1 KiB load instructions for the slice
+  constexpr int W_PER_WAVE = (W_INSTR + NW - 1) / NW;      // every wave issues this many
+  constexpr int W_LDS = stream_conv_weight_lds(K);
+  constexpr int LOG2_CI = CI == 32 ? 5 : CI == 64 ? 6 : CI == 128 ? 7 : 8;
+  constexpr int CP = CI / 16;                // 16-byte chunks per pixel
+  constexpr int FSHIFT = 8 - LOG2_CI, FMASK = CP - 1;
+  constexpr int STEPS_PER_TAP = CI / 32;
+  constexpr int kOutOfRange = (int)0x80000000;
+  static_assert(W_PER_WAVE * NW * 1024 <= W_LDS, "weight area");
+  static_assert(K % 32 == 0 && KS * 8 <= 160, "the filter slice must fit the registers");
+
+  extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
+  DQ8_TRACE_POINT(0);
+  DQ8_TRACE_WAVE(0);
+  int8_t* patch = smem;
+  int8_t* wlds = smem + p.patch_bytes;
+  float2* cp = reinterpret_cast<float2*>(smem + p.patch_bytes + W_LDS);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const EpiParams& e = p.epi;
+
+  const int tn = blockIdx.x % p.tiles_n;
+  const int rest = blockIdx.x / p.tiles_n;
+  const int tp = rest % p.tiles_per_image;
+  const int img = rest / p.tiles_per_image;
+  const int n0 = tn * 64;
+  const int hw = p.Ho * p.Wo;
+  const int p0 = tp * p.tile_px;                           // first output pixel of the tile
+  const int p_end = min(p0 + p.tile_px, hw);
+  const int y_base = p0 / p.Wo;
+  const int rows = (p_end - 1) / p.Wo - y_base + KH;       // patch rows in use
+  const int PW = p.Wo + KW - 1;
+
+  const v4i in_rsrc = make_rsrc(p.in, p.in_bytes);
+  const int8_t* w_base = p.w + (int64_t)n0 * K;
+  const int64_t w_valid = (int64_t)(p.Co - n0) * K;
+  const v4i w_rsrc = make_rsrc(w_base, w_valid < 0x7fffffff ? w_valid : 0x7fffffff);
+  const unsigned lds_base =
+      (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(size_t)(lds_void_t*)smem);
+
+  // ---- per-channel factors: the loads go out first and are used last
+  ColRaw raw = {1.0f, 1.0f, 1.0f, 0};
+  if (tid < 64) raw = col_fetch<EPI>(e, n0 + tid < e.N ? n0 + tid : e.N - 1);
+
+  // ---- the weight slice: LDS rows of ROWC chunks, chunk g = 64 j + lane of instruction j
+#pragma unroll
+  for (int i = 0; i < W_PER_WAVE; ++i) {
+    const int j = wave + i * NW;
+    const int g = j * 64 + lane;
+    const int row = g / ROWC, c = g - row * ROWC;
+    const bool ok = row < 64 && c < K / 16;
+    buffer_load_lds_b128(w_rsrc, lds_base + p.patch_bytes + j * 1024,
+                         ok ? row * K + (c << 4) : kOutOfRange);
+  }
+
+  // ---- the patch: instruction j of the workgroup fills LDS bytes [1024 j, 1024 j + 1024); patch
+  // rows have a pitch of PWp pixels, a multiple of 16, so that a step down a row leaves the
+  // swizzle of a pixel as it is (the pixels between the frame and the pitch are never read)
+  const int PWp = p.patch_pitch;
+  const int total = rows * PWp * CP;                       // chunks in use
+  const int n_patch = (((total + 63) >> 6) - wave + NW - 1) / NW;   // instructions of this wave
+  {
+    const int img_px = img * p.H * p.Wd;
+    constexpr int dq = (NW * 64) >> (LOG2_CI - 4);         // pixels per step
+    const int dq_y = dq / PWp, dq_x = dq - dq_y * PWp;
+    int g = wave * 64 + lane;
+    int q = g >> (LOG2_CI - 4);
+    int hy = q / PWp, hx = q - hy * PWp;
+    const int slot = g & (CP - 1);
+    for (int j = wave; j * 64 < total; j += NW) {
+      const int c = slot ^ ((q >> FSHIFT) & FMASK);
+      const int iy = y_base - p.pad_t + hy, ix = hx - p.pad_l;
+      const bool ok = g < total && hx < PW && (unsigned)iy < (unsigned)p.H &&
+                      (unsigned)ix < (unsigned)p.Wd;
+      const int voff = ok ? ((img_px + iy * p.Wd + ix) << LOG2_CI) + (c << 4) : kOutOfRange;
+      buffer_load_lds_b128(in_rsrc, (unsigned)__builtin_amdgcn_readfirstlane((int)(lds_base + j * 1024)),
+                           voff);
+      g += NW * 64;
+      q += dq;
+      hx += dq_x;
+      hy += dq_y;
+      if (hx >= PWp) {
+        hx -= PWp;
+        ++hy;
+      }
+    }
+  }
+
+  // ---- this wave's weight loads are the oldest in flight: they have landed once at most its
+  // patch loads remain.  (Weights from one half of the waves and the patch from the other, so
+  // that neither queues behind the other, was measured: both land 0.5 us later.)
+  if (n_patch >= 12) {
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(12));
+  } else {
+    static_for<12>([&](auto kc) {
+      constexpr int k = decltype(kc)::value;
+      if (n_patch == k) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(k));
+    });
+  }
+  __syncthreads();          // the weights are in LDS
+  DQ8_TRACE_WAVE(1);
+
+  // ---- weights into registers, MFMA operand layout: lane l holds channel l % 32 of a
+  // 32-channel group and the 16 bytes of k at 32 s + 16 (l / 32)
+  v4i wreg[KS][2];
+  {
+    const int8_t* wl = wlds + ((lane & 31) * ROWC + (lane >> 5)) * 16;
+    static_for<KS>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      wreg[s][0] = *reinterpret_cast<const v4i*>(wl + s * 32);
+      wreg[s][1] = *reinterpret_cast<const v4i*>(wl + 32 * ROWC * 16 + s * 32);
+    });
+  }
+
+  DQ8_TRACE_WAVE(2);
+  // ---- everything has landed for this wave; the factors are worked out and parked
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  if (tid < 64) {
+    const ColParams c = col_finish<EPI>(e, raw);
+    cp[tid] = make_float2(c.os, c.b);
+  }
+  __syncthreads();
+  DQ8_TRACE_POINT(1);
+  DQ8_TRACE_WAVE(3);
+
+  const bool plain = e.bias_kind == DQ8_BIAS_NONE && e.zo == 0;
+  int8_t* out = static_cast<int8_t*>(e.out);
+  const int nblocks = (p_end - p0 + 31) >> 5;
+  const int c0 = lane >> 5;
+  const int pitch_bytes = PWp << LOG2_CI;
+
+  for (int b = wave; b < nblocks; b += NW) {
+    // this lane's pixel: position in the patch at tap (0, 0)
+    const int px_raw = p0 + b * 32 + (lane & 31);
+    const int px = px_raw < p_end ? px_raw : p_end - 1;
+    const int y = (int)__umulhi((unsigned)px, p.wo_inv), x = px - y * p.Wo;
+    const int hq = (y - y_base) * PWp + x;
+    // byte offset of this lane's 16 bytes of k-half 0 at filter column kw, filter row 0; k-half
+    // h is the same with bit 5 + ... flipped (xor 32 h), filter row kh adds kh row pitches
+    int a0[KW];
+#pragma unroll
+    for (int kw = 0; kw < KW; ++kw) {
+      const int q = hq + kw;
+      a0[kw] = (q << LOG2_CI) + ((c0 ^ ((q >> FSHIFT) & FMASK)) << 4);
+    }
+
+    // pixel fragments, read PF steps ahead of their MFMAs
+    constexpr int PF = 4;
+    v4i fa[8];
+    auto load_frag = [&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      constexpr int tap = s / STEPS_PER_TAP;
+      constexpr int kh = tap / KW, kw = tap - KW * kh;
+      constexpr int h = s % STEPS_PER_TAP;
+      fa[s & 7] = *reinterpret_cast<const v4i*>(patch + (a0[kw] ^ (32 * h)) + kh * pitch_bytes);
+    };
+    static_for<PF>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      if constexpr (s < KS) load_frag(IntC<s>());
+    });
+    v16i acc[2];
+    static_for<KS>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      if constexpr (s + PF < KS) load_frag(IntC<s + PF>());
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (s == 0) {
+        // (the accumulators start from the instruction's constant zero, not from 32 moves)
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][0], fa[s & 7], zero, 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][1], fa[s & 7], zero, 0, 0, 0);
+      } else {
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][0], fa[s & 7], acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][1], fa[s & 7], acc[1], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+
+    DQ8_TRACE_WAVE(4 + 2 * ((b - wave) / NW));
+    // ---- requantise and store the block's 32 x 64 results: of a 32 x 32 fragment a lane holds
+    // pixel lane % 32 and the channel quads 8 g + 4 (lane / 32) .. + 3; two half-wave swaps
+    // leave it with 16 consecutive channels, one 16-byte store
+    const int64_t m = (int64_t)img * hw + px_raw;
+    auto finish = [&](auto mode_c) {
+      constexpr bool PLAIN = decltype(mode_c)::value == 1;
+      static_for<2>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const int cl0 = j * 32 + 4 * c0;
+        uint32_t w[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g]);
+          const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g + 2]);
+          const ColParams c[4] = {{p01[0], p01[1], 0}, {p01[2], p01[3], 0},
+                                  {p23[0], p23[1], 0}, {p23[2], p23[3], 0}};
+          w[g] = requant_pack4<EPI, PLAIN>(e, c, acc[j][4 * g + 0], acc[j][4 * g + 1],
+                                           acc[j][4 * g + 2], acc[j][4 * g + 3]);
+        }
+        const auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+        const auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+        const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+        const int n = n0 + j * 32 + 16 * c0;
+        if (px_raw < p_end && n < e.N) {
+          int8_t* dst = out + m * e.ldo + n;
+          if (n + 15 < e.N) {
+            *reinterpret_cast<v4i*>(dst) = v;
+          } else {
+#pragma unroll
+            for (int t = 0; t < 16; ++t)
+              if (n + t < e.N) dst[t] = (int8_t)((uint32_t)v[t >> 2] >> (8 * (t & 3)));
+          }
+        }
+      });
+    };
+    if (plain)
+      finish(IntC<1>());
+    else
+      finish(IntC<0>());
+    DQ8_TRACE_WAVE(5 + 2 * ((b - wave) / NW));
+  }
+  DQ8_TRACE_POINT(3);
+#else
+  (void)p;
+#endif
+}
+
+// ---- host side (qconv_direct.hip)
+// Whether the streaming kernel can run the problem (3 x 3 filter, 64 input channels, stride and
+// dilation 1 are the caller's to check; here: sizes, and a tile whose patch fits the LDS next to
+// the weights).  Chooses the pixel tile so that the workgroups come to whole rounds of the
+// compute units with the least work per workgroup and fills tile_px, tiles_per_image, tiles_n,
+// patch_bytes, in_bytes.
+bool stream_conv_plan(DirectConvParams* p);
+int launch_stream_conv(int epilogue, const DirectConvParams& p, hipStream_t st);
+
+}  // namespace dq8
+
+#endif  // DQ8_QCONV_STREAM_H_

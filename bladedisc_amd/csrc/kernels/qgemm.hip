@@ -10,6 +10,7 @@
 #include "qgemm_device.h"
 #include "qgemm_launch.h"
 #include "qconv_direct.h"
+#include "qconv_stream.h"
 
 #pragma clang fp contract(off)
 
@@ -1266,7 +1267,19 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
                 "patch that fits the LDS");
     return launch_direct_conv(config, epilogue, d, st);
   }
+  // 3 x 3 filters on 64 channels with int8 results: the filter in registers
+  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && Ci == 64 && !fused &&
+                            !e.fixedpoint && e.vec_store16 &&
+                            (epilogue == DQ8_EPI_REQUANT_CPU || epilogue == DQ8_EPI_REQUANT_GPU);
+  if (variant == kStreamConv) {
+    DQ8_REQUIRE(stream_shape && stream_conv_plan(&d),
+                "dq8_qconv2d: the streaming variant needs a 3 x 3 filter with stride and dilation "
+                "1 on 64 input channels, an int8 result without fused operators and 16-byte "
+                "aligned output rows");
+    return launch_stream_conv(epilogue, d, st);
+  }
   if (auto_pick) {
+    if (stream_shape && stream_conv_plan(&d)) return launch_stream_conv(epilogue, d, st);
     if (direct_shape) {
       const int c = pick_direct_conv(NB, Ho * Wo, Ci, Co);
       if (c >= 0 && direct_conv_plan(c, &d)) return launch_direct_conv(c, epilogue, d, st);

@@ -145,51 +145,90 @@ __device__ __forceinline__ float sat_rne_s32_as_float(float v) {
   return (float)(int)rintf(v);
 }
 
+// What col_params reads from memory for channel n, apart from the arithmetic on it: a kernel
+// that wants the loads in flight early and the divisions late calls the two halves itself.
+struct ColRaw {
+  float sx, sw, so;
+  int bias;   // the 32 bits of an f32 or s32 bias, an s8 bias sign-extended; 0 where none is read
+};
+
 template <int EPI>
-__device__ __forceinline__ ColParams col_params(const EpiParams& p, int n) {
+__device__ __forceinline__ int col_mode(const EpiParams& p) {
+  // the arithmetic the factors are for: a compile-time constant except under DEQUANT_F32
+  return EPI != DQ8_EPI_DEQUANT_F32 ? EPI
+         : p.requant == 1           ? DQ8_EPI_REQUANT_CPU
+         : p.requant == 2           ? DQ8_EPI_REQUANT_GPU
+                                    : DQ8_EPI_DEQUANT_F32;
+}
+
+template <int EPI>
+__device__ __forceinline__ ColRaw col_fetch(const EpiParams& p, int n) {
+  ColRaw r = {1.0f, 1.0f, 1.0f, 0};
+  if (EPI == DQ8_EPI_ACC_S32) return r;
+  r.sx = p.sx[(int64_t)n * p.sx_stride];
+  r.sw = p.sw[(int64_t)n * p.sw_stride];
+  const int mode = col_mode<EPI>(p);
+  if (mode == DQ8_EPI_DEQUANT_F32) {
+    if (p.bias_kind == DQ8_BIAS_F32) r.bias = ((const int32_t*)p.bias)[n];
+    return r;
+  }
+  r.so = p.so[(int64_t)n * p.so_stride];
+  if (mode == DQ8_EPI_REQUANT_CPU) {
+    if (p.bias_kind == DQ8_BIAS_S32 || (!p.fixedpoint && p.bias_kind == DQ8_BIAS_F32))
+      r.bias = ((const int32_t*)p.bias)[n];
+  } else {  // REQUANT_GPU
+    if (p.bias_kind == DQ8_BIAS_F32)
+      r.bias = ((const int32_t*)p.bias)[n];
+    else if (p.bias_kind == DQ8_BIAS_S8)
+      r.bias = ((const int8_t*)p.bias)[n];
+  }
+  return r;
+}
+
+template <int EPI>
+__device__ __forceinline__ ColParams col_finish(const EpiParams& p, const ColRaw& r) {
   ColParams c;
   c.os = 1.0f;
   c.b = 0.0f;
   c.sh = 0;
   if (EPI == DQ8_EPI_ACC_S32) return c;
-  const float sx = p.sx[(int64_t)n * p.sx_stride];
-  const float sw = p.sw[(int64_t)n * p.sw_stride];
-  const float prod = sx * sw;
-  // the arithmetic the factors are for: a compile-time constant except under DEQUANT_F32
-  const int mode = EPI != DQ8_EPI_DEQUANT_F32 ? EPI
-                   : p.requant == 1           ? DQ8_EPI_REQUANT_CPU
-                   : p.requant == 2           ? DQ8_EPI_REQUANT_GPU
-                                              : DQ8_EPI_DEQUANT_F32;
+  const float prod = r.sx * r.sw;
+  const int mode = col_mode<EPI>(p);
   if (mode == DQ8_EPI_DEQUANT_F32) {
     c.os = prod;
-    if (p.bias_kind == DQ8_BIAS_F32) c.b = ((const float*)p.bias)[n];
+    if (p.bias_kind == DQ8_BIAS_F32) c.b = __int_as_float(r.bias);
     return c;
   }
-  const float so = p.so[(int64_t)n * p.so_stride];
+  const float so = r.so;
   if (mode == DQ8_EPI_REQUANT_CPU && p.fixedpoint) {
     int m0, sh;
     fixedpoint_multiplier(prod / so, m0, sh);
     c.os = __int_as_float(m0);
     c.sh = sh;
-    c.b = __int_as_float(p.bias_kind == DQ8_BIAS_S32 ? ((const int32_t*)p.bias)[n] : 0);
+    c.b = __int_as_float(p.bias_kind == DQ8_BIAS_S32 ? r.bias : 0);
     return c;
   }
   if (mode == DQ8_EPI_REQUANT_CPU) {
     c.os = prod / (1.0f * so);
     if (p.bias_kind == DQ8_BIAS_S32) {
-      c.b = (float)((const int32_t*)p.bias)[n];
+      c.b = (float)r.bias;
     } else if (p.bias_kind == DQ8_BIAS_F32) {
       const float bs = (1.0f * 1.0f) / prod;
-      c.b = sat_rne_s32_as_float(((const float*)p.bias)[n] * bs);
+      c.b = sat_rne_s32_as_float(__int_as_float(r.bias) * bs);
     }
   } else {  // REQUANT_GPU
     c.os = prod / so;
     if (p.bias_kind == DQ8_BIAS_F32)
-      c.b = ((const float*)p.bias)[n];
+      c.b = __int_as_float(r.bias);
     else if (p.bias_kind == DQ8_BIAS_S8)
-      c.b = (float)((const int8_t*)p.bias)[n];
+      c.b = (float)r.bias;
   }
   return c;
+}
+
+template <int EPI>
+__device__ __forceinline__ ColParams col_params(const EpiParams& p, int n) {
+  return col_finish<EPI>(p, col_fetch<EPI>(p, n));
 }
 
 __device__ __forceinline__ int sat_rne_s8(float d) {

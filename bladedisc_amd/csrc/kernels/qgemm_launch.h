@@ -61,6 +61,9 @@ inline constexpr Variant kVariants[] = {
     {"direct3x3_512x64", 512, 64, 128, 512},
     // 64x64 with the k tiles split over 4 groups of waves (sixteen waves, 128 KiB LDS)
     {"pipe_64x64x128_k4", 64, 64, 128, 1024},
+    // 3 x 3 x 64-channel filters held in registers, pixel tile chosen per problem (convolution
+    // only, int8 results)
+    {"stream3x3_64", 32, 64, 32, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;
@@ -71,6 +74,7 @@ constexpr int kPersist256 = 14, kPersist128 = 15;
 constexpr int kPipe256x192 = 16, kPersist256x192 = 17;
 constexpr int kDirectConv2 = 18;   // the third direct variant (configuration 2)
 constexpr int kPipe64k4 = 19;
+constexpr int kStreamConv = 20;
 // largest M the heuristic hands to the small-M kernel
 constexpr int64_t kSkinnyMaxM = 32;
 // Above that many rows the small-M kernel still beats the 64 x 64 tiles while its workgroups

@@ -26,7 +26,8 @@ def host(t):
 
 def gemm_variants(K, k):
     """All variant ids of the GEMM."""
-    return [i for i, nm in enumerate(K.variant_names()) if not nm.startswith("direct3x3_")]
+    return [i for i, nm in enumerate(K.variant_names())
+            if not nm.startswith(("direct3x3_", "stream3x3_"))]
 
 
 def make_scales(rng, n, per_channel=True):
@@ -860,6 +861,73 @@ def test_qconv_direct_random_shapes(K):
                                  sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])),
                                  variant=v))
             np.testing.assert_array_equal(got, want, err_msg=tag + " variant %d" % v)
+
+
+
+def test_qconv_stream_variant(K):
+    """The 3 x 3 x 64-channel kernel that keeps the filter in registers: images whose pixel
+    tiles start and end anywhere in a row, one to many tiles per image, ragged and several
+    64-channel slices of output channels, asymmetric padding, both int8 epilogues with every
+    bias kind they take and an output zero point -- bit-exact against the oracle; then what it
+    must refuse."""
+    rng = np.random.default_rng(20260311)
+    sv = K.variant_names().index("stream3x3_64")
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    shapes = [(2, 56, 56, 64, [1, 1, 1, 1]), (1, 3, 3, 16, [1, 1, 1, 1]), (3, 9, 7, 80, [0, 0, 0, 0]),
+              (1, 6, 150, 64, [1, 1, 1, 1]), (1, 33, 17, 208, [2, 0, 1, 2]), (5, 28, 28, 128, [1, 1, 1, 1]),
+              (1, 112, 112, 64, [1, 1, 1, 1]), (40, 14, 14, 64, [0, 2, 2, 0])]
+    for nb, h, w_, co, pad in shapes:
+        ho, wo = h + pad[0] + pad[1] - 2, w_ + pad[2] + pad[3] - 2
+        x = rng.integers(-128, 128, (nb, h, w_, 64), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, 3, 3, 64), dtype=np.int8)
+        out_shape = [nb, ho, wo, co]
+        acc = O.conv_s32(x, wt, pad, md, out_shape)
+        sx, sw = make_scales(rng, co)
+        so = pick_so(acc, sx, sw)
+        scales = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])))
+        tag = "%dx%dx%dx64 -> %d pad %s" % (nb, h, w_, co, pad)
+        a2 = acc.reshape(-1, co)
+        # E1: plain, f32 bias (folded to s32 as the library does) with an output zero point, s32 bias
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_cpu(a2, sx, sw, so).reshape(out_shape), err_msg=tag)
+        bf = (rng.standard_normal(co) * 40 * so).astype(np.float32)
+        b32 = O.bias_f32_to_s32(bf, sx, sw)
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, bias=dev(bf), zo=3,
+                             variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_cpu(a2, sx, sw, so, b32=b32, zo=3).reshape(out_shape),
+                                      err_msg=tag + " f32 bias")
+        bi = rng.integers(-2000000, 2000000, co).astype(np.int32)
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, bias=dev(bi), zo=-5,
+                             variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_cpu(a2, sx, sw, so, b32=bi, zo=-5).reshape(out_shape),
+                                      err_msg=tag + " s32 bias")
+        # E2: f32 bias in output units, int8 bias
+        bo = (rng.standard_normal(co) * 30).astype(np.float32)
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(bo),
+                             variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_gpu(a2, sx, sw, so, bias_f32=bo).reshape(out_shape),
+                                      err_msg=tag + " E2 f32 bias")
+        b8 = rng.integers(-128, 128, co, dtype=np.int8)
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(b8),
+                             variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_gpu(a2, sx, sw, so, bias_i8=b8).reshape(out_shape),
+                                      err_msg=tag + " E2 s8 bias")
+        # the library's own choice for this shape gives the same bytes
+        auto = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(b8), **scales))
+        np.testing.assert_array_equal(auto, got, err_msg=tag + " heuristic")
+    # refusals: 4-byte results, other channel counts and filters, strides
+    x = dev(rng.integers(-128, 128, (1, 8, 8, 64), dtype=np.int8))
+    wt = dev(rng.integers(-128, 128, (64, 3, 3, 64), dtype=np.int8))
+    with pytest.raises(RuntimeError, match="streaming variant"):
+        K.qconv2d(x, wt, [1, 1, 1, 1], md, [1, 8, 8, 64], K.EPI_ACC_S32, variant=sv)
+    one = dev(np.array([0.01], np.float32))
+    x32 = dev(rng.integers(-128, 128, (1, 8, 8, 32), dtype=np.int8))
+    w32 = dev(rng.integers(-128, 128, (64, 3, 3, 32), dtype=np.int8))
+    with pytest.raises(RuntimeError, match="streaming variant"):
+        K.qconv2d(x32, w32, [1, 1, 1, 1], md, [1, 8, 8, 64], K.EPI_REQUANT_CPU, sx=one, sw=one, so=one, variant=sv)
+    md2 = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
+    with pytest.raises(RuntimeError, match="streaming variant"):
+        K.qconv2d(x, wt, [1, 1, 1, 1], md2, [1, 4, 4, 64], K.EPI_REQUANT_CPU, sx=one, sw=one, so=one, variant=sv)
 
 
 def test_qconv_direct_other_filter_sizes(K):
