@@ -83,18 +83,28 @@ bool direct_conv_plan(int config, DirectConvParams* p) {
   return true;
 }
 
+namespace {
+// output channels per workgroup of the streaming kernel for a filter, 0 if it has no instance
+int stream_conv_slice(int Kh, int Kw, int Ci) {
+  if (Kh == 3 && Kw == 3 && Ci == 64) return 64;
+  if (Kh == 3 && Kw == 3 && Ci == 128) return 32;
+  return 0;
+}
+}  // namespace
+
 bool stream_conv_plan(DirectConvParams* p) {
-  if (p->Ci != 64 || p->Kh != 3 || p->Kw != 3) return false;   // the instantiated filter
+  const int ns = stream_conv_slice(p->Kh, p->Kw, p->Ci);
+  if (ns == 0) return false;
   if (p->NB <= 0 || p->Ho <= 0 || p->Wo <= 1 || p->Co <= 0) return false;
-  constexpr int K = 3 * 3 * 64;
+  const int K = p->Kh * p->Kw * p->Ci;
   const int64_t in_bytes = (int64_t)p->NB * p->H * p->Wd * p->Ci;
-  if (in_bytes >= (1LL << 31) || (int64_t)(p->Co + 64) * K >= (1LL << 31)) return false;
+  if (in_bytes >= (1LL << 31) || (int64_t)(p->Co + ns) * K >= (1LL << 31)) return false;
   const int64_t hw = (int64_t)p->Ho * p->Wo;
   if (hw >= (1 << 24) || hw * p->Wo >= (1LL << 31)) return false;   // (exact umulhi division)
-  const int64_t pitch = (p->Wo + 2 + 15) / 16 * 16;
-  const int64_t tiles_n = ceil_div(p->Co, 64);
+  const int64_t pitch = (p->Wo + p->Kw - 1 + 15) / 16 * 16;
+  const int64_t tiles_n = ceil_div(p->Co, ns);
   const int64_t cus = compute_units();
-  const int fixed = kLdsBytes - stream_conv_weight_lds(K) - kStreamConvCpBytes;
+  const int fixed = kLdsBytes - stream_conv_weight_lds(K, ns) - stream_conv_cp_bytes(ns);
   // Time of a launch in units of one block of 32 pixels on one SIMD: rounds of workgroups x
   // (blocks of the busiest SIMD -- it runs waves 0 and 4, which take blocks 0, 8, ... and
   // 4, 12, ... -- plus about three block times of loading and of the last epilogue).
@@ -107,7 +117,7 @@ bool stream_conv_plan(DirectConvParams* p) {
       const int64_t first = t * tile, last = std::min(first + tile, hw) - 1;
       span = std::max(span, last / p->Wo - first / p->Wo + 1);
     }
-    const int64_t patch = ((span + 2) * pitch * 64 + 1023) / 1024 * 1024;
+    const int64_t patch = ((span + p->Kh - 1) * pitch * p->Ci + 1023) / 1024 * 1024;
     if (patch > fixed) continue;
     const int64_t blocks = ceil_div(tile, 32);
     const int64_t simd0 = ceil_div(blocks, 8) + (blocks > 4 ? ceil_div(blocks - 4, 8) : 0);
@@ -120,8 +130,10 @@ bool stream_conv_plan(DirectConvParams* p) {
     }
   }
   if (best_cost < 0) return false;
-  if ((int64_t)p->NB * best_tpi * tiles_n >= (1LL << 31)) return false;
-  p->log2_ci = 6;
+  if (((int64_t)p->NB * best_tpi + 7) / 8 * 8 * tiles_n >= (1LL << 31)) return false;
+  int log2_ci = 0;
+  while ((1 << log2_ci) < p->Ci) ++log2_ci;
+  p->log2_ci = log2_ci;
   p->kw_inv = 0;
   p->tile_px = (int)ceil_div(hw, best_tpi);
   p->patch_pitch = (int)pitch;
@@ -134,22 +146,30 @@ bool stream_conv_plan(DirectConvParams* p) {
 }
 
 namespace {
-template <int EPI>
+template <int KH, int KW, int CI, int NS, int EPI>
 int launch_stream_t(const DirectConvParams& p, hipStream_t st) {
-  const int lds = p.patch_bytes + stream_conv_weight_lds(3 * 3 * 64) + kStreamConvCpBytes;
-  auto kern = qconv_stream_kernel<3, 3, 64, EPI>;
+  const int lds = p.patch_bytes + stream_conv_weight_lds(KH * KW * CI, NS) + stream_conv_cp_bytes(NS);
+  auto kern = qconv_stream_kernel<KH, KW, CI, NS, EPI>;
   static std::atomic<uint64_t> lds_allowed{0};
   if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLdsBytes, &lds_allowed)) return s;
-  const int64_t grid = (int64_t)p.NB * p.tiles_per_image * p.tiles_n;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, st, p);
+  // (pixel tiles rounded up to a multiple of 8: workgroup b works on tile 8 (b / 8 / slices) + b % 8)
+  const int64_t tiles = ((int64_t)p.NB * p.tiles_per_image + 7) / 8 * 8;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles * p.tiles_n)), dim3(512), lds, st, p);
   return check_hip(hipGetLastError(), "qconv_stream launch");
+}
+
+template <int EPI>
+int launch_stream_epi(const DirectConvParams& p, hipStream_t st) {
+  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 64) return launch_stream_t<3, 3, 64, 64, EPI>(p, st);
+  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 128) return launch_stream_t<3, 3, 128, 32, EPI>(p, st);
+  return fail("the streaming convolution kernel has no instance for this filter");
 }
 }  // namespace
 
 int launch_stream_conv(int epilogue, const DirectConvParams& p, hipStream_t st) {
   switch (epilogue) {
-    case DQ8_EPI_REQUANT_CPU: return launch_stream_t<DQ8_EPI_REQUANT_CPU>(p, st);
-    case DQ8_EPI_REQUANT_GPU: return launch_stream_t<DQ8_EPI_REQUANT_GPU>(p, st);
+    case DQ8_EPI_REQUANT_CPU: return launch_stream_epi<DQ8_EPI_REQUANT_CPU>(p, st);
+    case DQ8_EPI_REQUANT_GPU: return launch_stream_epi<DQ8_EPI_REQUANT_GPU>(p, st);
   }
   return fail("the streaming convolution kernel has int8 results only");
 }

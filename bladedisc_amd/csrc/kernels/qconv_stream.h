@@ -1,5 +1,6 @@
 // int8 NHWC stride-1 convolution with the whole filter in registers ("streaming" form), for
-// filters whose 64-channel slice fits there: Kh * Kw * Ci <= 576 (3 x 3 x 64 in the first place).
+// filters of which a slice of NS output channels fits there: NS * Kh * Kw * Ci <= 36 KiB
+// (3 x 3 x 64 with 64-channel slices in the first place, 3 x 3 x 128 with 32-channel slices).
 //
 // Where the time of such a layer goes in the LDS-tiled kernels (32 x 56 x 56 x 64 -> 64, 9 us):
 // every workgroup loads, then multiplies, then requantises and stores, all in the same phase, so
@@ -7,13 +8,15 @@
 // issues about one VALU instruction per 5 cycles; 64 results per lane are 1.3 us of it), and the
 // k loop itself is paced by barriers and by LDS reads of both operands.  Here
 //  * a workgroup (8 waves, one per compute unit) takes `tile_px` consecutive output pixels of one
-//    image x 64 output channels; the input rows they touch, with the filter's frame, are loaded
+//    image x NS output channels (the slices of one pixel tile run on the same XCD, so that its
+//    L2 fetches their common patch once); the input rows they touch, with the filter's frame, are loaded
 //    into LDS once (as in qconv_direct.h, same swizzle);
-//  * the 64 x K weight slice is loaded into LDS once and from there into registers: every wave
-//    holds all of it in MFMA operand layout (K / 4 registers: 144 for 3 x 3 x 64), so the main
-//    loop reads only the pixel operand from LDS -- 1 KiB per two MFMAs -- and has no barrier;
-//  * a wave walks blocks of 32 pixels: K / 32 steps of two MFMAs (channels 0-31, 32-63), then
-//    requantises and stores that block's 32 x 64 results from registers and goes on to its next
+//  * the NS x K weight slice is loaded into LDS once and from there into registers: every wave
+//    holds all of it in MFMA operand layout (NS K / 256 registers: 144 for 3 x 3 x 64), so the
+//    main loop reads only the pixel operand from LDS -- 1 KiB per NS / 32 MFMAs -- and has no
+//    barrier;
+//  * a wave walks blocks of 32 pixels: K / 32 steps of NS / 32 MFMAs (one per 32 channels), then
+//    requantises and stores that block's 32 x NS results from registers and goes on to its next
 //    block.  The two waves of a SIMD drift apart by themselves (the older wave wins the matrix
 //    pipe), so one wave's epilogue runs under the other's MFMAs.
 // The weights go to LDS before the patch and are copied to registers while the patch is still
@@ -35,12 +38,12 @@ namespace dq8 {
 // LDS bytes the kernel needs on top of the patch: the padded weight slice (rows of K + 16
 // bytes, rounded up to the 8 KiB the eight waves' equal shares of load instructions cover) and
 // the per-channel (scale, addend) pairs.
-constexpr int stream_conv_weight_lds(int K) {
-  return ((64 * (K / 16 + 1) + 511) / 512) * 512 * 16;
+constexpr int stream_conv_weight_lds(int K, int NS) {
+  return ((NS * (K / 16 + 1) + 511) / 512) * 512 * 16;
 }
-constexpr int kStreamConvCpBytes = 64 * 8;
+constexpr int stream_conv_cp_bytes(int NS) { return NS * 8; }
 
-template <int KH, int KW, int CI, int EPI>
+template <int KH, int KW, int CI, int NS, int EPI>
 __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU, "int8 results only");
@@ -49,16 +52,17 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   constexpr int K = KH * KW * CI;
   constexpr int KS = K / 32;                 // MFMA steps per block
   constexpr int ROWC = K / 16 + 1;           // 16-byte chunks per weight row in LDS (one of padding)
-  constexpr int W_INSTR = (64 * ROWC + 63) / 64;           // 1 KiB load instructions for the slice
+  constexpr int NF = NS / 32;                // 32-channel fragments of the slice
+  constexpr int W_INSTR = (NS * ROWC + 63) / 64;           // 1 KiB load instructions for the slice
   constexpr int W_PER_WAVE = (W_INSTR + NW - 1) / NW;      // every wave issues this many
-  constexpr int W_LDS = stream_conv_weight_lds(K);
+  constexpr int W_LDS = stream_conv_weight_lds(K, NS);
   constexpr int LOG2_CI = CI == 32 ? 5 : CI == 64 ? 6 : CI == 128 ? 7 : 8;
   constexpr int CP = CI / 16;                // 16-byte chunks per pixel
   constexpr int FSHIFT = 8 - LOG2_CI, FMASK = CP - 1;
   constexpr int STEPS_PER_TAP = CI / 32;
   constexpr int kOutOfRange = (int)0x80000000;
   static_assert(W_PER_WAVE * NW * 1024 <= W_LDS, "weight area");
-  static_assert(K % 32 == 0 && KS * 8 <= 160, "the filter slice must fit the registers");
+  static_assert(NS % 32 == 0 && K % 32 == 0 && KS * NF * 4 <= 160, "the filter slice must fit the registers");
 
   extern __shared__ __attribute__((aligned(1024))) int8_t smem[];
   DQ8_TRACE_POINT(0);
@@ -72,11 +76,15 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const EpiParams& e = p.epi;
 
-  const int tn = blockIdx.x % p.tiles_n;
-  const int rest = blockIdx.x / p.tiles_n;
+  // workgroup -> (pixel tile, channel slice): consecutive workgroups go to the 8 XCDs in turn,
+  // so workgroups 8 apart share an L2; those are given the slices of one pixel tile
+  const int xcd = blockIdx.x & 7, r8 = blockIdx.x >> 3;
+  const int tn = r8 % p.tiles_n;
+  const int rest = (r8 / p.tiles_n) * 8 + xcd;
+  if (rest >= p.NB * p.tiles_per_image) return;            // (the grid is rounded up to 8 tiles)
   const int tp = rest % p.tiles_per_image;
   const int img = rest / p.tiles_per_image;
-  const int n0 = tn * 64;
+  const int n0 = tn * NS;
   const int hw = p.Ho * p.Wo;
   const int p0 = tp * p.tile_px;                           // first output pixel of the tile
   const int p_end = min(p0 + p.tile_px, hw);
@@ -93,7 +101,7 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
 
   // ---- per-channel factors: the loads go out first and are used last
   ColRaw raw = {1.0f, 1.0f, 1.0f, 0};
-  if (tid < 64) raw = col_fetch<EPI>(e, n0 + tid < e.N ? n0 + tid : e.N - 1);
+  if (tid < NS) raw = col_fetch<EPI>(e, n0 + tid < e.N ? n0 + tid : e.N - 1);
 
   // ---- the weight slice: LDS rows of ROWC chunks, chunk g = 64 j + lane of instruction j
 #pragma unroll
@@ -101,7 +109,7 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
     const int j = wave + i * NW;
     const int g = j * 64 + lane;
     const int row = g / ROWC, c = g - row * ROWC;
-    const bool ok = row < 64 && c < K / 16;
+    const bool ok = row < NS && c < K / 16;
     buffer_load_lds_b128(w_rsrc, lds_base + p.patch_bytes + j * 1024,
                          ok ? row * K + (c << 4) : kOutOfRange);
   }
@@ -155,20 +163,22 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
 
   // ---- weights into registers, MFMA operand layout: lane l holds channel l % 32 of a
   // 32-channel group and the 16 bytes of k at 32 s + 16 (l / 32)
-  v4i wreg[KS][2];
+  v4i wreg[KS][NF];
   {
     const int8_t* wl = wlds + ((lane & 31) * ROWC + (lane >> 5)) * 16;
     static_for<KS>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
-      wreg[s][0] = *reinterpret_cast<const v4i*>(wl + s * 32);
-      wreg[s][1] = *reinterpret_cast<const v4i*>(wl + 32 * ROWC * 16 + s * 32);
+      static_for<NF>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        wreg[s][j] = *reinterpret_cast<const v4i*>(wl + j * 32 * ROWC * 16 + s * 32);
+      });
     });
   }
 
   DQ8_TRACE_WAVE(2);
   // ---- everything has landed for this wave; the factors are worked out and parked
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-  if (tid < 64) {
+  if (tid < NS) {
     const ColParams c = col_finish<EPI>(e, raw);
     cp[tid] = make_float2(c.os, c.b);
   }
@@ -198,7 +208,7 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
     }
 
     // pixel fragments, read PF steps ahead of their MFMAs
-    constexpr int PF = 4;
+    constexpr int PF = NF >= 2 ? 4 : 7;
     v4i fa[8];
     auto load_frag = [&](auto sc) {
       constexpr int s = decltype(sc)::value;
@@ -211,31 +221,32 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
       constexpr int s = decltype(sc)::value;
       if constexpr (s < KS) load_frag(IntC<s>());
     });
-    v16i acc[2];
+    v16i acc[NF];
     static_for<KS>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
       if constexpr (s + PF < KS) load_frag(IntC<s + PF>());
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (s == 0) {
-        // (the accumulators start from the instruction's constant zero, not from 32 moves)
-        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][0], fa[s & 7], zero, 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][1], fa[s & 7], zero, 0, 0, 0);
-      } else {
-        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][0], fa[s & 7], acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][1], fa[s & 7], acc[1], 0, 0, 0);
-      }
+      static_for<NF>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (s == 0) {
+          // (the accumulators start from the instruction's constant zero, not from moves)
+          const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][j], fa[s & 7], zero, 0, 0, 0);
+        } else {
+          acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[s][j], fa[s & 7], acc[j], 0, 0, 0);
+        }
+      });
       __builtin_amdgcn_sched_barrier(0);
     });
 
     DQ8_TRACE_WAVE(4 + 2 * ((b - wave) / NW));
-    // ---- requantise and store the block's 32 x 64 results: of a 32 x 32 fragment a lane holds
+    // ---- requantise and store the block's 32 x NS results: of a 32 x 32 fragment a lane holds
     // pixel lane % 32 and the channel quads 8 g + 4 (lane / 32) .. + 3; two half-wave swaps
     // leave it with 16 consecutive channels, one 16-byte store
     const int64_t m = (int64_t)img * hw + px_raw;
     auto finish = [&](auto mode_c) {
       constexpr bool PLAIN = decltype(mode_c)::value == 1;
-      static_for<2>([&](auto jc) {
+      static_for<NF>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         const int cl0 = j * 32 + 4 * c0;
         uint32_t w[4];
@@ -277,9 +288,9 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
 }
 
 // ---- host side (qconv_direct.hip)
-// Whether the streaming kernel can run the problem (3 x 3 filter, 64 input channels, stride and
-// dilation 1 are the caller's to check; here: sizes, and a tile whose patch fits the LDS next to
-// the weights).  Chooses the pixel tile so that the workgroups come to whole rounds of the
+// Whether the streaming kernel can run the problem (stride and dilation 1 and a padding smaller
+// than the filter are the caller's to check; here: a 3 x 3 filter on 64 or 128 input channels,
+// sizes, and a tile whose patch fits the LDS next to the weights).  Chooses the pixel tile so that the workgroups come to whole rounds of the
 // compute units with the least work per workgroup and fills tile_px, tiles_per_image, tiles_n,
 // patch_bytes, in_bytes.
 bool stream_conv_plan(DirectConvParams* p);

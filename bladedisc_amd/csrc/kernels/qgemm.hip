@@ -1267,19 +1267,29 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
                 "patch that fits the LDS");
     return launch_direct_conv(config, epilogue, d, st);
   }
-  // 3 x 3 filters on 64 channels with int8 results: the filter in registers
-  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && Ci == 64 && !fused &&
+  // 3 x 3 filters on 64 or 128 channels with int8 results: the filter in registers
+  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && (Ci == 64 || Ci == 128) && !fused &&
                             !e.fixedpoint && e.vec_store16 &&
                             (epilogue == DQ8_EPI_REQUANT_CPU || epilogue == DQ8_EPI_REQUANT_GPU);
   if (variant == kStreamConv) {
     DQ8_REQUIRE(stream_shape && stream_conv_plan(&d),
                 "dq8_qconv2d: the streaming variant needs a 3 x 3 filter with stride and dilation "
-                "1 on 64 input channels, an int8 result without fused operators and 16-byte "
+                "1 on 64 or 128 input channels, an int8 result without fused operators and 16-byte "
                 "aligned output rows");
     return launch_stream_conv(epilogue, d, st);
   }
   if (auto_pick) {
-    if (stream_shape && stream_conv_plan(&d)) return launch_stream_conv(epilogue, d, st);
+    // The streaming kernel wins at every size on 64 input channels (batch 1 to 128 of
+    // 56 x 56 x 64 -> 64: 4.9-22.1 us against 6.3-32.7 for the best of the other kernels); on 128
+    // channels, where a pixel tile's patch is loaded by four 32-channel slices, while the
+    // workgroups are one round of the chip (32 x 28 x 28 x 128 -> 128: 8.3 against 9.3 us; batch
+    // 8: 5.1 / 6.7; batch 64, two rounds: 14.7 against 14.3 for the 128 x 128 tiles).
+    if (stream_shape) {
+      DirectConvParams sp = d;
+      if (stream_conv_plan(&sp) &&
+          (Ci == 64 || (int64_t)sp.NB * sp.tiles_per_image * sp.tiles_n <= compute_units()))
+        return launch_stream_conv(epilogue, sp, st);
+    }
     if (direct_shape) {
       const int c = pick_direct_conv(NB, Ho * Wo, Ci, Co);
       if (c >= 0 && direct_conv_plan(c, &d)) return launch_direct_conv(c, epilogue, d, st);
@@ -1290,6 +1300,12 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     if (variant == kPersist256) variant = kPipe256w8;
     if (variant == kPersist256x192) variant = kPipe256x192;
     if (variant == kPersist128) variant = kPipe128w8;
+    // Up to 256 output channels the 256-row tiles, which the estimate takes from two rounds of
+    // 128 x 128 tiles on, lose to the four-wave 128 x 128 tile as an implicit GEMM (3 x 3 x 128
+    // filters: 64 x 28 x 28 -> 128 14.3 against 16.3 us, 128 x 28 x 28 27.1 / 31.8,
+    // 32 x 56 x 56 27.3 / 32.0, 32 x 28 x 28 -> 256 15.4 / 17.0).
+    if (Co <= 256 && (variant == kPipe256w8 || variant == kPipe256x192) && pipe_ok(128, 128, p, true))
+      variant = kPipe128;
   }
   return launch_epi<true>(variant, p, epilogue, st);
 }

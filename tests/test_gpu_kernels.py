@@ -27,7 +27,7 @@ def host(t):
 def gemm_variants(K, k):
     """All variant ids of the GEMM."""
     return [i for i, nm in enumerate(K.variant_names())
-            if not nm.startswith(("direct3x3_", "stream3x3_"))]
+            if not nm.startswith(("direct3x3_", "stream3x3"))]
 
 
 def make_scales(rng, n, per_channel=True):
@@ -865,27 +865,32 @@ def test_qconv_direct_random_shapes(K):
 
 
 def test_qconv_stream_variant(K):
-    """The 3 x 3 x 64-channel kernel that keeps the filter in registers: images whose pixel
+    """The 3 x 3 kernel (64 or 128 input channels) that keeps the filter in registers: images whose pixel
     tiles start and end anywhere in a row, one to many tiles per image, ragged and several
     64-channel slices of output channels, asymmetric padding, both int8 epilogues with every
     bias kind they take and an output zero point -- bit-exact against the oracle; then what it
     must refuse."""
     rng = np.random.default_rng(20260311)
-    sv = K.variant_names().index("stream3x3_64")
+    sv = K.variant_names().index("stream3x3")
     md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
-    shapes = [(2, 56, 56, 64, [1, 1, 1, 1]), (1, 3, 3, 16, [1, 1, 1, 1]), (3, 9, 7, 80, [0, 0, 0, 0]),
-              (1, 6, 150, 64, [1, 1, 1, 1]), (1, 33, 17, 208, [2, 0, 1, 2]), (5, 28, 28, 128, [1, 1, 1, 1]),
-              (1, 112, 112, 64, [1, 1, 1, 1]), (40, 14, 14, 64, [0, 2, 2, 0])]
-    for nb, h, w_, co, pad in shapes:
+    shapes = [(2, 56, 56, 64, 64, [1, 1, 1, 1]), (1, 3, 3, 64, 16, [1, 1, 1, 1]), (3, 9, 7, 64, 80, [0, 0, 0, 0]),
+              (1, 6, 150, 64, 64, [1, 1, 1, 1]), (1, 33, 17, 64, 208, [2, 0, 1, 2]),
+              (5, 28, 28, 64, 128, [1, 1, 1, 1]), (1, 112, 112, 64, 64, [1, 1, 1, 1]),
+              (40, 14, 14, 64, 64, [0, 2, 2, 0]),
+              # 128 input channels: 32-channel slices, several slices per pixel tile
+              (3, 28, 28, 128, 128, [1, 1, 1, 1]), (1, 5, 4, 128, 16, [1, 1, 1, 1]),
+              (2, 17, 33, 128, 80, [0, 2, 2, 1]), (9, 14, 14, 128, 256, [1, 1, 1, 1]),
+              (1, 56, 56, 128, 48, [1, 1, 1, 1])]
+    for nb, h, w_, ci, co, pad in shapes:
         ho, wo = h + pad[0] + pad[1] - 2, w_ + pad[2] + pad[3] - 2
-        x = rng.integers(-128, 128, (nb, h, w_, 64), dtype=np.int8)
-        wt = rng.integers(-128, 128, (co, 3, 3, 64), dtype=np.int8)
+        x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, 3, 3, ci), dtype=np.int8)
         out_shape = [nb, ho, wo, co]
         acc = O.conv_s32(x, wt, pad, md, out_shape)
         sx, sw = make_scales(rng, co)
         so = pick_so(acc, sx, sw)
         scales = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])))
-        tag = "%dx%dx%dx64 -> %d pad %s" % (nb, h, w_, co, pad)
+        tag = "%dx%dx%dx%d -> %d pad %s" % (nb, h, w_, ci, co, pad)
         a2 = acc.reshape(-1, co)
         # E1: plain, f32 bias (folded to s32 as the library does) with an output zero point, s32 bias
         got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, variant=sv, **scales))
