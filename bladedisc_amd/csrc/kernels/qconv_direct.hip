@@ -146,10 +146,10 @@ bool stream_conv_plan(DirectConvParams* p) {
 }
 
 namespace {
-template <int KH, int KW, int CI, int NS, int EPI>
+template <int KH, int KW, int CI, int NS, int EPI, bool POST>
 int launch_stream_t(const DirectConvParams& p, hipStream_t st) {
   const int lds = p.patch_bytes + stream_conv_weight_lds(KH * KW * CI, NS) + stream_conv_cp_bytes(NS);
-  auto kern = qconv_stream_kernel<KH, KW, CI, NS, EPI>;
+  auto kern = qconv_stream_kernel<KH, KW, CI, NS, EPI, POST>;
   static std::atomic<uint64_t> lds_allowed{0};
   if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), kLdsBytes, &lds_allowed)) return s;
   // (pixel tiles rounded up to a multiple of 8: workgroup b works on tile 8 (b / 8 / slices) + b % 8)
@@ -160,8 +160,13 @@ int launch_stream_t(const DirectConvParams& p, hipStream_t st) {
 
 template <int EPI>
 int launch_stream_epi(const DirectConvParams& p, hipStream_t st) {
-  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 64) return launch_stream_t<3, 3, 64, 64, EPI>(p, st);
-  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 128) return launch_stream_t<3, 3, 128, 32, EPI>(p, st);
+  const bool post = p.epi.table != nullptr || p.epi.resid_kind != 0;
+  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 64)
+    return post ? launch_stream_t<3, 3, 64, 64, EPI, true>(p, st)
+                : launch_stream_t<3, 3, 64, 64, EPI, false>(p, st);
+  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 128)
+    return post ? launch_stream_t<3, 3, 128, 32, EPI, true>(p, st)
+                : launch_stream_t<3, 3, 128, 32, EPI, false>(p, st);
   return fail("the streaming convolution kernel has no instance for this filter");
 }
 }  // namespace

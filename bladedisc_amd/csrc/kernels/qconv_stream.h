@@ -20,7 +20,8 @@
 //    block.  The two waves of a SIMD drift apart by themselves (the older wave wins the matrix
 //    pipe), so one wave's epilogue runs under the other's MFMAs.
 // The weights go to LDS before the patch and are copied to registers while the patch is still
-// arriving.  int8 results only (REQUANT_CPU / REQUANT_GPU), 16-byte aligned output rows.
+// arriving.  int8 results only (REQUANT_CPU / REQUANT_GPU, with or without the fused operators of
+// dq8_qconv2d_fused), 16-byte aligned output rows.
 #ifndef DQ8_QCONV_STREAM_H_
 #define DQ8_QCONV_STREAM_H_
 
@@ -41,9 +42,11 @@ namespace dq8 {
 constexpr int stream_conv_weight_lds(int K, int NS) {
   return ((NS * (K / 16 + 1) + 511) / 512) * 512 * 16;
 }
-constexpr int stream_conv_cp_bytes(int NS) { return NS * 8; }
+constexpr int stream_conv_cp_bytes(int NS) { return NS * 8 + 256; }   // pairs + a fused table
 
-template <int KH, int KW, int CI, int NS, int EPI>
+// POST: the launch has operators fused behind the convolution (their code and registers are kept
+// out of the plain form).
+template <int KH, int KW, int CI, int NS, int EPI, bool POST>
 __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU, "int8 results only");
@@ -70,6 +73,7 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   int8_t* patch = smem;
   int8_t* wlds = smem + p.patch_bytes;
   float2* cp = reinterpret_cast<float2*>(smem + p.patch_bytes + W_LDS);
+  uint8_t* tab = reinterpret_cast<uint8_t*>(smem + p.patch_bytes + W_LDS + NS * 8);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -102,6 +106,9 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   // ---- per-channel factors: the loads go out first and are used last
   ColRaw raw = {1.0f, 1.0f, 1.0f, 0};
   if (tid < NS) raw = col_fetch<EPI>(e, n0 + tid < e.N ? n0 + tid : e.N - 1);
+  uint32_t tab_word = 0;
+  if (POST && e.table && tid >= 64 && tid < 128)      // (a fused table: 256 bytes, fetched by wave 1)
+    tab_word = reinterpret_cast<const uint32_t*>(e.table)[tid - 64];
 
   // ---- the weight slice: LDS rows of ROWC chunks, chunk g = 64 j + lane of instruction j
 #pragma unroll
@@ -182,6 +189,7 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
     const ColParams c = col_finish<EPI>(e, raw);
     cp[tid] = make_float2(c.os, c.b);
   }
+  if (POST && e.table && tid >= 64 && tid < 128) reinterpret_cast<uint32_t*>(tab)[tid - 64] = tab_word;
   __syncthreads();
   DQ8_TRACE_POINT(1);
   DQ8_TRACE_WAVE(3);
@@ -261,8 +269,10 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
         }
         const auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
         const auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
-        const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+        v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
         const int n = n0 + j * 32 + 16 * c0;
+        // (operators fused behind the convolution: a table, or + residual [, ReLU] and quantize)
+        if (POST && (e.table || e.resid_kind)) fused_tail16(e, tab, m, n, px_raw < p_end, v);
         if (px_raw < p_end && n < e.N) {
           int8_t* dst = out + m * e.ldo + n;
           if (n + 15 < e.N) {

@@ -1268,13 +1268,13 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     return launch_direct_conv(config, epilogue, d, st);
   }
   // 3 x 3 filters on 64 or 128 channels with int8 results: the filter in registers
-  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && (Ci == 64 || Ci == 128) && !fused &&
+  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && (Ci == 64 || Ci == 128) &&
                             !e.fixedpoint && e.vec_store16 &&
                             (epilogue == DQ8_EPI_REQUANT_CPU || epilogue == DQ8_EPI_REQUANT_GPU);
   if (variant == kStreamConv) {
     DQ8_REQUIRE(stream_shape && stream_conv_plan(&d),
                 "dq8_qconv2d: the streaming variant needs a 3 x 3 filter with stride and dilation "
-                "1 on 64 or 128 input channels, an int8 result without fused operators and 16-byte "
+                "1 on 64 or 128 input channels, an int8 result (float output stage) and 16-byte "
                 "aligned output rows");
     return launch_stream_conv(epilogue, d, st);
   }

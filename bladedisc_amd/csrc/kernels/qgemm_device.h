@@ -504,6 +504,62 @@ __device__ __forceinline__ void tile_coords(int bid, int nblocks, int tiles_m, i
   tn = in_panel / rows;
 }
 
+// Operators fused behind the quantized result of an int8 epilogue.  `v` holds the 16 consecutive
+// channels n .. n + 15 of output row m (which is also how the residual is read); `tab` is the
+// 256-entry table in LDS when e.table is set; `row_ok`: the row exists.  Table:
+// v = table[(uint8) v]; residual: v = quantize(resid_add(dequantize(v), r)) with the arithmetic
+// of the separate library calls.
+__device__ __forceinline__ void fused_tail16(const EpiParams& e, const uint8_t* tab, int64_t m,
+                                             int n, bool row_ok, v4i& v) {
+  if (e.table) {
+    static_for<4>([&](auto dc) {
+      constexpr int d = decltype(dc)::value;
+      const uint32_t x = (uint32_t)v[d];
+      v[d] = (int)((uint32_t)tab[x & 0xff] | ((uint32_t)tab[(x >> 8) & 0xff] << 8) |
+                   ((uint32_t)tab[(x >> 16) & 0xff] << 16) | ((uint32_t)tab[x >> 24] << 24));
+    });
+  } else if (row_ok && n < e.N) {
+    const float so_v = e.so[0], s2 = e.out_scale[0], z2 = (float)e.out_zp;
+    const bool whole = e.resid_vec && n + 15 < e.N;
+    const int64_t roff = m * e.ldr + n;
+    // the residual of the 16 channels, as f32 (channels past N: unused zeros)
+    v4f r[4];
+    if (whole && e.resid_kind == 1) {
+      const v4f* rp = reinterpret_cast<const v4f*>((const float*)e.resid + roff);
+      static_for<4>([&](auto dc) { r[decltype(dc)::value] = rp[decltype(dc)::value]; });
+    } else if (whole) {
+      const float rs = e.resid_scale[0];
+      const v4i rv = *reinterpret_cast<const v4i*>((const int8_t*)e.resid + roff);
+      static_for<4>([&](auto dc) {
+        constexpr int d = decltype(dc)::value;
+        static_for<4>([&](auto bc) {
+          constexpr int b = decltype(bc)::value;
+          r[d][b] = (float)((int)(int8_t)((uint32_t)rv[d] >> (8 * b)) - e.resid_zp) * rs;
+        });
+      });
+    } else {
+      static_for<4>([&](auto dc) {
+        constexpr int d = decltype(dc)::value;
+        static_for<4>([&](auto bc) {
+          constexpr int b = decltype(bc)::value;
+          r[d][b] = n + 4 * d + b < e.N ? resid_at(e, roff + 4 * d + b) : 0.0f;
+        });
+      });
+    }
+    static_for<4>([&](auto dc) {
+      constexpr int d = decltype(dc)::value;
+      uint32_t w2 = 0;
+      static_for<4>([&](auto bc) {
+        constexpr int b = decltype(bc)::value;
+        const int q = (int)(int8_t)((uint32_t)v[d] >> (8 * b));
+        const float t = resid_add(e, (float)(q - e.zo) * so_v, r[d][b]);
+        w2 |= ((uint32_t)quantize_s8(t, s2, z2) & 0xffu) << (8 * b);
+      });
+      v[d] = (int)w2;
+    });
+  }
+}
+
 // Hook of mfma_epilogue: called once, after the int8 results have been computed into
 // registers and before the first of them is stored (the default does nothing).
 // kPostOps: whether the epilogue carries the code of the fused operators (residual, table) and
@@ -825,57 +881,9 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
           const auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
           v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
           if (BeforeStores::kPostOps && (e.table || e.resid_kind)) {
-            // operators fused behind the quantized result: the lane holds 16 consecutive
-            // channels of one row, which is also how it reads the residual
             const int n = n_wave0 + j * 32 + 16 * (lane >> 5);
             const int64_t m = m_wave0 + i * 32 + (lane & 31);
-            if (e.table) {
-              static_for<4>([&](auto dc) {
-                constexpr int d = decltype(dc)::value;
-                const uint32_t x = (uint32_t)v[d];
-                v[d] = (int)((uint32_t)tab[x & 0xff] | ((uint32_t)tab[(x >> 8) & 0xff] << 8) |
-                             ((uint32_t)tab[(x >> 16) & 0xff] << 16) | ((uint32_t)tab[x >> 24] << 24));
-              });
-            } else if (m < m_end && n < e.N) {
-              const float so_v = e.so[0], s2 = e.out_scale[0], z2 = (float)e.out_zp;
-              const bool whole = e.resid_vec && n + 15 < e.N;
-              const int64_t roff = m * e.ldr + n;
-              // the residual of the 16 channels, as f32 (channels past N: unused zeros)
-              v4f r[4];
-              if (whole && e.resid_kind == 1) {
-                const v4f* rp = reinterpret_cast<const v4f*>((const float*)e.resid + roff);
-                static_for<4>([&](auto dc) { r[decltype(dc)::value] = rp[decltype(dc)::value]; });
-              } else if (whole) {
-                const float rs = e.resid_scale[0];
-                const v4i rv = *reinterpret_cast<const v4i*>((const int8_t*)e.resid + roff);
-                static_for<4>([&](auto dc) {
-                  constexpr int d = decltype(dc)::value;
-                  static_for<4>([&](auto bc) {
-                    constexpr int b = decltype(bc)::value;
-                    r[d][b] = (float)((int)(int8_t)((uint32_t)rv[d] >> (8 * b)) - e.resid_zp) * rs;
-                  });
-                });
-              } else {
-                static_for<4>([&](auto dc) {
-                  constexpr int d = decltype(dc)::value;
-                  static_for<4>([&](auto bc) {
-                    constexpr int b = decltype(bc)::value;
-                    r[d][b] = n + 4 * d + b < e.N ? resid_at(e, roff + 4 * d + b) : 0.0f;
-                  });
-                });
-              }
-              static_for<4>([&](auto dc) {
-                constexpr int d = decltype(dc)::value;
-                uint32_t w2 = 0;
-                static_for<4>([&](auto bc) {
-                  constexpr int b = decltype(bc)::value;
-                  const int q = (int)(int8_t)((uint32_t)v[d] >> (8 * b));
-                  const float t = resid_add(e, (float)(q - e.zo) * so_v, r[d][b]);
-                  w2 |= ((uint32_t)quantize_s8(t, s2, z2) & 0xffu) << (8 * b);
-                });
-                v[d] = (int)w2;
-              });
-            }
+            fused_tail16(e, tab, m, n, m < m_end, v);
           }
           if (kHook)
             held[kHook ? i : 0][kHook ? j : 0] = v;

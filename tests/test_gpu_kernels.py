@@ -920,6 +920,30 @@ def test_qconv_stream_variant(K):
         # the library's own choice for this shape gives the same bytes
         auto = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(b8), **scales))
         np.testing.assert_array_equal(auto, got, err_msg=tag + " heuristic")
+    # operators fused behind the convolution run in this kernel too (the library picks it for
+    # these shapes): residual (+ ReLU) + quantize and a table, against the separate calls
+    for nb, h, w_, ci, co in [(2, 56, 56, 64, 64), (3, 28, 28, 128, 128), (1, 9, 11, 64, 80)]:
+        x = dev(rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8))
+        wt = dev(rng.integers(-128, 128, (co, 3, 3, ci), dtype=np.int8))
+        out_shape = [nb, h, w_, co]
+        sc = dict(sx=dev(np.array([0.02], np.float32)), sw=dev(rng.uniform(0.001, 0.05, co).astype(np.float32)),
+                  so=dev(np.array([9.0], np.float32)))
+        plain = K.qconv2d(x, wt, [1, 1, 1, 1], md, out_shape, K.EPI_REQUANT_CPU, **sc)
+        z1 = torch.zeros(1, dtype=torch.int32, device="cuda")
+        res = dev(rng.standard_normal(out_shape).astype(np.float32) * 300)
+        s2 = dev(np.array([7.0], np.float32))
+        for relu in (False, True):
+            fused = K.qconv2d(x, wt, [1, 1, 1, 1], md, out_shape, K.EPI_REQUANT_CPU, **sc,
+                              post=K.make_postops(residual=res, relu=relu, out_scale=s2, out_zp=-3))
+            t = K.dequantize(plain, sc["so"], z1) + res
+            if relu:
+                t = torch.clamp_min(t, 0.0)
+            want = K.quantize(t, s2, torch.full((1,), -3, dtype=torch.int32, device="cuda"))
+            assert torch.equal(fused, want), (nb, h, w_, ci, co, relu)
+        table = K.activation_table(torch.nn.functional.gelu, sc["so"], z1, s2, z1)
+        fused = K.qconv2d(x, wt, [1, 1, 1, 1], md, out_shape, K.EPI_REQUANT_CPU, **sc,
+                          post=K.make_postops(table=table))
+        assert torch.equal(fused, K.lut8(plain, table))
     # refusals: 4-byte results, other channel counts and filters, strides
     x = dev(rng.integers(-128, 128, (1, 8, 8, 64), dtype=np.int8))
     wt = dev(rng.integers(-128, 128, (64, 3, 3, 64), dtype=np.int8))
