@@ -150,11 +150,11 @@ int launch_persist(const MainParams& p, int per_cu, hipStream_t st) {
   return check_hip(hipGetLastError(), "qgemm_persist launch");
 }
 
-template <int NW, int MT, int EPI>
+template <int NW, int MT, int EPI, int U = 4>
 int launch_skinny_t(const MainParams& p, hipStream_t st) {
   const dim3 grid((unsigned)ceil_div(p.N, 16), (unsigned)ceil_div(p.M, 16 * MT));
   DQ8_REQUIRE(grid.y <= 65535, "small-M qgemm: M too large for this variant");
-  hipLaunchKernelGGL((qgemm_skinny_kernel<NW, MT, EPI>), grid, dim3(NW * 64), 0, st, p);
+  hipLaunchKernelGGL((qgemm_skinny_kernel<NW, MT, EPI, U>), grid, dim3(NW * 64), 0, st, p);
   return check_hip(hipGetLastError(), "qgemm_skinny launch");
 }
 
@@ -188,8 +188,29 @@ int launch_skinny(const MainParams& p, hipStream_t st) {
   const int64_t weight_bytes = (int64_t)p.N * p.K;
   int mt = 1;
   while (mt < 4 && ceil_div(p.M, 16 * mt) * weight_bytes > (20LL << 20)) mt *= 2;
-  if (mt == 1) return deep ? launch_skinny_t<8, 1, EPI>(p, st) : launch_skinny_t<4, 1, EPI>(p, st);
-  if (mt == 2) return deep ? launch_skinny_t<8, 2, EPI>(p, st) : launch_skinny_t<4, 2, EPI>(p, st);
+  // k-steps a wave keeps in flight: as many as it has altogether up to six -- a batch that is
+  // not full still issues all its loads (3072 of k on eight waves, six steps each: 4.1 -> 3.8 us
+  // at M = 16, 7.5 -> 6.9 at M = 256; 768 of k on four waves, three steps: M = 128, -> 3072 5.4 ->
+  // 4.9 us; 1024 of k on eight, two steps: 3.5 -> 3.15 us) -- and four from seven steps on
+  // unless batches of six leave fewer idle slots.
+  const int64_t steps = ceil_div(ceil_div(p.K, 64), deep ? 8 : 4);
+  int u = 4;
+  if (steps <= 2) u = 2;
+  else if (steps == 3) u = 3;
+  else if (steps == 5 || steps == 6) u = 6;
+  else if (steps >= 7 && deep && ceil_div(steps, 6) * 6 < ceil_div(steps, 4) * 4) u = 6;
+  if (mt <= 2) {
+#define DQ8_SKINNY_CASE(NW_, U_)                                              \
+  if (u == U_) return mt == 1 ? launch_skinny_t<NW_, 1, EPI, U_>(p, st)      \
+                              : launch_skinny_t<NW_, 2, EPI, U_>(p, st);
+    if (deep) {
+      DQ8_SKINNY_CASE(8, 2) DQ8_SKINNY_CASE(8, 3) DQ8_SKINNY_CASE(8, 6) DQ8_SKINNY_CASE(8, 4)
+    } else {
+      DQ8_SKINNY_CASE(4, 2) DQ8_SKINNY_CASE(4, 3) DQ8_SKINNY_CASE(4, 4)
+      return mt == 1 ? launch_skinny_t<4, 1, EPI, 4>(p, st) : launch_skinny_t<4, 2, EPI, 4>(p, st);
+    }
+#undef DQ8_SKINNY_CASE
+  }
   return deep ? launch_skinny_t<8, 4, EPI>(p, st) : launch_skinny_t<4, 4, EPI>(p, st);
 }
 

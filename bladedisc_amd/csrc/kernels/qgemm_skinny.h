@@ -18,9 +18,9 @@
 
 namespace dq8 {
 
-template <int NW, int MT, int EPI>
+// U: k-steps a wave has in flight
+template <int NW, int MT, int EPI, int U = 4>
 __global__ void __launch_bounds__(NW * 64) qgemm_skinny_kernel(const MainParams p) {
-  constexpr int U = 4;  // k-steps in flight per wave
   __shared__ int red[NW][MT][256];
   // per wave: one k-step of weights and of each row tile ([16 rows][64 k], 1 KiB each) on its
   // way from load order (consecutive lanes along a row) to fragment order
