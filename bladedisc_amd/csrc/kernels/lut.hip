@@ -16,6 +16,8 @@ __device__ __forceinline__ unsigned map4(const uint8_t* t, unsigned w) {
 }
 
 // 16 bytes per thread, one sweep; `table` is indexed by the byte's bit pattern
+// (results leave with the streaming hint, a kilobyte per store instruction:
+// [65536,4096] 89.8 -> 74.7 us, 7.2 TB/s; [4096,4096] 6.0 -> 4.8 us)
 __global__ void __launch_bounds__(kThreads)
 lut_u8_v16(const vu4* __restrict__ in, vu4* __restrict__ out, int64_t n16,
            const uint8_t* __restrict__ table) {
@@ -25,7 +27,8 @@ lut_u8_v16(const vu4* __restrict__ in, vu4* __restrict__ out, int64_t n16,
   const int64_t stride = (int64_t)gridDim.x * kThreads;
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n16; i += stride) {
     const vu4 v = in[i];
-    out[i] = (vu4){map4(t, v[0]), map4(t, v[1]), map4(t, v[2]), map4(t, v[3])};
+    const vu4 r = (vu4){map4(t, v[0]), map4(t, v[1]), map4(t, v[2]), map4(t, v[3])};
+    __builtin_nontemporal_store(r, &out[i]);
   }
 }
 

@@ -9,6 +9,19 @@
 #include "dq8_common.h"
 
 namespace dq8 {
+
+// Streaming loads and stores (the "non-temporal" hint): for tensors that are swept once.  Every
+// wave instruction below covers whole 128-byte lines.
+typedef float dq8_v4f_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void st_stream(float4* p, const float4& v) {
+  __builtin_nontemporal_store((dq8_v4f_t){v.x, v.y, v.z, v.w}, reinterpret_cast<dq8_v4f_t*>(p));
+}
+__device__ __forceinline__ void st_stream(uint32_t* p, uint32_t v) { __builtin_nontemporal_store(v, p); }
+__device__ __forceinline__ float4 ld_stream(const float4* p) {
+  const dq8_v4f_t v = __builtin_nontemporal_load(reinterpret_cast<const dq8_v4f_t*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint32_t ld_stream(const uint32_t* p) { return __builtin_nontemporal_load(p); }
 namespace elementwise {
 
 constexpr int kThreads = 256;

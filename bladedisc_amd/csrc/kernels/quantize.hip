@@ -66,6 +66,10 @@ __device__ __forceinline__ float4 dequant_word4(uint32_t w, const int4& z, const
 // two words of a thread next to each other (one 8-byte load, stores 32 bytes apart between
 // neighbouring lanes) tensors that fit the last-level cache ran a quarter slower:
 // [4096,768] 5.35 -> 4.3 us, [32,56,56,64] 8.1 -> 6.1 us, [65536,4096] 221 -> 210 us.
+// The f32 results leave with the streaming hint (every store instruction is a whole kilobyte):
+// [4096,768] 4.37 -> 3.35 us, [32,56,56,64] 6.3 -> 5.1 us, [65536,4096] 216 -> 187 us, which
+// is 7.2 TB/s; the same hint on the loads made every size slower, and on quantize's stores (a
+// fifth of its traffic) it helped some sizes and hurt others, so neither is used.
 template <bool SIGNED>
 __global__ void __launch_bounds__(kThreads)
 dequantize_tensor_v4x2(const uint32_t* __restrict__ q, float4* __restrict__ out,
@@ -78,8 +82,8 @@ dequantize_tensor_v4x2(const uint32_t* __restrict__ q, float4* __restrict__ out,
     const bool two = i + kThreads < n4;
     const uint32_t w0 = q[i];
     const uint32_t w1 = two ? q[i + kThreads] : 0u;
-    out[i] = dequant_word<SIGNED>(w0, z, s);
-    if (two) out[i + kThreads] = dequant_word<SIGNED>(w1, z, s);
+    dq8::st_stream(&out[i], dequant_word<SIGNED>(w0, z, s));
+    if (two) dq8::st_stream(&out[i + kThreads], dequant_word<SIGNED>(w1, z, s));
   }
 }
 
@@ -111,12 +115,12 @@ quantize_lastaxis_v4(const float4* __restrict__ x, uint32_t* __restrict__ out,
   };
   for (; r + 3 * step < r_end; r += 4 * step, px += 4 * hop, po += 4 * hop) {
     const float4 v0 = px[0], v1 = px[hop], v2 = px[2 * hop], v3 = px[3 * hop];
-    po[0] = one(v0);
-    po[hop] = one(v1);
-    po[2 * hop] = one(v2);
-    po[3 * hop] = one(v3);
+    dq8::st_stream(&po[0], one(v0));
+    dq8::st_stream(&po[hop], one(v1));
+    dq8::st_stream(&po[2 * hop], one(v2));
+    dq8::st_stream(&po[3 * hop], one(v3));
   }
-  for (; r < r_end; r += step, px += hop, po += hop) po[0] = one(px[0]);
+  for (; r < r_end; r += step, px += hop, po += hop) dq8::st_stream(&po[0], one(px[0]));
 }
 
 template <bool SIGNED>
@@ -138,12 +142,13 @@ dequantize_lastaxis_v4(const uint32_t* __restrict__ q, float4* __restrict__ out,
   float4* po = out + r * nch4 + c4;
   for (; r + 3 * step < r_end; r += 4 * step, pq += 4 * hop, po += 4 * hop) {
     const uint32_t w0 = pq[0], w1 = pq[hop], w2 = pq[2 * hop], w3 = pq[3 * hop];
-    po[0] = dequant_word4<SIGNED>(w0, z, s);
-    po[hop] = dequant_word4<SIGNED>(w1, z, s);
-    po[2 * hop] = dequant_word4<SIGNED>(w2, z, s);
-    po[3 * hop] = dequant_word4<SIGNED>(w3, z, s);
+    dq8::st_stream(&po[0], dequant_word4<SIGNED>(w0, z, s));
+    dq8::st_stream(&po[hop], dequant_word4<SIGNED>(w1, z, s));
+    dq8::st_stream(&po[2 * hop], dequant_word4<SIGNED>(w2, z, s));
+    dq8::st_stream(&po[3 * hop], dequant_word4<SIGNED>(w3, z, s));
   }
-  for (; r < r_end; r += step, pq += hop, po += hop) po[0] = dequant_word4<SIGNED>(pq[0], z, s);
+  for (; r < r_end; r += step, pq += hop, po += hop)
+    dq8::st_stream(&po[0], dequant_word4<SIGNED>(pq[0], z, s));
 }
 
 // ------------------------------------- per channel, inner % 4 == 0 (any axis)
@@ -192,10 +197,10 @@ dequantize_rows(const uint32_t* __restrict__ q, float4* __restrict__ out,
       const bool two = i + kThreads < inner_words;
       const uint32_t w0 = pq[i];
       const uint32_t w1 = two ? pq[i + kThreads] : 0u;
-      po[i] = dequant_word<SIGNED>(w0, z, s);
-      if (two) po[i + kThreads] = dequant_word<SIGNED>(w1, z, s);
+      dq8::st_stream(&po[i], dequant_word<SIGNED>(w0, z, s));
+      if (two) dq8::st_stream(&po[i + kThreads], dequant_word<SIGNED>(w1, z, s));
     } else {
-      po[i] = dequant_word<SIGNED>(pq[i], z, s);
+      dq8::st_stream(&po[i], dequant_word<SIGNED>(pq[i], z, s));
     }
   }
 }
@@ -220,8 +225,8 @@ fake_quant_tensor_v4(const float4* __restrict__ x, float4* __restrict__ out, int
   const int64_t stride = (int64_t)gridDim.x * kThreads;
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n4; i += stride) {
     const float4 v = x[i];
-    out[i] = make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
-                         fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi));
+    dq8::st_stream(&out[i], make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
+                                        fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi)));
   }
 }
 
@@ -247,12 +252,12 @@ fake_quant_lastaxis_v4(const float4* __restrict__ x, float4* __restrict__ out, i
   };
   for (; r + 3 * step < r_end; r += 4 * step, px += 4 * hop, po += 4 * hop) {
     const float4 v0 = px[0], v1 = px[hop], v2 = px[2 * hop], v3 = px[3 * hop];
-    po[0] = one(v0);
-    po[hop] = one(v1);
-    po[2 * hop] = one(v2);
-    po[3 * hop] = one(v3);
+    dq8::st_stream(&po[0], one(v0));
+    dq8::st_stream(&po[hop], one(v1));
+    dq8::st_stream(&po[2 * hop], one(v2));
+    dq8::st_stream(&po[3 * hop], one(v3));
   }
-  for (; r < r_end; r += step, px += hop, po += hop) po[0] = one(px[0]);
+  for (; r < r_end; r += step, px += hop, po += hop) dq8::st_stream(&po[0], one(px[0]));
 }
 
 template <int ROUND>
@@ -268,9 +273,9 @@ fake_quant_rows_v4(const float4* __restrict__ x, float4* __restrict__ out, unsig
   const unsigned c = row % nch;
   const float s = scale[c];
   const int z = zp[c];
-  out[(int64_t)row * inner4 + i] =
-      make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
-                  fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi));
+  dq8::st_stream(&out[(int64_t)row * inner4 + i],
+                 make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
+                             fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi)));
 }
 
 template <int ROUND>
