@@ -83,6 +83,32 @@ __device__ __forceinline__ float4 div4_by_constant(const float4& x, float s, flo
   return q;
 }
 
+// The same with a divisor per component (per-channel scales on the last axis).
+__device__ __forceinline__ float4 div4_by_constants(const float4& x, const float4& s, const float4& y) {
+  float4 q;
+  {
+    const float a = x.x * y.x, b = x.y * y.y, c = x.z * y.z, d = x.w * y.w;
+    q.x = __builtin_fmaf(__builtin_fmaf(-a, s.x, x.x), y.x, a);
+    q.y = __builtin_fmaf(__builtin_fmaf(-b, s.y, x.y), y.y, b);
+    q.z = __builtin_fmaf(__builtin_fmaf(-c, s.z, x.z), y.z, c);
+    q.w = __builtin_fmaf(__builtin_fmaf(-d, s.w, x.w), y.w, d);
+  }
+  const float probe = (q.x + q.y) + (q.z + q.w);
+  if (__builtin_expect(!(probe == probe) || __builtin_fabsf(probe) == __builtin_inff(), 0)) {
+    q.x = x.x / s.x;
+    q.y = x.y / s.y;
+    q.z = x.z / s.z;
+    q.w = x.w / s.w;
+  }
+  return q;
+}
+
+// Whether div4_by_constant may be used with divisor s.
+__device__ __forceinline__ bool divisor_in_fast_range(float s) {
+  const float a = __builtin_fabsf(s);
+  return a >= 9.094947017729282e-13f && a <= 1099511627776.0f;   // 2^-40 .. 2^40
+}
+
 // quant_one from the quotient on (zero point 0)
 template <int ROUND>
 __device__ __forceinline__ int quant_from_quotient(float t0, float lo, float hi) {
@@ -96,11 +122,13 @@ __device__ __forceinline__ int quant_from_quotient(float t0, float lo, float hi)
 // quant_one's fmaxf / fminf pair does), then one addition of 1.5 * 2^23 per value rounds to the
 // nearest-even integer and leaves its two's-complement int8 in the low byte of the sum, which
 // the sub-dword form of the add writes straight into its byte of the word.
-__device__ __forceinline__ uint32_t quant4_pack_rne(const float4& t) {
-  const float c0 = __builtin_amdgcn_fmed3f(t.x, -128.0f, 127.0f);
-  const float c1 = __builtin_amdgcn_fmed3f(t.y, -128.0f, 127.0f);
-  const float c2 = __builtin_amdgcn_fmed3f(t.z, -128.0f, 127.0f);
-  const float c3 = __builtin_amdgcn_fmed3f(t.w, -128.0f, 127.0f);
+// (lo, hi: integers in [-128, 255] -- the bounds of an 8-bit type or inside them)
+__device__ __forceinline__ uint32_t quant4_pack_rne(const float4& t, float lo = -128.0f,
+                                                    float hi = 127.0f) {
+  const float c0 = __builtin_amdgcn_fmed3f(t.x, lo, hi);
+  const float c1 = __builtin_amdgcn_fmed3f(t.y, lo, hi);
+  const float c2 = __builtin_amdgcn_fmed3f(t.z, lo, hi);
+  const float c3 = __builtin_amdgcn_fmed3f(t.w, lo, hi);
   const float magic = 12582912.0f;
   uint32_t word = __float_as_uint(c0 + magic);   // byte 0; bytes 1 .. 3 are replaced below
 #if defined(__HIP_DEVICE_COMPILE__)
