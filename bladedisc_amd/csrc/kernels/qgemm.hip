@@ -1300,11 +1300,14 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     if (variant == kPersist256) variant = kPipe256w8;
     if (variant == kPersist256x192) variant = kPipe256x192;
     if (variant == kPersist128) variant = kPipe128w8;
-    // Up to 256 output channels the 256-row tiles, which the estimate takes from two rounds of
-    // 128 x 128 tiles on, lose to the four-wave 128 x 128 tile as an implicit GEMM (3 x 3 x 128
-    // filters: 64 x 28 x 28 -> 128 14.3 against 16.3 us, 128 x 28 x 28 27.1 / 31.8,
-    // 32 x 56 x 56 27.3 / 32.0, 32 x 28 x 28 -> 256 15.4 / 17.0).
-    if (Co <= 256 && (variant == kPipe256w8 || variant == kPipe256x192) && pipe_ok(128, 128, p, true))
+    // As implicit GEMMs the 256-row tiles, which the estimate takes from two rounds of 128 x 128
+    // tiles on, lose to the four-wave 128 x 128 tile where half their columns are empty (up to
+    // 128 output channels) or where they do not fill three quarters of the compute units (3 x 3
+    // x 128 filters: 64 x 28 x 28 -> 128 14.3 against 16.3 us, 128 x 28 x 28 27.1 / 31.8,
+    // 32 x 56 x 56 27.3 / 32.0, 32 x 28 x 28 -> 256 15.4 / 17.0; 64 x 28 x 28 x 256 -> 256, 196
+    // tiles of 256 x 256, keeps them: 33.7 against 44.5 us).
+    if ((variant == kPipe256w8 || variant == kPipe256x192) && pipe_ok(128, 128, p, true) &&
+        (Co <= 128 || (Co <= 256 && 4 * ceil_div(Mg, 256) * ceil_div(Co, 256) < 3 * compute_units())))
       variant = kPipe128;
   }
   return launch_epi<true>(variant, p, epilogue, st);
