@@ -112,11 +112,9 @@ bool stream_conv_plan(DirectConvParams* p) {
   for (int64_t tpi = 1; tpi <= ceil_div(hw, 32); ++tpi) {
     const int64_t tile = ceil_div(hw, tpi);
     if (ceil_div(hw, tile) != tpi) continue;               // the same tiling as a smaller tpi
-    int64_t span = 0;
-    for (int64_t t = 0; t < tpi; ++t) {
-      const int64_t first = t * tile, last = std::min(first + tile, hw) - 1;
-      span = std::max(span, last / p->Wo - first / p->Wo + 1);
-    }
+    // image rows a tile of `tile` consecutive pixels can span, wherever it starts in a row (an
+    // upper bound for this tiling, in closed form: the planner is called per launch)
+    const int64_t span = std::min<int64_t>((tile + p->Wo - 2) / p->Wo + 1, p->Ho);
     const int64_t patch = ((span + p->Kh - 1) * pitch * p->Ci + 1023) / 1024 * 1024;
     if (patch > fixed) continue;
     const int64_t blocks = ceil_div(tile, 32);
