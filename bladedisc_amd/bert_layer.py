@@ -146,13 +146,16 @@ class QuantBertLayer:
         return _layer_norm(h, self.f["emb_ln_g"], self.f["emb_ln_b"])
 
     def attention(self, qkv):
-        """softmax(q k^T / sqrt(d)) v in fp32.  qkv: [B, S, 3H] -> [B, S, H]."""
+        """softmax(q k^T / sqrt(d)) v in fp32, PyTorch's fused kernel.  qkv: [B, S, 3H] -> [B, S, H].
+        (Written out as two batched products, a scale and a softmax the same arithmetic is nine
+        launches, half of them copies into head-major layout: 73 -> 53 us for the whole layer at
+        batch 8 x seq 32, 248 -> 178 us at seq 384.)"""
         b, s, h3 = qkv.shape
         h = h3 // 3
         dh = h // self.heads
         q, k, v = (t.reshape(b, s, self.heads, dh).transpose(1, 2) for t in qkv.split(h, dim=-1))
-        p = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(dh), dim=-1)
-        return (p @ v).transpose(1, 2).reshape(b, s, h)
+        o = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+        return o.transpose(1, 2).reshape(b, s, h)
 
     def _linear_fp32(self, name, x):
         return x @ torch.from_numpy(self.fw[name]).to(self.device).T + self.bias[name]
