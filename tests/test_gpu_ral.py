@@ -389,7 +389,10 @@ def test_ral_pdll_weight_only_qgemm_weight_that_is_not_a_constant(rt, dtype):
 
 
 @pytest.mark.parametrize("nb,h,ci,co,k,stride,pad", [(2, 14, 64, 64, 3, 1, 1), (2, 7, 256, 128, 1, 1, 0),
-                                                      (1, 9, 32, 16, 3, 2, 1), (2, 30, 3, 64, 7, 2, 3)])
+                                                      (1, 9, 32, 16, 3, 2, 1), (2, 30, 3, 64, 7, 2, 3),
+                                                      # 3 x 3 on 128 channels: 32-channel slices of
+                                                      # the kernel that keeps the filter in registers
+                                                      (3, 28, 128, 128, 3, 1, 1)])
 def test_ral_qconv(rt, nb, h, ci, co, k, stride, pad):
     ctx, ral, ops = rt
     rng = np.random.default_rng(h + ci)
