@@ -257,18 +257,42 @@ __device__ __forceinline__ float fake_one(float x, float s, int zi, float lo, fl
   return (float)(q - zi) * s;
 }
 
+// fake_one on four values with one divisor through its reciprocal (the quotient's bits are those
+// of x / s, see div4_by_constant)
+template <int ROUND>
+__device__ __forceinline__ float4 fake4_by_constant(const float4& v, float s, float y, int zi,
+                                                    float lo, float hi) {
+  const float4 q = div4_by_constant(v, s, y);
+  const float z = (float)zi;
+  auto one = [&](float t0) {
+    const int qi = quant_from_quotient<ROUND>(t0 + z, lo, hi);
+    return (float)(qi - zi) * s;
+  };
+  return make_float4(one(q.x), one(q.y), one(q.z), one(q.w));
+}
+
 template <int ROUND>
 __global__ void __launch_bounds__(kThreads)
 fake_quant_tensor_v4(const float4* __restrict__ x, float4* __restrict__ out, int64_t n4,
                      const float* __restrict__ scale, const int32_t* __restrict__ zp, float lo,
                      float hi) {
+  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= n4) return;
+  float4 v = x[i];                        // (the data load first, as in quantize_tensor_v4)
+  __builtin_amdgcn_sched_barrier(0);
   const float s = scale[0];
   const int z = zp[0];
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n4; i += stride) {
-    const float4 v = x[i];
-    dq8::st_stream(&out[i], make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
-                                        fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi)));
+  const float y = 1.0f / s;
+  const bool fast = divisor_in_fast_range(s);
+  for (;;) {
+    dq8::st_stream(&out[i],
+                   fast ? fake4_by_constant<ROUND>(v, s, y, z, lo, hi)
+                        : make_float4(fake_one<ROUND>(v.x, s, z, lo, hi), fake_one<ROUND>(v.y, s, z, lo, hi),
+                                      fake_one<ROUND>(v.z, s, z, lo, hi), fake_one<ROUND>(v.w, s, z, lo, hi)));
+    i += stride;
+    if (i >= n4) break;
+    v = x[i];
   }
 }
 
