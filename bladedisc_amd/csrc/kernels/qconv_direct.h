@@ -43,6 +43,7 @@ struct DirectConvParams {
   int tile_px;          // output pixels per tile where that is not a template parameter
   int patch_pitch;      // (streaming kernel) pixels per patch row in LDS: Wo + Kw - 1 rounded up to 16
   unsigned wo_inv;      // (streaming kernel) floor(2^32 / Wo) + 1: pixel / Wo == umulhi(pixel, wo_inv)
+  int slice_n;          // (streaming kernel) output channels per workgroup
   int tiles_per_image;  // ceil(Ho * Wo / BM)
   int tiles_n;          // ceil(Co / BN)
   int patch_bytes;      // LDS reserved for the patch: (most rows a tile spans + Kh - 1) *

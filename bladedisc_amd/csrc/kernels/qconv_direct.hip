@@ -84,16 +84,28 @@ bool direct_conv_plan(int config, DirectConvParams* p) {
 }
 
 namespace {
-// output channels per workgroup of the streaming kernel for a filter, 0 if it has no instance
-int stream_conv_slice(int Kh, int Kw, int Ci) {
-  if (Kh == 3 && Kw == 3 && Ci == 64) return 64;
-  if (Kh == 3 && Kw == 3 && Ci == 128) return 32;
+// The (filter, slice) pairs the streaming kernel is instantiated for: 3 x 3 filters on 64 and 128
+// channels, and 1 x 1 filters (a GEMM over the pixels with a short k) on the same.  A slice is as
+// wide as the registers allow -- NS K / 256 of them hold it, next to 16 accumulators per 32
+// channels of it -- since every workgroup of a pixel tile loads the tile's patch again; `narrow`
+// is a second width for layers with no more output channels than that.
+struct StreamInstance {
+  int kh, kw, ci, ns, narrow;
+};
+constexpr StreamInstance kStreamInstances[] = {
+    {3, 3, 64, 64, 0}, {3, 3, 128, 32, 0}, {1, 1, 64, 128, 64}, {1, 1, 128, 128, 0},
+};
+int stream_conv_slice(int Kh, int Kw, int Ci, int Co) {
+  for (const StreamInstance& s : kStreamInstances)
+    if (s.kh == Kh && s.kw == Kw && s.ci == Ci) return s.narrow && Co <= s.narrow ? s.narrow : s.ns;
   return 0;
 }
 }  // namespace
 
+bool stream_conv_has_instance(int Kh, int Kw, int Ci) { return stream_conv_slice(Kh, Kw, Ci, 1) != 0; }
+
 bool stream_conv_plan(DirectConvParams* p) {
-  const int ns = stream_conv_slice(p->Kh, p->Kw, p->Ci);
+  const int ns = stream_conv_slice(p->Kh, p->Kw, p->Ci, p->Co);
   if (ns == 0) return false;
   if (p->NB <= 0 || p->Ho <= 0 || p->Wo <= 1 || p->Co <= 0) return false;
   const int K = p->Kh * p->Kw * p->Ci;
@@ -105,9 +117,14 @@ bool stream_conv_plan(DirectConvParams* p) {
   const int64_t tiles_n = ceil_div(p->Co, ns);
   const int64_t cus = compute_units();
   const int fixed = kLdsBytes - stream_conv_weight_lds(K, ns) - stream_conv_cp_bytes(ns);
-  // Time of a launch in units of one block of 32 pixels on one SIMD: rounds of workgroups x
-  // (blocks of the busiest SIMD -- it runs waves 0 and 4, which take blocks 0, 8, ... and
-  // 4, 12, ... -- plus about three block times of loading and of the last epilogue).
+  // Time of a launch in cycles of a SIMD: rounds of workgroups x (blocks of 32 pixels of the
+  // busiest SIMD -- it runs waves 0 and 4, which take blocks 0, 8, ... and 4, 12, ... -- each K / 32
+  // MFMAs of 32 cycles per 32 channels plus the part of their requantisation that does not
+  // run under another wave's MFMAs, plus the time of loading and of the last epilogue: three
+  // blocks of a 3 x 3 filter, which is the measure for the short blocks of a 1 x 1 filter too).
+  const int64_t nf = ns / 32;
+  const int64_t block_clk = (K / 32) * nf * 32 + nf * 230;
+  const int64_t fixed_clk = p->Kh * p->Kw > 1 ? 3 * block_clk : 3 * (18 * 2 * 32 + 2 * 230);
   int64_t best_cost = -1, best_tpi = 0, best_patch = 0;
   for (int64_t tpi = 1; tpi <= ceil_div(hw, 32); ++tpi) {
     const int64_t tile = ceil_div(hw, tpi);
@@ -115,12 +132,15 @@ bool stream_conv_plan(DirectConvParams* p) {
     // image rows a tile of `tile` consecutive pixels can span, wherever it starts in a row (an
     // upper bound for this tiling, in closed form: the planner is called per launch)
     const int64_t span = std::min<int64_t>((tile + p->Wo - 2) / p->Wo + 1, p->Ho);
-    const int64_t patch = ((span + p->Kh - 1) * pitch * p->Ci + 1023) / 1024 * 1024;
+    // (1 x 1: the tile's pixels as they come, whole blocks of 32)
+    const int64_t patch = p->Kh * p->Kw == 1
+                              ? (ceil_div(tile, 32) * 32 * p->Ci + 1023) / 1024 * 1024
+                              : ((span + p->Kh - 1) * pitch * p->Ci + 1023) / 1024 * 1024;
     if (patch > fixed) continue;
     const int64_t blocks = ceil_div(tile, 32);
     const int64_t simd0 = ceil_div(blocks, 8) + (blocks > 4 ? ceil_div(blocks - 4, 8) : 0);
     const int64_t wgs = (int64_t)p->NB * tpi * tiles_n;
-    const int64_t cost = ceil_div(wgs, cus) * (simd0 + 3);
+    const int64_t cost = ceil_div(wgs, cus) * (simd0 * block_clk + fixed_clk);
     if (best_cost < 0 || cost < best_cost || (cost == best_cost && wgs <= cus)) {
       best_cost = cost;
       best_tpi = tpi;
@@ -136,6 +156,7 @@ bool stream_conv_plan(DirectConvParams* p) {
   p->tile_px = (int)ceil_div(hw, best_tpi);
   p->patch_pitch = (int)pitch;
   p->wo_inv = (unsigned)((1ULL << 32) / (uint64_t)p->Wo + 1);
+  p->slice_n = ns;
   p->tiles_per_image = (int)best_tpi;
   p->tiles_n = (int)tiles_n;
   p->patch_bytes = (int)best_patch;
@@ -156,15 +177,21 @@ int launch_stream_t(const DirectConvParams& p, hipStream_t st) {
   return check_hip(hipGetLastError(), "qconv_stream launch");
 }
 
+template <int KH, int KW, int CI, int NS, int EPI>
+int launch_stream_post(const DirectConvParams& p, hipStream_t st) {
+  const bool post = p.epi.table != nullptr || p.epi.resid_kind != 0;
+  return post ? launch_stream_t<KH, KW, CI, NS, EPI, true>(p, st)
+              : launch_stream_t<KH, KW, CI, NS, EPI, false>(p, st);
+}
+
 template <int EPI>
 int launch_stream_epi(const DirectConvParams& p, hipStream_t st) {
-  const bool post = p.epi.table != nullptr || p.epi.resid_kind != 0;
-  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 64)
-    return post ? launch_stream_t<3, 3, 64, 64, EPI, true>(p, st)
-                : launch_stream_t<3, 3, 64, 64, EPI, false>(p, st);
-  if (p.Kh == 3 && p.Kw == 3 && p.Ci == 128)
-    return post ? launch_stream_t<3, 3, 128, 32, EPI, true>(p, st)
-                : launch_stream_t<3, 3, 128, 32, EPI, false>(p, st);
+  const int taps = p.Kh * p.Kw;
+  if (taps == 9 && p.Ci == 64 && p.slice_n == 64) return launch_stream_post<3, 3, 64, 64, EPI>(p, st);
+  if (taps == 9 && p.Ci == 128 && p.slice_n == 32) return launch_stream_post<3, 3, 128, 32, EPI>(p, st);
+  if (taps == 1 && p.Ci == 64 && p.slice_n == 128) return launch_stream_post<1, 1, 64, 128, EPI>(p, st);
+  if (taps == 1 && p.Ci == 64 && p.slice_n == 64) return launch_stream_post<1, 1, 64, 64, EPI>(p, st);
+  if (taps == 1 && p.Ci == 128 && p.slice_n == 128) return launch_stream_post<1, 1, 128, 128, EPI>(p, st);
   return fail("the streaming convolution kernel has no instance for this filter");
 }
 }  // namespace

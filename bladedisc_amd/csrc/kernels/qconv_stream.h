@@ -1,6 +1,7 @@
 // int8 NHWC stride-1 convolution with the whole filter in registers ("streaming" form), for
 // filters of which a slice of NS output channels fits there: NS * Kh * Kw * Ci <= 36 KiB
-// (3 x 3 x 64 with 64-channel slices in the first place, 3 x 3 x 128 with 32-channel slices).
+// (3 x 3 x 64 with 64-channel slices in the first place, 3 x 3 x 128 with 32-channel slices,
+// 1 x 1 x 64 and 1 x 1 x 128 with 128-channel slices).
 //
 // Where the time of such a layer goes in the LDS-tiled kernels (32 x 56 x 56 x 64 -> 64, 9 us):
 // every workgroup loads, then multiplies, then requantises and stores, all in the same phase, so
@@ -20,7 +21,13 @@
 //    block.  The two waves of a SIMD drift apart by themselves (the older wave wins the matrix
 //    pipe), so one wave's epilogue runs under the other's MFMAs.
 // The weights go to LDS before the patch and are copied to registers while the patch is still
-// arriving.  int8 results only (REQUANT_CPU / REQUANT_GPU, with or without the fused operators of
+// arriving.
+// A 1 x 1 filter (a GEMM over the pixels with k = Ci) runs the same way on 64 or 128 channels,
+// where the GEMM kernels' k tile of 128 is short or half empty and their lock-step
+// requantisation is most of the time; its blocks share no pixels, so a wave loads those of its
+// own blocks and waits for no other wave's: the first block's before the weights' barrier, the
+// others' while the first is multiplied.
+// int8 results only (REQUANT_CPU / REQUANT_GPU, with or without the fused operators of
 // dq8_qconv2d_fused), 16-byte aligned output rows.
 #ifndef DQ8_QCONV_STREAM_H_
 #define DQ8_QCONV_STREAM_H_
@@ -50,7 +57,7 @@ template <int KH, int KW, int CI, int NS, int EPI, bool POST>
 __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU, "int8 results only");
-  static_assert(CI == 32 || CI == 64 || CI == 128 || CI == 256, "channels per pixel");
+  static_assert(CI == 32 || CI == 64 || CI == 128 || CI == 256 || CI == 512, "channels per pixel");
   constexpr int NW = 8;
   constexpr int K = KH * KW * CI;
   constexpr int KS = K / 32;                 // MFMA steps per block
@@ -59,9 +66,10 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   constexpr int W_INSTR = (NS * ROWC + 63) / 64;           // 1 KiB load instructions for the slice
   constexpr int W_PER_WAVE = (W_INSTR + NW - 1) / NW;      // every wave issues this many
   constexpr int W_LDS = stream_conv_weight_lds(K, NS);
-  constexpr int LOG2_CI = CI == 32 ? 5 : CI == 64 ? 6 : CI == 128 ? 7 : 8;
+  constexpr int LOG2_CI = CI == 32 ? 5 : CI == 64 ? 6 : CI == 128 ? 7 : CI == 256 ? 8 : 9;
   constexpr int CP = CI / 16;                // 16-byte chunks per pixel
-  constexpr int FSHIFT = 8 - LOG2_CI, FMASK = CP - 1;
+  // (swizzle of the chunks inside a 256-byte bank row, as in qconv_direct.h)
+  constexpr int FSHIFT = LOG2_CI >= 8 ? 0 : 8 - LOG2_CI, FMASK = CP > 16 ? 15 : CP - 1;
   constexpr int STEPS_PER_TAP = CI / 32;
   constexpr int kOutOfRange = (int)0x80000000;
   static_assert(W_PER_WAVE * NW * 1024 <= W_LDS, "weight area");
@@ -121,13 +129,39 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
                          ok ? row * K + (c << 4) : kOutOfRange);
   }
 
-  // ---- the patch: instruction j of the workgroup fills LDS bytes [1024 j, 1024 j + 1024); patch
-  // rows have a pitch of PWp pixels, a multiple of 16, so that a step down a row leaves the
-  // swizzle of a pixel as it is (the pixels between the frame and the pitch are never read)
+  // ---- the patch.  1 x 1 filter: a wave loads the pixels of its own blocks, block by block, and
+  // waits for no other wave's (pixel t of the tile at LDS bytes [CI t, CI t + CI), chunks swizzled)
+  constexpr bool POINT = KH == 1 && KW == 1;
+  constexpr int IPB = CI / 32;                             // load instructions per block of 32 pixels
+  const int nblocks = (p_end - p0 + 31) >> 5;
   const int PWp = p.patch_pitch;
-  const int total = rows * PWp * CP;                       // chunks in use
-  const int n_patch = (((total + 63) >> 6) - wave + NW - 1) / NW;   // instructions of this wave
-  {
+  int n_patch;                       // patch load instructions of this wave issued ahead of the weights' wait
+  auto load_block = [&](int b) {
+#pragma unroll
+    for (int i = 0; i < IPB; ++i) {
+      const int g = i * 64 + lane;
+      const int t = b * 32 + (g >> (LOG2_CI - 4));
+      const int c = (g & (CP - 1)) ^ ((t >> FSHIFT) & FMASK);
+      const int voff = p0 + t < p_end ? ((img * hw + p0 + t) << LOG2_CI) + (c << 4) : kOutOfRange;
+      buffer_load_lds_b128(in_rsrc,
+                           (unsigned)__builtin_amdgcn_readfirstlane((int)(lds_base + (b * 32 << LOG2_CI) + i * 1024)),
+                           voff);
+    }
+  };
+  if constexpr (POINT) {
+    // (the first block now; the others once the per-channel factors, whose loads the compiler
+    // waits for with a count that knows nothing of these, have been used)
+    n_patch = 0;
+    if (wave < nblocks) {
+      load_block(wave);
+      n_patch = IPB;
+    }
+  } else {
+    // instruction j of the workgroup fills LDS bytes [1024 j, 1024 j + 1024); patch
+    // rows have a pitch of PWp pixels, a multiple of 16, so that a step down a row leaves the
+    // swizzle of a pixel as it is (the pixels between the frame and the pitch are never read)
+    const int total = rows * PWp * CP;                       // chunks in use
+    n_patch = (((total + 63) >> 6) - wave + NW - 1) / NW;
     const int img_px = img * p.H * p.Wd;
     constexpr int dq = (NW * 64) >> (LOG2_CI - 4);         // pixels per step
     const int dq_y = dq / PWp, dq_x = dq - dq_y * PWp;
@@ -157,14 +191,18 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   // ---- this wave's weight loads are the oldest in flight: they have landed once at most its
   // patch loads remain.  (Weights from one half of the waves and the patch from the other, so
   // that neither queues behind the other, was measured: both land 0.5 us later.)
-  if (n_patch >= 12) {
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(12));
-  } else {
-    static_for<12>([&](auto kc) {
-      constexpr int k = decltype(kc)::value;
-      if (n_patch == k) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(k));
-    });
-  }
+  auto wait_patch_loads = [&](int left) {   // until at most `left` of this wave's loads are in flight
+    constexpr int kMost = POINT ? 32 : 12;
+    if (left >= kMost) {
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kMost));
+    } else {
+      static_for<kMost>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        if (left == k) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(k));
+      });
+    }
+  };
+  wait_patch_loads(n_patch);
   __syncthreads();          // the weights are in LDS
   DQ8_TRACE_WAVE(1);
 
@@ -183,29 +221,43 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   }
 
   DQ8_TRACE_WAVE(2);
-  // ---- everything has landed for this wave; the factors are worked out and parked
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  // ---- everything has landed for this wave (1 x 1: all but its own pixels, which no other
+  // wave reads); the factors are worked out and parked
+  if constexpr (!POINT) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   if (tid < NS) {
     const ColParams c = col_finish<EPI>(e, raw);
     cp[tid] = make_float2(c.os, c.b);
   }
   if (POST && e.table && tid >= 64 && tid < 128) reinterpret_cast<uint32_t*>(tab)[tid - 64] = tab_word;
+  int later = 0;                     // (1 x 1) load instructions of this wave's blocks after the current one
+  if constexpr (POINT) {
+    for (int b = wave + NW; b < nblocks; b += NW) {
+      load_block(b);
+      later += IPB;
+    }
+  }
   __syncthreads();
   DQ8_TRACE_POINT(1);
   DQ8_TRACE_WAVE(3);
 
   const bool plain = e.bias_kind == DQ8_BIAS_NONE && e.zo == 0;
   int8_t* out = static_cast<int8_t*>(e.out);
-  const int nblocks = (p_end - p0 + 31) >> 5;
   const int c0 = lane >> 5;
   const int pitch_bytes = PWp << LOG2_CI;
 
   for (int b = wave; b < nblocks; b += NW) {
     // this lane's pixel: position in the patch at tap (0, 0)
     const int px_raw = p0 + b * 32 + (lane & 31);
-    const int px = px_raw < p_end ? px_raw : p_end - 1;
-    const int y = (int)__umulhi((unsigned)px, p.wo_inv), x = px - y * p.Wo;
-    const int hq = (y - y_base) * PWp + x;
+    int hq;
+    if constexpr (POINT) {
+      hq = b * 32 + (lane & 31);
+      wait_patch_loads(later);        // the block's pixels have landed (later blocks' may be on their way)
+      later -= IPB;
+    } else {
+      const int px = px_raw < p_end ? px_raw : p_end - 1;
+      const int y = (int)__umulhi((unsigned)px, p.wo_inv), x = px - y * p.Wo;
+      hq = (y - y_base) * PWp + x;
+    }
     // byte offset of this lane's 16 bytes of k-half 0 at filter column kw, filter row 0; k-half
     // h is the same with bit 5 + ... flipped (xor 32 h), filter row kh adds kh row pitches
     int a0[KW];
@@ -299,11 +351,13 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
 
 // ---- host side (qconv_direct.hip)
 // Whether the streaming kernel can run the problem (stride and dilation 1 and a padding smaller
-// than the filter are the caller's to check; here: a 3 x 3 filter on 64 or 128 input channels,
-// sizes, and a tile whose patch fits the LDS next to the weights).  Chooses the pixel tile so that the workgroups come to whole rounds of the
+// than the filter are the caller's to check; here: a 3 x 3 or 1 x 1 filter on 64 or 128 input
+// channels, sizes, and a tile whose patch fits the LDS next to the weights).  Chooses the pixel tile so that the workgroups come to whole rounds of the
 // compute units with the least work per workgroup and fills tile_px, tiles_per_image, tiles_n,
 // patch_bytes, in_bytes.
 bool stream_conv_plan(DirectConvParams* p);
+// whether the kernel is instantiated for a Kh x Kw filter on Ci channels
+bool stream_conv_has_instance(int Kh, int Kw, int Ci);
 int launch_stream_conv(int epilogue, const DirectConvParams& p, hipStream_t st);
 
 }  // namespace dq8

@@ -1211,10 +1211,46 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
         epilogue, g, Mg * Co, st);
   }
 
-  // A 1x1 filter with stride 1 and no padding is a plain GEMM over the pixels: the GEMM
-  // instantiations load their rows without the per-tap address arithmetic.
-  if (auto_pick && Kh == 1 && Kw == 1 && sh == 1 && sw_ == 1 && padding[0] == 0 &&
-      padding[1] == 0 && padding[2] == 0 && padding[3] == 0) {
+  // A 1x1 filter with stride 1 and no padding is a plain GEMM over the pixels.
+  const bool pointwise = Kh == 1 && Kw == 1 && sh == 1 && sw_ == 1 && padding[0] == 0 &&
+                         padding[1] == 0 && padding[2] == 0 && padding[3] == 0;
+  // what the streaming kernel asks of the output side
+  const bool stream_out = !e.fixedpoint && e.vec_store16 &&
+                          (epilogue == DQ8_EPI_REQUANT_CPU || epilogue == DQ8_EPI_REQUANT_GPU);
+  // On 64 or 128 input channels the filter fits the registers of the streaming kernel; its
+  // pixels are then one long row, cut into patch rows of 16 where the count allows, so that a
+  // tile is any run of pixels, across images.
+  if (pointwise && (auto_pick || variant == kStreamConv)) {
+    DirectConvParams sp = {};
+    sp.in = in;
+    sp.w = w;
+    sp.Ci = (int)Ci; sp.Co = (int)Co;
+    sp.Kh = 1; sp.Kw = 1;
+    if (Mg % 16 == 0 && Mg / 16 < (1LL << 24)) {
+      sp.NB = 1; sp.H = sp.Ho = (int)(Mg / 16); sp.Wd = sp.Wo = 16;
+    } else {
+      sp.NB = (int)NB; sp.H = sp.Ho = (int)Ho; sp.Wd = sp.Wo = (int)Wo;
+    }
+    sp.epi = e;
+    const bool ok = stream_out && Ci <= 128 && stream_conv_has_instance(1, 1, (int)Ci) &&
+                    stream_conv_plan(&sp);
+    if (!auto_pick)
+      DQ8_REQUIRE(ok, "dq8_qconv2d: the streaming variant needs a 3 x 3 or 1 x 1 filter on 64 or "
+                      "128 input channels, stride and dilation 1, an int8 result (float output "
+                      "stage) and 16-byte aligned output rows");
+    // Against the GEMM kernels, whose k tile of 128 is half empty at 64 channels and whose
+    // workgroups requantise in lock step, it wins once the launch has a few million results
+    // (us per launch, streaming / GEMM; 64 -> 256 channels on 56 x 56 images: batch 1 4.1 / 3.5,
+    // batch 4 4.7 / 4.7, batch 8 5.45 / 7.6, batch 32 11.2 / 15.3, batch 64 17.6 / 26.3; 64 -> 64,
+    // batch 32: 28 x 28 3.7 / 4.5, 56 x 56 5.5 / 7.0, 112 x 112 12.7 / 19.3; 128 -> 128, batch 32:
+    // 28 x 28 5.0 / 4.7, 56 x 56 8.7 / 12.1; 128 -> 256 on 28 x 28: 5.8 / 7.7; 128 -> 512: 8.6 / 8.8,
+    // batch 64 12.6 / 15.4.  Filters on 256 and 512 input channels were built and lost at every
+    // size: 32 x 14 x 14 x 256 -> 1024 7.85 / 7.6).
+    if (ok && (!auto_pick || Mg * Co >= (Ci == 64 ? (3LL << 19) : (6LL << 20))))
+      return launch_stream_conv(epilogue, sp, st);
+  }
+  // Otherwise the GEMM instantiations load its rows without the per-tap address arithmetic.
+  if (auto_pick && pointwise) {
     MainParams g = {};
     g.A = in;
     g.W = w;
@@ -1268,14 +1304,12 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     return launch_direct_conv(config, epilogue, d, st);
   }
   // 3 x 3 filters on 64 or 128 channels with int8 results: the filter in registers
-  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && (Ci == 64 || Ci == 128) &&
-                            !e.fixedpoint && e.vec_store16 &&
-                            (epilogue == DQ8_EPI_REQUANT_CPU || epilogue == DQ8_EPI_REQUANT_GPU);
+  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && (Ci == 64 || Ci == 128) && stream_out;
   if (variant == kStreamConv) {
     DQ8_REQUIRE(stream_shape && stream_conv_plan(&d),
-                "dq8_qconv2d: the streaming variant needs a 3 x 3 filter with stride and dilation "
-                "1 on 64 or 128 input channels, an int8 result (float output stage) and 16-byte "
-                "aligned output rows");
+                "dq8_qconv2d: the streaming variant needs a 3 x 3 or 1 x 1 filter on 64 or "
+                "128 input channels, stride and dilation 1, an int8 result (float output "
+                "stage) and 16-byte aligned output rows");
     return launch_stream_conv(epilogue, d, st);
   }
   if (auto_pick) {

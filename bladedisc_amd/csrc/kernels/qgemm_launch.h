@@ -61,9 +61,9 @@ inline constexpr Variant kVariants[] = {
     {"direct3x3_512x64", 512, 64, 128, 512},
     // 64x64 with the k tiles split over 4 groups of waves (sixteen waves, 128 KiB LDS)
     {"pipe_64x64x128_k4", 64, 64, 128, 1024},
-    // 3 x 3 filters on 64 or 128 channels held in registers, pixel tile chosen per problem
-    // (convolution only, int8 results)
-    {"stream3x3", 32, 64, 32, 512},
+    // a filter slice held in registers (3 x 3 or 1 x 1 on 64 or 128 channels), pixel tile chosen
+    // per problem (convolution only, int8 results)
+    {"stream", 32, 64, 32, 512},
 };
 constexpr int kPipe256 = 4, kPipe128 = 5, kPipe64 = 6, kPipe256x64 = 7;
 constexpr int kPipe64k2 = 8;

@@ -27,7 +27,7 @@ def host(t):
 def gemm_variants(K, k):
     """All variant ids of the GEMM."""
     return [i for i, nm in enumerate(K.variant_names())
-            if not nm.startswith(("direct3x3_", "stream3x3"))]
+            if not nm.startswith(("direct3x3_", "stream"))]
 
 
 def make_scales(rng, n, per_channel=True):
@@ -871,7 +871,7 @@ def test_qconv_stream_variant(K):
     bias kind they take and an output zero point -- bit-exact against the oracle; then what it
     must refuse."""
     rng = np.random.default_rng(20260311)
-    sv = K.variant_names().index("stream3x3")
+    sv = K.variant_names().index("stream")
     md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
     shapes = [(2, 56, 56, 64, 64, [1, 1, 1, 1]), (1, 3, 3, 64, 16, [1, 1, 1, 1]), (3, 9, 7, 64, 80, [0, 0, 0, 0]),
               (1, 6, 150, 64, 64, [1, 1, 1, 1]), (1, 33, 17, 64, 208, [2, 0, 1, 2]),
@@ -957,6 +957,96 @@ def test_qconv_stream_variant(K):
     md2 = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
     with pytest.raises(RuntimeError, match="streaming variant"):
         K.qconv2d(x, wt, [1, 1, 1, 1], md2, [1, 4, 4, 64], K.EPI_REQUANT_CPU, sx=one, sw=one, so=one, variant=sv)
+
+
+def test_qconv_stream_pointwise(K):
+    """1 x 1 filters on 64 and 128 input channels in the kernel that keeps the filter in registers
+    (a GEMM over the pixels with a short k): pixel counts that are and are not a multiple of 16
+    (one long row of pixels cut anywhere, or tiles per image), one pixel tile to many, tiles
+    that end inside a block of 32 pixels, ragged channel slices, both slice widths of the
+    64-channel filter, every bias kind of the int8 epilogues, fused operators -- bit-exact
+    against the oracle and against the library's choice; then what it must refuse."""
+    rng = np.random.default_rng(20260412)
+    names = K.variant_names()
+    sv = names.index("stream")
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    pad = [0, 0, 0, 0]
+    shapes = [(8, 56, 56, 64, 256), (2, 56, 56, 64, 64), (4, 28, 28, 128, 512), (3, 7, 7, 128, 2048),
+              (1, 4, 4, 128, 16), (5, 9, 7, 64, 208), (1, 1, 48, 64, 80), (7, 13, 3, 128, 144),
+              (2, 23, 5, 128, 96), (1, 56, 56, 128, 64), (1, 1, 16, 64, 16), (3, 5, 11, 64, 400),
+              (1, 1, 33, 64, 48), (16, 112, 112, 64, 64), (1, 300, 301, 128, 128)]
+    for nb, h, w_, ci, co in shapes:
+        x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, 1, 1, ci), dtype=np.int8)
+        out_shape = [nb, h, w_, co]
+        acc = x.reshape(-1, ci).astype(np.int32) @ wt.reshape(co, ci).astype(np.int32).T
+        sx, sw = make_scales(rng, co)
+        so = pick_so(acc, sx, sw)
+        scales = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])))
+        tag = "%dx%dx%dx%d -> %d" % (nb, h, w_, ci, co)
+        for v in (sv,):
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, variant=v, **scales))
+            np.testing.assert_array_equal(got, O.requant_cpu(acc, sx, sw, so).reshape(out_shape), err_msg=tag)
+            bf = (rng.standard_normal(co) * 40 * so).astype(np.float32)
+            b32 = O.bias_f32_to_s32(bf, sx, sw)
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, bias=dev(bf), zo=3,
+                                 variant=v, **scales))
+            np.testing.assert_array_equal(got, O.requant_cpu(acc, sx, sw, so, b32=b32, zo=3).reshape(out_shape),
+                                          err_msg=tag + " f32 bias")
+            bi = rng.integers(-2000000, 2000000, co).astype(np.int32)
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, bias=dev(bi), zo=-5,
+                                 variant=v, **scales))
+            np.testing.assert_array_equal(got, O.requant_cpu(acc, sx, sw, so, b32=bi, zo=-5).reshape(out_shape),
+                                          err_msg=tag + " s32 bias")
+            bo = (rng.standard_normal(co) * 30).astype(np.float32)
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(bo),
+                                 variant=v, **scales))
+            np.testing.assert_array_equal(got, O.requant_gpu(acc, sx, sw, so, bias_f32=bo).reshape(out_shape),
+                                          err_msg=tag + " E2 f32 bias")
+            b8 = rng.integers(-128, 128, co, dtype=np.int8)
+            got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(b8),
+                                 variant=v, **scales))
+            np.testing.assert_array_equal(got, O.requant_gpu(acc, sx, sw, so, bias_i8=b8).reshape(out_shape),
+                                          err_msg=tag + " E2 s8 bias")
+            auto = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(b8), **scales))
+            np.testing.assert_array_equal(auto, got, err_msg=tag + " heuristic")
+    # fused operators: residual (+ ReLU) + quantize and a table, against the separate calls
+    for nb, h, w_, ci, co in [(32, 28, 28, 64, 256), (2, 28, 28, 128, 512), (1, 9, 11, 64, 80), (40, 56, 56, 128, 128)]:
+        x = dev(rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8))
+        wt = dev(rng.integers(-128, 128, (co, 1, 1, ci), dtype=np.int8))
+        out_shape = [nb, h, w_, co]
+        sc = dict(sx=dev(np.array([0.02], np.float32)), sw=dev(rng.uniform(0.001, 0.05, co).astype(np.float32)),
+                  so=dev(np.array([4.0], np.float32)))
+        z1 = torch.zeros(1, dtype=torch.int32, device="cuda")
+        res = dev(rng.standard_normal(out_shape).astype(np.float32) * 300)
+        s2 = dev(np.array([7.0], np.float32))
+        plain = K.qconv2d(x, wt, pad, md, out_shape, K.EPI_REQUANT_CPU, variant=sv, **sc)
+        for relu in (False, True):
+            fused = K.qconv2d(x, wt, pad, md, out_shape, K.EPI_REQUANT_CPU, **sc,
+                              post=K.make_postops(residual=res, relu=relu, out_scale=s2, out_zp=-3))
+            t = K.dequantize(plain, sc["so"], z1) + res
+            if relu:
+                t = torch.clamp_min(t, 0.0)
+            want = K.quantize(t, s2, torch.full((1,), -3, dtype=torch.int32, device="cuda"))
+            assert torch.equal(fused, want), (nb, h, w_, ci, co, relu)
+        table = K.activation_table(torch.nn.functional.gelu, sc["so"], z1, s2, z1)
+        fused = K.qconv2d(x, wt, pad, md, out_shape, K.EPI_REQUANT_CPU, **sc,
+                          post=K.make_postops(table=table))
+        assert torch.equal(fused, K.lut8(plain, table)), (nb, h, w_, ci, co)
+    # refusals: channel counts without an instance, strides, 4-byte results
+    one = dev(np.array([0.01], np.float32))
+    for ci, v in ((32, sv), (256, sv)):
+        x = dev(rng.integers(-128, 128, (1, 8, 8, ci), dtype=np.int8))
+        wt = dev(rng.integers(-128, 128, (64, 1, 1, ci), dtype=np.int8))
+        with pytest.raises(RuntimeError, match="streaming variant"):
+            K.qconv2d(x, wt, pad, md, [1, 8, 8, 64], K.EPI_REQUANT_CPU, sx=one, sw=one, so=one, variant=v)
+    x = dev(rng.integers(-128, 128, (1, 8, 8, 64), dtype=np.int8))
+    wt = dev(rng.integers(-128, 128, (64, 1, 1, 64), dtype=np.int8))
+    with pytest.raises(RuntimeError, match="streaming variant"):
+        K.qconv2d(x, wt, pad, md, [1, 8, 8, 64], K.EPI_ACC_S32, variant=sv)
+    md2 = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
+    with pytest.raises(RuntimeError, match="streaming variant"):
+        K.qconv2d(x, wt, pad, md2, [1, 4, 4, 64], K.EPI_REQUANT_CPU, sx=one, sw=one, so=one, variant=sv)
 
 
 def test_qconv_direct_other_filter_sizes(K):
