@@ -93,7 +93,7 @@ struct StreamInstance {
   int kh, kw, ci, ns, narrow;
 };
 constexpr StreamInstance kStreamInstances[] = {
-    {3, 3, 64, 64, 0}, {3, 3, 128, 32, 0}, {1, 1, 64, 128, 64}, {1, 1, 128, 128, 0},
+    {3, 3, 64, 64, 0}, {3, 3, 128, 32, 0}, {1, 1, 64, 128, 64}, {1, 1, 128, 128, 0}, {4, 4, 16, 64, 0},
 };
 int stream_conv_slice(int Kh, int Kw, int Ci, int Co) {
   for (const StreamInstance& s : kStreamInstances)
@@ -189,6 +189,7 @@ int launch_stream_epi(const DirectConvParams& p, hipStream_t st) {
   const int taps = p.Kh * p.Kw;
   if (taps == 9 && p.Ci == 64 && p.slice_n == 64) return launch_stream_post<3, 3, 64, 64, EPI>(p, st);
   if (taps == 9 && p.Ci == 128 && p.slice_n == 32) return launch_stream_post<3, 3, 128, 32, EPI>(p, st);
+  if (p.Kh == 4 && p.Kw == 4 && p.Ci == 16 && p.slice_n == 64) return launch_stream_post<4, 4, 16, 64, EPI>(p, st);
   if (taps == 1 && p.Ci == 64 && p.slice_n == 128) return launch_stream_post<1, 1, 64, 128, EPI>(p, st);
   if (taps == 1 && p.Ci == 64 && p.slice_n == 64) return launch_stream_post<1, 1, 64, 64, EPI>(p, st);
   if (taps == 1 && p.Ci == 128 && p.slice_n == 128) return launch_stream_post<1, 1, 128, 128, EPI>(p, st);

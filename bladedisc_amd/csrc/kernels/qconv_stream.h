@@ -1,7 +1,8 @@
 // int8 NHWC stride-1 convolution with the whole filter in registers ("streaming" form), for
 // filters of which a slice of NS output channels fits there: NS * Kh * Kw * Ci <= 36 KiB
 // (3 x 3 x 64 with 64-channel slices in the first place, 3 x 3 x 128 with 32-channel slices,
-// 1 x 1 x 64 and 1 x 1 x 128 with 128-channel slices).
+// 1 x 1 x 64 and 1 x 1 x 128 with 128-channel slices, 4 x 4 x 16 -- a 7 x 7 stride-2 stem after
+// space to depth -- with 64-channel slices).
 //
 // Where the time of such a layer goes in the LDS-tiled kernels (32 x 56 x 56 x 64 -> 64, 9 us):
 // every workgroup loads, then multiplies, then requantises and stores, all in the same phase, so
@@ -57,7 +58,8 @@ template <int KH, int KW, int CI, int NS, int EPI, bool POST>
 __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU, "int8 results only");
-  static_assert(CI == 32 || CI == 64 || CI == 128 || CI == 256 || CI == 512, "channels per pixel");
+  static_assert(CI == 16 || CI == 32 || CI == 64 || CI == 128 || CI == 256 || CI == 512, "channels per pixel");
+  static_assert(CI >= 32 || KW % 2 == 0, "16 channels: an MFMA step takes two taps next to each other");
   constexpr int NW = 8;
   constexpr int K = KH * KW * CI;
   constexpr int KS = K / 32;                 // MFMA steps per block
@@ -66,11 +68,11 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   constexpr int W_INSTR = (NS * ROWC + 63) / 64;           // 1 KiB load instructions for the slice
   constexpr int W_PER_WAVE = (W_INSTR + NW - 1) / NW;      // every wave issues this many
   constexpr int W_LDS = stream_conv_weight_lds(K, NS);
-  constexpr int LOG2_CI = CI == 32 ? 5 : CI == 64 ? 6 : CI == 128 ? 7 : CI == 256 ? 8 : 9;
+  constexpr int LOG2_CI = CI == 16 ? 4 : CI == 32 ? 5 : CI == 64 ? 6 : CI == 128 ? 7 : CI == 256 ? 8 : 9;
   constexpr int CP = CI / 16;                // 16-byte chunks per pixel
   // (swizzle of the chunks inside a 256-byte bank row, as in qconv_direct.h)
   constexpr int FSHIFT = LOG2_CI >= 8 ? 0 : 8 - LOG2_CI, FMASK = CP > 16 ? 15 : CP - 1;
-  constexpr int STEPS_PER_TAP = CI / 32;
+  constexpr int STEPS_PER_TAP = CI >= 32 ? CI / 32 : 1;
   constexpr int kOutOfRange = (int)0x80000000;
   static_assert(W_PER_WAVE * NW * 1024 <= W_LDS, "weight area");
   static_assert(NS % 32 == 0 && K % 32 == 0 && KS * NF * 4 <= 160, "the filter slice must fit the registers");
@@ -261,10 +263,14 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
     // byte offset of this lane's 16 bytes of k-half 0 at filter column kw, filter row 0; k-half
     // h is the same with bit 5 + ... flipped (xor 32 h), filter row kh adds kh row pitches
     int a0[KW];
+    if constexpr (CI == 16) {
+      a0[0] = (hq + c0) << 4;
+    } else {
 #pragma unroll
-    for (int kw = 0; kw < KW; ++kw) {
-      const int q = hq + kw;
-      a0[kw] = (q << LOG2_CI) + ((c0 ^ ((q >> FSHIFT) & FMASK)) << 4);
+      for (int kw = 0; kw < KW; ++kw) {
+        const int q = hq + kw;
+        a0[kw] = (q << LOG2_CI) + ((c0 ^ ((q >> FSHIFT) & FMASK)) << 4);
+      }
     }
 
     // pixel fragments, read PF steps ahead of their MFMAs
@@ -272,10 +278,17 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
     v4i fa[8];
     auto load_frag = [&](auto sc) {
       constexpr int s = decltype(sc)::value;
-      constexpr int tap = s / STEPS_PER_TAP;
-      constexpr int kh = tap / KW, kw = tap - KW * kh;
-      constexpr int h = s % STEPS_PER_TAP;
-      fa[s & 7] = *reinterpret_cast<const v4i*>(patch + (a0[kw] ^ (32 * h)) + kh * pitch_bytes);
+      if constexpr (CI == 16) {
+        // a pixel is one chunk (no swizzle): the step's 32 bytes of k are the taps 2 j and
+        // 2 j + 1 of a filter row, i.e. two neighbouring patch pixels, one per half-wave
+        constexpr int kh = s / (KW / 2), j = s - (KW / 2) * kh;
+        fa[s & 7] = *reinterpret_cast<const v4i*>(patch + a0[0] + 32 * j + kh * pitch_bytes);
+      } else {
+        constexpr int tap = s / STEPS_PER_TAP;
+        constexpr int kh = tap / KW, kw = tap - KW * kh;
+        constexpr int h = s % STEPS_PER_TAP;
+        fa[s & 7] = *reinterpret_cast<const v4i*>(patch + (a0[kw] ^ (32 * h)) + kh * pitch_bytes);
+      }
     };
     static_for<PF>([&](auto sc) {
       constexpr int s = decltype(sc)::value;

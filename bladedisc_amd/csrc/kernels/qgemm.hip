@@ -160,38 +160,72 @@ int transpose_batched(const void* src, void* dst, int64_t B, int64_t R, int64_t 
 // K x K stride-2 convolution of src is then a ceil(K / 2)^2 stride-1 convolution of dst.  With
 // H = Kh, W = Kw, no padding and B = Co the same kernel re-lays out the weights.  One 16-byte
 // store per thread.
+// One launch does two such jobs (image and weights): blockIdx.y < a.B belongs to the first.
+struct SpaceToDepthJob {
+  const int8_t* src;
+  int8_t* dst;
+  int B, H, W, Hb, Wb, pad_t, pad_l;
+};
+template <int C>
 __global__ void __launch_bounds__(256)
-space_to_depth2_s8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, int64_t B,
-                          int H, int W, int C, int Hb, int Wb, int pad_t, int pad_l) {
-  const int64_t total = B * Hb * Wb;
-  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total;
-       idx += (int64_t)gridDim.x * 256) {
-    const int bx = (int)(idx % Wb);
-    const int by = (int)((idx / Wb) % Hb);
-    const int64_t b = idx / ((int64_t)Wb * Hb);
-    uint32_t w[4] = {0, 0, 0, 0};
+space_to_depth2_s8_kernel(const SpaceToDepthJob ja, const SpaceToDepthJob jb) {
+  // blockIdx.y: image; threads over its Hb * Wb output pixels
+  const bool first = (int)blockIdx.y < ja.B;
+  const SpaceToDepthJob& j = first ? ja : jb;
+  const int8_t* __restrict__ src = j.src;
+  int8_t* __restrict__ dst = j.dst;
+  const int H = j.H, W = j.W, Hb = j.Hb, Wb = j.Wb, pad_t = j.pad_t, pad_l = j.pad_l;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= Hb * Wb) return;
+  const int by = idx / Wb, bx = idx - by * Wb;
+  const int64_t b = first ? (int)blockIdx.y : (int)blockIdx.y - ja.B;
+  // the two pixels of an image row that go into one output pixel are 2 C consecutive bytes
+  // there and here: one (unaligned) load where both are inside the image, bytes otherwise
+  uint64_t lo = 0, hi = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int iy = 2 * by + (q >> 1) - pad_t, ix = 2 * bx + (q & 1) - pad_l;
-      if ((unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W) {
-        const int8_t* px = src + ((b * H + iy) * W + ix) * C;
-        for (int c = 0; c < C; ++c) {
-          const int e = q * C + c;
-          w[e >> 2] |= (uint32_t)(uint8_t)px[c] << (8 * (e & 3));
+  for (int r = 0; r < 2; ++r) {
+    const int iy = 2 * by + r - pad_t, ix = 2 * bx - pad_l;
+    if ((unsigned)iy >= (unsigned)H) continue;
+    const int8_t* px = src + ((b * H + iy) * W + ix) * C;
+    uint64_t v = 0;
+    if (ix >= 0 && ix + 1 < W) {
+      __builtin_memcpy(&v, px, 2 * C);
+    } else {
+#pragma unroll
+      for (int dx = 0; dx < 2; ++dx)
+        if ((unsigned)(ix + dx) < (unsigned)W) {
+#pragma unroll
+          for (int c = 0; c < C; ++c) v |= (uint64_t)(uint8_t)px[dx * C + c] << (8 * (dx * C + c));
         }
-      }
     }
-    *reinterpret_cast<v4i*>(dst + idx * 16) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    constexpr int kBytes = 2 * C;                 // row r lands at bytes [r kBytes, r kBytes + kBytes)
+    if (r == 0) {
+      lo = v;
+    } else if constexpr (kBytes == 8) {
+      hi = v;
+    } else {
+      lo |= v << (8 * kBytes);
+      hi = v >> (64 - 8 * kBytes);
+    }
   }
+  *reinterpret_cast<v4i*>(dst + ((int64_t)b * Hb * Wb + idx) * 16) =
+      (v4i){(int)(uint32_t)lo, (int)(uint32_t)(lo >> 32), (int)(uint32_t)hi, (int)(uint32_t)(hi >> 32)};
 }
 
-int space_to_depth2_s8(const int8_t* src, int8_t* dst, int64_t B, int64_t H, int64_t W,
-                       int64_t C, int64_t Hb, int64_t Wb, int pad_t, int pad_l, hipStream_t st) {
-  const int64_t total = B * Hb * Wb;
-  if (total == 0) return 0;
-  const int64_t blocks = std::min<int64_t>(ceil_div(total, 256), 1 << 20);
-  hipLaunchKernelGGL(space_to_depth2_s8_kernel, dim3((unsigned)blocks), dim3(256), 0, st, src,
-                     dst, B, (int)H, (int)W, (int)C, (int)Hb, (int)Wb, pad_t, pad_l);
+// Both jobs in one launch (jb.B may be 0); C channels in both.
+int space_to_depth2_s8(const SpaceToDepthJob& ja, const SpaceToDepthJob& jb, int C, hipStream_t st) {
+  const int64_t px = std::max<int64_t>((int64_t)ja.Hb * ja.Wb, (int64_t)jb.Hb * jb.Wb);
+  if (px == 0 || ja.B + jb.B == 0) return 0;
+  DQ8_REQUIRE(px < (1LL << 31) - 256 && (int64_t)ja.B + jb.B <= 65535 && C >= 1 && C <= 4,
+              "space to depth: at most 65535 images of fewer than 2^31 pixels, 1 to 4 channels");
+  const dim3 grid((unsigned)ceil_div(px, 256), (unsigned)(ja.B + jb.B));
+  auto launch = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(256), 0, st, ja, jb); };
+  switch (C) {
+    case 1: launch(space_to_depth2_s8_kernel<1>); break;
+    case 2: launch(space_to_depth2_s8_kernel<2>); break;
+    case 3: launch(space_to_depth2_s8_kernel<3>); break;
+    default: launch(space_to_depth2_s8_kernel<4>); break;
+  }
   return check_hip(hipGetLastError(), "space-to-depth launch");
 }
 
@@ -357,10 +391,14 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
     const int64_t cus = compute_units();
     // (256 x 64 tiles for a narrow N once they occupy three quarters of the compute units)
     if (N <= 64 && 4 * tiles(kPipe256x64) >= 3 * cus) return kPipe256x64;
+    // A wide tile is a candidate while at least 0.7 of the columns of its tiles are columns of
+    // the problem (M = 100352, 256 -> 128: 256 x 192 tiles 14.6 us, 128 x 128 12.9; M = 25088,
+    // 512 -> 256: 10.9 against 8.9).
+    auto columns_used = [&](int v) { return 10 * N >= 7 * ceil_div(N, kVariants[v].bn) * kVariants[v].bn; };
     const int64_t t256 = tiles(kPipe256w8);
     const int64_t rounds = ceil_div(t256, cus);
     const bool big256 = t256 >= 140 && (rounds == 1 || 10 * t256 >= 7 * cus * rounds) &&
-                        (out_bytes == 1 || K >= 2048);
+                        (out_bytes == 1 || K >= 2048) && columns_used(kPipe256w8);
     if (out_bytes == 1) {
       // estimated time in us of a launch of `t` tiles whose k tile costs `per_k` us with all
       // compute units busy and whose fixed parts cost `fixed` us
@@ -376,7 +414,7 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
       bool p256 = false, p192 = false;
       const double e256 = big256 ? estimate(t256, 1.6, 5.4, &p256) : 1e30;
       // (from 180 tiles: M = 1152, 2048 -> 7424, 195 tiles: 24.3 against 27.2 us on 145 of 256 x 256)
-      const double e192 = t192 >= 180 ? estimate(t192, 1.27, 4.7, &p192) : 1e30;
+      const double e192 = t192 >= 180 && columns_used(kPipe256x192) ? estimate(t192, 1.27, 4.7, &p192) : 1e30;
       if (e192 < e256) return p192 ? kPersist256x192 : kPipe256x192;
       if (big256) return p256 ? kPersist256 : kPipe256w8;
     } else if (big256) {
@@ -397,7 +435,7 @@ int pick_variant(int64_t M, int64_t N, int64_t K, bool pipe, int out_bytes = 1) 
         return (double)ceil_div(t, cus) * (kt * per_k * (1.0 + 0.65 * busy * std::sqrt(busy)) / 1.65 + fixed);
       };
       const int64_t t192 = tiles(kPipe256x192);
-      if (t256 <= cus && t192 <= cus)
+      if (t256 <= cus && t192 <= cus && columns_used(kPipe256x192) && columns_used(kPipe256w8))
         return one_round(t192, 1.27, 4.7) < one_round(t256, 1.6, 5.4) ? kPipe256x192 : kPipe256w8;
     }
     // (int32 / f32 results, four times the bytes to store: eight waves throughout, and the
@@ -1075,7 +1113,8 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   // 62-65 us that way).
   if (variant == -1 && is_nhwc_ohwi(md) && Ci >= 1 && Ci <= 4 && sh == 2 && sw_ == 2 &&
       dh == 1 && dw == 1 && workspace != nullptr && aligned(workspace, 256) && Ho > 0 && Wo > 0 &&
-      NB > 0 && Co > 0 && in && w && out && H < (1 << 30) && Wd < (1 << 30)) {
+      NB > 0 && Co > 0 && NB + Co <= 65535 && Kh < (1 << 15) && Kw < (1 << 15) && in && w && out &&
+      H < (1 << 15) && Wd < (1 << 15)) {
     const int64_t kbh = (Kh + 1) / 2, kbw = (Kw + 1) / 2;
     const int64_t Hb = Ho + kbh - 1, Wb = Wo + kbw - 1;
     const size_t in_b = pad256(NB * Hb * Wb * 16), w_b = pad256(Co * kbh * kbw * 16);
@@ -1083,9 +1122,9 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
       hipStream_t st0 = (hipStream_t)stream;
       int8_t* in_t = static_cast<int8_t*>(workspace);
       int8_t* w_t = in_t + in_b;
-      if (int s = space_to_depth2_s8(in, in_t, NB, H, Wd, Ci, Hb, Wb, padding[0], padding[2], st0))
-        return s;
-      if (int s = space_to_depth2_s8(w, w_t, Co, Kh, Kw, Ci, kbh, kbw, 0, 0, st0)) return s;
+      const SpaceToDepthJob job_in = {in, in_t, (int)NB, (int)H, (int)Wd, (int)Hb, (int)Wb, padding[0], padding[2]};
+      const SpaceToDepthJob job_w = {w, w_t, (int)Co, (int)Kh, (int)Kw, (int)kbh, (int)kbw, 0, 0};
+      if (int s = space_to_depth2_s8(job_in, job_w, (int)Ci, st0)) return s;
       const int64_t in2[4] = {NB, Hb, Wb, 16}, w2[4] = {Co, kbh, kbw, 16};
       const int32_t pad2[4] = {0, 0, 0, 0};
       int32_t md2[17];
@@ -1304,12 +1343,13 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     return launch_direct_conv(config, epilogue, d, st);
   }
   // 3 x 3 filters on 64 or 128 channels with int8 results: the filter in registers
-  const bool stream_shape = direct_shape && Kh == 3 && Kw == 3 && (Ci == 64 || Ci == 128) && stream_out;
+  const bool stream_shape = direct_shape && Ci <= 128 && stream_conv_has_instance((int)d.Kh, (int)d.Kw, (int)Ci) &&
+                            stream_out;
   if (variant == kStreamConv) {
     DQ8_REQUIRE(stream_shape && stream_conv_plan(&d),
                 "dq8_qconv2d: the streaming variant needs a 3 x 3 or 1 x 1 filter on 64 or "
-                "128 input channels, stride and dilation 1, an int8 result (float output "
-                "stage) and 16-byte aligned output rows");
+                "128 input channels (or 4 x 4 on 16), stride and dilation 1, an int8 result "
+                "(float output stage) and 16-byte aligned output rows");
     return launch_stream_conv(epilogue, d, st);
   }
   if (auto_pick) {
@@ -1321,7 +1361,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     if (stream_shape) {
       DirectConvParams sp = d;
       if (stream_conv_plan(&sp) &&
-          (Ci == 64 || (int64_t)sp.NB * sp.tiles_per_image * sp.tiles_n <= compute_units()))
+          (Ci <= 64 || (int64_t)sp.NB * sp.tiles_per_image * sp.tiles_n <= compute_units()))
         return launch_stream_conv(epilogue, sp, st);
     }
     if (direct_shape) {

@@ -959,6 +959,55 @@ def test_qconv_stream_variant(K):
         K.qconv2d(x, wt, [1, 1, 1, 1], md2, [1, 4, 4, 64], K.EPI_REQUANT_CPU, sx=one, sw=one, so=one, variant=sv)
 
 
+def test_qconv_stream_16_channels(K):
+    """4 x 4 filters on 16 channels (what a 7 x 7 stride-2 stem becomes after space to depth) in
+    the kernel that keeps the filter in registers: an MFMA step's 32 bytes of k are two
+    neighbouring patch pixels.  Bit-exact against the oracle, forced and as the library's choice,
+    and the stem itself (3 channels, stride 2) through the library against the oracle."""
+    rng = np.random.default_rng(20260413)
+    sv = K.variant_names().index("stream")
+    md = list(O.NHWC_OHWI_METADATA) + [1, 1, 1, 1, 1]
+    for nb, h, w_, co, pad in [(2, 115, 115, 64, [0, 0, 0, 0]), (1, 9, 12, 80, [1, 2, 0, 3]),
+                               (3, 30, 31, 16, [0, 0, 0, 0]), (1, 131, 67, 96, [3, 0, 1, 1]),
+                               (9, 20, 20, 64, [0, 0, 0, 0])]:
+        ho, wo = h + pad[0] + pad[1] - 3, w_ + pad[2] + pad[3] - 3
+        x = rng.integers(-128, 128, (nb, h, w_, 16), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, 4, 4, 16), dtype=np.int8)
+        out_shape = [nb, ho, wo, co]
+        acc = O.conv_s32(x, wt, pad, md, out_shape)
+        sx, sw = make_scales(rng, co)
+        so = pick_so(acc, sx, sw)
+        scales = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])))
+        tag = "%dx%dx%dx16 -> %d pad %s" % (nb, h, w_, co, pad)
+        a2 = acc.reshape(-1, co)
+        bi = rng.integers(-200000, 200000, co).astype(np.int32)
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, bias=dev(bi), zo=-5,
+                             variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_cpu(a2, sx, sw, so, b32=bi, zo=-5).reshape(out_shape),
+                                      err_msg=tag + " s32 bias")
+        bo = (rng.standard_normal(co) * 30).astype(np.float32)
+        got = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(bo),
+                             variant=sv, **scales))
+        np.testing.assert_array_equal(got, O.requant_gpu(a2, sx, sw, so, bias_f32=bo).reshape(out_shape),
+                                      err_msg=tag + " E2 f32 bias")
+        auto = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(bo), **scales))
+        np.testing.assert_array_equal(auto, got, err_msg=tag + " heuristic")
+    # the stem: 7 x 7, stride 2, padding 3, three channels
+    md2 = list(O.NHWC_OHWI_METADATA) + [2, 2, 1, 1, 1]
+    for nb, h in [(2, 224), (1, 97)]:
+        ho = (h + 6 - 7) // 2 + 1
+        x = rng.integers(-128, 128, (nb, h, h, 3), dtype=np.int8)
+        wt = rng.integers(-128, 128, (64, 7, 7, 3), dtype=np.int8)
+        out_shape = [nb, ho, ho, 64]
+        acc = O.conv_s32(x, wt, [3, 3, 3, 3], md2, out_shape)
+        sx, sw = make_scales(rng, 64)
+        so = pick_so(acc, sx, sw)
+        got = host(K.qconv2d(dev(x), dev(wt), [3, 3, 3, 3], md2, out_shape, K.EPI_REQUANT_CPU,
+                             sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so]))))
+        np.testing.assert_array_equal(got, O.requant_cpu(acc.reshape(-1, 64), sx, sw, so).reshape(out_shape),
+                                      err_msg="stem %d x %d" % (nb, h))
+
+
 def test_qconv_stream_pointwise(K):
     """1 x 1 filters on 64 and 128 input channels in the kernel that keeps the filter in registers
     (a GEMM over the pixels with a short k): pixel counts that are and are not a multiple of 16
