@@ -61,7 +61,8 @@ def parse():
     p.add_argument("--workload", default="headline",
                    help="'headline' (default), or one parity-test configuration on its own, "
                         "e.g. for a profiler: 'gemm:MxKxN' (dynamic-M sweep shape, requant to "
-                        "int8), 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS), "
+                        "int8), 'conv:NAME' (NAME from baseline_configs.RESNET_CONVS), 'layer:NAME' (a layer of "
+                        "the ResNet-50 sweep, HxHxCI_KxKxCO_sS), "
                         "'wo:MxKxN' (weight-only linear, f16 x uint8) or 'qlinear:MxKxN' "
                         "(quantize -> qgemm -> dequantize of f32 activations in one launch)")
     p.add_argument("--operands", choices=("config", "uniform", "ones", "zeros"), default="config",
@@ -384,6 +385,32 @@ def config_reports(torch, K):
         convs[conv["name"]] = r
         del cols
     rep["4_resnet_convs_requant"] = convs
+
+    # ---- 4b: every distinct convolution of ResNet-50 at batch 32 (GPU only; operands drawn as
+    # in config 4: activations max(N(0, 1), 0), weights N(0, 1) per output channel, both
+    # quantized symmetrically to their maximum.  Uniform random bytes, which toggle far more
+    # bits, run up to a third slower under sustained load: the clocks drop)
+    sweep = {}
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4)
+    for h, ci, co, k, stride, pad in cfg.RESNET50_LAYERS:
+        ho = (h + 2 * pad - k) // stride + 1
+        xf = torch.randn((32, h, h, ci), device="cuda", generator=gen).clamp_min_(0)
+        xq = torch.round(xf * (127.0 / xf.max())).to(torch.int8)
+        wf = torch.randn((co, k, k, ci), device="cuda", generator=gen)
+        wq = torch.round(wf * (127.0 / wf.abs().amax(dim=(1, 2, 3), keepdim=True))).to(torch.int8)
+        del xf, wf
+        md = list(O.NHWC_OHWI_METADATA) + [stride, stride, 1, 1, 1]
+        osh = [32, ho, ho, co]
+        sx, so = f1(0.02), f1(20.0)
+        sw = torch.rand(co, device="cuda", generator=gen) * 0.049 + 0.001
+        o = torch.empty(tuple(osh), dtype=torch.int8, device="cuda")
+        gpu_s = time_graph(torch, [FnCall(lambda: K.qconv2d(xq, wq, [pad] * 4, md, osh, K.EPI_REQUANT_CPU,
+                                                            sx=sx, sw=sw, so=so, out=o))])
+        sweep["%dx%dx%d_%dx%dx%d_s%d" % (h, h, ci, k, k, co, stride)] = roof(
+            2.0 * 32 * ho * ho * co * k * k * ci, xq.numel() + wq.numel() + o.numel() + 4 * co, gpu_s)
+        del xq, wq, o
+    rep["4b_resnet50_layers_batch32_requant"] = sweep
 
     # ---- 5: quantized BERT-base encoder layer, batch 8
     from bladedisc_amd import bert_layer as B
@@ -725,6 +752,30 @@ def single_workload(torch, args):
         mg, kg = nb * osh[1] * osh[2], kk * kk * ci
         ops, byts = 2.0 * mg * co * kg, nb * h * w_ * ci + co * kg + mg * co + 4 * co
         name = "int8 NHWC conv %s, batch %d, requant to int8 (E1)" % (what, nb)
+    elif kind == "layer":
+        # one layer of the ResNet-50 sweep, named as in the report: HxHxCI_KxKxCO_sS
+        names = {"%dx%dx%d_%dx%dx%d_s%d" % (h, h, ci, kk, kk, co, s_): (h, ci, co, kk, s_, pd)
+                 for h, ci, co, kk, s_, pd in cfg.RESNET50_LAYERS}
+        if what not in names:
+            raise SystemExit("bench.py: --workload layer:NAME, NAME one of %s" % ", ".join(names))
+        h, ci, co, kk, stride, pd = names[what]
+        ho = (h + 2 * pd - kk) // stride + 1
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(4)
+        xf = torch.randn((32, h, h, ci), device="cuda", generator=gen).clamp_min_(0)
+        xq = torch.round(xf * (127.0 / xf.max())).to(torch.int8)
+        wf = torch.randn((co, kk, kk, ci), device="cuda", generator=gen)
+        wq = torch.round(wf * (127.0 / wf.abs().amax(dim=(1, 2, 3), keepdim=True))).to(torch.int8)
+        md = list(O.NHWC_OHWI_METADATA) + [stride, stride, 1, 1, 1]
+        osh = [32, ho, ho, co]
+        sx, so = f1(0.02), f1(20.0)
+        sw = torch.rand(co, device="cuda", generator=gen) * 0.049 + 0.001
+        o = torch.empty(tuple(osh), dtype=torch.int8, device="cuda")
+        call = lambda: K.qconv2d(xq, wq, [pd] * 4, md, osh, K.EPI_REQUANT_CPU, sx=sx, sw=sw,  # noqa: E731
+                                 so=so, out=o)
+        ops = 2.0 * 32 * ho * ho * co * kk * kk * ci
+        byts = xq.numel() + wq.numel() + o.numel() + 4 * co
+        name = "int8 NHWC conv %s (ResNet-50 sweep), batch 32, requant to int8 (E1)" % what
     elif kind == "wo":
         # weight-only quantized linear: f16 activations x uint8 weights [N,K]
         m, k, n = (int(v) for v in what.split("x"))

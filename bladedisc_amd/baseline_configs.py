@@ -15,6 +15,18 @@ RESNET_CONVS = (                                                # NHWC x OHWI
     dict(name="28x28x128_3x3x128", nb=32, h=28, w=28, ci=128, co=128, k=3, stride=1, pad=1),
     dict(name="14x14x256_1x1x1024", nb=32, h=14, w=14, ci=256, co=1024, k=1, stride=1, pad=0),
 )
+# Every distinct convolution of ResNet-50 (h = w: input size; batch 32 in the sweep): the layers
+# around the three above, timed on the GPU only.  (h, ci, co, k, stride, pad)
+RESNET50_LAYERS = (
+    (224, 3, 64, 7, 2, 3),
+    (56, 64, 64, 1, 1, 0), (56, 64, 64, 3, 1, 1), (56, 64, 256, 1, 1, 0), (56, 256, 64, 1, 1, 0),
+    (56, 256, 128, 1, 1, 0), (56, 128, 128, 3, 2, 1), (56, 256, 512, 1, 2, 0),
+    (28, 128, 512, 1, 1, 0), (28, 512, 128, 1, 1, 0), (28, 128, 128, 3, 1, 1),
+    (28, 512, 256, 1, 1, 0), (28, 256, 256, 3, 2, 1), (28, 512, 1024, 1, 2, 0),
+    (14, 256, 1024, 1, 1, 0), (14, 1024, 256, 1, 1, 0), (14, 256, 256, 3, 1, 1),
+    (14, 1024, 512, 1, 1, 0), (14, 512, 512, 3, 2, 1), (14, 1024, 2048, 1, 2, 0),
+    (7, 512, 2048, 1, 1, 0), (7, 2048, 512, 1, 1, 0), (7, 512, 512, 3, 1, 1),
+)
 BERT_SEQ_LENS = (32, 128, 384)
 
 

@@ -50,7 +50,9 @@ namespace dq8 {
 constexpr int stream_conv_weight_lds(int K, int NS) {
   return ((NS * (K / 16 + 1) + 511) / 512) * 512 * 16;
 }
-constexpr int stream_conv_cp_bytes(int NS) { return NS * 8 + 256; }   // pairs + a fused table
+// (the per-channel factors, a fused table, and -- from 64 channels a slice on -- a 32 x NS result
+// tile per wave)
+constexpr int stream_conv_cp_bytes(int NS) { return NS * 8 + 256 + (NS >= 64 ? 8 * 32 * NS : 0); }
 
 // POST: the launch has operators fused behind the convolution (their code and registers are kept
 // out of the plain form).
@@ -74,6 +76,20 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   constexpr int FSHIFT = LOG2_CI >= 8 ? 0 : 8 - LOG2_CI, FMASK = CP > 16 ? 15 : CP - 1;
   constexpr int STEPS_PER_TAP = CI >= 32 ? CI / 32 : 1;
   constexpr int kOutOfRange = (int)0x80000000;
+  // The factors of a lane's channels (16 per 32-channel fragment) stay in registers over all
+  // blocks where the filter slice leaves room for them; otherwise they are read from LDS per
+  // fragment, all reads of a fragment ahead of its arithmetic (read one by one as they are
+  // needed, each exposes the LDS latency under the other waves' fragment reads: 1750 cycles per
+  // 32 x 64 block instead of 700).
+  // Results leave through a wave-private LDS tile where a slice row is 64 bytes or more: of a
+  // fragment a lane pair holds 32 bytes of a pixel's row; read back in row order, a store
+  // instruction covers whole 64- or 128-byte pieces, which can be written through the L2 (see
+  // st_through: an ordinary store's dirty lines are written back after the kernel's last wave,
+  // 25 MB of results in about 2.5 us; 32-byte pieces written through are slower than that).
+  constexpr bool STAGE = NS >= 64;
+  constexpr int LPR = NS / 16;                // lanes (16-byte chunks) per row of the tile
+  constexpr bool HOIST_OS = KS * NF * 4 + NF * 16 + NF * 16 + 60 <= 240;
+  constexpr bool HOIST_B = KS * NF * 4 + NF * 16 + NF * 32 + 60 <= 240;
   static_assert(W_PER_WAVE * NW * 1024 <= W_LDS, "weight area");
   static_assert(NS % 32 == 0 && K % 32 == 0 && KS * NF * 4 <= 160, "the filter slice must fit the registers");
 
@@ -82,7 +98,10 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   DQ8_TRACE_WAVE(0);
   int8_t* patch = smem;
   int8_t* wlds = smem + p.patch_bytes;
-  float2* cp = reinterpret_cast<float2*>(smem + p.patch_bytes + W_LDS);
+  // per-channel factors: the scales, then the addends (a launch without bias and zero point
+  // reads only the first)
+  float* cp_os = reinterpret_cast<float*>(smem + p.patch_bytes + W_LDS);
+  float* cp_b = cp_os + NS;
   uint8_t* tab = reinterpret_cast<uint8_t*>(smem + p.patch_bytes + W_LDS + NS * 8);
 
   const int tid = threadIdx.x;
@@ -228,7 +247,8 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   if constexpr (!POINT) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
   if (tid < NS) {
     const ColParams c = col_finish<EPI>(e, raw);
-    cp[tid] = make_float2(c.os, c.b);
+    cp_os[tid] = c.os;
+    cp_b[tid] = c.b;
   }
   if (POST && e.table && tid >= 64 && tid < 128) reinterpret_cast<uint32_t*>(tab)[tid - 64] = tab_word;
   int later = 0;                     // (1 x 1) load instructions of this wave's blocks after the current one
@@ -246,6 +266,25 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   int8_t* out = static_cast<int8_t*>(e.out);
   const int c0 = lane >> 5;
   const int pitch_bytes = PWp << LOG2_CI;
+  int8_t* stg = reinterpret_cast<int8_t*>(tab) + 256 + wave * (32 * NS);
+  // lane's channels of fragment j: j * 32 + 4 * c0 + 8 * g + 0 .. 3, g = 0 .. 3
+  v4f hos[HOIST_OS ? NF : 1][4], hb[HOIST_B ? NF : 1][4];
+  if constexpr (HOIST_OS) {
+    static_for<NF>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) hos[j][g] = *reinterpret_cast<const v4f*>(&cp_os[j * 32 + 4 * c0 + 8 * g]);
+    });
+  }
+  if constexpr (HOIST_B) {
+    if (!plain) {
+      static_for<NF>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) hb[j][g] = *reinterpret_cast<const v4f*>(&cp_b[j * 32 + 4 * c0 + 8 * g]);
+      });
+    }
+  }
 
   for (int b = wave; b < nblocks; b += NW) {
     // this lane's pixel: position in the patch at tap (0, 0)
@@ -322,13 +361,27 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
       static_for<NF>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         const int cl0 = j * 32 + 4 * c0;
+        v4f os4[4], b4[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          if constexpr (HOIST_OS)
+            os4[g] = hos[j][g];
+          else
+            os4[g] = *reinterpret_cast<const v4f*>(&cp_os[cl0 + 8 * g]);
+          if constexpr (PLAIN)
+            b4[g] = (v4f){0.f, 0.f, 0.f, 0.f};
+          else if constexpr (HOIST_B)
+            b4[g] = hb[j][g];
+          else
+            b4[g] = *reinterpret_cast<const v4f*>(&cp_b[cl0 + 8 * g]);
+        }
+        // (the instantiations with fused operators have no registers to spare for that)
+        if constexpr (!POST && (!HOIST_OS || (!PLAIN && !HOIST_B))) __builtin_amdgcn_sched_barrier(0);
         uint32_t w[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const v4f p01 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g]);
-          const v4f p23 = *reinterpret_cast<const v4f*>(&cp[cl0 + 8 * g + 2]);
-          const ColParams c[4] = {{p01[0], p01[1], 0}, {p01[2], p01[3], 0},
-                                  {p23[0], p23[1], 0}, {p23[2], p23[3], 0}};
+          const ColParams c[4] = {{os4[g][0], b4[g][0], 0}, {os4[g][1], b4[g][1], 0},
+                                  {os4[g][2], b4[g][2], 0}, {os4[g][3], b4[g][3], 0}};
           w[g] = requant_pack4<EPI, PLAIN>(e, c, acc[j][4 * g + 0], acc[j][4 * g + 1],
                                            acc[j][4 * g + 2], acc[j][4 * g + 3]);
         }
@@ -338,7 +391,13 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
         const int n = n0 + j * 32 + 16 * c0;
         // (operators fused behind the convolution: a table, or + residual [, ReLU] and quantize)
         if (POST && (e.table || e.resid_kind)) fused_tail16(e, tab, m, n, px_raw < p_end, v);
-        if (px_raw < p_end && n < e.N) {
+        if constexpr (STAGE) {
+          // chunk c of tile row r in slot c ^ f(r), f such that the 16 lanes of a write phase
+          // (16 consecutive rows, the same chunk) cover all banks
+          const int r = lane & 31;
+          const int slot = (2 * j + c0) ^ (NS == 64 ? (r >> 2) & 3 : (r >> 1) & (LPR - 1));
+          *reinterpret_cast<v4i*>(stg + r * NS + slot * 16) = v;
+        } else if (px_raw < p_end && n < e.N) {
           int8_t* dst = out + m * e.ldo + n;
           if (n + 15 < e.N) {
             *reinterpret_cast<v4i*>(dst) = v;
@@ -354,6 +413,19 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
       finish(IntC<1>());
     else
       finish(IntC<0>());
+    if constexpr (STAGE) {
+      // (the wave's own writes, in order: no barrier)
+#pragma unroll
+      for (int i = 0; i < NF; ++i) {
+        const int u = i * 64 + lane;
+        const int r = u / LPR;
+        const int c = (u % LPR) ^ (NS == 64 ? (r >> 2) & 3 : (r >> 1) & (LPR - 1));
+        const v4i v = *reinterpret_cast<const v4i*>(stg + u * 16);
+        const int px2 = p0 + b * 32 + r;
+        if (px2 < p_end && n0 + c * 16 < e.N)
+          st_through(out + ((int64_t)img * hw + px2) * e.ldo + n0 + c * 16, v);
+      }
+    }
     DQ8_TRACE_WAVE(5 + 2 * ((b - wave) / NW));
   }
   DQ8_TRACE_POINT(3);

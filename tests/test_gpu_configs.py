@@ -142,6 +142,30 @@ def test_config4_resnet_convs(K, C, idx):
     assert np.array_equal(small.reshape(-1, co), acc[:ho * wo])
 
 
+def test_resnet50_layer_sweep(K, C):
+    """Every distinct convolution of ResNet-50 (the layers bench.py times next to config 4), at
+    batch 4 so that each goes to the kernel its full-size form goes to or a neighbour of it:
+    bit-exact against im2col + the oracle's int8 GEMM, with an s32 bias and an output zero
+    point."""
+    rng = np.random.default_rng(50)
+    for h, ci, co, k, stride, pad in C.RESNET50_LAYERS:
+        nb = 4
+        x = rng.integers(-128, 128, (nb, h, h, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8)
+        cols, ho, wo = _im2col(x, k, stride, pad)
+        acc, _ = O.gemm_s32_fast(cols, wt.reshape(co, -1))
+        sw = rng.uniform(0.001, 0.05, co).astype(np.float32)
+        sx = 0.02
+        so = float(np.abs(acc * (sx * sw)).max() / 200.0)
+        bi = rng.integers(-20000, 20000, co).astype(np.int32)
+        md = list(O.NHWC_OHWI_METADATA) + [stride, stride, 1, 1, 1]
+        out_shape = [nb, ho, wo, co]
+        y = K.qconv2d(dev(x), dev(wt), [pad] * 4, md, out_shape, K.EPI_REQUANT_CPU, sx=f1(sx), sw=dev(sw),
+                      so=f1(so), bias=dev(bi), zo=2)
+        ref = O.requant_cpu(acc, sx, sw, so, b32=bi, zo=2).reshape(out_shape)
+        assert np.array_equal(y.cpu().numpy(), ref), (h, ci, co, k, stride)
+
+
 @pytest.mark.parametrize("seq", [32, 128, 384])
 @pytest.mark.parametrize("backend", ["raw", "ral"])
 def test_config5_bert_layer(C, seq, backend):
