@@ -584,7 +584,7 @@ struct NoHook {
   __device__ __forceinline__ void operator()() const {}
 };
 
-template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores = NoHook>
+template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores = NoHook, bool BLOCK_STAGE = false>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
                                               int n_blk0, const ColParams* early = nullptr,
@@ -773,7 +773,17 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
 // that a lane holds 16 consecutive channels of its row, and stored from the registers;
 // int32 / f32 results are staged through LDS one fragment at a time so that they leave as
 // full 128-byte row segments.
-template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores>
+// BLOCK_STAGE (int8 results, every wave of the workgroup active, (NT / 64) wave tiles side by
+// side covering the BN columns): the waves put their packed results into one row-major tile of
+// the whole block in LDS, behind the factors, and after a barrier the workgroup stores it row
+// by row -- whole rows of BN bytes per group of BN / 16 lanes -- with stores that write through
+// the L2 (st_through: a wave's own 32-byte row pieces would be too small for those).  Measured,
+// us per launch before / after: M = 6272, 256 -> 1024 7.65 / 7.0; M = 100352, 256 -> 128 13.0 /
+// 11.7; M = 4096, 768 -> 3072 15.2 / 14.6; 4096^3 unchanged.  Not for the persistent kernels: a
+// workgroup that walks several tiles writes most of its results long before the kernel ends,
+// and there the extra barrier and LDS trip per tile cost more than the shorter tail saves
+// (M = 16384, 768 -> 3072: 50.0 -> 52.0 us).
+template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores, bool BLOCK_STAGE>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
                                               int n_blk0, const ColParams* early,
@@ -834,9 +844,24 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     // With a hook the results of the whole wave tile are formed first (32 registers per
     // 128 x 64), the hook runs, and the stores follow in one go; without one each fragment is
     // stored as soon as it is packed.
-    constexpr bool kHook = !__is_same(BeforeStores, NoHook);
+    constexpr bool kHook = !BLOCK_STAGE && !__is_same(BeforeStores, NoHook);
     v4i held[kHook ? FM : 1][kHook ? FN : 1];
+    // block tile in LDS: chunk c (16 bytes) of row r in slot c ^ f(r % 32), f such that the 16
+    // lanes of a write phase -- 16 consecutive rows, the same chunk -- cover all banks
+    constexpr int kWN = BN / (FN * 32), kWM = (NT / 64) / kWN, kBM = kWM * FM * 32;
+    constexpr int kChunks = BN / 16;
+    auto swz = [](int r) {
+      return BN % 256 == 0 ? (r & 15) : BN % 128 == 0 ? ((r >> 1) & 7) : ((r >> 2) & 3);
+    };
+    int8_t* tile = smem + CP_BYTES + BN * 4 + 256;
+    const int row_wave0 = (wave / kWN) * (FM * 32);
     auto store_frag = [&](const v4i v, int i, int j) {
+      if constexpr (BLOCK_STAGE) {
+        const int r = lane & 31;
+        const int c = ((wn_off + j * 32) >> 4) + (lane >> 5);
+        *reinterpret_cast<v4i*>(tile + (row_wave0 + i * 32 + r) * BN + ((c ^ swz(r)) << 4)) = v;
+        return;
+      }
       const int n = n_wave0 + j * 32 + 16 * (lane >> 5);
       const int m = m_wave0 + i * 32 + (lane & 31);
       if (m < m_end && n < e.N) {
@@ -919,6 +944,30 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
 #pragma unroll
         for (int i = 0; i < FM; ++i) store_frag(held[kHook ? i : 0][kHook ? j : 0], i, j);
     }
+    if constexpr (BLOCK_STAGE) {
+      static_assert(kWM * kWN * 64 == NT && (kBM * kChunks) % NT == 0, "block tile over the workgroup");
+      __syncthreads();
+      before_stores();
+      const int m_blk0 = m_wave0 - row_wave0;
+#pragma unroll
+      for (int k = 0; k < kBM * kChunks / NT; ++k) {
+        const int u = tid + k * NT;
+        const int row = u / kChunks;
+        const int c = (u % kChunks) ^ swz(row & 31);
+        const int m = m_blk0 + row, n = n_blk0 + c * 16;
+        if (m < m_end && n < e.N) {
+          const v4i v = *reinterpret_cast<const v4i*>(tile + u * 16);
+          int8_t* dst = out + (int64_t)m * e.ldo + n;
+          if (n + 15 < e.N) {
+            st_through(dst, v);
+          } else {
+#pragma unroll
+            for (int b = 0; b < 16; ++b)
+              if (n + b < e.N) dst[b] = (int8_t)((uint32_t)v[b >> 2] >> (8 * (b & 3)));
+          }
+        }
+      }
+    }
     DQ8_TRACE_POINT(6);
     return;
   }
@@ -985,7 +1034,7 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
               }
             }
             if (n + 3 < e.N) {
-              __builtin_nontemporal_store(v, reinterpret_cast<v4i*>(dst));
+              st_through(dst, v);
             } else {
 #pragma unroll
               for (int q = 0; q < 4; ++q)

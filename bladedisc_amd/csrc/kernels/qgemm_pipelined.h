@@ -392,8 +392,12 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
     }
   }
 
-  mfma_epilogue<EPI, FM, FN, NT, BN>(acc, p.epi, smem_all, m0 + wm * TM, n0 + wn * TN, n0,
-                                     early.c, wave, kg == 0);
+  // (one k group: the whole workgroup takes part in the epilogue, and its LDS holds the block's
+  // int8 tile behind the factors)
+  constexpr bool kBlockStage = KSPLIT == 1 && (EPI == DQ8_EPI_REQUANT_CPU || EPI == DQ8_EPI_REQUANT_GPU) &&
+                               BN * 12 + 512 + BM * BN <= 2 * STAGE;
+  mfma_epilogue<EPI, FM, FN, NT, BN, NoHook, kBlockStage>(acc, p.epi, smem_all, m0 + wm * TM, n0 + wn * TN, n0,
+                                                          early.c, wave, kg == 0);
   DQ8_TRACE_POINT(3);
 #else
   (void)p;
