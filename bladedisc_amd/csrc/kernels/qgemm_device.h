@@ -855,11 +855,20 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
     };
     int8_t* tile = smem + CP_BYTES + BN * 4 + 256;
     const int row_wave0 = (wave / kWN) * (FM * 32);
+    // With 64 channels to a wave tile a wave's own rows are whole 64-byte pieces: each wave
+    // stages and stores its own tile, and the workgroup needs no barrier for it.
+    constexpr bool kWavePrivate = FN == 2;
     auto store_frag = [&](const v4i v, int i, int j) {
       if constexpr (BLOCK_STAGE) {
         const int r = lane & 31;
-        const int c = ((wn_off + j * 32) >> 4) + (lane >> 5);
-        *reinterpret_cast<v4i*>(tile + (row_wave0 + i * 32 + r) * BN + ((c ^ swz(r)) << 4)) = v;
+        if constexpr (kWavePrivate) {
+          // (a wave tile of 64 channels: rows of 64 bytes in the wave's own part of the area)
+          *reinterpret_cast<v4i*>(tile + wave * (FM * 32 * 64) + (i * 32 + r) * 64 +
+                                  (((2 * j + (lane >> 5)) ^ ((r >> 2) & 3)) << 4)) = v;
+        } else {
+          const int c = ((wn_off + j * 32) >> 4) + (lane >> 5);
+          *reinterpret_cast<v4i*>(tile + (row_wave0 + i * 32 + r) * BN + ((c ^ swz(r)) << 4)) = v;
+        }
         return;
       }
       const int n = n_wave0 + j * 32 + 16 * (lane >> 5);
@@ -939,12 +948,68 @@ __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiPara
       store_all(IntC<0>());
     if (kHook) {
       before_stores();
+      // A wave tile of 64 channels (the persistent 256 x 256 kernel): the 32 x 64 results of a
+      // row of fragments go through the wave's own 4 KiB of staging (where the 4-byte epilogues
+      // stage theirs) and leave as whole 64-byte row pieces, written through the L2 -- no
+      // barrier, and nothing left dirty for the write-back after the last wave.
+      constexpr bool kWaveStage = FN == 2;
+      if constexpr (kWaveStage) {
+        int8_t* stg = (stage_base ? stage_base : smem + CP_BYTES) + wave * 4096;
+        static_for<FM>([&](auto ic) {
+          constexpr int i = decltype(ic)::value;
+          const int r = lane & 31;
 #pragma unroll
-      for (int j = 0; j < FN; ++j)
+          for (int j = 0; j < 2; ++j)
+            *reinterpret_cast<v4i*>(stg + r * 64 + (((2 * j + (lane >> 5)) ^ ((r >> 2) & 3)) << 4)) =
+                held[kHook ? i : 0][kHook ? j : 0];
 #pragma unroll
-        for (int i = 0; i < FM; ++i) store_frag(held[kHook ? i : 0][kHook ? j : 0], i, j);
+          for (int k = 0; k < 2; ++k) {
+            const int u = k * 64 + lane;
+            const int row = u >> 2;
+            const int c = (u & 3) ^ ((row >> 2) & 3);
+            const v4i v = *reinterpret_cast<const v4i*>(stg + u * 16);
+            const int m = m_wave0 + i * 32 + row, n = n_wave0 + c * 16;
+            if (m < m_end && n < e.N) {
+              int8_t* dst = out + (int64_t)m * e.ldo + n;
+              if (n + 15 < e.N) {
+                st_through(dst, v);
+              } else {
+#pragma unroll
+                for (int b = 0; b < 16; ++b)
+                  if (n + b < e.N) dst[b] = (int8_t)((uint32_t)v[b >> 2] >> (8 * (b & 3)));
+              }
+            }
+          }
+        });
+      } else {
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int i = 0; i < FM; ++i) store_frag(held[kHook ? i : 0][kHook ? j : 0], i, j);
+      }
     }
-    if constexpr (BLOCK_STAGE) {
+    if constexpr (BLOCK_STAGE && kWavePrivate) {
+      before_stores();
+      const int8_t* mine = tile + wave * (FM * 32 * 64);
+#pragma unroll
+      for (int k = 0; k < FM * 2; ++k) {
+        const int u = k * 64 + lane;
+        const int row = u >> 2;
+        const int c = (u & 3) ^ ((row >> 2) & 3);
+        const int m = m_wave0 + row, n = n_wave0 + c * 16;
+        if (m < m_end && n < e.N) {
+          const v4i v = *reinterpret_cast<const v4i*>(mine + u * 16);
+          int8_t* dst = out + (int64_t)m * e.ldo + n;
+          if (n + 15 < e.N) {
+            st_through(dst, v);
+          } else {
+#pragma unroll
+            for (int b = 0; b < 16; ++b)
+              if (n + b < e.N) dst[b] = (int8_t)((uint32_t)v[b >> 2] >> (8 * (b & 3)));
+          }
+        }
+      }
+    } else if constexpr (BLOCK_STAGE) {
       static_assert(kWM * kWN * 64 == NT && (kBM * kChunks) % NT == 0, "block tile over the workgroup");
       __syncthreads();
       before_stores();
