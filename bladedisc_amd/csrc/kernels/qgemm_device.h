@@ -774,15 +774,17 @@ __global__ void __launch_bounds__(WM* WN * 64) qgemm_mfma_kernel(const MainParam
 // int32 / f32 results are staged through LDS one fragment at a time so that they leave as
 // full 128-byte row segments.
 // BLOCK_STAGE (int8 results, every wave of the workgroup active, (NT / 64) wave tiles side by
-// side covering the BN columns): the waves put their packed results into one row-major tile of
-// the whole block in LDS, behind the factors, and after a barrier the workgroup stores it row
-// by row -- whole rows of BN bytes per group of BN / 16 lanes -- with stores that write through
-// the L2 (st_through: a wave's own 32-byte row pieces would be too small for those).  Measured,
-// us per launch before / after: M = 6272, 256 -> 1024 7.65 / 7.0; M = 100352, 256 -> 128 13.0 /
-// 11.7; M = 4096, 768 -> 3072 15.2 / 14.6; 4096^3 unchanged.  Not for the persistent kernels: a
-// workgroup that walks several tiles writes most of its results long before the kernel ends,
-// and there the extra barrier and LDS trip per tile cost more than the shorter tail saves
-// (M = 16384, 768 -> 3072: 50.0 -> 52.0 us).
+// side covering the BN columns): results leave through LDS, behind the factors, in row order, with
+// stores that write through the L2 (st_through; a lane pair's own 32-byte row pieces would be too
+// small for those).  A wave tile of 64 channels stages and stores its own rows -- whole 64-byte
+// pieces, no barrier; narrower or odd wave tiles are collected in one row-major tile of the
+// whole block, and after a barrier the workgroup stores it BN bytes a row.  Measured, us per
+// launch before / after: M = 6272, 256 -> 1024 7.65 / 7.0; M = 100352, 256 -> 128 13.0 / 11.7;
+// M = 4096, 768 -> 3072 15.2 / 14.3; 4096^3 61.3 / 59.5.  The persistent kernels, whose epilogue
+// holds its results in registers until the next tile's loads have landed, do the same per row
+// of fragments where a wave tile is 64 channels wide (M = 16384, 768 -> 3072: 48.5 / 45.5); the
+// block-wide form was measured there and lost (50.0 / 52.0: a barrier and an LDS trip per tile
+// for results most of which are written long before the kernel ends).
 template <int EPI, int FM, int FN, int NT, int BN, typename BeforeStores, bool BLOCK_STAGE>
 __device__ __forceinline__ void mfma_epilogue(v16i (&acc)[FM][FN], const EpiParams& e,
                                               int8_t* smem, int m_wave0, int n_wave0,
