@@ -65,13 +65,39 @@ def _compile(src, force, hdr_m, hooks=False):
             and os.path.getmtime(obj) > max(os.path.getmtime(src), hdr_m)):
         return obj, ""
     cmd = [HIPCC] + COMMON + DEVICE + (["-DDQ8_TEST_HOOKS"] if hooks else []) + \
-        ["-x", "hip", "-c", src, "-o", obj]
+        ["-Rpass-analysis=kernel-resource-usage", "-x", "hip", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
-    log = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
-                    if "packed-fp32-ops" not in l)
+    lines = (r.stdout + r.stderr).splitlines()
+    log = "\n".join(l for l in lines if "packed-fp32-ops" not in l and "remark:" not in l)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+    _record_resources(obj, lines)
     return obj, log
+
+
+def _record_resources(obj, lines):
+    """Registers and scratch of every kernel in the object, from the compiler's resource remarks,
+    as <obj>.resources.json (read by tests/test_build_resources.py: the kernels that are meant
+    to keep everything in registers must not spill)."""
+    import json
+    import re
+    kernels, name = {}, None
+    for l in lines:
+        m = re.search(r"remark: .*Function Name: (\S+)", l)
+        if m:
+            name = m.group(1)
+            kernels[name] = {}
+            continue
+        if name is None:
+            continue
+        for key, pat in (("vgprs", r"VGPRs: (\d+)"), ("agprs", r"AGPRs: (\d+)"),
+                         ("scratch_bytes_per_lane", r"ScratchSize \[bytes/lane\]: (\d+)"),
+                         ("lds_bytes", r"LDS Size \[bytes/block\]: (\d+)")):
+            m = re.search("remark: .* " + pat, l)
+            if m:
+                kernels[name][key] = int(m.group(1))
+    with open(obj + ".resources.json", "w") as f:
+        json.dump(kernels, f, indent=0, sort_keys=True)
 
 
 def build_test_code_objects():

@@ -86,7 +86,8 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   // instruction covers whole 64- or 128-byte pieces, which can be written through the L2 (see
   // st_through: an ordinary store's dirty lines are written back after the kernel's last wave,
   // 25 MB of results in about 2.5 us; 32-byte pieces written through are slower than that).
-  constexpr bool STAGE = NS >= 64;
+  // (not where the fused operators come on top of a filter slice of 144 registers: no room)
+  constexpr bool STAGE = NS >= 64 && !(POST && KS * NF * 4 + NF * 16 > 170);
   constexpr int LPR = NS / 16;                // lanes (16-byte chunks) per row of the tile
   constexpr bool HOIST_OS = KS * NF * 4 + NF * 16 + NF * 16 + 60 <= 240;
   constexpr bool HOIST_B = KS * NF * 4 + NF * 16 + NF * 32 + 60 <= 240;
@@ -333,6 +334,10 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
       constexpr int s = decltype(sc)::value;
       if constexpr (s < KS) load_frag(IntC<s>());
     });
+    // (A 32-channel slice is one chain of MFMAs, each waiting for the one before it -- 48.6
+    // cycles apiece instead of 32 for a wave on its own; even and odd steps on two accumulators
+    // were measured on one box: 32 x 28 x 28 x 128 -> 128 8.63 against 8.74 us -- the other wave
+    // of the SIMD fills the gaps already; not worth 16 more registers.)
     v16i acc[NF];
     static_for<KS>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
@@ -361,27 +366,38 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
       static_for<NF>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         const int cl0 = j * 32 + 4 * c0;
-        v4f os4[4], b4[4];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
+        auto factors = [&](int g, v4f& os, v4f& b) {
           if constexpr (HOIST_OS)
-            os4[g] = hos[j][g];
+            os = hos[j][g];
           else
-            os4[g] = *reinterpret_cast<const v4f*>(&cp_os[cl0 + 8 * g]);
+            os = *reinterpret_cast<const v4f*>(&cp_os[cl0 + 8 * g]);
           if constexpr (PLAIN)
-            b4[g] = (v4f){0.f, 0.f, 0.f, 0.f};
+            b = (v4f){0.f, 0.f, 0.f, 0.f};
           else if constexpr (HOIST_B)
-            b4[g] = hb[j][g];
+            b = hb[j][g];
           else
-            b4[g] = *reinterpret_cast<const v4f*>(&cp_b[cl0 + 8 * g]);
+            b = *reinterpret_cast<const v4f*>(&cp_b[cl0 + 8 * g]);
+        };
+        // all LDS reads of the fragment ahead of its arithmetic (the instantiations with fused
+        // operators have no registers to spare for that and read as they go)
+        constexpr bool kAhead = !POST && (!HOIST_OS || (!PLAIN && !HOIST_B));
+        v4f os4[kAhead ? 4 : 1], b4[kAhead ? 4 : 1];
+        if constexpr (kAhead) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) factors(g, os4[g], b4[g]);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        // (the instantiations with fused operators have no registers to spare for that)
-        if constexpr (!POST && (!HOIST_OS || (!PLAIN && !HOIST_B))) __builtin_amdgcn_sched_barrier(0);
         uint32_t w[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const ColParams c[4] = {{os4[g][0], b4[g][0], 0}, {os4[g][1], b4[g][1], 0},
-                                  {os4[g][2], b4[g][2], 0}, {os4[g][3], b4[g][3], 0}};
+          v4f os, b;
+          if constexpr (kAhead) {
+            os = os4[g];
+            b = b4[g];
+          } else {
+            factors(g, os, b);
+          }
+          const ColParams c[4] = {{os[0], b[0], 0}, {os[1], b[1], 0}, {os[2], b[2], 0}, {os[3], b[3], 0}};
           w[g] = requant_pack4<EPI, PLAIN>(e, c, acc[j][4 * g + 0], acc[j][4 * g + 1],
                                            acc[j][4 * g + 2], acc[j][4 * g + 3]);
         }
