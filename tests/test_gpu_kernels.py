@@ -1296,6 +1296,32 @@ def test_qgemm_strided_rows_all_variants(K, m, n, k, pad):
         assert (got[:, n:] == 77).all(), "variant %d wrote past the row" % v
 
 
+@pytest.mark.parametrize("m,n,k,ldo", [(300, 200, 256, 208), (1000, 100, 768, 112), (513, 72, 128, 80),
+                                       (4100, 1000, 768, 1008), (260, 328, 512, 336)])
+def test_qgemm_ragged_channels_in_16_byte_aligned_rows(K, m, n, k, ldo):
+    """Output rows that take 16-byte stores (aligned buffer, row stride a multiple of 16) while
+    the channel count is not a multiple of 16: the last chunk of a row is written byte by byte,
+    and nothing lands in the columns behind it -- every variant, both int8 epilogues."""
+    rng = np.random.default_rng(m * 7 + n)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    acc, _ = O.gemm_s32_fast(a, w)
+    sx, sw = make_scales(rng, n)
+    so = pick_so(acc, sx, sw)
+    bias = rng.standard_normal(n).astype(np.float32) * 5
+    want1 = O.requant_cpu(acc, sx, sw, so)
+    want2 = O.requant_gpu(acc, sx, sw, so, bias_f32=bias)
+    da, dw = dev(a), dev(w)
+    scales = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])))
+    for v in [-1] + gemm_variants(K, k):
+        for epi, want, b in ((K.EPI_REQUANT_CPU, want1, None), (K.EPI_REQUANT_GPU, want2, dev(bias))):
+            out_full = torch.full((m, ldo), 77, dtype=torch.int8, device="cuda")
+            K.qgemm(da, dw, epi, bias=b, out=out_full[:, :n], variant=v, **scales)
+            got = host(out_full)
+            np.testing.assert_array_equal(got[:, :n], want, err_msg="variant %d epilogue %d" % (v, epi))
+            assert (got[:, n:] == 77).all(), "variant %d wrote past the row" % v
+
+
 def test_qgemm_random_shapes_epilogues_variants(K):
     """Seeded sweep over ragged shapes, every epilogue / bias kind and every kernel
     variant (heuristic included), bit-exact against the oracle."""
