@@ -76,19 +76,18 @@ __global__ void __launch_bounds__(512) qconv_stream_kernel(const DirectConvParam
   constexpr int FSHIFT = LOG2_CI >= 8 ? 0 : 8 - LOG2_CI, FMASK = CP > 16 ? 15 : CP - 1;
   constexpr int STEPS_PER_TAP = CI >= 32 ? CI / 32 : 1;
   constexpr int kOutOfRange = (int)0x80000000;
-  // The factors of a lane's channels (16 per 32-channel fragment) stay in registers over all
-  // blocks where the filter slice leaves room for them; otherwise they are read from LDS per
-  // fragment, all reads of a fragment ahead of its arithmetic (read one by one as they are
-  // needed, each exposes the LDS latency under the other waves' fragment reads: 1750 cycles per
-  // 32 x 64 block instead of 700).
   // Results leave through a wave-private LDS tile where a slice row is 64 bytes or more: of a
   // fragment a lane pair holds 32 bytes of a pixel's row; read back in row order, a store
   // instruction covers whole 64- or 128-byte pieces, which can be written through the L2 (see
   // st_through: an ordinary store's dirty lines are written back after the kernel's last wave,
   // 25 MB of results in about 2.5 us; 32-byte pieces written through are slower than that).
-  // (not where the fused operators come on top of a filter slice of 144 registers: no room)
+  // Not where the fused operators come on top of a filter slice of 144 registers: no room.
   constexpr bool STAGE = NS >= 64 && !(POST && KS * NF * 4 + NF * 16 > 170);
-  constexpr int LPR = NS / 16;                // lanes (16-byte chunks) per row of the tile
+  constexpr int LPR = NS / 16;                // lanes (16-byte chunks) per row of that tile
+  // The factors of a lane's channels (16 scales and 16 addends per 32-channel fragment) stay in
+  // registers over all blocks where the filter slice leaves room for them; otherwise they are
+  // read from LDS per fragment, all reads of a fragment ahead of its arithmetic (read one by one
+  // as they are needed, each read exposes the LDS latency under the other waves' fragment reads).
   constexpr bool HOIST_OS = KS * NF * 4 + NF * 16 + NF * 16 + 60 <= 240;
   constexpr bool HOIST_B = KS * NF * 4 + NF * 16 + NF * 32 + 60 <= 240;
   static_assert(W_PER_WAVE * NW * 1024 <= W_LDS, "weight area");
