@@ -85,15 +85,18 @@ bool direct_conv_plan(int config, DirectConvParams* p) {
 
 namespace {
 // The (filter, slice) pairs the streaming kernel is instantiated for: 3 x 3 filters on 64 and 128
-// channels, and 1 x 1 filters (a GEMM over the pixels with a short k) on the same.  A slice is as
-// wide as the registers allow -- NS K / 256 of them hold it, next to 16 accumulators per 32
-// channels of it -- since every workgroup of a pixel tile loads the tile's patch again; `narrow`
-// is a second width for layers with no more output channels than that.
+// channels, 1 x 1 filters (a GEMM over the pixels with a short k) on 64 to 256, and the 4 x 4 x 16
+// form of a stem.  A slice is as wide as the registers allow -- NS K / 256 of them hold it, next
+// to 16 accumulators per 32 channels of it -- since every workgroup of a pixel tile loads the
+// tile's patch again; `narrow` is a second width for layers with no more output channels than
+// that.  (1 x 1 x 256 with 128-channel slices spills; 1 x 1 x 512 was measured and lost to the
+// GEMM tiles at every size.)
 struct StreamInstance {
   int kh, kw, ci, ns, narrow;
 };
 constexpr StreamInstance kStreamInstances[] = {
     {3, 3, 64, 64, 0}, {3, 3, 128, 32, 0}, {1, 1, 64, 128, 64}, {1, 1, 128, 128, 0}, {4, 4, 16, 64, 0},
+    {1, 1, 256, 64, 0},
 };
 int stream_conv_slice(int Kh, int Kw, int Ci, int Co) {
   for (const StreamInstance& s : kStreamInstances)
@@ -193,6 +196,10 @@ int launch_stream_epi(const DirectConvParams& p, hipStream_t st) {
   if (taps == 1 && p.Ci == 64 && p.slice_n == 128) return launch_stream_post<1, 1, 64, 128, EPI>(p, st);
   if (taps == 1 && p.Ci == 64 && p.slice_n == 64) return launch_stream_post<1, 1, 64, 64, EPI>(p, st);
   if (taps == 1 && p.Ci == 128 && p.slice_n == 128) return launch_stream_post<1, 1, 128, 128, EPI>(p, st);
+  // (256 channels: without fused operators only -- with them the kernel would spill)
+  if (taps == 1 && p.Ci == 256 && !(p.epi.table != nullptr || p.epi.resid_kind != 0)) {
+    if (p.slice_n == 64) return launch_stream_t<1, 1, 256, 64, EPI, false>(p, st);
+  }
   return fail("the streaming convolution kernel has no instance for this filter");
 }
 }  // namespace

@@ -1,7 +1,8 @@
 // int8 NHWC stride-1 convolution with the whole filter in registers ("streaming" form), for
 // filters of which a slice of NS output channels fits there: NS * Kh * Kw * Ci <= 36 KiB
 // (3 x 3 x 64 with 64-channel slices in the first place, 3 x 3 x 128 with 32-channel slices,
-// 1 x 1 x 64 and 1 x 1 x 128 with 128-channel slices, 4 x 4 x 16 -- a 7 x 7 stride-2 stem after
+// 1 x 1 x 64 and 1 x 1 x 128 with 128-channel slices, 1 x 1 x 256 with 64-channel slices,
+// 4 x 4 x 16 -- a 7 x 7 stride-2 stem after
 // space to depth -- with 64-channel slices).
 //
 // Where the time of such a layer goes in the LDS-tiled kernels (32 x 56 x 56 x 64 -> 64, 9 us):
@@ -23,7 +24,7 @@
 //    pipe), so one wave's epilogue runs under the other's MFMAs.
 // The weights go to LDS before the patch and are copied to registers while the patch is still
 // arriving.
-// A 1 x 1 filter (a GEMM over the pixels with k = Ci) runs the same way on 64 or 128 channels,
+// A 1 x 1 filter (a GEMM over the pixels with k = Ci) runs the same way on 64 to 256 channels,
 // where the GEMM kernels' k tile of 128 is short or half empty and their lock-step
 // requantisation is most of the time; its blocks share no pixels, so a wave loads those of its
 // own blocks and waits for no other wave's: the first block's before the weights' barrier, the

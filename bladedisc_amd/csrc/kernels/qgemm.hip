@@ -1256,7 +1256,7 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
   // what the streaming kernel asks of the output side
   const bool stream_out = !e.fixedpoint && e.vec_store16 &&
                           (epilogue == DQ8_EPI_REQUANT_CPU || epilogue == DQ8_EPI_REQUANT_GPU);
-  // On 64 or 128 input channels the filter fits the registers of the streaming kernel; its
+  // On 64 to 256 input channels the filter fits the registers of the streaming kernel; its
   // pixels are then one long row, cut into patch rows of 16 where the count allows, so that a
   // tile is any run of pixels, across images.
   if (pointwise && (auto_pick || variant == kStreamConv)) {
@@ -1271,21 +1271,32 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
       sp.NB = (int)NB; sp.H = sp.Ho = (int)Ho; sp.Wd = sp.Wo = (int)Wo;
     }
     sp.epi = e;
-    const bool ok = stream_out && Ci <= 128 && stream_conv_has_instance(1, 1, (int)Ci) &&
+    const bool ok = stream_out && Ci <= 256 && (Ci <= 128 || !fused) && stream_conv_has_instance(1, 1, (int)Ci) &&
                     stream_conv_plan(&sp);
     if (!auto_pick)
       DQ8_REQUIRE(ok, "dq8_qconv2d: the streaming variant needs a 3 x 3 or 1 x 1 filter on 64 or "
-                      "128 input channels, stride and dilation 1, an int8 result (float output "
-                      "stage) and 16-byte aligned output rows");
+                      "128 input channels (1 x 1 without fused operators also on 256), stride and "
+                      "dilation 1, an int8 result (float output stage) and 16-byte aligned output "
+                      "rows");
     // Against the GEMM kernels, whose k tile of 128 is half empty at 64 channels and whose
     // workgroups requantise in lock step, it wins once the launch has a few million results
     // (us per launch, streaming / GEMM; 64 -> 256 channels on 56 x 56 images: batch 1 4.1 / 3.5,
     // batch 4 4.7 / 4.7, batch 8 5.45 / 7.6, batch 32 11.2 / 15.3, batch 64 17.6 / 26.3; 64 -> 64,
     // batch 32: 28 x 28 3.7 / 4.5, 56 x 56 5.5 / 7.0, 112 x 112 12.7 / 19.3; 128 -> 128, batch 32:
     // 28 x 28 5.0 / 4.7, 56 x 56 8.7 / 12.1; 128 -> 256 on 28 x 28: 5.8 / 7.7; 128 -> 512: 8.6 / 8.8,
-    // batch 64 12.6 / 15.4.  Filters on 256 and 512 input channels were built and lost at every
-    // size: 32 x 14 x 14 x 256 -> 1024 7.85 / 7.6).
-    if (ok && (!auto_pick || Mg * Co >= (Ci == 64 ? (3LL << 19) : (6LL << 20))))
+    // batch 64 12.6 / 15.4).
+    // 256 channels (64-channel slices; every slice of a pixel tile loads the tile's pixels again):
+    // while the workgroups are one round of the chip or the slices are at most two -- 32 x 14 x 14
+    // x 256 -> 1024 5.5 / 6.55, 32 x 56 x 56 x 256 -> 64 6.4 / 7.65, -> 128 10.3 / 11.5, 32 x 28 x 28
+    // x 256 -> 256 5.7 / 6.7; several rounds of many slices lose: 64 x 28 x 28 x 256 -> 256
+    // 9.9 / 8.8, 32 x 56 x 56 x 256 -> 512 31.1 / 28.4; below 1.5 M results the GEMM tiles are
+    // as fast (4 x 14 x 14 x 256 -> 1024 3.85 / 3.8).
+    const bool take = Ci == 64    ? Mg * Co >= (3LL << 19)
+                      : Ci == 128 ? Mg * Co >= (6LL << 20)
+                                  : Mg * Co >= (3LL << 19) &&
+                                        (Co <= 128 || (int64_t)sp.NB * sp.tiles_per_image * sp.tiles_n <=
+                                                          compute_units());
+    if (ok && (!auto_pick || take))
       return launch_stream_conv(epilogue, sp, st);
   }
   // Otherwise the GEMM instantiations load its rows without the per-tap address arithmetic.

@@ -1009,7 +1009,7 @@ def test_qconv_stream_16_channels(K):
 
 
 def test_qconv_stream_pointwise(K):
-    """1 x 1 filters on 64 and 128 input channels in the kernel that keeps the filter in registers
+    """1 x 1 filters on 64 to 256 input channels in the kernel that keeps the filter in registers
     (a GEMM over the pixels with a short k): pixel counts that are and are not a multiple of 16
     (one long row of pixels cut anywhere, or tiles per image), one pixel tile to many, tiles
     that end inside a block of 32 pixels, ragged channel slices, both slice widths of the
@@ -1023,7 +1023,9 @@ def test_qconv_stream_pointwise(K):
     shapes = [(8, 56, 56, 64, 256), (2, 56, 56, 64, 64), (4, 28, 28, 128, 512), (3, 7, 7, 128, 2048),
               (1, 4, 4, 128, 16), (5, 9, 7, 64, 208), (1, 1, 48, 64, 80), (7, 13, 3, 128, 144),
               (2, 23, 5, 128, 96), (1, 56, 56, 128, 64), (1, 1, 16, 64, 16), (3, 5, 11, 64, 400),
-              (1, 1, 33, 64, 48), (16, 112, 112, 64, 64), (1, 300, 301, 128, 128)]
+              (1, 1, 33, 64, 48), (16, 112, 112, 64, 64), (1, 300, 301, 128, 128),
+              # 256 input channels: 64-channel slices, one round of workgroups and several
+              (32, 14, 14, 256, 1024), (3, 9, 7, 256, 208), (2, 56, 56, 256, 64), (1, 5, 3, 256, 16)]
     for nb, h, w_, ci, co in shapes:
         x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
         wt = rng.integers(-128, 128, (co, 1, 1, ci), dtype=np.int8)
@@ -1060,7 +1062,8 @@ def test_qconv_stream_pointwise(K):
             auto = host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(b8), **scales))
             np.testing.assert_array_equal(auto, got, err_msg=tag + " heuristic")
     # fused operators: residual (+ ReLU) + quantize and a table, against the separate calls
-    for nb, h, w_, ci, co in [(32, 28, 28, 64, 256), (2, 28, 28, 128, 512), (1, 9, 11, 64, 80), (40, 56, 56, 128, 128)]:
+    for nb, h, w_, ci, co in [(32, 28, 28, 64, 256), (2, 28, 28, 128, 512), (1, 9, 11, 64, 80), (40, 56, 56, 128, 128),
+                              (8, 14, 14, 256, 1024)]:   # fused on 256 channels: the GEMM tiles' result
         x = dev(rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8))
         wt = dev(rng.integers(-128, 128, (co, 1, 1, ci), dtype=np.int8))
         out_shape = [nb, h, w_, co]
@@ -1084,7 +1087,7 @@ def test_qconv_stream_pointwise(K):
         assert torch.equal(fused, K.lut8(plain, table)), (nb, h, w_, ci, co)
     # refusals: channel counts without an instance, strides, 4-byte results
     one = dev(np.array([0.01], np.float32))
-    for ci, v in ((32, sv), (256, sv)):
+    for ci, v in ((32, sv), (512, sv)):
         x = dev(rng.integers(-128, 128, (1, 8, 8, ci), dtype=np.int8))
         wt = dev(rng.integers(-128, 128, (64, 1, 1, ci), dtype=np.int8))
         with pytest.raises(RuntimeError, match="streaming variant"):
