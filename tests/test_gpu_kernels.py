@@ -864,6 +864,53 @@ def test_qconv_direct_random_shapes(K):
 
 
 
+def test_qconv_library_choice_on_random_shapes(K):
+    """Seeded sweep over what decides the kernel of a convolution -- channel counts with and
+    without a register-filter instance, 1 x 1 to 7 x 7 filters, strides, paddings, batch and
+    image sizes from one pixel tile to many, ragged output channels, every int8 epilogue and
+    bias kind: whatever the library picks gives the bytes of the generic kernel (one thread
+    per result; pinned to the oracle by the tests above)."""
+    rng = np.random.default_rng(20260507)
+    gen = K.variant_names().index("generic")
+    md0 = list(O.NHWC_OHWI_METADATA)
+    done = 0
+    for case in range(500):
+        ci = int(rng.choice([3, 4, 16, 32, 64, 64, 128, 128, 256, 256, 512]))
+        k = int(rng.choice([7, 3, 5])) if ci <= 4 else int(rng.choice([1, 1, 1, 3, 3, 2]))
+        s = int(rng.choice([1, 1, 1, 2]))
+        pad = int(rng.choice([0, k // 2, 1 if k > 1 else 0]))
+        big = rng.random() < 0.3
+        nb = int(rng.integers(1, 40 if big else 6))
+        lo, hi = max(k - 2 * pad, 1), 30 if big else 60
+        h, w_ = int(rng.integers(lo, hi)), int(rng.integers(lo, hi))
+        if ci <= 4:
+            h, w_ = 3 * h + 7, 3 * w_ + 7
+        co = int(rng.choice([16, 32, 48, 64, 80, 128, 144, 208, 256, 512, 1024, int(rng.integers(1, 300))]))
+        ho, wo = (h + 2 * pad - k) // s + 1, (w_ + 2 * pad - k) // s + 1
+        if ho < 1 or wo < 1 or nb * ho * wo * co > 3e7 or nb * h * w_ * ci > 3e7:
+            continue
+        x = dev(rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8))
+        wt = dev(rng.integers(-128, 128, (co, k, k, ci), dtype=np.int8))
+        out_shape, md = [nb, ho, wo, co], md0 + [s, s, 1, 1, 1]
+        so = np.float32(0.02 * 0.025 * 74.0 * 74.0 * np.sqrt(k * k * ci) / 40.0)
+        kw = dict(sx=dev(np.array([0.02], np.float32)), sw=dev(rng.uniform(0.001, 0.05, co).astype(np.float32)),
+                  so=dev(np.array([so])))
+        kind, epi = int(rng.integers(0, 4)), K.EPI_REQUANT_CPU
+        if kind == 1:
+            kw.update(bias=dev((rng.standard_normal(co) * 3 * so).astype(np.float32)), zo=int(rng.integers(-10, 10)))
+        elif kind == 2:
+            kw.update(bias=dev(rng.integers(-100000, 100000, co).astype(np.int32)))
+        elif kind == 3:
+            epi = K.EPI_REQUANT_GPU
+            kw.update(bias=dev((rng.standard_normal(co) * 30).astype(np.float32)))
+        got = K.qconv2d(x, wt, [pad] * 4, md, out_shape, epi, **kw)
+        want = K.qconv2d(x, wt, [pad] * 4, md, out_shape, epi, variant=gen, **kw)
+        assert torch.equal(got, want), "case %d: %dx%dx%dx%d, %dx%d stride %d pad %d -> %d, bias kind %d" % (
+            case, nb, h, w_, ci, k, k, s, pad, co, kind)
+        done += 1
+    assert done > 400
+
+
 def test_qconv_stream_variant(K):
     """The 3 x 3 kernel (64 or 128 input channels) that keeps the filter in registers: images whose pixel
     tiles start and end anywhere in a row, one to many tiles per image, ragged and several
