@@ -1393,7 +1393,9 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     // tiles of 256 x 256, keeps them: 33.7 against 44.5 us).
     if ((variant == kPipe256w8 || variant == kPipe256x192) && pipe_ok(128, 128, p, true) &&
         (Co <= 128 || (Co <= 256 && 4 * ceil_div(Mg, 256) * ceil_div(Co, 256) < 3 * compute_units())))
-      variant = kPipe128;
+      // (eight waves while the 128 x 128 tiles are at most one per compute unit, as for the
+      // plain GEMM: 32 x 56 x 56 x 128 -> 128, 3 x 3 stride 2, 196 tiles: 8.9 against 9.7 us)
+      variant = es == 1 && ceil_div(Mg, 128) * ceil_div(Co, 128) <= compute_units() ? kPipe128w8 : kPipe128;
   }
   return launch_epi<true>(variant, p, epilogue, st);
 }

@@ -160,7 +160,8 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   const int kc = (ls ^ lr ^ (wave & 1)) << 4;   // byte offset of the lane's chunk in a k tile
   int a_off[A_LD], b_off[B_LD];      // GEMM: byte offset of the lane's chunk in row 0 of the tile
   int a_lds[A_LD], b_lds[B_LD];      // wave-uniform LDS byte offset of the 1 KiB block
-  int a_h[CONV ? A_LD : 1], a_w[CONV ? A_LD : 1], a_n[CONV ? A_LD : 1];   // conv: row geometry
+  // conv: the row's first input pixel (coordinates, and byte offset of its channel 0)
+  int a_h[CONV ? A_LD : 1], a_w[CONV ? A_LD : 1], a_pix[CONV ? A_LD : 1];
 #pragma unroll
   for (int i = 0; i < A_LD; ++i) {
     const int q = wave + i * NW;
@@ -173,7 +174,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
       // rows past M get a coordinate no tap can bring back into the image
       a_h[i] = m < p.M ? ho * p.sh - p.pad_t : -(1 << 24);
       a_w[i] = wo * p.sw_ - p.pad_l;
-      a_n[i] = n_img * p.H * p.Wd;
+      a_pix[i] = m < p.M ? ((n_img * p.H + ho * p.sh - p.pad_t) * p.Wd + a_w[i]) * p.Ci : 0;
       a_off[i] = 0;
     } else {
       a_off[i] = (q * 8 + lr) * (int)p.lda + kc;
@@ -187,21 +188,47 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   }
 
   // Per k tile: is the lane's chunk inside K, and (conv) which tap does it belong to.
-  // tile_setup(kt) precedes the issue_load calls of tile kt.
-  int t_koff = kOutOfRange, t_dh = 0, t_dw = 0, t_ci = 0;
+  // tile_setup(kt) precedes the issue_load calls of tile kt and is called with kt = 0, 1, 2, ...
+  // in turn: the lane's chunk moves on by BK channels per call, i.e. by BK / Ci taps, BK % Ci
+  // channels and at most one carry each from the channels into the taps and from the filter's
+  // columns into its rows.  (Two integer divisions per call instead were a fifth of the VALU
+  // instructions of a 64 x 64 tile's k loop, a hundred per k tile and wave next to four MFMAs;
+  // such a tile's time is its wave's instruction count: 32 x 7 x 7 x 512, 3 x 3 -> 512: 12.7 ->
+  // 11.5 us.)
+  int t_koff = kOutOfRange, t_dh = 0, t_dw = 0, t_off = 0;
+  int c_ci = 0, c_kh = 0, c_kw = 0;                  // the chunk's place in the filter, next call
+  int d_ci = 0, d_kh = 0, d_kw = 0;                  // what BK channels add to it
+  if (CONV) {
+    const unsigned k = (unsigned)(kt0 * BK + kc);
+    const unsigned tap = k / (unsigned)p.Ci;
+    c_ci = (int)(k - tap * (unsigned)p.Ci);
+    c_kh = (int)(tap / (unsigned)p.Kw);
+    c_kw = (int)(tap - (unsigned)c_kh * (unsigned)p.Kw);
+    const int d_tap = BK / p.Ci;
+    d_ci = BK - d_tap * p.Ci;
+    d_kh = d_tap / p.Kw;
+    d_kw = d_tap - d_kh * p.Kw;
+  }
+  // (The same state kept per wave in scalar registers where Ci is a multiple of BK was measured
+  // and is slower: a wave issues scalar and vector instructions from one stream, and the scalar
+  // form has more of them.)
   auto tile_setup = [&](int kt) {
     const int k = (kt0 + kt) * BK + kc;
     const bool in = kt < KT && k < p.K;
     t_koff = in ? (kt0 + kt) * BK : kOutOfRange;
     if (CONV) {
-      const unsigned tap = (unsigned)k / (unsigned)p.Ci;
-      t_ci = k - (int)tap * p.Ci;
-      const unsigned kh = tap / (unsigned)p.Kw;
-      t_dh = (int)kh * p.dh;
-      t_dw = (int)(tap - kh * p.Kw) * p.dw;
+      t_dh = c_kh * p.dh;
+      t_dw = c_kw * p.dw;
+      t_off = (t_dh * p.Wd + t_dw) * p.Ci + c_ci;
+      c_ci += d_ci;
+      const bool carry = c_ci >= p.Ci;
+      c_ci -= carry ? p.Ci : 0;
+      c_kw += d_kw + (carry ? 1 : 0);                  // (< 2 Kw)
+      const bool wrap = c_kw >= p.Kw;
+      c_kw -= wrap ? p.Kw : 0;
+      c_kh += d_kh + (wrap ? 1 : 0);
     }
   };
-
   // issues load number `idx` (0 .. LD-1) of tile `kt` into stage `st`; chunks past the
   // end of K (and conv taps in the padding) get an out-of-range offset: zeros arrive,
   // no memory is touched
@@ -215,7 +242,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
           const int hi = a_h[i] + t_dh, wi = a_w[i] + t_dw;
           const bool ok = t_koff != kOutOfRange && (unsigned)hi < (unsigned)p.H &&
                           (unsigned)wi < (unsigned)p.Wd;
-          voff = ok ? (a_n[i] + hi * p.Wd + wi) * p.Ci + t_ci : kOutOfRange;
+          voff = ok ? a_pix[i] + t_off : kOutOfRange;
         } else {
           voff = t_koff != kOutOfRange ? a_off[i] + t_koff : kOutOfRange;
         }
