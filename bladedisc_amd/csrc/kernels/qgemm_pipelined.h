@@ -142,9 +142,11 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   // image (convolution)
   constexpr int64_t kMaxRecords = 0x7fffffff;
   constexpr int kOutOfRange = (int)0x80000000;
-  const int8_t* a_base = CONV ? p.A : p.A + (int64_t)m0 * p.lda;
+  const bool rowmap = !CONV && p.rowmap != 0;       // rows are the pixels of a strided 1 x 1 filter
+  const int8_t* a_base = CONV || rowmap ? p.A : p.A + (int64_t)m0 * p.lda;
   const int8_t* w_base = p.W + (int64_t)n0 * p.ldw;
-  const int64_t a_valid = CONV ? p.conv_bytes : (int64_t)(p.M - m0 - 1) * p.lda + p.K;
+  const int64_t a_valid =
+      CONV || rowmap ? p.conv_bytes : (int64_t)(p.M - m0 - 1) * p.lda + p.K;
   const int64_t w_valid = (int64_t)(p.N - n0 - 1) * p.ldw + p.K;
   const v4i a_rsrc = make_rsrc(a_base, a_valid < kMaxRecords ? a_valid : kMaxRecords);
   const v4i w_rsrc = make_rsrc(w_base, w_valid < kMaxRecords ? w_valid : kMaxRecords);
@@ -176,6 +178,13 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
       a_w[i] = wo * p.sw_ - p.pad_l;
       a_pix[i] = m < p.M ? ((n_img * p.H + ho * p.sh - p.pad_t) * p.Wd + a_w[i]) * p.Ci : 0;
       a_off[i] = 0;
+    } else if (rowmap) {
+      // (rows past M read the last row again; their results are not stored)
+      const int m = min(m0 + q * 8 + lr, p.M - 1);
+      const int hw = p.Ho * p.Wo;
+      const int n_img = m / hw, rem = m - n_img * hw;
+      const int ho = rem / p.Wo, wo = rem - ho * p.Wo;
+      a_off[i] = ((n_img * p.H + ho * p.sh) * p.Wd + wo * p.sw_) * p.Ci + kc;
     } else {
       a_off[i] = (q * 8 + lr) * (int)p.lda + kc;
     }

@@ -702,6 +702,11 @@ CONVS = [  # nb, h, w, ci, co, k, stride, pad, dil
     (1, 33, 17, 64, 200, 3, 1, 2, 1),
     (1, 36, 36, 256, 64, 3, 1, 1, 1),  # a patch of 107 KiB: LDS addresses beyond 128 KiB
     (1, 6, 150, 64, 64, 3, 1, 1, 1),   # a wide image: tiles of 256 pixels span 2-3 rows
+    # 1 x 1 filters with a stride: the library runs them as a GEMM over the pixels they read
+    (3, 14, 14, 256, 512, 1, 2, 0, 1),
+    (2, 9, 11, 48, 80, 1, 2, 0, 1),    # odd image sizes, K = 48, ragged Co
+    (5, 28, 28, 128, 256, 1, 2, 0, 1),  # several row tiles, images ending inside a tile
+    (1, 7, 5, 512, 1024, 1, 3, 0, 1),
 ]
 
 
@@ -862,6 +867,42 @@ def test_qconv_direct_random_shapes(K):
                                  variant=v))
             np.testing.assert_array_equal(got, want, err_msg=tag + " variant %d" % v)
 
+
+
+def test_qconv_strided_pointwise_rows_are_pixels(K):
+    """1 x 1 filters with unequal strides, and with fused operators, on the path that finds each
+    GEMM row's input pixel once and then runs the plain GEMM's loop: against the oracle, the
+    implicit-GEMM kernel and the separate calls."""
+    rng = np.random.default_rng(20260618)
+    names = K.variant_names()
+    pipe128 = names.index("pipe_128x128x128")
+    for nb, h, w_, ci, co, sh, sw_ in [(2, 13, 17, 64, 96, 2, 1), (3, 16, 9, 128, 200, 1, 2), (1, 30, 31, 32, 64, 3, 2),
+                                      (16, 28, 28, 256, 512, 2, 2), (4, 56, 56, 64, 128, 2, 2)]:
+        x = rng.integers(-128, 128, (nb, h, w_, ci), dtype=np.int8)
+        wt = rng.integers(-128, 128, (co, 1, 1, ci), dtype=np.int8)
+        ho, wo = (h - 1) // sh + 1, (w_ - 1) // sw_ + 1
+        md = list(O.NHWC_OHWI_METADATA) + [sh, sw_, 1, 1, 1]
+        out_shape, pad = [nb, ho, wo, co], [0, 0, 0, 0]
+        acc = O.conv_s32(x, wt, pad, md, out_shape)
+        tag = "%dx%dx%dx%d -> %d, strides %d %d" % (nb, h, w_, ci, co, sh, sw_)
+        np.testing.assert_array_equal(host(K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_ACC_S32)), acc,
+                                      err_msg=tag)
+        sx, sw = make_scales(rng, co)
+        so = pick_so(acc, sx, sw)
+        sc = dict(sx=dev(np.array([sx])), sw=dev(sw), so=dev(np.array([so])))
+        bf = (rng.standard_normal(co) * 30).astype(np.float32)
+        got = K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(bf), **sc)
+        np.testing.assert_array_equal(host(got), O.requant_gpu(acc.reshape(-1, co), sx, sw, so, bias_f32=bf).reshape(out_shape),
+                                      err_msg=tag)
+        assert torch.equal(got, K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_GPU, bias=dev(bf),
+                                          variant=pipe128, **sc)), tag
+        plain = K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, **sc)
+        res = dev(rng.standard_normal(out_shape).astype(np.float32) * 300)
+        s2, z1 = dev(np.array([7.0], np.float32)), torch.zeros(1, dtype=torch.int32, device="cuda")
+        fused = K.qconv2d(dev(x), dev(wt), pad, md, out_shape, K.EPI_REQUANT_CPU, **sc,
+                          post=K.make_postops(residual=res, relu=True, out_scale=s2, out_zp=-3))
+        t = torch.clamp_min(K.dequantize(plain, sc["so"], z1) + res, 0.0)
+        assert torch.equal(fused, K.quantize(t, s2, torch.full((1,), -3, dtype=torch.int32, device="cuda"))), tag
 
 
 def test_qconv_library_choice_on_random_shapes(K):
