@@ -309,7 +309,8 @@ mfma_probe_kernel(const int8_t* a, const int8_t* b, int32_t* d32, const int8_t* 
 }  // namespace
 #define DQ8_DECLARE_LAUNCH(CONV, EPI) \
   extern template int launch_variant<CONV, EPI>(int, MainParams&, hipStream_t); \
-  extern template int launch_f32a<CONV, EPI>(const MainParams&, hipStream_t);
+  extern template int launch_f32a<CONV, EPI>(const MainParams&, hipStream_t); \
+  extern template int launch_rowmap<CONV, EPI>(int, MainParams&, hipStream_t);
 DQ8_DECLARE_LAUNCH(false, DQ8_EPI_ACC_S32)
 DQ8_DECLARE_LAUNCH(false, DQ8_EPI_REQUANT_CPU)
 DQ8_DECLARE_LAUNCH(false, DQ8_EPI_REQUANT_GPU)
@@ -344,6 +345,17 @@ int launch_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
     case DQ8_EPI_REQUANT_CPU: return launch_variant<CONV, DQ8_EPI_REQUANT_CPU>(variant, p, st);
     case DQ8_EPI_REQUANT_GPU: return launch_variant<CONV, DQ8_EPI_REQUANT_GPU>(variant, p, st);
     case DQ8_EPI_DEQUANT_F32: return launch_variant<CONV, DQ8_EPI_DEQUANT_F32>(variant, p, st);
+  }
+  return fail("unknown epilogue");
+}
+
+// (the GEMM over the pixels of a strided 1 x 1 filter; its kernels sit with the convolution's)
+int launch_rowmap_epi(int variant, MainParams& p, int epilogue, hipStream_t st) {
+  switch (epilogue) {
+    case DQ8_EPI_ACC_S32: return launch_rowmap<true, DQ8_EPI_ACC_S32>(variant, p, st);
+    case DQ8_EPI_REQUANT_CPU: return launch_rowmap<true, DQ8_EPI_REQUANT_CPU>(variant, p, st);
+    case DQ8_EPI_REQUANT_GPU: return launch_rowmap<true, DQ8_EPI_REQUANT_GPU>(variant, p, st);
+    case DQ8_EPI_DEQUANT_F32: return launch_rowmap<true, DQ8_EPI_DEQUANT_F32>(variant, p, st);
   }
   return fail("unknown epilogue");
 }
@@ -1337,14 +1349,13 @@ int qconv2d_impl(int variant, const int8_t* in, const int64_t in_sizes[4], const
     g.H = (int)H; g.Wd = (int)Wd; g.Ci = (int)Ci; g.Ho = (int)Ho; g.Wo = (int)Wo;
     g.sh = sh; g.sw_ = sw_;
     g.conv_bytes = NB * H * Wd * Ci;
-    g.rowmap = 1;
     g.epi = e;
     int v = pick_any(Mg, Co, Ci, pipe_ok(256, 256, g, false), es);
     if (v == kPersist256) v = kPipe256w8;
     if (v == kPersist256x192) v = kPipe256x192;
     if (v == kPersist128) v = kPipe128w8;
-    if (is_pipe_variant(v) && pipe_ok(kVariants[v].bm, kVariants[v].bn, g, false))
-      return launch_epi<false>(v, g, epilogue, st);
+    if (rowmap_has_variant(v) && pipe_ok(kVariants[v].bm, kVariants[v].bn, g, false))
+      return launch_rowmap_epi(v, g, epilogue, st);
   }
 
   MainParams p = {};

@@ -82,10 +82,6 @@ struct MainParams {
   int H, Wd, Ci, Ho, Wo, Kh, Kw;
   int pad_t, pad_l, sh, sw_, dh, dw;
   int64_t conv_bytes;   // size of the NHWC image tensor in bytes
-  // Plain GEMM over the pixels a strided 1 x 1 filter reads (pipelined one-tile kernels only):
-  // row m of A is input pixel (m / (Ho Wo), sh ((m / Wo) % Ho), sw_ (m % Wo)) of the image
-  // described by H, Wd, Ci, Ho, Wo, sh, sw_, conv_bytes; lda is not used
-  int rowmap;
   int tiles_m, tiles_n;
   // Zero-point corrections (pipelined GEMM kernels; null = none): the accumulator of
   // output (m, n) starts at corr_n[n] + corr_m[m] instead of 0.

@@ -119,13 +119,13 @@ inline bool pipe_ok(int bm, int bn, const MainParams& p, bool conv) {
   return (int64_t)bm * p.lda + p.K + 2 * BK < (1LL << 31);
 }
 
-template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI>
+template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI, bool ROWMAP = false>
 int launch_pipe(const MainParams& p, hipStream_t st) {
   constexpr int BK = 128;
   constexpr int lds = KSPLIT * 2 * (BM + BN) * BK;
-  DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV),
+  DQ8_REQUIRE(pipe_ok(BM, BN, p, CONV) && (!ROWMAP || p.conv_bytes < (1LL << 31)),
               "pipelined qgemm needs K % 16 == 0 and operands that fit 32-bit buffer offsets");
-  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, KSPLIT, CONV, EPI>;
+  auto kern = qgemm_pipe_kernel<BM, BN, WM, WN, KSPLIT, CONV, EPI, ROWMAP>;
   static std::atomic<uint64_t> lds_allowed{0};
   if (int s = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds, &lds_allowed)) return s;
   hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(WM * WN * KSPLIT * 64), lds, st, p);
@@ -258,6 +258,30 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
   return fail("unknown or unsupported qgemm variant for this operation");
 }
 
+// The tiles a strided 1 x 1 convolution runs on as a GEMM over the pixels it reads (instantiated
+// next to the convolution kernels: CONV true; the GEMM files carry a stub).
+inline bool rowmap_has_variant(int variant) {
+  return variant == kPipe128 || variant == kPipe128w8 || variant == kPipe64 || variant == kPipe64k2 ||
+         variant == kPipe256w8 || variant == kPipe256x192;
+}
+template <bool CONV, int EPI>
+int launch_rowmap(int variant, MainParams& p, hipStream_t st) {
+  if constexpr (CONV) {
+    const Variant& v = kVariants[variant];
+    p.tiles_m = (int)ceil_div(p.M, v.bm);
+    p.tiles_n = (int)ceil_div(p.N, v.bn);
+    switch (variant) {
+      case kPipe128: return launch_pipe<128, 128, 2, 2, 1, false, EPI, true>(p, st);
+      case kPipe128w8: return launch_pipe<128, 128, 2, 4, 1, false, EPI, true>(p, st);
+      case kPipe64: return launch_pipe<64, 64, 2, 2, 1, false, EPI, true>(p, st);
+      case kPipe64k2: return launch_pipe<64, 64, 2, 2, 2, false, EPI, true>(p, st);
+      case kPipe256w8: return launch_pipe<256, 256, 2, 4, 1, false, EPI, true>(p, st);
+      case kPipe256x192: return launch_pipe<256, 192, 4, 2, 1, false, EPI, true>(p, st);
+    }
+  }
+  return fail("no kernel with rows mapped to pixels for this variant");
+}
+
 }  // namespace dq8
 
 // the body of one qgemm_launch_*.hip
@@ -265,6 +289,7 @@ int launch_variant(int variant, MainParams& p, hipStream_t st) {
   namespace dq8 {                          \
   template int launch_variant<CONV, EPI>(int, MainParams&, hipStream_t); \
   template int launch_f32a<CONV, EPI>(const MainParams&, hipStream_t);   \
+  template int launch_rowmap<CONV, EPI>(int, MainParams&, hipStream_t);  \
   }
 
 #endif  // DQ8_QGEMM_LAUNCH_H_

@@ -99,7 +99,11 @@ __device__ __forceinline__ void buffer_load_lds_b128(v4i rsrc, unsigned lds_addr
 // s_waitcnt immediate for gfx9: vmcnt = n (6 bits, split), lgkmcnt = 0, expcnt = any
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4); }
 
-template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI>
+// ROWMAP (with CONV false): the plain GEMM over the pixels a strided 1 x 1 filter reads.  Row m
+// of A is input pixel (m / (Ho Wo), sh ((m / Wo) % Ho), sw_ (m % Wo)) of the NHWC image that H,
+// Wd, Ci, Ho, Wo, sh, sw_ and conv_bytes describe (lda is not used): found once, before the k
+// loop, which is the GEMM's -- half the instructions of the implicit GEMM's.
+template <int BM, int BN, int WM, int WN, int KSPLIT, bool CONV, int EPI, bool ROWMAP = false>
 __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const MainParams p) {
   // The inline assembly only assembles in the device compilation; the host pass
   // just needs the kernel's stub.
@@ -142,11 +146,11 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   // image (convolution)
   constexpr int64_t kMaxRecords = 0x7fffffff;
   constexpr int kOutOfRange = (int)0x80000000;
-  const bool rowmap = !CONV && p.rowmap != 0;       // rows are the pixels of a strided 1 x 1 filter
-  const int8_t* a_base = CONV || rowmap ? p.A : p.A + (int64_t)m0 * p.lda;
+  static_assert(!(CONV && ROWMAP), "rows mapped to pixels: a form of the plain GEMM");
+  const int8_t* a_base = CONV || ROWMAP ? p.A : p.A + (int64_t)m0 * p.lda;
   const int8_t* w_base = p.W + (int64_t)n0 * p.ldw;
   const int64_t a_valid =
-      CONV || rowmap ? p.conv_bytes : (int64_t)(p.M - m0 - 1) * p.lda + p.K;
+      CONV || ROWMAP ? p.conv_bytes : (int64_t)(p.M - m0 - 1) * p.lda + p.K;
   const int64_t w_valid = (int64_t)(p.N - n0 - 1) * p.ldw + p.K;
   const v4i a_rsrc = make_rsrc(a_base, a_valid < kMaxRecords ? a_valid : kMaxRecords);
   const v4i w_rsrc = make_rsrc(w_base, w_valid < kMaxRecords ? w_valid : kMaxRecords);
@@ -178,7 +182,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
       a_w[i] = wo * p.sw_ - p.pad_l;
       a_pix[i] = m < p.M ? ((n_img * p.H + ho * p.sh - p.pad_t) * p.Wd + a_w[i]) * p.Ci : 0;
       a_off[i] = 0;
-    } else if (rowmap) {
+    } else if (ROWMAP) {
       // (rows past M read the last row again; their results are not stored)
       const int m = min(m0 + q * 8 + lr, p.M - 1);
       const int hw = p.Ho * p.Wo;
