@@ -683,6 +683,65 @@ def test_activation_table_equals_the_operator_chain(K):
     np.testing.assert_array_equal(table, want)
 
 
+def test_qgemm_library_choice_on_random_shapes(K):
+    """Seeded sweep over what decides the kernel of a GEMM -- rows from one to 16384, contraction
+    lengths and channel counts that are and are not multiples of the tiles, transposed operands,
+    zero points, every epilogue and bias kind: whatever the library picks gives the bytes
+    (the floats, to 1e-6 relative) of the generic kernel, which the tests above pin to the
+    oracle."""
+    rng = np.random.default_rng(20260702)
+    gen = K.variant_names().index("generic")
+    done = 0
+    for case in range(400):
+        r = rng.random()
+        if r < 0.5:
+            m = int(rng.integers(1, 300))
+            k = int(rng.choice([64, 128, 768, 1024, 3072, 4096, int(rng.integers(1, 3000))]))
+            n = int(rng.choice([16, 64, 768, 3072, 4096, int(rng.integers(1, 2000))]))
+        elif r < 0.92:
+            m = int(rng.integers(300, 5000))
+            k = int(rng.choice([128, 256, 768, 2304, int(rng.integers(1, 1500))]))
+            n = int(rng.choice([64, 256, 768, 1024, 3072, int(rng.integers(1, 1500))]))
+        else:
+            m, k, n = int(rng.choice([8192, 16384, 12000])), int(rng.choice([768, 512])), int(rng.choice([768, 3072, 1000]))
+        tp_b, tp_a = bool(rng.random() < 0.8), bool(rng.random() < 0.1)
+        a = dev(rng.integers(-128, 128, (k, m) if tp_a else (m, k), dtype=np.int8))
+        w = dev(rng.integers(-128, 128, (n, k) if tp_b else (k, n), dtype=np.int8))
+        epi = int(rng.choice([K.EPI_ACC_S32, K.EPI_REQUANT_CPU, K.EPI_REQUANT_CPU, K.EPI_REQUANT_GPU, K.EPI_REQUANT_GPU,
+                              K.EPI_DEQUANT_F32, K.EPI_REQUANT_CPU_DEQUANT_F32, K.EPI_REQUANT_GPU_DEQUANT_F32]))
+        kw = dict(tp_a=tp_a, tp_b=tp_b)
+        so = np.float32(0.02 * 0.025 * 74.0 * 74.0 * np.sqrt(k) / 40.0)
+        if epi != K.EPI_ACC_S32:
+            kw.update(sx=dev(np.array([0.02], np.float32)), so=dev(np.array([so])),
+                      sw=dev(rng.uniform(0.001, 0.05, n if rng.random() < 0.8 else 1).astype(np.float32)))
+        bk = int(rng.integers(0, 3))
+        cpu_kind = epi in (K.EPI_REQUANT_CPU, K.EPI_REQUANT_CPU_DEQUANT_F32)
+        gpu_kind = epi in (K.EPI_REQUANT_GPU, K.EPI_REQUANT_GPU_DEQUANT_F32)
+        if cpu_kind and bk == 1:
+            kw.update(bias=dev((rng.standard_normal(n) * 3 * so).astype(np.float32)))
+        if cpu_kind and bk == 2:
+            kw.update(bias=dev(rng.integers(-100000, 100000, n).astype(np.int32)))
+        if gpu_kind and bk == 1:
+            kw.update(bias=dev((rng.standard_normal(n) * 30).astype(np.float32)))
+        if gpu_kind and bk == 2:
+            kw.update(bias=dev(rng.integers(-128, 128, n, dtype=np.int8)))
+        if epi == K.EPI_DEQUANT_F32 and bk:
+            kw.update(bias=dev(rng.standard_normal(n).astype(np.float32)))
+        kw.update(zx=int(rng.integers(-5, 5)) if rng.random() < 0.15 else 0,
+                  zw=int(rng.integers(-5, 5)) if rng.random() < 0.1 else 0,
+                  zo=int(rng.integers(-10, 10)) if epi == K.EPI_REQUANT_CPU else 0)
+        got = K.qgemm(a, w, epi, **kw)
+        want = K.qgemm(a, w, epi, variant=gen, **kw)
+        tag = "case %d: %dx%dx%d, epilogue %d, bias kind %d, transposes %d %d, zero points %d %d %d" % (
+            case, m, k, n, epi, bk, tp_a, tp_b, kw["zx"], kw["zw"], kw["zo"])
+        if got.dtype == torch.float32:
+            assert torch.allclose(got, want, rtol=1e-6, atol=0), tag
+        else:
+            assert torch.equal(got, want), tag
+        done += 1
+    assert done == 400
+
+
 # ------------------------------------------------------------------------- conv
 CONVS = [  # nb, h, w, ci, co, k, stride, pad, dil
     (2, 30, 30, 3, 64, 7, 2, 3, 1),      # an RGB first layer: channels padded into scratch
