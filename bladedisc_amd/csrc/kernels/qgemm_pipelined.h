@@ -49,6 +49,8 @@
 #ifndef DQ8_QGEMM_PIPELINED_H_
 #define DQ8_QGEMM_PIPELINED_H_
 
+#include <type_traits>
+
 #include "qgemm_device.h"
 
 // Timeline hook for profiling builds: a harness may define DQ8_TRACE_POINT(i) before
@@ -350,8 +352,9 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
 #pragma unroll
   for (int j = 0; j < FN; ++j) load_frag_b(0, 0, 0, j);
 
-  for (int kt = 0; kt < KT; ++kt) {
-    const int cur = kt & 1, nxt = cur ^ 1;
+  // One k tile out of stage `cur` (an int, or a compile-time constant: see below).
+  auto k_tile = [&](auto cur_v, int kt) {
+    const int cur = cur_v, nxt = cur ^ 1;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       if (ks == 2) {
@@ -397,6 +400,21 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  };
+  // The small tiles are a few MFMAs per k tile and wave, and their time is the wave's
+  // instruction count: two k tiles per trip with the stage a constant turn the stage offsets of
+  // the LDS reads and of the loads into immediate operands (a third of the vector instructions
+  // of a 64 x 64 tile's k tile).
+  constexpr bool kTwoPerTrip = BM * BN <= 64 * 64;
+  if constexpr (kTwoPerTrip) {
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+      k_tile(std::integral_constant<int, 0>{}, kt);
+      k_tile(std::integral_constant<int, 1>{}, kt + 1);
+    }
+    if (kt < KT) k_tile(std::integral_constant<int, 0>{}, kt);
+  } else {
+    for (int kt = 0; kt < KT; ++kt) k_tile(kt & 1, kt);
   }
   // nothing of this wave may still be writing LDS when the workgroup retires
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
