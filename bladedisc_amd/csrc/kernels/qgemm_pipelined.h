@@ -405,7 +405,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
   // instruction count: two k tiles per trip with the stage a constant turn the stage offsets of
   // the LDS reads and of the loads into immediate operands (a third of the vector instructions
   // of a 64 x 64 tile's k tile).
-  constexpr bool kTwoPerTrip = BM * BN <= 64 * 64;
+  constexpr bool kTwoPerTrip = BM * BN <= 128 * 128;
   if constexpr (kTwoPerTrip) {
     int kt = 0;
     for (; kt + 1 < KT; kt += 2) {
