@@ -259,7 +259,9 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
                           (unsigned)wi < (unsigned)p.Wd;
           voff = ok ? a_pix[i] + t_off : kOutOfRange;
         } else {
-          voff = t_koff != kOutOfRange ? a_off[i] + t_koff : kOutOfRange;
+          // (t_koff out of range: 2^31 plus a row's offset, which the host keeps below 2^31, is
+          // past every descriptor as well -- no select)
+          voff = a_off[i] + t_koff;
         }
         buffer_load_lds_b128(a_rsrc, base + a_lds[i], voff);
       }
@@ -267,7 +269,7 @@ __global__ void __launch_bounds__(WM* WN* KSPLIT * 64) qgemm_pipe_kernel(const M
     for (int i = 0; i < B_LD; ++i)
       if (A_LD + i == idx)
         buffer_load_lds_b128(w_rsrc, base + b_lds[i],
-                             t_koff != kOutOfRange ? b_off[i] + t_koff : kOutOfRange);
+                             b_off[i] + t_koff);
   };
 
   // ---- fragment addressing.  Operand row R = R0 + lane%32 sits in block R/8 at row
